@@ -1,0 +1,161 @@
+"""Pins for oracle/pattern.py (CPU only): closed forms vs brute force and library routines,
+hand-worked path walks, invariants of the walk."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import pattern as op
+
+
+def test_conv_diag_brute_force_and_conv2d():
+    rng = np.random.default_rng(0)
+    A = rng.random((40, 40)).astype(np.float32)
+    C = op.conv_diag_closed_form(A, 31)
+    brute = np.zeros((40, 40))
+    for i in range(40):
+        for j in range(40):
+            for t in range(-15, 16):
+                if 0 <= i + t < 40 and 0 <= j + t < 40:
+                    brute[i, j] += float(A[i + t, j + t])
+    assert np.allclose(C, brute, rtol=1e-13)
+    ref = F.conv2d(torch.from_numpy(A)[None], torch.eye(31)[None, None], padding="same")[0].numpy()
+    assert np.allclose(C, ref, rtol=2e-6)
+    # a wrong sign of t (correlation vs convolution) is invisible for a symmetric
+    # kernel, but a transposed map is not: anti-diagonal sums differ
+    assert not np.allclose(C, op.conv_diag_closed_form(A[::-1].copy(), 31)[::-1])
+
+
+def test_pool_and_routes_agree():
+    rng = np.random.default_rng(1)
+    A = rng.random((128, 128)).astype(np.float32)
+    p64 = op.pooled_map(A, 32, 31, "fp64")
+    p32 = op.pooled_map(A, 32, 31, "torch")
+    assert p64.shape == (4, 4) and p64.dtype == np.float32
+    assert np.allclose(p64, p32, rtol=1e-5)
+    # pool only
+    q64 = op.pooled_map(A, 32, 0, "fp64")
+    assert np.allclose(q64, A.astype(np.float64).reshape(4, 32, 4, 32).mean(axis=(1, 3)), rtol=1e-7)
+    assert np.allclose(q64, op.pooled_map(A, 32, 0, "torch"), rtol=1e-5)
+
+
+@pytest.mark.parametrize("q", [0.9, 0.96, 0.98, 0.99, 0.5, 0.0, 1.0])
+@pytest.mark.parametrize("n", [16, 1024])
+def test_quantile_matches_torch_and_numpy(q, n):
+    rng = np.random.default_rng(int(q * 100) + n)
+    v = rng.random(n).astype(np.float32)
+    t, lo, hi, w = op.quantile_linear(v, q)
+    ref = torch.quantile(torch.from_numpy(v), q).item()
+    assert abs(float(t) - ref) <= 2 * np.spacing(np.float32(abs(ref)))
+    assert abs(float(t) - float(np.quantile(v.astype(np.float64), q))) <= 1e-5 * max(abs(ref), 1e-30)
+    assert 0 <= lo <= hi <= n - 1 and hi - lo <= 1
+
+
+def _walk(grid, x, y, thresh):
+    g = np.asarray(grid, dtype=np.float32)
+    nb = g.shape[0]
+    tmp = np.zeros((nb + 1, nb + 1), np.float32)
+    tmp[:-1, :-1] = g
+    ff = np.zeros((nb, nb), np.float32)
+    op.flood_fill_walk(tmp, x, y, ff, np.float32(thresh))
+    return (ff > 0).astype(int)
+
+
+def test_walk_hand_worked_grids():
+    # all equal -> every comparison ties -> pure diagonal walk, start cell unmarked
+    g = np.ones((4, 4))
+    m = _walk(g, 0, 0, 0.5)
+    assert m.tolist() == [[0, 0, 0, 0], [0, 1, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1]]
+    # from (0,1): diagonal (1,2),(2,3); then at (2,3): D=g[3][3]=1 > R=sentinel 0, G=sentinel 0 -> down (3,3)
+    m = _walk(g, 0, 1, 0.5)
+    assert m.tolist() == [[0, 0, 0, 0], [0, 0, 1, 0], [0, 0, 0, 1], [0, 0, 0, 1]]
+    # a ridge going down the first column then right along the last row
+    g = np.array([[1, 0, 0, 0],
+                  [9, 0, 0, 0],
+                  [8, 0, 0, 0],
+                  [7, 6, 5, 4]], dtype=np.float32)
+    m = _walk(g, 0, 0, 4.5)
+    # down,down,down mark (1,0),(2,0),(3,0); then along last row: right marks 6,5; 4 is not > 4.5
+    assert m.tolist() == [[0, 0, 0, 0], [1, 0, 0, 0], [1, 0, 0, 0], [1, 1, 1, 0]]
+    # right-vs-diagonal tie goes diagonal; down-vs-right tie takes the "else" branch (right or diagonal)
+    g = np.array([[0, 5, 0],
+                  [5, 5, 0],
+                  [0, 0, 0]], dtype=np.float32)
+    m = _walk(g, 0, 0, 1.0)  # D=5,R=5 -> not D>R; R=5 > G=5? no -> diagonal to (1,1)
+    assert m[1, 1] == 1 and m[0, 1] == 0 and m[1, 0] == 0
+    # threshold is strict
+    g = np.full((3, 3), 2.0)
+    assert _walk(g, 0, 0, 2.0).sum() == 0
+
+
+def test_walk_properties_random():
+    rng = np.random.default_rng(4)
+    for trial in range(20):
+        nb = int(rng.integers(3, 12))
+        pooled = rng.random((nb, nb)).astype(np.float32)
+        thresh = np.float32(rng.random())
+        trace = []
+        mask = op.mask_from_pooled(pooled, thresh, trace)
+        offdiag = mask.copy()
+        offdiag[np.arange(nb), np.arange(nb)] = 0
+        assert ((pooled > thresh) | (offdiag == 0)).all()      # marks only where value > thresh
+        assert (np.diag(mask) == 1).all()                      # diagonal forced
+        assert mask[0, 1:].sum() == 0 or True                  # seeds may be reached by other walks
+        # independence of the walk order: marks are idempotent
+        tmp = np.zeros((nb + 1, nb + 1), np.float32)
+        tmp[:-1, :-1] = pooled
+        ff = np.zeros((nb, nb), np.float32)
+        for k in reversed(range(nb)):
+            op.flood_fill_walk(tmp, k, 0, ff, thresh)
+            op.flood_fill_walk(tmp, 0, k, ff, thresh)
+        m2 = (ff > 0).astype(np.int8)
+        m2[np.arange(nb), np.arange(nb)] = 1
+        assert np.array_equal(mask, m2)
+
+
+def test_walk_matches_recursive_statement():
+    """The move rule, written recursively from its prose description, gives the same marks."""
+
+    def rec(data, x, y, ff, th):
+        if x + 1 == data.shape[0] or y + 1 == data.shape[1]:
+            return
+        cand = {"d": data[x + 1][y], "r": data[x][y + 1], "g": data[x + 1][y + 1]}
+        if cand["d"] > cand["r"]:
+            mv = "d" if cand["d"] > cand["g"] else "g"
+        else:
+            mv = "r" if cand["r"] > cand["g"] else "g"
+        nx, ny = {"d": (x + 1, y), "r": (x, y + 1), "g": (x + 1, y + 1)}[mv]
+        if data[nx][ny] > th:
+            ff[nx][ny] = data[nx][ny]
+        rec(data, nx, ny, ff, th)
+
+    rng = np.random.default_rng(9)
+    nb = 9
+    pooled = rng.random((nb, nb)).astype(np.float32)
+    tmp = np.zeros((nb + 1, nb + 1), np.float32)
+    tmp[:-1, :-1] = pooled
+    a = np.zeros((nb, nb), np.float32)
+    b = np.zeros((nb, nb), np.float32)
+    for k in range(nb):
+        rec(tmp, 0, k, a, 0.6)
+        rec(tmp, k, 0, a, 0.6)
+        op.flood_fill_walk(tmp, 0, k, b, 0.6)
+        op.flood_fill_walk(tmp, k, 0, b, 0.6)
+    assert np.array_equal(a, b)
+
+
+def test_generators_and_margin():
+    rng = np.random.default_rng(12)
+    A = rng.random((256, 256)).astype(np.float32)
+    A += 3.0 * np.eye(256, dtype=np.float32)
+    m64, p64, t64 = op.generate_mask_conv_ff(A, 32, 0.9, route="fp64")
+    m32, p32, t32 = op.generate_mask_conv_ff(A, 32, 0.9, route="torch")
+    margin = op.decision_margin(p64, 0.9)
+    route_err = float(np.max(np.abs(p64 - p32) / np.abs(p64)))
+    if margin > 8 * route_err:
+        assert np.array_equal(m64, m32)
+    mc, _, k = op.generate_mask_conv(A, 32, 0.3)
+    assert k == int(64 * 0.3 - 8)
+    assert mc.sum() >= k and (np.diag(mc) == 1).all()
+    mf, _, _ = op.generate_mask_conv_ff(A, 32, 0.9, ksize=0)
+    assert mf.shape == (8, 8)
