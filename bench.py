@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config4]
+
+A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
+layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
+already resident in HBM.  The default workload is the north-star configuration: B=32, H=2, L=4096,
+d=32, 32x32 blocks, diagonal band of 3 plus random blocks up to 10 % block density, fp32.
+
+Prints ONE JSON line.  ``value`` is the effective TFLOP/s of the step (algorithmic FLOPs
+12*n*d*NB divided by the step time); ``roofline`` describes the slowest kernel (its share of the
+algorithmic FLOPs over its own HIP-event time); ``cpu_baseline`` is the dense PyTorch statement of
+the same semantics (the oracle) timed on the host cores over a bounded sample of the batch.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def _event_ms(fn, iters, warm=3):
+    """Average duration of fn() in ms from HIP events on the current (= the library's) stream."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    end.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def build_workload(name):
+    from spion_amd import workloads
+    from spion_amd.csr import block_mask_to_csr_host
+
+    if name == "north_star":
+        B, H, L, d, bs = 32, 2, 4096, 32, 32
+        mat = workloads.north_star_mask(bs)
+        scale = 1.0
+    elif name == "config1":
+        B, H, L, d, bs = 8, 2, 1024, 32, 32
+        mat = workloads.config1_mask()
+        scale = 1.0 / np.sqrt(32.0)
+    elif name == "config4":
+        B, H, L, d, bs = 32, 2, 4096, 32, 1
+        mat = None
+        scale = 1.0
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    wl = dict(name=name, B=B, H=H, L=L, d=d, bs=bs, mat=mat, scale=scale)
+    if mat is not None:
+        sm, off, col = block_mask_to_csr_host(mat, bs)
+        wl["block_density"] = float(mat.mean())
+    else:
+        sm, off, col = workloads.window_random_csr(L, 64, 205, seed=3)
+        wl["block_density"] = None
+    wl.update(sum_mat=sm, offsets=off, columns=col, nnz=int(off[-1]))
+    return wl
+
+
+def cpu_baseline(wl, budget_s=20.0):
+    """The oracle's dense PyTorch statement (forward + autograd backward) on the host cores, on as many
+    whole samples of the batch as fit in the time budget."""
+    from oracle import sparse_attention as osa
+    from spion_amd import workloads
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    H, L, d = wl["H"], wl["L"], wl["d"]
+    rows = osa.csr_row_index(wl["offsets"])
+    pat = torch.zeros(L, L)
+    pat[torch.from_numpy(rows), torch.from_numpy(wl["columns"].astype(np.int64))] = 1.0
+    key_mask = workloads.valid_length_mask(1, L, L // 2, L, seed=5) if wl["name"] == "config4" else None
+    q, k, v, do = workloads.qkv(1, H, L, d, scale=wl["scale"], seed=0)
+    for t in (q, k, v):
+        t.requires_grad_()
+
+    def one():
+        for t in (q, k, v):
+            t.grad = None
+        o, _ = osa.dense_masked_attention(q, k, v, pat, key_mask)
+        o.backward(do)
+
+    one()  # warm-up
+    t0 = time.perf_counter()
+    n = 0
+    while True:
+        one()
+        n += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or n >= wl["B"]:
+            break
+    flops = 12.0 * wl["nnz"] * d * H * n
+    return dict(value=flops / el / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                ms_per_sample=1e3 * el / n,
+                sample=f"{n} of {wl['B']} samples (H={H}, L={L}, d={d}) of the same workload, dense masked "
+                       f"softmax attention forward+autograd backward in PyTorch fp32; effective rate on the "
+                       f"algorithmic 12*n*d FLOPs (dense FLOPs actually executed: {12.0 * L * L * d * H * n:.3e})")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="north_star")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU; there is no CPU fallback")
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda:0")
+
+    import spion_amd
+    from spion_amd import _lib, workloads
+    from spion_amd.attention import Attention
+
+    wl = build_workload(args.workload)
+    B, H, L, d, bs, nnz = wl["B"], wl["H"], wl["L"], wl["d"], wl["bs"], wl["nnz"]
+    NB = B * H
+    q, k, v, do = workloads.qkv(B, H, L, d, scale=wl["scale"], seed=0, device=dev)
+    for t in (q, k, v):
+        t.requires_grad_()
+    with_mask = wl["name"] == "config4"
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    if with_mask:
+        cpp = Attention._blockcuda_mask_compile_module()
+        mod_cls = spion_amd.CUDABlockMaskAttention
+        key_mask = workloads.valid_length_mask(B, L, L // 2, L, seed=5).to(dev)
+        pattern = torch.zeros(L, L)
+        rows = np.repeat(np.arange(L), wl["sum_mat"])
+        pattern[torch.from_numpy(rows), torch.from_numpy(wl["columns"].astype(np.int64))] = 1.0
+        mat = pattern.to(dev)
+    else:
+        cpp = Attention._blockcuda_compile_module()
+        mod_cls = spion_amd.CUDABlockAttention
+        key_mask = torch.ones(B, L, device=dev)
+        mat = torch.from_numpy(wl["mat"]).to(dev)
+    handle = cpp.init(d, L, NB, bs)
+    _lib.check_error("init")
+    module = mod_cls(cfg, cpp, handle)
+
+    def step():
+        for t in (q, k, v):
+            t.grad = None
+        out, _ = module(q, k, v, key_mask, mat)
+        out.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    path = _lib.core().spion_last_path(handle)
+
+    # ---- per-kernel times at the C ABI, HIP events on the library's stream -----------------------
+    core = _lib.core()
+    idx = module.csr_cache.get(mat, bs)
+    Q = q.detach().reshape(NB, L, d).contiguous()
+    K = k.detach().reshape(NB, L, d).contiguous()
+    V = v.detach().reshape(NB, L, d).contiguous()
+    dO = do.reshape(NB, L, d).contiguous()
+    Kt = K.transpose(1, 2).contiguous()
+    Vt = V.transpose(1, 2).contiguous()
+    P = torch.empty(NB * nnz, device=dev)
+    O = torch.empty_like(Q)
+    dP = torch.empty(NB * nnz, device=dev)
+    dS = torch.empty(NB * nnz, device=dev)
+    dQ, dK, dV = torch.empty_like(Q), torch.empty_like(Q), torch.empty_like(Q)
+    pen = (1e6 * (1.0 - key_mask.repeat(1, H))).contiguous() if with_mask else None
+
+    def fwd():
+        a = [handle, Q.data_ptr(), Kt.data_ptr(), V.data_ptr()] + ([pen.data_ptr()] if with_mask else [])
+        cpp.attn_forward(*a, P.data_ptr(), O.data_ptr(), idx.offsets.data_ptr(), idx.columns.data_ptr(),
+                         idx.sum_mat.data_ptr(), nnz)
+
+    def bwd():
+        cpp.attn_backward(handle, Q.data_ptr(), K.data_ptr(), Vt.data_ptr(), P.data_ptr(), dO.data_ptr(),
+                          dP.data_ptr(), dS.data_ptr(), dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
+                          idx.offsets.data_ptr(), idx.columns.data_ptr(), idx.sum_mat.data_ptr(), nnz)
+
+    it = max(10, args.steps)
+    t_fwd = _event_ms(fwd, it)
+    t_bwd = _event_ms(bwd, it)
+    core.spion_set_backward_passes(handle, 1)
+    t_row = _event_ms(bwd, it)
+    core.spion_set_backward_passes(handle, 2)
+    t_col = _event_ms(bwd, it)
+    core.spion_set_backward_passes(handle, 3)
+    _lib.check_error("bench kernels")
+
+    alg_flops = workloads.sparse_flops(nnz, d, NB)
+    alg_bytes = workloads.sparse_bytes(nnz, L, d, NB)
+    third = alg_flops / 3.0  # forward, row pass and column pass carry 4*n*d*NB each
+    names = {1: ("tile_fwd_kernel", "tile_bwd_row_kernel", "tile_bwd_col_kernel"),
+             2: ("elem_fwd_kernel", "elem_bwd_row_kernel", "elem_bwd_col_kernel")}[path]
+    kernels = dict(zip(names, (t_fwd, t_row, t_col)))
+    dom = max(kernels, key=kernels.get)
+    dom_ms = kernels[dom]
+    if path == 1:
+        roof = dict(bound="mfma", kernel=dom, achieved=third / dom_ms / 1e9, peak=PEAK_FP32_MFMA_TFLOPS,
+                    unit="TFLOP/s", traffic=None)
+    else:
+        # element path: HBM-bound by design; the slowest kernel's share of the algorithmic bytes
+        share = {names[0]: 4.0 * (4 * L * d + nnz) * NB, names[1]: 4.0 * (4 * L * d + nnz) * NB,
+                 names[2]: 4.0 * (3 * L * d) * NB}[dom]
+        roof = dict(bound="hbm", kernel=dom, achieved=share / dom_ms / 1e6, peak=PEAK_HBM_GBS, unit="GB/s",
+                    traffic=None)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
+
+    result = {
+        "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
+        "value": alg_flops / ms_step / 1e9,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded N(0,1) tensors, seeded block mask)",
+        "config": {"workload": f"{wl['name']}: sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, "
+                               f"block {bs}, nnz/head={nnz}, block density="
+                               f"{wl['block_density'] if wl['block_density'] is None else round(wl['block_density'], 4)}",
+                   "kernel_path": {1: "mfma-tile", 2: "element"}[path]},
+        "abi_ms": {"attn_forward": round(t_fwd, 4), "attn_backward": round(t_bwd, 4),
+                   "fwd_plus_bwd": round(t_fwd + t_bwd, 4)},
+        "abi_effective_tflops": alg_flops / (t_fwd + t_bwd) / 1e9,
+        "abi_fraction_of_fp32_mfma_peak": alg_flops / (t_fwd + t_bwd) / 1e9 / PEAK_FP32_MFMA_TFLOPS,
+        "abi_effective_hbm_gbs": alg_bytes / (t_fwd + t_bwd) / 1e6,
+        "algorithmic": {"gflop": alg_flops / 1e9, "mbytes": alg_bytes / 1e6},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,168 @@
+/*
+ * spion_hip.h -- C ABI of libspion_hip.so: SPION layer-wise sparse attention for AMD MI355X (gfx950).
+ *
+ * Every pointer argument is a DEVICE pointer unless a comment says "host".  float = IEEE fp32,
+ * int = int32.  The caller owns every buffer it passes (inputs, outputs and the dP / dS scratch
+ * arrays); the library owns only the handle and the private workspace hanging off it.  All work is
+ * enqueued on the handle's stream (the HIP null stream unless spion_set_stream was called), which is
+ * the stream PyTorch-ROCm uses by default, so results are ordered with the surrounding torch ops and
+ * no call synchronises the host in steady state.  The first call that sees a new (Offsets, Columns,
+ * nnz) triple copies the index to the host once to analyse it (tile detection, transposed index).
+ *
+ * The four entry points of each family have the signatures the reference's ctypes declarations bind
+ * (reference: models/attention.py:141-191); the drop-in libraries attn.so, attn_mask.so,
+ * block_attn.so and block_attn_mask.so re-export them under the reference's un-prefixed names
+ * init / attn_forward / attn_backward / destroy.
+ *
+ * Like the reference, the attention entry points return void.  Failures (bad handle, inconsistent
+ * CSR, HIP errors) are recorded and can be read with spion_last_error(); after a failure the call
+ * launches nothing.
+ */
+#ifndef SPION_HIP_H
+#define SPION_HIP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------------------------------
+ * Sparse attention on an element-level CSR pattern, no key mask.
+ * Replaces models/block_attn.cu:547-568 (init / attn_forward / attn_backward / destroy).
+ *
+ *   NB = num_batches = batch * heads,  L = seq_len,  d = emb_dim,  n = nnz per (batch, head).
+ *   Offsets[L+1]  exclusive prefix sum of per-row counts, shared by all NB problems.
+ *   Columns[>=n]  sorted column indices per row; only the first n entries are read (the reference
+ *                 passes NB identical copies, models/attention_blockcuda.py:43).
+ *   SumMat[L]     per-row counts (= Offsets[i+1]-Offsets[i]); accepted for compatibility, not read.
+ *   Attn[NB*n]    out: probabilities P in CSR order, problem stride n.
+ *
+ * Semantics (models/block_attn.cu:33-88): off-pattern logits count as 0 in the softmax denominator:
+ *   v = (q_i . k_j)/sqrt(d);  m = max(-100, max_j v);  Z = sum_j exp(v-m) + (L-n_i) exp(-m);  P = exp(v-m)/Z.
+ * ---------------------------------------------------------------------------------------------- */
+void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size);
+
+/* Q [NB][L][d], Kt [NB][d][L] (K transposed), V [NB][L][d]; out: Attn [NB*n], Out [NB][L][d].
+ * Reference: models/block_attn.cu:552-556. */
+void spion_block_attn_forward(void* handle, const float* Q, const float* Kt, const float* V,
+                              float* Attn, float* Out,
+                              const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+/* Q, K [NB][L][d], Vt [NB][d][L] (V transposed), P = Attn of the forward, dO [NB][L][d];
+ * dP, dS: caller-owned scratch of NB*n floats each, contents unspecified on return;
+ * out: dQ, dK, dV [NB][L][d] (need not be zeroed).  Reference: models/block_attn.cu:558-563. */
+void spion_block_attn_backward(void* handle, const float* Q, const float* K, const float* Vt,
+                               const float* P, const float* dO, float* dP, float* dS,
+                               float* dQ, float* dK, float* dV,
+                               const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+void spion_block_destroy(void* handle);
+
+/* ------------------------------------------------------------------------------------------------
+ * Sparse attention on an element-level CSR pattern with an additive key-padding penalty.
+ * Replaces models/block_attn_mask.cu:655-674.
+ *   Mask[NB*L]: 0 for valid keys, 1e6 for padded keys, index (b*H+h)*L + key
+ *   (models/attention_blockcuda_mask.py:42-43).
+ *   v = (q_i . k_j)/sqrt(d) - Mask[bh*L + j];  m = max(0, max_j v)  (models/block_attn_mask.cu:88-140).
+ * ---------------------------------------------------------------------------------------------- */
+void* spion_blockmask_init(int emb_dim, int seq_len, int num_batches, int block_size);
+
+void spion_blockmask_attn_forward(void* handle, const float* Q, const float* Kt, const float* V,
+                                  const float* Mask, float* Attn, float* Out,
+                                  const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+void spion_blockmask_attn_backward(void* handle, const float* Q, const float* K, const float* Vt,
+                                   const float* P, const float* dO, float* dP, float* dS,
+                                   float* dQ, float* dK, float* dV,
+                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+void spion_blockmask_destroy(void* handle);
+
+/* ------------------------------------------------------------------------------------------------
+ * Dense-phase attention (produces the full probability map that feeds pattern discovery).
+ * Replaces models/attn.cu:265-280.  Operands follow the reference's column-major convention:
+ *   forward : Qt [NB][d][L], K [NB][L][d], Vt [NB][d][L];
+ *             out Attn [NB][L(key)][L(query)] (Attn[h][j][i] = P[i][j]), Out [NB][d][L].
+ *   backward: Qt, Kt [NB][d][L], V [NB][L][d], P = Attn, dOt [NB][d][L];
+ *             dP, dScale, dS: caller scratch [NB][L][L] (dScale is never touched);
+ *             out dQ, dK, dV as [NB][d][L].
+ *   v = (q_i . k_j)/sqrt(d);  m = max(-10, max_j v);  P = softmax_j  (models/attn.cu:9-36).
+ * ---------------------------------------------------------------------------------------------- */
+void* spion_dense_init(int emb_dim, int seq_len, int num_batches);
+
+void spion_dense_attn_forward(void* handle, const float* Qt, const float* K, const float* Vt,
+                              float* Attn, float* Out);
+
+void spion_dense_attn_backward(void* handle, const float* Qt, const float* Kt, const float* V,
+                               const float* P, const float* dOt, float* dP, float* dScale, float* dS,
+                               float* dQ, float* dK, float* dV);
+
+void spion_dense_destroy(void* handle);
+
+/* Dense-phase attention with the key-padding penalty Mask[NB*L] subtracted from the logits.
+ * Replaces models/attn_mask.cu:280-298. */
+void* spion_densemask_init(int emb_dim, int seq_len, int num_batches);
+
+void spion_densemask_attn_forward(void* handle, const float* Qt, const float* K, const float* Vt,
+                                  const float* Mask, float* Attn, float* Out);
+
+void spion_densemask_attn_backward(void* handle, const float* Qt, const float* Kt, const float* V,
+                                   const float* P, const float* dOt, float* dP, float* dScale, float* dS,
+                                   float* dQ, float* dK, float* dV);
+
+void spion_densemask_destroy(void* handle);
+
+/* ------------------------------------------------------------------------------------------------
+ * Pattern discovery on the device.  The reference does this in Python on the host CPU
+ * (main_conv_ff.py:254-278, main_conv.py:236-256, main_ff.py:253-272); there is no reference FFI.
+ *
+ *   Score  [n_maps][L][L]  head/batch-averaged probability maps (one per layer).
+ *   Mat    [n_maps][nb][nb] out: 0.0 / 1.0 block masks, nb = L / block_size.
+ *   Pooled [n_maps][nb][nb] out, optional (may be NULL): pooled filtered map, fp32.
+ *   Thresh [n_maps]         out, optional (may be NULL): the quantile threshold used.
+ *   conv_ksize : odd size of the diagonal (identity) filter, 31 in the reference; 0 = no filter.
+ *   mode       : SPION_PATTERN_FLOOD  -> param = quantile q in [0,1], greedy path walk from the
+ *                                        top row and left column, then the diagonal is set;
+ *                SPION_PATTERN_TOPK   -> param = density; the int(nb*nb*density - nb) largest
+ *                                        pooled blocks (ties: lower index first), then the diagonal.
+ *   stream     : a hipStream_t, or NULL for the null stream.
+ * Filter and pooling accumulate in fp64 and round once to fp32.  Returns 0 on success.
+ * ---------------------------------------------------------------------------------------------- */
+#define SPION_PATTERN_FLOOD 0
+#define SPION_PATTERN_TOPK 1
+
+int spion_pattern_generate(const float* Score, int n_maps, int seq_len, int block_size,
+                           int conv_ksize, int mode, double param,
+                           float* Mat, float* Pooled, float* Thresh, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Additions with no counterpart in the reference (which reports no errors at all).
+ * ---------------------------------------------------------------------------------------------- */
+
+/* Message of the most recent failure in this process, or "" if none since spion_clear_error(). */
+const char* spion_last_error(void);
+void spion_clear_error(void);
+
+/* Launch this handle's work on `stream` (a hipStream_t; NULL = null stream).  Any family. */
+void spion_set_stream(void* handle, void* stream);
+
+/* Forget the analysed pattern of a sparse handle.  The analysis is cached under the key
+ * (Offsets pointer, Columns pointer, nnz); call this if index arrays were rewritten in place. */
+void spion_invalidate_pattern(void* handle);
+
+/* Which kernel family the last forward/backward of a sparse handle used:
+ * 0 = none yet, 1 = MFMA 32x32 tile path, 2 = element (gather) path. */
+int spion_last_path(void* handle);
+
+/* Force the element path even for tile-structured patterns (testing / comparison). */
+void spion_force_element_path(void* handle, int on);
+
+/* Profiling aid: run only part of a sparse handle's backward.  bit 0 = row pass (row sums and dQ),
+ * bit 1 = column pass (dK, dV; needs the row sums of an earlier row pass).  Default 3 = both. */
+void spion_set_backward_passes(void* handle, int mask);
+
+const char* spion_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPION_HIP_H */

@@ -1,0 +1,118 @@
+"""ctypes loaders for the built HIP libraries (spion_amd/lib/*.so).
+
+``libspion_hip.so`` carries the prefixed C ABI of include/spion_hip.h; ``attn.so``,
+``attn_mask.so``, ``block_attn.so`` and ``block_attn_mask.so`` re-export one family each under the
+un-prefixed names the reference binds (models/attention.py:141-191).  Loading fails loudly when a
+library has not been built: there is no fallback path.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_double, c_int, c_void_p
+
+import torch  # noqa: F401  (first: the HIP runtime PyTorch ships must be the one in the process)
+
+LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+
+_P = c_void_p
+_cache: dict = {}
+
+
+class SpionLibraryError(RuntimeError):
+    pass
+
+
+def lib_path(name: str) -> str:
+    return os.path.join(LIB_DIR, name)
+
+
+def _cdll(name: str) -> ctypes.CDLL:
+    if name in _cache:
+        return _cache[name]
+    path = lib_path(name)
+    if not os.path.exists(path):
+        raise SpionLibraryError(
+            f"{path} is missing: build the HIP libraries first (python -m spion_amd.build). "
+            "spion_amd has no CPU fallback."
+        )
+    lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+    _cache[name] = lib
+    return lib
+
+
+def core() -> ctypes.CDLL:
+    """libspion_hip.so with argtypes of the entry points that have no reference counterpart."""
+    lib = _cdll("libspion_hip.so")
+    if getattr(lib, "_spion_typed", False):
+        return lib
+    lib.spion_last_error.restype = c_char_p
+    lib.spion_last_error.argtypes = []
+    lib.spion_clear_error.argtypes = []
+    lib.spion_clear_error.restype = None
+    lib.spion_set_stream.argtypes = [_P, _P]
+    lib.spion_set_stream.restype = None
+    lib.spion_invalidate_pattern.argtypes = [_P]
+    lib.spion_invalidate_pattern.restype = None
+    lib.spion_last_path.argtypes = [_P]
+    lib.spion_last_path.restype = c_int
+    lib.spion_force_element_path.argtypes = [_P, c_int]
+    lib.spion_force_element_path.restype = None
+    lib.spion_set_backward_passes.argtypes = [_P, c_int]
+    lib.spion_set_backward_passes.restype = None
+    lib.spion_version.restype = c_char_p
+    lib.spion_version.argtypes = []
+    lib.spion_pattern_generate.argtypes = [_P, c_int, c_int, c_int, c_int, c_int, c_double, _P, _P, _P, _P]
+    lib.spion_pattern_generate.restype = c_int
+    for fam, extra in (("block", 0), ("blockmask", 1)):
+        getattr(lib, f"spion_{fam}_init").argtypes = [c_int, c_int, c_int, c_int]
+        getattr(lib, f"spion_{fam}_init").restype = _P
+        getattr(lib, f"spion_{fam}_attn_forward").argtypes = [_P] * (9 + extra) + [c_int]
+        getattr(lib, f"spion_{fam}_attn_forward").restype = None
+        getattr(lib, f"spion_{fam}_attn_backward").argtypes = [_P] * 14 + [c_int]
+        getattr(lib, f"spion_{fam}_attn_backward").restype = None
+        getattr(lib, f"spion_{fam}_destroy").argtypes = [_P]
+        getattr(lib, f"spion_{fam}_destroy").restype = None
+    for fam, extra in (("dense", 0), ("densemask", 1)):
+        getattr(lib, f"spion_{fam}_init").argtypes = [c_int, c_int, c_int]
+        getattr(lib, f"spion_{fam}_init").restype = _P
+        getattr(lib, f"spion_{fam}_attn_forward").argtypes = [_P] * (6 + extra)
+        getattr(lib, f"spion_{fam}_attn_forward").restype = None
+        getattr(lib, f"spion_{fam}_attn_backward").argtypes = [_P] * 12
+        getattr(lib, f"spion_{fam}_attn_backward").restype = None
+        getattr(lib, f"spion_{fam}_destroy").argtypes = [_P]
+        getattr(lib, f"spion_{fam}_destroy").restype = None
+    lib._spion_typed = True
+    return lib
+
+
+def check_error(where: str = "") -> None:
+    """Raise if the library recorded a failure since the last check (the C entry points return void)."""
+    lib = core()
+    msg = lib.spion_last_error()
+    if msg:
+        text = msg.decode("utf-8", "replace")
+        lib.spion_clear_error()
+        raise SpionLibraryError(f"{where}: {text}" if where else text)
+
+
+def load_dropin(name: str, n_init: int, n_fwd: int, n_bwd: int, trailing_int: bool) -> ctypes.CDLL:
+    """Load one drop-in library and declare the ABI exactly as the reference's loaders do
+    (models/attention.py:141-191): ``init`` takes ``n_init`` ints and returns an opaque pointer,
+    ``attn_forward`` / ``attn_backward`` take ``n_fwd`` / ``n_bwd`` pointers (plus ``nnz`` for the
+    block libraries), ``destroy`` takes the handle."""
+    core()  # the drop-ins depend on libspion_hip.so; load it (and fail) first
+    lib = _cdll(name)
+    if getattr(lib, "_spion_typed", False):
+        return lib
+    tail = [c_int] if trailing_int else []
+    lib.init.argtypes = [c_int] * n_init
+    lib.init.restype = _P
+    lib.attn_forward.argtypes = [_P] * n_fwd + tail
+    lib.attn_forward.restype = None
+    lib.attn_backward.argtypes = [_P] * n_bwd + tail
+    lib.attn_backward.restype = None
+    lib.destroy.argtypes = [_P]
+    lib.destroy.restype = None
+    lib._spion_typed = True
+    return lib

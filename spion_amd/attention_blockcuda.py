@@ -1,0 +1,104 @@
+"""``CUDABlockAttention``: sparse attention on a block mask, no key mask.
+
+Drop-in for the reference module of the same name (models/attention_blockcuda.py): same constructor
+``(config, attn_cpp, attn_handle)``, same ``forward(query, key, value, mask, mat)`` returning
+``(out [B,H,L,d], P_flat [B*H*nnz])`` and the same autograd contract (gradients for query, key and value
+only; the gradient of the returned probabilities is ignored, models/attention_blockcuda.py:73-112).
+``attn_cpp`` is the ctypes library exporting init / attn_forward / attn_backward
+(models/block_attn.cu:547-568), ``attn_handle`` the pointer its ``init`` returned.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .csr import CsrCache
+
+
+class _BlockAttnFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, query, key, value, mask, mat, module):
+        m = module
+        idx = m.csr_cache.get(mat, m.block_size)
+        nb_, L, d = m.num_batches, m.seq_len, m.emb_dim
+        if tuple(query.shape) != (m.batch_size, m.num_heads, L, d):
+            raise ValueError(
+                f"query shape {tuple(query.shape)} does not match the handle "
+                f"({m.batch_size}, {m.num_heads}, {L}, {d})"
+            )
+        dev = query.device
+        q = query.contiguous()
+        kt = key.permute(0, 1, 3, 2).contiguous()  # the ABI takes K transposed in the forward
+        v = value.contiguous()
+        p_flat = torch.empty(nb_ * idx.nnz, dtype=torch.float32, device=dev)
+        out = torch.empty((m.batch_size, m.num_heads, L, d), dtype=torch.float32, device=dev)
+        if m.with_mask:
+            pen = (1e6 * (1.0 - mask.repeat(1, m.num_heads))).to(torch.float32).contiguous()  # [B, H*L]
+            m.attn_cpp.attn_forward(m.attn_handle, q.data_ptr(), kt.data_ptr(), v.data_ptr(), pen.data_ptr(),
+                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
+                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
+        else:
+            m.attn_cpp.attn_forward(m.attn_handle, q.data_ptr(), kt.data_ptr(), v.data_ptr(),
+                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
+                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
+        _lib.check_error("attn_forward")
+        ctx.save_for_backward(q, key, value, p_flat, idx.offsets, idx.columns, idx.sum_mat)
+        ctx.module = m
+        ctx.nnz = idx.nnz
+        if m.with_mask:
+            ctx.mark_non_differentiable(p_flat)
+            return out, p_flat
+        return out, p_flat
+
+    @staticmethod
+    def backward(ctx, grad_output, grad_weight):
+        m = ctx.module
+        q, key, value, p_flat, offsets, columns, sum_mat = ctx.saved_tensors
+        dev = q.device
+        n_total = m.num_batches * ctx.nnz
+        k = key.contiguous()
+        vt = value.permute(0, 1, 3, 2).contiguous()  # the ABI takes V transposed in the backward
+        go = grad_output.contiguous()
+        scratch_dp = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
+        scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
+        shape = (m.batch_size, m.num_heads, m.seq_len, m.emb_dim)
+        dq = torch.empty(shape, dtype=torch.float32, device=dev)
+        dk = torch.empty(shape, dtype=torch.float32, device=dev)
+        dv = torch.empty(shape, dtype=torch.float32, device=dev)
+        m.attn_cpp.attn_backward(m.attn_handle, q.data_ptr(), k.data_ptr(), vt.data_ptr(), p_flat.data_ptr(),
+                                 go.data_ptr(), scratch_dp.data_ptr(), scratch_ds.data_ptr(), dq.data_ptr(),
+                                 dk.data_ptr(), dv.data_ptr(), offsets.data_ptr(), columns.data_ptr(),
+                                 sum_mat.data_ptr(), ctx.nnz)
+        _lib.check_error("attn_backward")
+        return dq, dk, dv, None, None, None
+
+
+class _BlockAttentionBase(nn.Module):
+    with_mask = False
+
+    def __init__(self, config, attn_cpp, attn_handle):
+        super().__init__()
+        if attn_cpp is None or not attn_handle:
+            raise _lib.SpionLibraryError(
+                f"{type(self).__name__} needs the loaded HIP library and a handle from its init(); "
+                "there is no fallback implementation"
+            )
+        self.emb_dim = config["head_dim"]
+        self.num_heads = config["num_head"]
+        self.seq_len = config["max_seq_len"]
+        self.batch_size = config["batch_size"]
+        self.block_size = config["block_size"]
+        self.num_batches = self.batch_size * self.num_heads
+        self.num_blocks = int(self.seq_len / self.block_size)
+        self.attn_cpp = attn_cpp
+        self.attn_handle = attn_handle
+        self.csr_cache = CsrCache()
+        self.attn_func = _BlockAttnFunction
+
+
+class CUDABlockAttention(_BlockAttentionBase):
+    with_mask = False
+
+    def forward(self, query, key, value, mask, mat):
+        return self.attn_func.apply(query, key, value, mask, mat, self)

@@ -1,0 +1,65 @@
+"""Build libspion_hip.so and the four drop-in libraries for gfx950, in-tree under spion_amd/lib/.
+
+    python -m spion_amd.build
+
+hipcc cross-compiles without a GPU.  Object files go to spion_amd/lib/obj/.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+OBJ = os.path.join(LIB, "obj")
+
+HIP_SOURCES = ["capi.hip", "sparse_attn.hip", "dense_attn.hip", "pattern.hip"]
+DROPINS = {1: "attn.so", 2: "attn_mask.so", 3: "block_attn.so", 4: "block_attn_mask.so"}
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+HIP_FLAGS = [
+    "-O3", "-std=c++17", "--offload-arch=gfx950", "-fPIC",
+    # packed-fp32 instruction selection is switched off on purpose for this hardware pool
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd, verbose):
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "is not a recognized feature" not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"command failed ({r.returncode}): {' '.join(cmd)}\n{out}")
+    if verbose and out.strip():
+        print(out, flush=True)
+
+
+def build_all(verbose: bool = False, jobs: int = 4) -> str:
+    os.makedirs(OBJ, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(OBJ, src.replace(".hip", ".o"))
+        _run([HIPCC, *HIP_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj], verbose)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(compile_one, HIP_SOURCES))
+    main_lib = os.path.join(LIB, "libspion_hip.so")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", main_lib, *objs,
+          "-Wl,-soname,libspion_hip.so"], verbose)
+    for k, name in DROPINS.items():
+        _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", f"-DSPION_DROPIN={k}",
+              os.path.join(CSRC, "dropin.cpp"), "-o", os.path.join(LIB, name),
+              f"-L{LIB}", "-lspion_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed", "-Wl,-z,defs"], verbose)
+    return main_lib
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", sorted(f for f in os.listdir(LIB) if f.endswith(".so")))
+    sys.exit(0)

@@ -1,0 +1,149 @@
+// extern "C" surface of libspion_hip.so (declared in include/spion_hip.h) and the error slot.
+#include "common.h"
+#include "../../include/spion_hip.h"
+
+namespace spion {
+
+static std::mutex g_err_mutex;
+static std::string g_err;
+
+void set_error(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    g_err = buf;
+}
+bool error_pending() {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    return !g_err.empty();
+}
+
+// implemented in sparse_attn.hip / dense_attn.hip / pattern.hip
+void* sparse_init(int, int, int, int, bool);
+void sparse_destroy(void*);
+void sparse_forward(void*, const float*, const float*, const float*, const float*, float*, float*, const int*,
+                    const int*, int, bool);
+void sparse_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
+                     float*, float*, float*, const int*, const int*, int);
+void sparse_invalidate(void*);
+int sparse_last_path(void*);
+void sparse_force_element(void*, int);
+void sparse_set_bwd_passes(void*, int);
+void* dense_init(int, int, int, bool);
+void dense_destroy(void*);
+void dense_forward(void*, const float*, const float*, const float*, const float*, float*, float*, bool);
+void dense_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
+                    float*);
+int pattern_generate(const float*, int, int, int, int, int, double, float*, float*, float*, hipStream_t);
+
+}  // namespace spion
+
+using namespace spion;
+
+extern "C" {
+
+// ---- sparse, no key mask -----------------------------------------------------------------------
+void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    return sparse_init(emb_dim, seq_len, num_batches, block_size, false);
+}
+void spion_block_attn_forward(void* h, const float* Q, const float* Kt, const float* V, float* Attn, float* Out,
+                              const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_forward(h, Q, Kt, V, nullptr, Attn, Out, Offsets, Columns, nnz, false);
+}
+void spion_block_attn_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P,
+                               const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
+                               const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz);
+}
+void spion_block_destroy(void* h) { sparse_destroy(h); }
+
+// ---- sparse, key mask --------------------------------------------------------------------------
+void* spion_blockmask_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    return sparse_init(emb_dim, seq_len, num_batches, block_size, true);
+}
+void spion_blockmask_attn_forward(void* h, const float* Q, const float* Kt, const float* V, const float* Mask,
+                                  float* Attn, float* Out, const int* Offsets, const int* Columns,
+                                  const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_forward(h, Q, Kt, V, Mask, Attn, Out, Offsets, Columns, nnz, true);
+}
+void spion_blockmask_attn_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P,
+                                   const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
+                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz);
+}
+void spion_blockmask_destroy(void* h) { sparse_destroy(h); }
+
+// ---- dense phase ---------------------------------------------------------------------------------
+void* spion_dense_init(int emb_dim, int seq_len, int num_batches) {
+    return dense_init(emb_dim, seq_len, num_batches, false);
+}
+void spion_dense_attn_forward(void* h, const float* Qt, const float* K, const float* Vt, float* Attn, float* Out) {
+    dense_forward(h, Qt, K, Vt, nullptr, Attn, Out, false);
+}
+void spion_dense_attn_backward(void* h, const float* Qt, const float* Kt, const float* V, const float* P,
+                               const float* dOt, float* dP, float* dScale, float* dS, float* dQ, float* dK,
+                               float* dV) {
+    (void)dP;
+    (void)dScale;
+    (void)dS;
+    dense_backward(h, Qt, Kt, V, P, dOt, dQ, dK, dV);
+}
+void spion_dense_destroy(void* h) { dense_destroy(h); }
+
+void* spion_densemask_init(int emb_dim, int seq_len, int num_batches) {
+    return dense_init(emb_dim, seq_len, num_batches, true);
+}
+void spion_densemask_attn_forward(void* h, const float* Qt, const float* K, const float* Vt, const float* Mask,
+                                  float* Attn, float* Out) {
+    dense_forward(h, Qt, K, Vt, Mask, Attn, Out, true);
+}
+void spion_densemask_attn_backward(void* h, const float* Qt, const float* Kt, const float* V, const float* P,
+                                   const float* dOt, float* dP, float* dScale, float* dS, float* dQ, float* dK,
+                                   float* dV) {
+    (void)dP;
+    (void)dScale;
+    (void)dS;
+    dense_backward(h, Qt, Kt, V, P, dOt, dQ, dK, dV);
+}
+void spion_densemask_destroy(void* h) { dense_destroy(h); }
+
+// ---- pattern discovery ---------------------------------------------------------------------------
+int spion_pattern_generate(const float* Score, int n_maps, int seq_len, int block_size, int conv_ksize, int mode,
+                           double param, float* Mat, float* Pooled, float* Thresh, void* stream) {
+    return pattern_generate(Score, n_maps, seq_len, block_size, conv_ksize, mode, param, Mat, Pooled, Thresh,
+                            static_cast<hipStream_t>(stream));
+}
+
+// ---- additions -----------------------------------------------------------------------------------
+const char* spion_last_error(void) {
+    static thread_local std::string copy;
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    copy = g_err;
+    return copy.c_str();
+}
+void spion_clear_error(void) {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    g_err.clear();
+}
+void spion_set_stream(void* h, void* stream) {
+    HandleHeader* hd = static_cast<HandleHeader*>(h);
+    if (!hd || (hd->magic != KIND_SPARSE && hd->magic != KIND_DENSE)) {
+        set_error("spion_set_stream: not a spion handle");
+        return;
+    }
+    hd->stream = static_cast<hipStream_t>(stream);
+}
+void spion_invalidate_pattern(void* h) { sparse_invalidate(h); }
+int spion_last_path(void* h) { return sparse_last_path(h); }
+void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
+void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
+const char* spion_version(void) { return "spion_hip 0.1 (gfx950)"; }
+
+}  // extern "C"

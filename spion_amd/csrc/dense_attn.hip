@@ -1,0 +1,300 @@
+// Dense-phase attention (forward + backward) for gfx950: ordinary softmax attention that also
+// materialises the full probability map, which the dense training phase hands to pattern discovery.
+//
+// Operand layouts are the reference's column-major ones (models/attn.cu:179-262,
+// models/attention_cuda.py:18-74): Qt/Vt/dOt and all gradients are feature-major [NB][d][L], K (forward) and
+// V (backward) are row-major [NB][L][d], and the map is stored key-major: Attn[h][j][i] = P[i][j].
+// One work-group owns 32 queries (forward, row pass) or 32 keys (column pass) of one head and walks all
+// L/32 tiles of the other dimension with v_mfma_f32_32x32x2_f32; see tile_ops.h for the register layout.
+#include "common.h"
+#include "tile_ops.h"
+#include "../../include/spion_hip.h"
+
+#include <cmath>
+
+namespace spion {
+
+constexpr int DENSE_WAVES = 4;
+
+template <int D, bool MASK>
+__global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
+    const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
+    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, int L, int nbr, int NB,
+    float scale) {
+    constexpr int WAVES = DENSE_WAVES;
+    __shared__ float lds[WAVES * (D / 32) * 16 * 64];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const float* penh = MASK ? pen + (size_t)bh * L : nullptr;
+    float* Ah = Attn + (size_t)bh * L * L + I * 32 + li;
+
+    float q[D / 2];
+    load_cols<D>(Qt + hb, L, I * 32, li, h, q);
+
+    float m = -10.f, z = 0.f;  // models/attn.cu:17
+    for (int J = w; J < nbr; J += WAVES) {
+        float k[D / 2];
+        load_rows<D>(K + hb, J * 32, li, h, k);
+        f32x16 s = mma_feat<D>(k, q);  // s[r] = q_i . k_j, i = I*32+li, j = J*32+acc_row(r,h)
+        float v[16], tm = m;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            v[r] = s[r] * scale;
+            if (MASK) v[r] -= penh[J * 32 + acc_row(r, h)];
+            tm = fmaxf(tm, v[r]);
+        }
+        float zz = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zz += __expf(v[r] - tm);
+        z = z * __expf(m - tm) + zz;
+        m = tm;
+    }
+    {
+        float m2 = __shfl_xor(m, 32, 64), z2 = __shfl_xor(z, 32, 64);
+        float M = fmaxf(m, m2);
+        z = z * __expf(m - M) + z2 * __expf(m2 - M);
+        m = M;
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
+        float Mx = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __expf(lds_m[ww][li] - Mx);
+        m = Mx;
+        z = Z;
+    }
+    const float rinv = 1.0f / z;
+
+    f32x16 o[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) o[c] = (f32x16){0};
+    for (int J = w; J < nbr; J += WAVES) {
+        float k[D / 2];
+        load_rows<D>(K + hb, J * 32, li, h, k);
+        f32x16 s = mma_feat<D>(k, q);
+        float p[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = s[r] * scale;
+            if (MASK) v -= penh[J * 32 + acc_row(r, h)];
+            p[r] = __expf(v - m) * rinv;
+            Ah[(size_t)(J * 32 + acc_row(r, h)) * L] = p[r];
+        }
+        mma_tile_t<D>(p, Vt + hb, L, J * 32, li, h, o);
+    }
+    reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+}
+
+// Row pass: g_i = sum_j dP_ij P_ij (kept in G), dS = (dP*P - P*g)*scale, dQ^T = K^T-tiles . dS^T.
+template <int D>
+__global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_row_kernel(
+    const float* __restrict__ Kt, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dOt, float* __restrict__ G, float* __restrict__ dQ, int L, int nbr, int NB,
+    float scale) {
+    constexpr int WAVES = DENSE_WAVES;
+    __shared__ float lds[WAVES * (D / 32) * 16 * 64];
+    __shared__ float lds_g[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const float* Ah = Attn + (size_t)bh * L * L + I * 32 + li;
+
+    float go[D / 2];
+    load_cols<D>(dOt + hb, L, I * 32, li, h, go);
+
+    float g = 0.f;
+    for (int J = w; J < nbr; J += WAVES) {
+        float v[D / 2];
+        load_rows<D>(V + hb, J * 32, li, h, v);
+        f32x16 dp = mma_feat<D>(v, go);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) g = fmaf(dp[r], Ah[(size_t)(J * 32 + acc_row(r, h)) * L], g);
+    }
+    g += __shfl_xor(g, 32, 64);
+    if (h == 0) lds_g[w][li] = g;
+    __syncthreads();
+    g = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = g;
+
+    f32x16 acc[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] = (f32x16){0};
+    for (int J = w; J < nbr; J += WAVES) {
+        float v[D / 2];
+        load_rows<D>(V + hb, J * 32, li, h, v);
+        f32x16 dp = mma_feat<D>(v, go);
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float p = Ah[(size_t)(J * 32 + acc_row(r, h)) * L];
+            ds[r] = (dp[r] * p - p * g) * scale;
+        }
+        mma_tile_t<D>(ds, Kt + hb, L, J * 32, li, h, acc);
+    }
+    reduce_store<D, WAVES, true>(acc, dQ + hb, I * 32, w, li, h, lds, L);
+}
+
+// Column pass: dK^T = Q^T-tiles . dS, dV^T = dO^T-tiles . P for 32 keys of one head.
+template <int D>
+__global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_col_kernel(
+    const float* __restrict__ Qt, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dOt, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
+    int L, int nbr, int NB, float scale) {
+    constexpr int WAVES = DENSE_WAVES;
+    __shared__ float lds[WAVES * (D / 32) * 16 * 64];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const float* Arow = Attn + (size_t)bh * L * L + (size_t)(J * 32 + li) * L + 4 * h;
+    const float* Gh = G + (size_t)bh * L;
+
+    float v[D / 2];
+    load_rows<D>(V + hb, J * 32, li, h, v);
+
+    f32x16 ak[D / 32], av[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        ak[c] = (f32x16){0};
+        av[c] = (f32x16){0};
+    }
+    for (int I = w; I < nbr; I += WAVES) {
+        float go[D / 2];
+        load_cols<D>(dOt + hb, L, I * 32, li, h, go);
+        f32x16 dp = mma_feat<D>(go, v);  // dp[r] = dO_i . v_j, i = I*32+acc_row(r,h), j = J*32+li
+        float p[16], ds[16];
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            float4 pv = *reinterpret_cast<const float4*>(Arow + I * 32 + 8 * g4);
+            p[4 * g4] = pv.x;
+            p[4 * g4 + 1] = pv.y;
+            p[4 * g4 + 2] = pv.z;
+            p[4 * g4 + 3] = pv.w;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float g = Gh[I * 32 + acc_row(r, h)];
+            ds[r] = (dp[r] * p[r] - p[r] * g) * scale;
+        }
+        mma_tile_t<D>(ds, Qt + hb, L, I * 32, li, h, ak);
+        mma_tile_t<D>(p, dOt + hb, L, I * 32, li, h, av);
+    }
+    reduce_store<D, WAVES, true>(ak, dK + hb, J * 32, w, li, h, lds, L);
+    __syncthreads();
+    reduce_store<D, WAVES, true>(av, dV + hb, J * 32, w, li, h, lds, L);
+}
+
+// -------------------------------------------------------------------------------------------------
+struct DenseAttn {
+    HandleHeader hdr;
+    int d, L, NB;
+    bool has_mask;
+    float scale;
+    float* ws_rowsum = nullptr;  // [NB][L]
+};
+
+static DenseAttn* as_dense(void* h, const char* who) {
+    DenseAttn* a = static_cast<DenseAttn*>(h);
+    if (!a || a->hdr.magic != KIND_DENSE) {
+        set_error("%s: not a dense-attention handle", who);
+        return nullptr;
+    }
+    return a;
+}
+
+void* dense_init(int emb_dim, int seq_len, int num_batches, bool has_mask) {
+    if (seq_len <= 0 || num_batches <= 0 || seq_len % 32) {
+        set_error("dense init: seq_len must be a positive multiple of 32 and num_batches positive (got %d, %d)",
+                  seq_len, num_batches);
+        return nullptr;
+    }
+    if (emb_dim != 32 && emb_dim != 64) {
+        set_error("dense init: emb_dim %d unsupported (32 or 64)", emb_dim);
+        return nullptr;
+    }
+    DenseAttn* a = new DenseAttn();
+    a->hdr.magic = KIND_DENSE;
+    a->hdr.stream = nullptr;
+    a->d = emb_dim;
+    a->L = seq_len;
+    a->NB = num_batches;
+    a->has_mask = has_mask;
+    a->scale = 1.0f / sqrtf((float)emb_dim);  // models/attn.cu:153
+    return a;
+}
+
+void dense_destroy(void* h) {
+    DenseAttn* a = as_dense(h, "destroy");
+    if (!a) return;
+    if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
+    a->hdr.magic = 0;
+    delete a;
+}
+
+template <int D>
+static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, const float* Vt, const float* Mask,
+                             float* Attn, float* Out) {
+    const int nbr = a->L / 32;
+    dim3 grid(nbr * a->NB), block(64 * DENSE_WAVES);
+    if (a->has_mask)
+        hipLaunchKernelGGL((dense_fwd_kernel<D, true>), grid, block, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
+                           a->L, nbr, a->NB, a->scale);
+    else
+        hipLaunchKernelGGL((dense_fwd_kernel<D, false>), grid, block, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
+                           a->L, nbr, a->NB, a->scale);
+}
+
+template <int D>
+static void dense_bwd_launch(DenseAttn* a, const float* Qt, const float* Kt, const float* V, const float* P,
+                             const float* dOt, float* dQ, float* dK, float* dV) {
+    const int nbr = a->L / 32;
+    dim3 grid(nbr * a->NB), block(64 * DENSE_WAVES);
+    hipLaunchKernelGGL((dense_bwd_row_kernel<D>), grid, block, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_rowsum, dQ, a->L,
+                       nbr, a->NB, a->scale);
+    hipLaunchKernelGGL((dense_bwd_col_kernel<D>), grid, block, 0, a->hdr.stream, Qt, V, P, dOt, a->ws_rowsum, dK, dV,
+                       a->L, nbr, a->NB, a->scale);
+}
+
+void dense_forward(void* h, const float* Qt, const float* K, const float* Vt, const float* Mask, float* Attn,
+                   float* Out, bool mask_entry) {
+    DenseAttn* a = as_dense(h, "attn_forward");
+    if (!a) return;
+    if (a->has_mask != mask_entry) {
+        set_error("attn_forward: handle was created by the %s init", a->has_mask ? "mask" : "no-mask");
+        return;
+    }
+    if (!Qt || !K || !Vt || !Attn || !Out || (mask_entry && !Mask)) {
+        set_error("attn_forward: null pointer argument");
+        return;
+    }
+    if (a->d == 32) dense_fwd_launch<32>(a, Qt, K, Vt, Mask, Attn, Out);
+    else dense_fwd_launch<64>(a, Qt, K, Vt, Mask, Attn, Out);
+    check_launch("dense_fwd_kernel");
+}
+
+void dense_backward(void* h, const float* Qt, const float* Kt, const float* V, const float* P, const float* dOt,
+                    float* dQ, float* dK, float* dV) {
+    DenseAttn* a = as_dense(h, "attn_backward");
+    if (!a) return;
+    if (!Qt || !Kt || !V || !P || !dOt || !dQ || !dK || !dV) {
+        set_error("attn_backward: null pointer argument");
+        return;
+    }
+    if (!a->ws_rowsum && !SPION_HIP_OK(hipMalloc((void**)&a->ws_rowsum, sizeof(float) * (size_t)a->NB * a->L))) return;
+    if (a->d == 32) dense_bwd_launch<32>(a, Qt, Kt, V, P, dOt, dQ, dK, dV);
+    else dense_bwd_launch<64>(a, Qt, Kt, V, P, dOt, dQ, dK, dV);
+    check_launch("dense_bwd kernels");
+}
+
+}  // namespace spion

@@ -1,0 +1,237 @@
+// Pattern discovery on the device: diagonal filter + block pooling in one pass over the score map,
+// then (one work-group per map) the quantile threshold, the greedy path walks and the binarised mask.
+//
+// Restates what the reference does on the host CPU with PyTorch ops and a recursive Python function
+// (main_conv_ff.py:35-62 and :254-278; top-k variant main_conv.py:236-256; pool-only main_ff.py:253-272).
+#include "common.h"
+#include "../../include/spion_hip.h"
+
+#include <cmath>
+#include <mutex>
+
+namespace spion {
+
+constexpr int POOL_THREADS = 256;
+constexpr int WALK_THREADS = 1024;
+
+// pooled[I][J] = (1/bs^2) sum_{i in I, j in J} sum_{t=-hk..hk} A[i+t][j+t]  (zero outside the map).
+// Regrouped per source element A[p][q]: its weight is the number of shifts t that land in the block.
+// fp64 accumulation in a fixed order, one rounding to fp32.
+__global__ __launch_bounds__(POOL_THREADS) void conv_pool_kernel(const float* __restrict__ A, float* __restrict__ pooled,
+                                                                 int L, int bs, int nb, int hk) {
+    __shared__ double red[POOL_THREADS];
+    const int I = blockIdx.y, J = blockIdx.x, map = blockIdx.z;
+    const float* Am = A + (size_t)map * L * L;
+    const int p0 = max(0, I * bs - hk), p1 = min(L, I * bs + bs + hk);
+    const int q0 = max(0, J * bs - hk), q1 = min(L, J * bs + bs + hk);
+    const int w = q1 - q0, total = (p1 - p0) * w;
+    double acc = 0.0;
+    for (int e = threadIdx.x; e < total; e += POOL_THREADS) {
+        const int p = p0 + e / w, q = q0 + e % w;
+        const int dp = p - I * bs, dq = q - J * bs;  // t must satisfy dp-bs+1 <= t <= dp, same for dq
+        const int lo = max(-hk, max(dp, dq) - bs + 1);
+        const int hi = min(hk, min(dp, dq));
+        if (hi >= lo) acc += (double)Am[(size_t)p * L + q] * (double)(hi - lo + 1);
+    }
+    red[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s = POOL_THREADS / 2; s > 0; s >>= 1) {
+        if (threadIdx.x < s) red[threadIdx.x] += red[threadIdx.x + s];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) pooled[((size_t)map * nb + I) * nb + J] = (float)(red[0] / ((double)bs * (double)bs));
+}
+
+__device__ __forceinline__ uint32_t float_key(float f) {  // order-preserving map to unsigned
+    uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// Key of the element of ascending rank `rank` (0-based) among v[0..N): 8-bit radix select by the whole
+// work-group.  hist: 256 ints of LDS, sh: 2 ints of LDS.
+__device__ uint32_t block_select(const float* __restrict__ v, int N, int rank, int* hist, int* sh) {
+    uint32_t prefix = 0, mask = 0;
+    int rem = rank;
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+        __syncthreads();
+        for (int i = threadIdx.x; i < N; i += blockDim.x) {
+            uint32_t k = float_key(v[i]);
+            if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            int c = 0, b = 0;
+            for (; b < 255; ++b) {
+                if (c + hist[b] > rem) break;
+                c += hist[b];
+            }
+            sh[0] = b;
+            sh[1] = rem - c;
+        }
+        __syncthreads();
+        prefix |= (uint32_t)sh[0] << shift;
+        mask |= 255u << shift;
+        rem = sh[1];
+        __syncthreads();
+    }
+    return prefix;
+}
+
+// One work-group per map.
+__global__ __launch_bounds__(WALK_THREADS) void threshold_walk_kernel(const float* __restrict__ pooled_all,
+                                                                      float* __restrict__ mat_all,
+                                                                      float* __restrict__ thresh_out, int nb, int mode,
+                                                                      float q, int topk) {
+    __shared__ int hist[256];
+    __shared__ int sh[2];
+    __shared__ int s_cnt;
+    __shared__ uint32_t s_min;
+    const int map = blockIdx.x, N = nb * nb;
+    const float* pooled = pooled_all + (size_t)map * N;
+    float* mat = mat_all + (size_t)map * N;
+
+    for (int i = threadIdx.x; i < N; i += blockDim.x) mat[i] = 0.f;
+
+    if (mode == SPION_PATTERN_FLOOD) {
+        // torch.quantile, linear interpolation, every step in fp32 (main_conv_ff.py:268)
+        const float r = q * (float)(N - 1);
+        const int lo = (int)floorf(r), hi = (int)ceilf(r);
+        const float wgt = r - (float)lo;
+        const uint32_t klo = block_select(pooled, N, lo, hist, sh);
+        if (threadIdx.x == 0) {
+            s_cnt = 0;
+            s_min = 0xffffffffu;
+        }
+        __syncthreads();
+        int c = 0;
+        uint32_t mn = 0xffffffffu;
+        for (int i = threadIdx.x; i < N; i += blockDim.x) {
+            uint32_t k = float_key(pooled[i]);
+            if (k <= klo) ++c;
+            else mn = min(mn, k);
+        }
+        atomicAdd(&s_cnt, c);
+        atomicMin(&s_min, mn);
+        __syncthreads();
+        const float a = key_float(klo);
+        const float b = (hi < s_cnt) ? a : key_float(s_min);  // sorted[hi]
+        const float diff = b - a;
+        float thresh;
+        if (wgt < 0.5f) thresh = a + __fmul_rn(wgt, diff);
+        else thresh = b - __fmul_rn(diff, 1.0f - wgt);
+        if (threadIdx.x == 0 && thresh_out) thresh_out[map] = thresh;
+        __syncthreads();  // mat is zeroed for everyone
+
+        // greedy walks: walker k < nb starts at (0, k), walker nb + k at (k, 0)  (main_conv_ff.py:271-274)
+        for (int wk = threadIdx.x; wk < 2 * nb; wk += blockDim.x) {
+            int x = wk < nb ? 0 : wk - nb, y = wk < nb ? wk : 0;
+            auto at = [&](int xx, int yy) -> float { return (xx < nb && yy < nb) ? pooled[xx * nb + yy] : 0.f; };
+            while (x < nb && y < nb) {  // x+1 != nb+1 and y+1 != nb+1 on the sentinel-padded map
+                const float Dn = at(x + 1, y), Rt = at(x, y + 1), Dg = at(x + 1, y + 1);
+                int nx, ny;
+                float val;
+                if (Dn > Rt) {
+                    if (Dn > Dg) { nx = x + 1; ny = y; val = Dn; }
+                    else { nx = x + 1; ny = y + 1; val = Dg; }
+                } else {
+                    if (Rt > Dg) { nx = x; ny = y + 1; val = Rt; }
+                    else { nx = x + 1; ny = y + 1; val = Dg; }
+                }
+                // ff_mat[nx][ny] = val, later binarised with ff_mat > 0
+                if (val > thresh && val > 0.f && nx < nb && ny < nb) mat[nx * nb + ny] = 1.f;
+                x = nx;
+                y = ny;
+            }
+        }
+    } else {
+        // the topk largest pooled blocks (main_conv.py:246-249); ties at the boundary: lower index first
+        if (threadIdx.x == 0 && thresh_out) thresh_out[map] = 0.f;
+        if (topk > 0) {
+            const int k = min(topk, N);
+            const uint32_t kk = block_select(pooled, N, N - k, hist, sh);  // k-th largest
+            if (threadIdx.x == 0) s_cnt = 0;
+            __syncthreads();
+            int c = 0;
+            for (int i = threadIdx.x; i < N; i += blockDim.x)
+                if (float_key(pooled[i]) > kk) {
+                    mat[i] = 1.f;
+                    ++c;
+                }
+            atomicAdd(&s_cnt, c);
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                int need = k - s_cnt;
+                for (int i = 0; i < N && need > 0; ++i)
+                    if (float_key(pooled[i]) == kk) {
+                        mat[i] = 1.f;
+                        --need;
+                    }
+            }
+            if (threadIdx.x == 0 && thresh_out) thresh_out[map] = key_float(kk);
+        }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) mat[i * nb + i] = 1.f;  // main_conv_ff.py:277-278
+}
+
+static std::mutex g_ws_mutex;
+static float* g_pool_ws = nullptr;
+static size_t g_pool_ws_count = 0;
+
+int pattern_generate(const float* Score, int n_maps, int L, int bs, int ksize, int mode, double param, float* Mat,
+                     float* Pooled, float* Thresh, hipStream_t stream) {
+    if (!Score || !Mat) {
+        set_error("spion_pattern_generate: null Score or Mat");
+        return 1;
+    }
+    if (n_maps <= 0 || L <= 0 || bs <= 0 || L % bs) {
+        set_error("spion_pattern_generate: need n_maps > 0 and seq_len a positive multiple of block_size (got %d, %d, %d)",
+                  n_maps, L, bs);
+        return 1;
+    }
+    if (ksize < 0 || (ksize && ksize % 2 == 0)) {
+        set_error("spion_pattern_generate: conv_ksize must be 0 or odd (got %d)", ksize);
+        return 1;
+    }
+    if (mode != SPION_PATTERN_FLOOD && mode != SPION_PATTERN_TOPK) {
+        set_error("spion_pattern_generate: unknown mode %d", mode);
+        return 1;
+    }
+    const int nb = L / bs;
+    if (nb > 16384 || n_maps > 65535 || nb > 65535) {
+        set_error("spion_pattern_generate: block grid %d or map count %d too large", nb, n_maps);
+        return 1;
+    }
+    if (mode == SPION_PATTERN_FLOOD && !(param >= 0.0 && param <= 1.0)) {
+        set_error("spion_pattern_generate: quantile %g outside [0, 1]", param);
+        return 1;
+    }
+    float* pooled = Pooled;
+    if (!pooled) {
+        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        const size_t need = (size_t)n_maps * nb * nb;
+        if (g_pool_ws_count < need) {
+            if (g_pool_ws) (void)hipFree(g_pool_ws);
+            g_pool_ws = nullptr;
+            g_pool_ws_count = 0;
+            if (!SPION_HIP_OK(hipMalloc((void**)&g_pool_ws, sizeof(float) * need))) return 1;
+            g_pool_ws_count = need;
+        }
+        pooled = g_pool_ws;
+    }
+    hipLaunchKernelGGL(conv_pool_kernel, dim3(nb, nb, n_maps), dim3(POOL_THREADS), 0, stream, Score, pooled, L, bs, nb,
+                       ksize / 2);
+    if (!check_launch("conv_pool_kernel")) return 1;
+    int topk = 0;
+    if (mode == SPION_PATTERN_TOPK) topk = (int)((double)(nb * nb) * param - (double)nb);  // main_conv.py:247
+    hipLaunchKernelGGL(threshold_walk_kernel, dim3(n_maps), dim3(WALK_THREADS), 0, stream, pooled, Mat, Thresh, nb, mode,
+                       (float)param, topk);
+    if (!check_launch("threshold_walk_kernel")) return 1;
+    return 0;
+}
+
+}  // namespace spion

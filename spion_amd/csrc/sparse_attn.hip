@@ -1,0 +1,831 @@
+// Sparse attention (forward + backward) on an element-level CSR pattern for gfx950 (MI355X).
+//
+// Two kernel families serve the same C ABI:
+//   * tile path    -- the pattern is a union of aligned 32x32 tiles (what a block mask of block size
+//                     32, 64, ... expands to).  Every contraction is a dense 32x32xd product done with
+//                     v_mfma_f32_32x32x2_f32; operands go straight from global memory into the MFMA
+//                     register layout (every access is a coalesced 128-byte row segment), the tile
+//                     list of a block row / block column is walked per wavefront.
+//   * element path -- any other CSR (element-sparse patterns, odd head sizes): one wavefront per
+//                     row gathers K/V rows; a transposed (CSC) index built on the host once per
+//                     pattern makes dK/dV deterministic without atomics.
+//
+// Semantics follow the reference kernels (models/block_attn.cu:33-130, models/block_attn_mask.cu:88-173):
+// the softmax denominator counts every off-pattern key with logit 0.
+#include "common.h"
+#include "tile_ops.h"
+#include "../../include/spion_hip.h"
+
+#include <algorithm>
+#include <cmath>
+#include <vector>
+
+namespace spion {
+
+// =================================================================================================
+// element path
+// =================================================================================================
+constexpr int ELEM_WAVES = 4;
+
+// [NB][D][L] -> [NB][L][D]
+__global__ __launch_bounds__(256) void transpose_dl_kernel(const float* __restrict__ Xt, float* __restrict__ X,
+                                                           int D, int L) {
+    __shared__ float tile[32][33];
+    const size_t base = (size_t)blockIdx.z * D * L;
+    const int l0 = blockIdx.x * 32, d0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8) {
+        int dd = d0 + r, ll = l0 + tx;
+        tile[r][tx] = (dd < D && ll < L) ? Xt[base + (size_t)dd * L + ll] : 0.f;
+    }
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8) {
+        int ll = l0 + r, dd = d0 + tx;
+        if (ll < L && dd < D) X[base + (size_t)ll * D + dd] = tile[tx][r];
+    }
+}
+
+template <int D>
+__device__ __forceinline__ float row_dot(const float* __restrict__ a, const float* __restrict__ b) {
+    float s = 0.f;
+    const float4* a4 = reinterpret_cast<const float4*>(a);
+    const float4* b4 = reinterpret_cast<const float4*>(b);
+#pragma unroll
+    for (int t = 0; t < D / 4; ++t) {
+        float4 x = a4[t], y = b4[t];
+        s = fmaf(x.x, y.x, s);
+        s = fmaf(x.y, y.y, s);
+        s = fmaf(x.z, y.z, s);
+        s = fmaf(x.w, y.w, s);
+    }
+    return s;
+}
+
+// acc[c] += sum_k w_k * X[col_k][c] over the entries of one CSR row, the entries being held one per
+// lane in chunks of 64 (w_l, col_l); LPR lanes cover one X row, 64/LPR entries are processed at once.
+template <int D>
+struct RowAcc {
+    static constexpr int LPR = D >= 64 ? 64 : D;
+    static constexpr int G = 64 / LPR;
+    static constexpr int CPL = D / LPR;
+    float acc[CPL];
+    __device__ __forceinline__ void clear() {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
+    }
+    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int lane) {
+        const int grp = lane / LPR, cl = lane % LPR;
+        // Uniform trip count: every lane takes part in every shuffle.  Slots past nk carry w = 0
+        // and row 0 (set by the caller), so they add nothing.
+        for (int kb = 0; kb < nk; kb += G) {
+            const int kk = kb + grp;
+            float w = __shfl(w_l, kk, 64);
+            int rr = __shfl(row_l, kk, 64);
+            const float* xr = X + (size_t)rr * D + cl;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) acc[c] = fmaf(w, xr[c * LPR], acc[c]);
+        }
+    }
+    __device__ __forceinline__ void finish(float* __restrict__ out_row, int lane) {
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            float a = acc[c];
+#pragma unroll
+            for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, 64);
+            if (lane < LPR) out_row[lane + c * LPR] = a;
+        }
+    }
+};
+
+// One wavefront per (head, row).  K is row-major here ([NB][L][D], transposed copy in the workspace).
+template <int D, bool MASK>
+__global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
+    const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+    const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
+    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
+    const int lane = threadIdx.x & 63;
+    const long long wrow = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    if (wrow >= (long long)NB * L) return;
+    const int bh = (int)(wrow / L), row = (int)(wrow % L);
+    const int r0 = offs[row], cnt = offs[row + 1] - r0;
+    const size_t hb = (size_t)bh * L * D;
+    const float* q = Q + hb + (size_t)row * D;
+    float* p = P + (size_t)bh * nnz + r0;
+    const int* cj = cols + r0;
+
+    float m = MASK ? 0.f : -100.f;
+    for (int k = lane; k < cnt; k += 64) {
+        int col = cj[k];
+        float v = row_dot<D>(q, K + hb + (size_t)col * D) * scale;
+        if (MASK) v -= pen[(size_t)bh * L + col];
+        p[k] = v;
+        m = fmaxf(m, v);
+    }
+    m = wave_max(m);
+    float z = 0.f;
+    for (int k = lane; k < cnt; k += 64) z += __expf(p[k] - m);
+    z = wave_sum(z);
+    z += (float)(L - cnt) * __expf(-m);
+    const float r = 1.0f / z;
+
+    RowAcc<D> acc;
+    acc.clear();
+    for (int c0 = 0; c0 < cnt; c0 += 64) {
+        const int k = c0 + lane;
+        float w = 0.f;
+        int col = 0;
+        if (k < cnt) {
+            w = __expf(p[k] - m) * r;
+            col = cj[k];
+            p[k] = w;
+        }
+        acc.chunk(w, col, min(64, cnt - c0), V + hb, lane);
+    }
+    acc.finish(O + hb + (size_t)row * D, lane);
+}
+
+// Row pass of the backward: dP = dO.V^T on the pattern, g = sum_row dP*P, dS = (dP*P - P*g)*scale
+// (written to the caller's dS scratch for the column pass), dQ = dS.K.
+template <int D>
+__global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
+    const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ P,
+    const float* __restrict__ dO, float* __restrict__ dS, float* __restrict__ dQ,
+    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
+    const int lane = threadIdx.x & 63;
+    const long long wrow = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    if (wrow >= (long long)NB * L) return;
+    const int bh = (int)(wrow / L), row = (int)(wrow % L);
+    const int r0 = offs[row], cnt = offs[row + 1] - r0;
+    const size_t hb = (size_t)bh * L * D;
+    const float* go = dO + hb + (size_t)row * D;
+    const float* p = P + (size_t)bh * nnz + r0;
+    float* ds = dS + (size_t)bh * nnz + r0;
+    const int* cj = cols + r0;
+
+    float g = 0.f;
+    for (int k = lane; k < cnt; k += 64) {
+        float t = row_dot<D>(go, V + hb + (size_t)cj[k] * D) * p[k];
+        ds[k] = t;
+        g += t;
+    }
+    g = wave_sum(g);
+
+    RowAcc<D> acc;
+    acc.clear();
+    for (int c0 = 0; c0 < cnt; c0 += 64) {
+        const int k = c0 + lane;
+        float w = 0.f;
+        int col = 0;
+        if (k < cnt) {
+            w = (ds[k] - p[k] * g) * scale;
+            col = cj[k];
+            ds[k] = w;
+        }
+        acc.chunk(w, col, min(64, cnt - c0), K + hb, lane);
+    }
+    acc.finish(dQ + hb + (size_t)row * D, lane);
+}
+
+// Column pass of the backward: dK_j = sum_i dS_ij Q_i, dV_j = sum_i P_ij dO_i over the transposed index.
+template <int D>
+__global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
+    const float* __restrict__ Q, const float* __restrict__ dO, const float* __restrict__ P,
+    const float* __restrict__ dS, float* __restrict__ dK, float* __restrict__ dV,
+    const int* __restrict__ colptr, const int* __restrict__ crow, const int* __restrict__ cpos, int L, int NB,
+    int nnz) {
+    const int lane = threadIdx.x & 63;
+    const long long wcol = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    if (wcol >= (long long)NB * L) return;
+    const int bh = (int)(wcol / L), col = (int)(wcol % L);
+    const int c0p = colptr[col], cnt = colptr[col + 1] - c0p;
+    const size_t hb = (size_t)bh * L * D;
+    const float* p = P + (size_t)bh * nnz;
+    const float* ds = dS + (size_t)bh * nnz;
+
+    RowAcc<D> ak, av;
+    ak.clear();
+    av.clear();
+    for (int c0 = 0; c0 < cnt; c0 += 64) {
+        const int e = c0 + lane;
+        float wk = 0.f, wv = 0.f;
+        int row = 0;
+        if (e < cnt) {
+            int pos = cpos[c0p + e];
+            row = crow[c0p + e];
+            wk = ds[pos];
+            wv = p[pos];
+        }
+        const int nk = min(64, cnt - c0);
+        ak.chunk(wk, row, nk, Q + hb, lane);
+        av.chunk(wv, row, nk, dO + hb, lane);
+    }
+    ak.finish(dK + hb + (size_t)col * D, lane);
+    av.finish(dV + hb + (size_t)col * D, lane);
+}
+
+// =================================================================================================
+// tile path (MFMA); the operand conventions are described in tile_ops.h
+// =================================================================================================
+// Forward, one work-group per (head, block row): sweep 1 finds the row maxima and denominators
+// (online over the tiles), sweep 2 recomputes the logits, writes P and accumulates O = P.V.
+template <int D, int WAVES, bool MASK>
+__global__ __launch_bounds__(64 * WAVES) void tile_fwd_kernel(
+    const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
+    const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
+    const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
+    int NB, int nnz, float scale) {
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int rn = cnt * 32;
+    const size_t hb = (size_t)bh * L * D;
+    const float* Kth = Kt + hb;
+    const float* penh = MASK ? pen + (size_t)bh * L : nullptr;
+    float* Prow = P + (size_t)bh * nnz + offs[I * 32] + (size_t)li * rn + 4 * h;
+
+    float q[D / 2];
+    load_rows<D>(Q + hb, I * 32, li, h, q);
+
+    float m = MASK ? 0.f : -100.f, z = 0.f;
+    for (int t = w; t < cnt; t += WAVES) {
+        const int J = tcol[t0 + t];
+        float k[D / 2];
+        load_cols<D>(Kth, L, J * 32, li, h, k);
+        f32x16 s = mma_feat<D>(k, q);  // s[r] = q_i . k_j, i = I*32+li, j = J*32+acc_row(r,h)
+        float v[16], tm = m;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            v[r] = s[r] * scale;
+            if (MASK) v[r] -= penh[J * 32 + acc_row(r, h)];
+            tm = fmaxf(tm, v[r]);
+        }
+        float zz = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) zz += __expf(v[r] - tm);
+        z = z * __expf(m - tm) + zz;
+        m = tm;
+    }
+    {   // merge the two half-waves, then the waves, of every row
+        float m2 = __shfl_xor(m, 32, 64), z2 = __shfl_xor(z, 32, 64);
+        float M = fmaxf(m, m2);
+        z = z * __expf(m - M) + z2 * __expf(m2 - M);
+        m = M;
+        if (WAVES > 1) {
+            if (h == 0) {
+                lds_m[w][li] = m;
+                lds_z[w][li] = z;
+            }
+            __syncthreads();
+            float Mx = lds_m[0][li];
+#pragma unroll
+            for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+            float Z = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __expf(lds_m[ww][li] - Mx);
+            m = Mx;
+            z = Z;
+        }
+    }
+    z += (float)(L - rn) * __expf(-m);
+    const float rinv = 1.0f / z;  // +inf denominator -> 0 -> P = 0, as in the reference
+
+    f32x16 o[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) o[c] = (f32x16){0};
+    for (int t = w; t < cnt; t += WAVES) {
+        const int J = tcol[t0 + t];
+        float k[D / 2];
+        load_cols<D>(Kth, L, J * 32, li, h, k);
+        f32x16 s = mma_feat<D>(k, q);
+        float p[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float v = s[r] * scale;
+            if (MASK) v -= penh[J * 32 + acc_row(r, h)];
+            p[r] = __expf(v - m) * rinv;
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            *reinterpret_cast<float4*>(Prow + t * 32 + 8 * g) =
+                make_float4(p[4 * g], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]);
+        mma_tile<D>(p, V + hb, J * 32, li, h, o);
+    }
+    reduce_store<D, WAVES>(o, O + hb, I * 32, w, li, h, lds);
+}
+
+// Backward, row pass, one work-group per (head, block row): g_i = sum_j dP_ij P_ij (kept in G for the
+// column pass), dS = (dP*P - P*g)*scale, dQ = dS.K.
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void tile_bwd_row_kernel(
+    const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
+    const float* __restrict__ dO, float* __restrict__ G, float* __restrict__ dQ, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    __shared__ float lds_g[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int rn = cnt * 32;
+    const size_t hb = (size_t)bh * L * D;
+    const float* Vth = Vt + hb;
+    const float* Prow = P + (size_t)bh * nnz + offs[I * 32] + (size_t)li * rn + 4 * h;
+
+    float go[D / 2];
+    load_rows<D>(dO + hb, I * 32, li, h, go);
+
+    float g = 0.f;
+    for (int t = w; t < cnt; t += WAVES) {
+        const int J = tcol[t0 + t];
+        float vt[D / 2];
+        load_cols<D>(Vth, L, J * 32, li, h, vt);
+        f32x16 dp = mma_feat<D>(vt, go);  // dp[r] = dO_i . v_j
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            float4 pv = *reinterpret_cast<const float4*>(Prow + t * 32 + 8 * q4);
+            g = fmaf(dp[4 * q4], pv.x, g);
+            g = fmaf(dp[4 * q4 + 1], pv.y, g);
+            g = fmaf(dp[4 * q4 + 2], pv.z, g);
+            g = fmaf(dp[4 * q4 + 3], pv.w, g);
+        }
+    }
+    g += __shfl_xor(g, 32, 64);
+    if (WAVES > 1) {
+        if (h == 0) lds_g[w][li] = g;
+        __syncthreads();
+        g = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
+    }
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = g;
+
+    f32x16 acc[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] = (f32x16){0};
+    for (int t = w; t < cnt; t += WAVES) {
+        const int J = tcol[t0 + t];
+        float vt[D / 2];
+        load_cols<D>(Vth, L, J * 32, li, h, vt);
+        f32x16 dp = mma_feat<D>(vt, go);
+        float ds[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+            float4 pv = *reinterpret_cast<const float4*>(Prow + t * 32 + 8 * q4);
+            ds[4 * q4] = (dp[4 * q4] * pv.x - pv.x * g) * scale;
+            ds[4 * q4 + 1] = (dp[4 * q4 + 1] * pv.y - pv.y * g) * scale;
+            ds[4 * q4 + 2] = (dp[4 * q4 + 2] * pv.z - pv.z * g) * scale;
+            ds[4 * q4 + 3] = (dp[4 * q4 + 3] * pv.w - pv.w * g) * scale;
+        }
+        mma_tile<D>(ds, K + hb, J * 32, li, h, acc);
+    }
+    reduce_store<D, WAVES>(acc, dQ + hb, I * 32, w, li, h, lds);
+}
+
+// Backward, column pass, one work-group per (head, block column): dK_J = sum_I dS_IJ^T Q_I,
+// dV_J = sum_I P_IJ^T dO_I, walking the transposed tile index.
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void tile_bwd_col_kernel(
+    const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
+    const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
+    const int* __restrict__ trp, const int* __restrict__ tcp, const int* __restrict__ tcrow,
+    const int* __restrict__ tcord, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
+    const size_t hb = (size_t)bh * L * D;
+    const float* Ph = P + (size_t)bh * nnz;
+    const float* Gh = G + (size_t)bh * L;
+
+    float vt[D / 2];
+    load_cols<D>(Vt + hb, L, J * 32, li, h, vt);
+
+    f32x16 ak[D / 32], av[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        ak[c] = (f32x16){0};
+        av[c] = (f32x16){0};
+    }
+    for (int e = w; e < cnt; e += WAVES) {
+        const int I = tcrow[e0 + e], ord = tcord[e0 + e];
+        const int rn = (trp[I + 1] - trp[I]) * 32;
+        float go[D / 2];
+        load_rows<D>(dO + hb, I * 32, li, h, go);
+        f32x16 dp = mma_feat<D>(go, vt);  // dp[r] = dO_i . v_j, i = I*32+acc_row(r,h), j = J*32+li
+        const float* pt = Ph + offs[I * 32] + ord * 32 + li;
+        float p[16], ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int ir = acc_row(r, h);
+            p[r] = pt[(size_t)ir * rn];
+            const float g = Gh[I * 32 + ir];
+            ds[r] = (dp[r] * p[r] - p[r] * g) * scale;
+        }
+        mma_tile<D>(ds, Q + hb, I * 32, li, h, ak);
+        mma_tile<D>(p, dO + hb, I * 32, li, h, av);
+    }
+    reduce_store<D, WAVES>(ak, dK + hb, J * 32, w, li, h, lds);
+    if (WAVES > 1) __syncthreads();
+    reduce_store<D, WAVES>(av, dV + hb, J * 32, w, li, h, lds);
+}
+
+// =================================================================================================
+// host side
+// =================================================================================================
+struct PatternIndex {
+    const int* key_off = nullptr;
+    const int* key_col = nullptr;
+    int key_nnz = -1;
+    bool valid = false;
+    bool tiled = false;
+    int ntiles = 0;
+    int max_row_tiles = 0, max_col_tiles = 0;
+    int* d_blob = nullptr;  // one allocation holding every array below
+    int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr, *d_tcrow = nullptr, *d_tcord = nullptr;
+    int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
+    void release() {
+        if (d_blob) (void)hipFree(d_blob);
+        *this = PatternIndex();
+    }
+};
+
+struct SparseAttn {
+    HandleHeader hdr;
+    int d, L, NB, bs;
+    bool has_mask;
+    float scale;
+    PatternIndex pat;
+    float* ws_rowsum = nullptr;  // [NB][L]   g of the backward (tile path)
+    float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
+    int last_path = 0;
+    bool force_element = false;
+    int bwd_passes = 3;  // bit 0: row pass (g, dQ), bit 1: column pass (dK, dV); profiling only
+};
+
+static SparseAttn* as_sparse(void* h, const char* who) {
+    SparseAttn* a = static_cast<SparseAttn*>(h);
+    if (!a || a->hdr.magic != KIND_SPARSE) {
+        set_error("%s: not a sparse-attention handle", who);
+        return nullptr;
+    }
+    return a;
+}
+
+static bool tile_supported(int d) { return d == 32 || d == 64; }
+static bool elem_supported(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
+
+void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, bool has_mask) {
+    if (emb_dim <= 0 || seq_len <= 0 || num_batches <= 0) {
+        set_error("init: emb_dim, seq_len and num_batches must be positive (got %d, %d, %d)", emb_dim, seq_len,
+                  num_batches);
+        return nullptr;
+    }
+    if (!elem_supported(emb_dim)) {
+        set_error("init: emb_dim %d unsupported (16, 32, 64 or 128)", emb_dim);
+        return nullptr;
+    }
+    SparseAttn* a = new SparseAttn();
+    a->hdr.magic = KIND_SPARSE;
+    a->hdr.stream = nullptr;
+    a->d = emb_dim;
+    a->L = seq_len;
+    a->NB = num_batches;
+    a->bs = block_size;
+    a->has_mask = has_mask;
+    a->scale = 1.0f / sqrtf((float)emb_dim);  // models/block_attn.cu:420
+    return a;
+}
+
+void sparse_destroy(void* h) {
+    SparseAttn* a = as_sparse(h, "destroy");
+    if (!a) return;
+    a->pat.release();
+    if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
+    if (a->ws_trans) (void)hipFree(a->ws_trans);
+    a->hdr.magic = 0;
+    delete a;
+}
+
+// Copy the index to the host once, validate it, detect the tile structure and build the transposed
+// index.  Returns false (error recorded) if the CSR is inconsistent.
+static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Columns, int nnz) {
+    PatternIndex& pi = a->pat;
+    pi.release();
+    const int L = a->L;
+    if (nnz < 0) {
+        set_error("pattern: nnz %d is negative", nnz);
+        return false;
+    }
+    std::vector<int> off(L + 1), col((size_t)nnz);
+    if (!SPION_HIP_OK(hipMemcpyAsync(off.data(), Offsets, sizeof(int) * (L + 1), hipMemcpyDeviceToHost, a->hdr.stream)))
+        return false;
+    if (nnz && !SPION_HIP_OK(hipMemcpyAsync(col.data(), Columns, sizeof(int) * (size_t)nnz, hipMemcpyDeviceToHost,
+                                            a->hdr.stream)))
+        return false;
+    if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
+
+    if (off[0] != 0 || off[L] != nnz) {
+        set_error("pattern: Offsets[0]=%d, Offsets[L]=%d do not match nnz=%d", off[0], off[L], nnz);
+        return false;
+    }
+    for (int i = 0; i < L; ++i) {
+        if (off[i + 1] < off[i]) {
+            set_error("pattern: Offsets not monotone at row %d", i);
+            return false;
+        }
+        for (int k = off[i]; k < off[i + 1]; ++k) {
+            if (col[k] < 0 || col[k] >= L) {
+                set_error("pattern: column %d out of range at row %d", col[k], i);
+                return false;
+            }
+            if (k > off[i] && col[k] <= col[k - 1]) {
+                set_error("pattern: columns of row %d are not strictly increasing", i);
+                return false;
+            }
+        }
+    }
+
+    // --- tile detection: every 32-row strip has identical rows made of aligned runs of 32 columns
+    bool tiled = !a->force_element && tile_supported(a->d) && (L % 32 == 0);
+    const int nbr = L / 32;
+    std::vector<int> trp, tcol;
+    if (tiled) {
+        trp.assign(nbr + 1, 0);
+        for (int I = 0; I < nbr && tiled; ++I) {
+            const int r0 = I * 32, a0 = off[r0], n0 = off[r0 + 1] - a0;
+            if (n0 % 32) tiled = false;
+            for (int k = 0; k < n0 && tiled; ++k) {
+                int c = col[a0 + k];
+                if ((k % 32 == 0 && c % 32 != 0) || (k % 32 && c != col[a0 + k - 1] + 1)) tiled = false;
+            }
+            for (int r = 1; r < 32 && tiled; ++r) {
+                const int ar = off[r0 + r];
+                if (off[r0 + r + 1] - ar != n0 || (n0 && memcmp(&col[ar], &col[a0], sizeof(int) * n0))) tiled = false;
+            }
+            if (tiled) {
+                for (int k = 0; k < n0; k += 32) tcol.push_back(col[a0 + k] / 32);
+                trp[I + 1] = (int)tcol.size();
+            }
+        }
+    }
+
+    std::vector<int> blob;
+    auto append = [&](const std::vector<int>& v) {
+        size_t o = blob.size();
+        blob.insert(blob.end(), v.begin(), v.end());
+        while (blob.size() % 4) blob.push_back(0);
+        return o;
+    };
+    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcrow = 0, o_tcord = 0, o_ccp = 0, o_crow = 0, o_cpos = 0;
+    if (tiled) {
+        const int nt = (int)tcol.size();
+        std::vector<int> tcp(nbr + 1, 0), tcrow(std::max(nt, 1)), tcord(std::max(nt, 1));
+        for (int t = 0; t < nt; ++t) tcp[tcol[t] + 1]++;
+        for (int J = 0; J < nbr; ++J) tcp[J + 1] += tcp[J];
+        std::vector<int> fill(tcp.begin(), tcp.end() - 1);
+        int mr = 0, mc = 0;
+        for (int I = 0; I < nbr; ++I) {
+            mr = std::max(mr, trp[I + 1] - trp[I]);
+            for (int t = trp[I]; t < trp[I + 1]; ++t) {
+                int e = fill[tcol[t]]++;
+                tcrow[e] = I;
+                tcord[e] = t - trp[I];
+            }
+        }
+        for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
+        if (tcol.empty()) tcol.push_back(0);
+        o_trp = append(trp);
+        o_tcol = append(tcol);
+        o_tcp = append(tcp);
+        o_tcrow = append(tcrow);
+        o_tcord = append(tcord);
+        pi.ntiles = nt;
+        pi.max_row_tiles = mr;
+        pi.max_col_tiles = mc;
+    } else {
+        std::vector<int> ccp(L + 1, 0), crow(std::max(nnz, 1)), cpos(std::max(nnz, 1));
+        for (int k = 0; k < nnz; ++k) ccp[col[k] + 1]++;
+        for (int j = 0; j < L; ++j) ccp[j + 1] += ccp[j];
+        std::vector<int> fill(ccp.begin(), ccp.end() - 1);
+        for (int i = 0; i < L; ++i)
+            for (int k = off[i]; k < off[i + 1]; ++k) {
+                int e = fill[col[k]]++;
+                crow[e] = i;
+                cpos[e] = k;
+            }
+        o_ccp = append(ccp);
+        o_crow = append(crow);
+        o_cpos = append(cpos);
+    }
+    if (!SPION_HIP_OK(hipMalloc((void**)&pi.d_blob, sizeof(int) * blob.size()))) return false;
+    if (!SPION_HIP_OK(hipMemcpy(pi.d_blob, blob.data(), sizeof(int) * blob.size(), hipMemcpyHostToDevice))) {
+        pi.release();
+        return false;
+    }
+    if (tiled) {
+        pi.d_trp = pi.d_blob + o_trp;
+        pi.d_tcol = pi.d_blob + o_tcol;
+        pi.d_tcp = pi.d_blob + o_tcp;
+        pi.d_tcrow = pi.d_blob + o_tcrow;
+        pi.d_tcord = pi.d_blob + o_tcord;
+    } else {
+        pi.d_ccp = pi.d_blob + o_ccp;
+        pi.d_crow = pi.d_blob + o_crow;
+        pi.d_cpos = pi.d_blob + o_cpos;
+    }
+    pi.tiled = tiled;
+    pi.key_off = Offsets;
+    pi.key_col = Columns;
+    pi.key_nnz = nnz;
+    pi.valid = true;
+    return true;
+}
+
+static bool ensure_pattern(SparseAttn* a, const int* Offsets, const int* Columns, int nnz) {
+    PatternIndex& pi = a->pat;
+    if (pi.valid && pi.key_off == Offsets && pi.key_col == Columns && pi.key_nnz == nnz) return true;
+    return analyse_pattern(a, Offsets, Columns, nnz);
+}
+
+static bool ensure_ws(float** p, size_t count) {
+    if (*p) return true;
+    return SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * count));
+}
+
+static int pick_waves(const PatternIndex& pi, int nbr, bool by_col) {
+    // average tiles per strip decides how many wavefronts share one strip
+    const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
+    (void)by_col;
+    if (avg <= 1) return 1;
+    if (avg <= 3) return 2;
+    return 4;
+}
+
+template <int D, bool MASK>
+static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, const float* V, const float* pen, float* P,
+                            float* O, const int* offs, int nnz) {
+    const PatternIndex& pi = a->pat;
+    const int nbr = a->L / 32;
+    const dim3 grid(nbr * a->NB);
+    const int wv = pick_waves(pi, nbr, false);
+#define SPION_LAUNCH(W)                                                                                             \
+    hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V, pen, P, O,    \
+                       pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale)
+    if (wv == 1) SPION_LAUNCH(1);
+    else if (wv == 2) SPION_LAUNCH(2);
+    else SPION_LAUNCH(4);
+#undef SPION_LAUNCH
+}
+
+template <int D>
+static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
+                            const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz) {
+    const PatternIndex& pi = a->pat;
+    const int nbr = a->L / 32;
+    const dim3 grid(nbr * a->NB);
+    const int wv = pick_waves(pi, nbr, false);
+#define SPION_LAUNCH(W)                                                                                             \
+    do {                                                                                                            \
+        if (a->bwd_passes & 1)                                                                                      \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P, dO,     \
+                               a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);       \
+        if (a->bwd_passes & 2)                                                                                      \
+            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
+                               a->ws_rowsum, dK, dV, pi.d_trp, pi.d_tcp, pi.d_tcrow, pi.d_tcord, offs, a->L, nbr,   \
+                               a->NB, nnz, a->scale);                                                               \
+    } while (0)
+    if (wv == 1) SPION_LAUNCH(1);
+    else if (wv == 2) SPION_LAUNCH(2);
+    else SPION_LAUNCH(4);
+#undef SPION_LAUNCH
+}
+
+static void launch_transpose(SparseAttn* a, const float* Xt, float* X) {
+    dim3 grid((a->L + 31) / 32, (a->d + 31) / 32, a->NB);
+    hipLaunchKernelGGL(transpose_dl_kernel, grid, dim3(256), 0, a->hdr.stream, Xt, X, a->d, a->L);
+}
+
+template <int D>
+static void launch_elem_fwd(SparseAttn* a, const float* Q, const float* Krm, const float* V, const float* pen,
+                            float* P, float* O, const int* offs, const int* cols, int nnz) {
+    const long long rows = (long long)a->NB * a->L;
+    dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
+    if (a->has_mask)
+        hipLaunchKernelGGL((elem_fwd_kernel<D, true>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V, pen,
+                           P, O, offs, cols, a->L, a->NB, nnz, a->scale);
+    else
+        hipLaunchKernelGGL((elem_fwd_kernel<D, false>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V, pen,
+                           P, O, offs, cols, a->L, a->NB, nnz, a->scale);
+}
+
+template <int D>
+static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vrm, const float* P,
+                            const float* dO, float* dS, float* dQ, float* dK, float* dV, const int* offs,
+                            const int* cols, int nnz) {
+    const PatternIndex& pi = a->pat;
+    const long long rows = (long long)a->NB * a->L;
+    dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
+    if (a->bwd_passes & 1)
+        hipLaunchKernelGGL((elem_bwd_row_kernel<D>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, K, Vrm, P, dO, dS,
+                           dQ, offs, cols, a->L, a->NB, nnz, a->scale);
+    if (a->bwd_passes & 2)
+        hipLaunchKernelGGL((elem_bwd_col_kernel<D>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, dO, P, dS, dK,
+                           dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz);
+}
+
+void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, const float* Mask, float* Attn,
+                    float* Out, const int* Offsets, const int* Columns, int nnz, bool mask_entry) {
+    SparseAttn* a = as_sparse(h, "attn_forward");
+    if (!a) return;
+    if (a->has_mask != mask_entry) {
+        set_error("attn_forward: handle was created by the %s init", a->has_mask ? "mask" : "no-mask");
+        return;
+    }
+    if (!Q || !Kt || !V || !Attn || !Out || !Offsets || (nnz > 0 && !Columns) || (mask_entry && !Mask)) {
+        set_error("attn_forward: null pointer argument");
+        return;
+    }
+    if (!ensure_pattern(a, Offsets, Columns, nnz)) return;
+    if (a->pat.tiled) {
+        a->last_path = 1;
+        if (a->d == 32) {
+            if (a->has_mask) launch_tile_fwd<32, true>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
+            else launch_tile_fwd<32, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+        } else {
+            if (a->has_mask) launch_tile_fwd<64, true>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
+            else launch_tile_fwd<64, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+        }
+        check_launch("tile_fwd_kernel");
+        return;
+    }
+    a->last_path = 2;
+    if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+    launch_transpose(a, Kt, a->ws_trans);
+    switch (a->d) {
+        case 16: launch_elem_fwd<16>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        case 32: launch_elem_fwd<32>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        case 64: launch_elem_fwd<64>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        default: launch_elem_fwd<128>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+    }
+    check_launch("elem_fwd_kernel");
+}
+
+void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P, const float* dO,
+                     float* dP, float* dS, float* dQ, float* dK, float* dV, const int* Offsets, const int* Columns,
+                     int nnz) {
+    SparseAttn* a = as_sparse(h, "attn_backward");
+    if (!a) return;
+    (void)dP;
+    if (!Q || !K || !Vt || !P || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("attn_backward: null pointer argument");
+        return;
+    }
+    if (!ensure_pattern(a, Offsets, Columns, nnz)) return;
+    if (a->pat.tiled) {
+        a->last_path = 1;
+        if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+        if (a->d == 32) launch_tile_bwd<32>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz);
+        else launch_tile_bwd<64>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz);
+        check_launch("tile_bwd kernels");
+        return;
+    }
+    a->last_path = 2;
+    if (!dS) {
+        set_error("attn_backward: the element path needs the dS scratch buffer");
+        return;
+    }
+    if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+    launch_transpose(a, Vt, a->ws_trans);
+    switch (a->d) {
+        case 16: launch_elem_bwd<16>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        case 32: launch_elem_bwd<32>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        case 64: launch_elem_bwd<64>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        default: launch_elem_bwd<128>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+    }
+    check_launch("elem_bwd kernels");
+}
+
+void sparse_invalidate(void* h) {
+    SparseAttn* a = as_sparse(h, "spion_invalidate_pattern");
+    if (a) a->pat.release();
+}
+int sparse_last_path(void* h) {
+    SparseAttn* a = as_sparse(h, "spion_last_path");
+    return a ? a->last_path : 0;
+}
+void sparse_set_bwd_passes(void* h, int mask) {
+    SparseAttn* a = as_sparse(h, "spion_set_backward_passes");
+    if (a) a->bwd_passes = mask & 3;
+}
+void sparse_force_element(void* h, int on) {
+    SparseAttn* a = as_sparse(h, "spion_force_element_path");
+    if (!a) return;
+    a->force_element = on != 0;
+    a->pat.release();
+}
+
+}  // namespace spion

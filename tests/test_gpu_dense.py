@@ -1,0 +1,94 @@
+"""Parity of the dense-phase HIP kernels with the float64 oracle, through the C ABI (GPU box only)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dense_attention as oda
+from oracle import sparse_attention as osa
+from spion_amd import _lib, workloads
+from spion_amd.attention import Attention
+from tests.abi_utils import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_dense(d, L, NB, Q, K, V, dO, pen=None):
+    """Drive attn.so / attn_mask.so with the reference's operand layouts (models/attention_cuda.py:18-74)."""
+    lib = Attention._cuda_mask_compile_module() if pen is not None else Attention._cuda_compile_module()
+    h = lib.init(d, L, NB)
+    _lib.check_error("init")
+    nan = float("nan")
+    Qt, Kt, Vt, dOt = (t.transpose(1, 2).contiguous() for t in (Q, K, V, dO))
+    attn = torch.full((NB, L, L), nan, device="cuda")
+    out_t = torch.full((NB, d, L), nan, device="cuda")
+    args = [h, Qt.data_ptr(), K.data_ptr(), Vt.data_ptr()]
+    if pen is not None:
+        args.append(pen.data_ptr())
+    lib.attn_forward(*args, attn.data_ptr(), out_t.data_ptr())
+    _lib.check_error("attn_forward")
+    dq, dk, dv = (torch.full((NB, d, L), nan, device="cuda") for _ in range(3))
+    lib.attn_backward(h, Qt.data_ptr(), Kt.data_ptr(), V.data_ptr(), attn.data_ptr(), dOt.data_ptr(), None, None,
+                      None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr())
+    _lib.check_error("attn_backward")
+    torch.cuda.synchronize()
+    lib.destroy(h)
+    tr = lambda t: t.transpose(1, 2).cpu().numpy()
+    return dict(O=tr(out_t), P=tr(attn), dQ=tr(dq), dK=tr(dk), dV=tr(dv))
+
+
+@pytest.mark.parametrize("L,d,NB,with_mask", [(128, 32, 3, False), (256, 64, 2, False), (256, 32, 4, True),
+                                              (1024, 32, 2, False)])
+def test_dense_matches_oracle(L, d, NB, with_mask):
+    g = torch.Generator().manual_seed(L + d)
+    Q, K, V, dO = (torch.randn(NB, L, d, generator=g).cuda() for _ in range(4))
+    pen = None
+    pen_np = None
+    if with_mask:
+        km = np.ones((NB // 2, L), np.float32)
+        km[0, 130:] = 0
+        km[1, 33:] = 0
+        pen_np = osa.key_penalty_from_mask(km, 2)
+        pen = torch.from_numpy(pen_np).cuda()
+    got = _run_dense(d, L, NB, Q, K, V, dO, pen)
+    f = lambda t: t.cpu().numpy().astype(np.float64)
+    O, P = oda.dense_attention_forward(f(Q), f(K), f(V), None if pen_np is None else pen_np.astype(np.float64))
+    dQ, dK, dV = oda.dense_attention_backward(f(Q), f(K), f(V), P, f(dO))
+    for name, ref in (("P", P), ("O", O), ("dQ", dQ), ("dK", dK), ("dV", dV)):
+        assert_close(got[name], ref, what=f"dense L={L} d={d} {name}")
+    assert_close(got["P"].sum(-1), np.ones((NB, L)), what="rows of P sum to one")
+    if with_mask:
+        assert (got["P"][0][:, 130:] == 0).all() and (got["P"][2][:, 33:] == 0).all()
+
+
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_dense_modules_autograd(with_mask):
+    import spion_amd
+
+    B, H, L, d = 2, 2, 128, 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
+    if with_mask:
+        cpp = Attention._cuda_mask_compile_module()
+        mod = spion_amd.CUDAMaskAttention(cfg, cpp, cpp.init(d, L, B * H))
+    else:
+        cpp = Attention._cuda_compile_module()
+        mod = spion_amd.CUDAAttention(cfg, cpp, cpp.init(d, L, B * H))
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=7, device="cuda")
+    key_mask = torch.ones(B, L)
+    if with_mask:
+        key_mask[1, 90:] = 0
+    for t in (q, k, v):
+        t.requires_grad_()
+    out, attn = mod(q, k, v, key_mask.cuda())
+    assert out.shape == (B, H, L, d) and attn.shape == (B, H, L, L)
+    out.backward(do)
+    qc, kc, vc = (t.detach().double().cpu().requires_grad_() for t in (q, k, v))
+    s = qc @ kc.transpose(-1, -2) * float(np.float32(1.0) / np.sqrt(np.float32(d)))
+    if with_mask:
+        s = s - 1e6 * (1 - key_mask.double())[:, None, None, :]
+    p = torch.softmax(s, -1)
+    o = p @ vc
+    o.backward(do.double().cpu())
+    assert_close(out.detach().cpu().numpy(), o.detach().numpy(), what="dense module out")
+    assert_close(attn.detach().cpu().numpy(), p.detach().numpy(), what="dense module attn")
+    for name, a, b in (("dq", q, qc), ("dk", k, kc), ("dv", v, vc)):
+        assert_close(a.grad.cpu().numpy(), b.grad.numpy(), what=f"dense module {name}")

@@ -1,0 +1,73 @@
+"""Pattern discovery kernels vs the oracle: pooled maps to 1 ulp-level, masks bit-exact (GPU box only)."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import pattern as op
+from spion_amd import discover_block_masks, generate_pattern_conv, generate_pattern_conv_ff, generate_pattern_ff
+from spion_amd import workloads
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _check_maps(maps, bs, q, ksize):
+    mode = "conv_ff" if ksize else "ff"
+    mat, pooled, thresh = discover_block_masks(maps.cuda(), bs, mode=mode, threshold=q, ksize=ksize or 31,
+                                               return_aux=True)
+    mat, pooled, thresh = mat.cpu().numpy(), pooled.cpu().numpy(), thresh.cpu().numpy()
+    for i in range(maps.shape[0]):
+        ref_mask, ref_pooled, ref_thresh = op.generate_mask_conv_ff(maps[i].numpy(), bs, q, ksize=ksize, route="fp64")
+        # fp64 accumulation on both sides, one rounding: equal except for double-rounding ties
+        assert np.max(np.abs(pooled[i] - ref_pooled) / np.abs(ref_pooled).max()) < 2e-7
+        # the walk is checked on the GPU's own pooled map: bit-exact by construction of the oracle
+        t_gpu = op.quantile_linear(pooled[i], q)[0]
+        assert abs(float(thresh[i]) - float(t_gpu)) <= np.spacing(np.float32(abs(t_gpu)))
+        assert np.array_equal(mat[i].astype(np.int8), op.mask_from_pooled(pooled[i], np.float32(thresh[i])))
+        if np.array_equal(pooled[i], ref_pooled) and thresh[i] == ref_thresh:
+            assert np.array_equal(mat[i].astype(np.int8), ref_mask)
+    return mat, pooled, thresh
+
+
+@pytest.mark.parametrize("L,bs,q,ksize", [(256, 32, 0.9, 31), (512, 64, 0.96, 31), (256, 16, 0.75, 31),
+                                          (256, 32, 0.9, 0), (128, 32, 0.5, 7)])
+def test_pattern_small_maps(L, bs, q, ksize):
+    g = torch.Generator().manual_seed(L + bs)
+    maps = torch.softmax(torch.randn(3, L, L, generator=g) * 2, -1)
+    maps[1] += 0.02 * torch.eye(L)
+    _check_maps(maps, bs, q, ksize)
+
+
+def test_pattern_config2_bit_exact_against_both_routes():
+    """Config 2: two 1024x1024 maps, 31x31 diagonal filter, 32x32 pooling, q = 0.90.
+    The seed is one whose decision margin exceeds the float32-route error (tests/golden/config2.json),
+    so the reference's float32 PyTorch route, the float64 route and the GPU must give the same masks."""
+    meta = json.load(open(os.path.join(GOLDEN, "config2.json")))
+    maps = workloads.score_maps_config2(2, 1024, 32, seed=meta["seed"])
+    mat, pooled, thresh = _check_maps(maps, 32, 0.90, 31)
+    golden = np.load(os.path.join(GOLDEN, "config2_masks.npy"))
+    assert np.array_equal(mat.astype(np.int8), golden)
+    for i in range(2):
+        m32, _, _ = op.generate_mask_conv_ff(maps[i].numpy(), 32, 0.90, route="torch")
+        assert np.array_equal(mat[i].astype(np.int8), m32)
+
+
+def test_pattern_topk_and_generators():
+    L, bs = 256, 32
+    g = torch.Generator().manual_seed(3)
+    maps = torch.softmax(torch.randn(2, L, L, generator=g) * 2, -1)
+    mat = discover_block_masks(maps.cuda(), bs, mode="conv", density=0.3).cpu().numpy()
+    for i in range(2):
+        ref, _, k = op.generate_mask_conv(maps[i].numpy(), bs, 0.3)
+        assert np.array_equal(mat[i].astype(np.int8), ref)
+    cfg = dict(max_seq_len=L, block_size=bs, num_layers=2, threshold=0.9, density=0.3)
+    attn_lst = [torch.cat([m, m], 0).cuda() for m in maps]  # gathered maps carry extra rows; only the first L count
+    for fn in (generate_pattern_conv_ff, generate_pattern_ff, generate_pattern_conv):
+        ml = fn(attn_lst, cfg)
+        assert ml.shape == (4, 2, L // bs, L // bs) and ml.dtype == torch.float32
+        assert torch.equal(ml[0], ml[3]) and set(ml.unique().tolist()) <= {0.0, 1.0}
+        assert (torch.diagonal(ml[0], dim1=-2, dim2=-1) == 1).all()

@@ -1,0 +1,307 @@
+"""Parity of the sparse-attention HIP kernels with the float64 oracle, through the C ABI (GPU box only).
+
+Tolerance: fp32 results within 1e-4 relative (see abi_utils.assert_close).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sparse_attention as osa
+from spion_amd import workloads
+from tests.abi_utils import SparseABI, assert_close, run_and_check
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(NB, L, d, seed, scale=1.0, dev="cuda"):
+    g = torch.Generator().manual_seed(seed)
+    return tuple((torch.randn(NB, L, d, generator=g) * s).to(dev) for s in (scale, scale, 1.0, 1.0))
+
+
+def _random_block_mask(nb, p, seed, empty_row=None, empty_col=None):
+    rng = np.random.default_rng(seed)
+    mat = (rng.random((nb, nb)) < p).astype(np.float32)
+    mat[np.arange(nb), np.arange(nb)] = 1
+    if empty_row is not None:
+        mat[empty_row, :] = 0
+    if empty_col is not None:
+        mat[:, empty_col] = 0
+    return mat
+
+
+# ---------------------------------------------------------------------------------- tile (MFMA) path
+@pytest.mark.parametrize(
+    "L,bs,d,NB,p",
+    [
+        (128, 32, 32, 3, 0.15),   # about one tile per strip  -> 1 wavefront per strip
+        (256, 32, 32, 2, 0.30),   # 2-3 tiles per strip       -> 2 wavefronts
+        (256, 32, 32, 5, 0.80),   # many tiles                -> 4 wavefronts
+        (256, 64, 32, 2, 0.40),   # 64x64 blocks = 2x2 tiles
+        (256, 32, 64, 2, 0.50),   # head dim 64
+        (512, 128, 64, 1, 0.50),
+    ],
+)
+def test_tile_path_matches_oracle(L, bs, d, NB, p):
+    nb = L // bs
+    mat = _random_block_mask(nb, p, seed=L + bs + d)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=1, scale=1.5)
+    run_and_check(abi, Q, K, V, dO, tag=f"tile L={L} bs={bs} d={d}")
+    assert abi.last_path() == 1
+    abi.close()
+
+
+def test_tile_path_empty_block_row_and_column():
+    L, bs, d, NB = 256, 32, 32, 2
+    mat = _random_block_mask(L // bs, 0.4, seed=5, empty_row=2, empty_col=5)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=2)
+    got, _ = run_and_check(abi, Q, K, V, dO, tag="empty strip")
+    assert (got["O"][:, 64:96] == 0).all() and (got["dQ"][:, 64:96] == 0).all()
+    assert (got["dK"][:, 160:192] == 0).all() and (got["dV"][:, 160:192] == 0).all()
+    abi.close()
+
+
+def test_tile_path_full_pattern_is_softmax_attention():
+    L, bs, d, NB = 128, 32, 32, 2
+    sm, off, col = osa.build_csr_from_block_mask(np.ones((4, 4), np.float32), bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=3)
+    O, P = abi.forward(Q, K, V)
+    ref = torch.nn.functional.scaled_dot_product_attention(Q.double().cpu(), K.double().cpu(), V.double().cpu())
+    assert_close(O.cpu().numpy(), ref.numpy(), what="full pattern O")
+    assert_close(P.view(NB, L, L).sum(-1).cpu().numpy(), np.ones((NB, L)), what="row sums")
+    abi.close()
+
+
+@pytest.mark.parametrize("d", [32, 64])
+def test_tile_path_with_key_mask(d):
+    L, bs, B, H = 256, 32, 3, 2
+    NB = B * H
+    mat = _random_block_mask(L // bs, 0.35, seed=8)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    key_mask = np.ones((B, L), np.float32)
+    key_mask[0, 200:] = 0
+    key_mask[1, 77:] = 0       # not tile aligned
+    pen = torch.from_numpy(osa.key_penalty_from_mask(key_mask, H)).cuda()
+    abi = SparseABI(d, L, NB, bs, with_mask=True)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=4)
+    got, _ = run_and_check(abi, Q, K, V, dO, penalty=pen, tag="key mask")
+    # probabilities of padded keys are exactly zero
+    rows = osa.csr_row_index(off)
+    padded = torch.from_numpy(col.astype(np.int64) >= 77).cuda()
+    assert (got["P"][2][padded] == 0).all() and (got["P"][3][padded] == 0).all()
+    abi.close()
+
+
+def test_row_sum_invariant_large_logits_and_guard():
+    # logits of +-30: exp range exercised; every row still obeys sum P = 1 - (L-n) e^{-m} / Z
+    L, bs, d, NB = 128, 32, 32, 2
+    mat = _random_block_mask(4, 0.5, seed=9)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=6, scale=3.0)
+    run_and_check(abi, Q, K, V, dO, tag="large logits")
+    # every logit below -88.7 -> denominator overflows in fp32 -> P == 0 exactly (reference guard)
+    Q2 = torch.full_like(Q, 8.0)
+    K2 = torch.full_like(K, -8.0)          # q.k/sqrt(32) = -362
+    O, P = abi.forward(Q2, K2, V)
+    sparse_rows = torch.from_numpy(np.repeat(sm < L, sm)).cuda()
+    assert (P[:, sparse_rows] == 0).all()
+    abi.close()
+
+
+# ---------------------------------------------------------------------------------- element path
+def _random_element_csr(L, p, seed, empty_row=None):
+    rng = np.random.default_rng(seed)
+    pat = rng.random((L, L)) < p
+    pat[np.arange(L), np.arange(L)] = True
+    if empty_row is not None:
+        pat[empty_row, :] = False
+    return osa.csr_from_dense_pattern(pat)
+
+
+@pytest.mark.parametrize("L,d,NB,p", [(96, 32, 3, 0.2), (100, 16, 2, 0.5), (160, 64, 2, 0.9), (70, 128, 2, 0.3)])
+def test_element_path_matches_oracle(L, d, NB, p):
+    sm, off, col = _random_element_csr(L, p, seed=L + d, empty_row=7)
+    abi = SparseABI(d, L, NB, 1, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=10, scale=1.2)
+    got, _ = run_and_check(abi, Q, K, V, dO, tag=f"element L={L} d={d}")
+    assert abi.last_path() == 2
+    assert (got["O"][:, 7] == 0).all() and (got["dQ"][:, 7] == 0).all()
+    abi.close()
+
+
+def test_element_path_with_key_mask():
+    L, d, B, H = 192, 32, 2, 2
+    sm, off, col = _random_element_csr(L, 0.25, seed=21)
+    key_mask = np.ones((B, L), np.float32)
+    key_mask[0, 150:] = 0
+    key_mask[1, 31:] = 0
+    pen = torch.from_numpy(osa.key_penalty_from_mask(key_mask, H)).cuda()
+    abi = SparseABI(d, L, B * H, 1, with_mask=True)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(B * H, L, d, seed=11)
+    run_and_check(abi, Q, K, V, dO, penalty=pen, tag="element key mask")
+    abi.close()
+
+
+def test_tile_and_element_paths_agree():
+    """Two independent kernel families on the same block pattern."""
+    L, bs, d, NB = 512, 32, 32, 4
+    mat = _random_block_mask(L // bs, 0.2, seed=31)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    Q, K, V, dO = _inputs(NB, L, d, seed=12)
+    res = []
+    for force in (False, True):
+        abi = SparseABI(d, L, NB, bs, with_mask=False)
+        abi.force_element(force)
+        abi.set_pattern(sm, off, col)
+        O, P = abi.forward(Q, K, V)
+        dQ, dK, dV = abi.backward(Q, K, V, P, dO)
+        assert abi.last_path() == (2 if force else 1)
+        res.append([t.cpu().numpy() for t in (O, P, dQ, dK, dV)])
+        abi.close()
+    for a, b, name in zip(res[0], res[1], ["O", "P", "dQ", "dK", "dV"]):
+        assert_close(a, b, what=f"tile vs element {name}")
+
+
+# ---------------------------------------------------------------------------------- benchmark configurations
+def test_config1_block_sparse_l1024():
+    """B=8, H=2, L=1024, d=32, 32x32 blocks, band of 3 + 5 % random blocks; inputs N(0,1)/sqrt(32)."""
+    B, H, L, d, bs = 8, 2, 1024, 32, 32
+    mat = workloads.config1_mask()
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    q, k, v, do = workloads.qkv(B, H, L, d, scale=1.0 / np.sqrt(32.0), seed=0, device="cuda")
+    abi = SparseABI(d, L, B * H, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    f = lambda t: t.reshape(B * H, L, d).contiguous()
+    run_and_check(abi, f(q), f(k), f(v), f(do), tag="config 1")
+    assert abi.last_path() == 1
+    abi.close()
+
+
+def test_config4_element_sparse_small_heads():
+    """Config 4 shape (L=4096, d=32, window +-64 plus random columns to 5 %, key padding) on 2x2 heads."""
+    B, H, L, d = 2, 2, 4096, 32
+    sm, off, col = workloads.window_random_csr(L, 64, 205, seed=3)
+    key_mask = workloads.valid_length_mask(B, L, 2048, 4096, seed=5)
+    pen = torch.from_numpy(osa.key_penalty_from_mask(key_mask.numpy(), H)).cuda()
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=0, device="cuda")
+    abi = SparseABI(d, L, B * H, 1, with_mask=True)
+    abi.set_pattern(sm, off, col)
+    f = lambda t: t.reshape(B * H, L, d).contiguous()
+    run_and_check(abi, f(q), f(k), f(v), f(do), penalty=pen, tag="config 4")
+    assert abi.last_path() == 2
+    abi.close()
+
+
+def test_north_star_shape_properties():
+    """L=4096, H=2, d=32, 10 % block density at the benchmark batch: size-independent checks
+    (row-sum invariant, linearity of the backward in dO, tile path == element path on one head pair)
+    plus the oracle on two of the 64 heads."""
+    B, H, L, d, bs = 32, 2, 4096, 32, 32
+    NB = B * H
+    mat = workloads.north_star_mask(bs)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=0, device="cuda")
+    f = lambda t: t.reshape(NB, L, d).contiguous()
+    Q, K, V, dO = f(q), f(k), f(v), f(do)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    O, P = abi.forward(Q, K, V)
+    dQ, dK, dV = abi.backward(Q, K, V, P, dO)
+    assert abi.last_path() == 1
+    # (a) oracle on heads 0 and 63
+    from tests.abi_utils import oracle_fwd_bwd
+    for hsel in (0, NB - 1):
+        s = slice(hsel, hsel + 1)
+        ref = oracle_fwd_bwd(Q[s], K[s], V[s], dO[s], sm, off, col)
+        for name, got in (("O", O), ("P", P), ("dQ", dQ), ("dK", dK), ("dV", dV)):
+            assert_close(got[s].cpu().numpy(), ref[name], what=f"north star head {hsel} {name}")
+    # (b) rows of P sum to less than one and are non-negative; all finite
+    rows = torch.from_numpy(osa.csr_row_index(off)).cuda()
+    rs = torch.zeros(NB, L, device="cuda").index_add_(1, rows, P)
+    assert torch.isfinite(P).all() and (P >= 0).all() and (rs <= 1 + 1e-5).all() and (rs > 0).all()
+    # (c) the backward is linear in dO
+    dQ2, dK2, dV2 = abi.backward(Q, K, V, P, 2.0 * dO)
+    for a, b in ((dQ, dQ2), (dK, dK2), (dV, dV2)):
+        assert torch.allclose(2.0 * a, b, rtol=1e-5, atol=1e-5)
+    abi.close()
+    # (d) element path on the first 4 heads agrees with the tile path
+    abi2 = SparseABI(d, L, 4, bs, with_mask=False)
+    abi2.force_element(True)
+    abi2.set_pattern(sm, off, col)
+    O2, P2 = abi2.forward(Q[:4], K[:4], V[:4])
+    e = abi2.backward(Q[:4], K[:4], V[:4], P2, dO[:4])
+    assert abi2.last_path() == 2
+    for a, b, name in ((O[:4], O2, "O"), (P[:4], P2, "P"), (dQ[:4], e[0], "dQ"), (dK[:4], e[1], "dK"), (dV[:4], e[2], "dV")):
+        assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"north star tile vs element {name}")
+    abi2.close()
+
+
+# ---------------------------------------------------------------------------------- module level (autograd)
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_block_modules_autograd_match_dense_statement(with_mask):
+    import spion_amd
+
+    B, H, L, d, bs = 2, 2, 256, 32, 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    mat_np = _random_block_mask(L // bs, 0.3, seed=41)
+    mat = torch.from_numpy(mat_np).cuda()
+    if with_mask:
+        cpp = spion_amd.Attention._blockcuda_mask_compile_module()
+        mod = spion_amd.CUDABlockMaskAttention(cfg, cpp, cpp.init(d, L, B * H, bs))
+    else:
+        cpp = spion_amd.Attention._blockcuda_compile_module()
+        mod = spion_amd.CUDABlockAttention(cfg, cpp, cpp.init(d, L, B * H, bs))
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=3, device="cuda")
+    key_mask = torch.ones(B, L)
+    if with_mask:
+        key_mask[0, 100:] = 0
+    for t in (q, k, v):
+        t.requires_grad_()
+    for it in range(2):  # second call goes through the CSR cache
+        out, attn = mod(q, k, v, key_mask.cuda(), mat)
+        out.backward(do)
+    if with_mask:
+        assert attn == 0
+    else:
+        assert attn.shape == (B * H * int(mat_np.sum()) * bs * bs,)
+    qc, kc, vc = (t.detach().double().cpu().requires_grad_() for t in (q, k, v))
+    pat = torch.from_numpy(np.repeat(np.repeat(mat_np, bs, 0), bs, 1)).double()
+    O, _ = osa.dense_masked_attention(qc, kc, vc, pat, key_mask.double() if with_mask else None)
+    O.backward(do.double().cpu())
+    assert_close(out.detach().cpu().numpy(), O.detach().numpy(), what="module out")
+    for name, a, b in (("dq", q, qc), ("dk", k, kc), ("dv", v, vc)):
+        assert_close(a.grad.cpu().numpy() / 2.0, b.grad.numpy(), what=f"module {name}")  # two backward passes accumulated
+
+
+# ---------------------------------------------------------------------------------- error handling (host side)
+def test_inconsistent_csr_is_reported_not_launched():
+    from spion_amd import _lib
+
+    L, d, NB = 64, 32, 1
+    abi = SparseABI(d, L, NB, 32, with_mask=False)
+    sm, off, col = osa.build_csr_from_block_mask(np.eye(2, dtype=np.float32), 32)
+    bad = col.copy()
+    bad[5] = 9999
+    abi.set_pattern(sm, off, bad)
+    Q, K, V, dO = _inputs(NB, L, d, seed=1)
+    with pytest.raises(_lib.SpionLibraryError, match="out of range"):
+        abi.forward(Q, K, V)
+    off2 = off.copy()
+    off2[-1] += 1
+    abi.set_pattern(sm, off2, col)
+    abi.nnz = int(off[-1])
+    with pytest.raises(_lib.SpionLibraryError, match="do not match"):
+        abi.forward(Q, K, V)
+    abi.close()
