@@ -124,6 +124,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="north_star")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy a few times (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -135,6 +137,14 @@ def main():
     import spion_amd
     from spion_amd import _lib, workloads
     from spion_amd.attention import Attention
+
+    if args.copy_probe:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)  # 256 MiB read + 256 MiB written
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     wl = build_workload(args.workload)
     B, H, L, d, bs, nnz = wl["B"], wl["H"], wl["L"], wl["d"], wl["bs"], wl["nnz"]
