@@ -160,6 +160,12 @@ void spion_force_element_path(void* handle, int on);
  * bit 1 = column pass (dK, dV; needs the row sums of an earlier row pass).  Default 3 = both. */
 void spion_set_backward_passes(void* handle, int mask);
 
+/* The forward of the MFMA tile path keeps a private copy of Out, filed under the Attn pointer it filled
+ * (up to 4 per handle, NB*L*d floats each); a backward given the same P pointer then gets its softmax
+ * row sums from dO.Out in one step.  on = 0 switches the copies off (the backward then recomputes the
+ * row sums with one more sweep over the tiles); default on. */
+void spion_use_output_cache(void* handle, int on);
+
 const char* spion_version(void);
 
 #ifdef __cplusplus

@@ -60,6 +60,8 @@ def core() -> ctypes.CDLL:
     lib.spion_force_element_path.restype = None
     lib.spion_set_backward_passes.argtypes = [_P, c_int]
     lib.spion_set_backward_passes.restype = None
+    lib.spion_use_output_cache.argtypes = [_P, c_int]
+    lib.spion_use_output_cache.restype = None
     lib.spion_version.restype = c_char_p
     lib.spion_version.argtypes = []
     lib.spion_pattern_generate.argtypes = [_P, c_int, c_int, c_int, c_int, c_int, c_double, _P, _P, _P, _P]

@@ -32,6 +32,7 @@ void sparse_invalidate(void*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
+void sparse_use_ocache(void*, int);
 void* dense_init(int, int, int, bool);
 void dense_destroy(void*);
 void dense_forward(void*, const float*, const float*, const float*, const float*, float*, float*, bool);
@@ -144,6 +145,7 @@ void spion_invalidate_pattern(void* h) { sparse_invalidate(h); }
 int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
+void spion_use_output_cache(void* h, int on) { sparse_use_ocache(h, on); }
 const char* spion_version(void) { return "spion_hip 0.1 (gfx950)"; }
 
 }  // extern "C"

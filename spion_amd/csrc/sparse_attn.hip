@@ -13,11 +13,12 @@
 // Semantics follow the reference kernels (models/block_attn.cu:33-130, models/block_attn_mask.cu:88-173):
 // the softmax denominator counts every off-pattern key with logit 0.
 #include "common.h"
-#include "tile_ops.h"
+#include "tile_kernels.h"
 #include "../../include/spion_hip.h"
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <vector>
 
 namespace spion {
@@ -224,216 +225,6 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
 }
 
 // =================================================================================================
-// tile path (MFMA); the operand conventions are described in tile_ops.h
-// =================================================================================================
-// Forward, one work-group per (head, block row): sweep 1 finds the row maxima and denominators
-// (online over the tiles), sweep 2 recomputes the logits, writes P and accumulates O = P.V.
-template <int D, int WAVES, bool MASK>
-__global__ __launch_bounds__(64 * WAVES) void tile_fwd_kernel(
-    const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
-    const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
-    const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
-    int NB, int nnz, float scale) {
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
-    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
-    const int rn = cnt * 32;
-    const size_t hb = (size_t)bh * L * D;
-    const float* Kth = Kt + hb;
-    const float* penh = MASK ? pen + (size_t)bh * L : nullptr;
-    float* Prow = P + (size_t)bh * nnz + offs[I * 32] + (size_t)li * rn + 4 * h;
-
-    float q[D / 2];
-    load_rows<D>(Q + hb, I * 32, li, h, q);
-
-    float m = MASK ? 0.f : -100.f, z = 0.f;
-    for (int t = w; t < cnt; t += WAVES) {
-        const int J = tcol[t0 + t];
-        float k[D / 2];
-        load_cols<D>(Kth, L, J * 32, li, h, k);
-        f32x16 s = mma_feat<D>(k, q);  // s[r] = q_i . k_j, i = I*32+li, j = J*32+acc_row(r,h)
-        float v[16], tm = m;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            v[r] = s[r] * scale;
-            if (MASK) v[r] -= penh[J * 32 + acc_row(r, h)];
-            tm = fmaxf(tm, v[r]);
-        }
-        float zz = 0.f;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) zz += __expf(v[r] - tm);
-        z = z * __expf(m - tm) + zz;
-        m = tm;
-    }
-    {   // merge the two half-waves, then the waves, of every row
-        float m2 = __shfl_xor(m, 32, 64), z2 = __shfl_xor(z, 32, 64);
-        float M = fmaxf(m, m2);
-        z = z * __expf(m - M) + z2 * __expf(m2 - M);
-        m = M;
-        if (WAVES > 1) {
-            if (h == 0) {
-                lds_m[w][li] = m;
-                lds_z[w][li] = z;
-            }
-            __syncthreads();
-            float Mx = lds_m[0][li];
-#pragma unroll
-            for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
-            float Z = 0.f;
-#pragma unroll
-            for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __expf(lds_m[ww][li] - Mx);
-            m = Mx;
-            z = Z;
-        }
-    }
-    z += (float)(L - rn) * __expf(-m);
-    const float rinv = 1.0f / z;  // +inf denominator -> 0 -> P = 0, as in the reference
-
-    f32x16 o[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) o[c] = (f32x16){0};
-    for (int t = w; t < cnt; t += WAVES) {
-        const int J = tcol[t0 + t];
-        float k[D / 2];
-        load_cols<D>(Kth, L, J * 32, li, h, k);
-        f32x16 s = mma_feat<D>(k, q);
-        float p[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float v = s[r] * scale;
-            if (MASK) v -= penh[J * 32 + acc_row(r, h)];
-            p[r] = __expf(v - m) * rinv;
-        }
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-            *reinterpret_cast<float4*>(Prow + t * 32 + 8 * g) =
-                make_float4(p[4 * g], p[4 * g + 1], p[4 * g + 2], p[4 * g + 3]);
-        mma_tile<D>(p, V + hb, J * 32, li, h, o);
-    }
-    reduce_store<D, WAVES>(o, O + hb, I * 32, w, li, h, lds);
-}
-
-// Backward, row pass, one work-group per (head, block row): g_i = sum_j dP_ij P_ij (kept in G for the
-// column pass), dS = (dP*P - P*g)*scale, dQ = dS.K.
-template <int D, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void tile_bwd_row_kernel(
-    const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
-    const float* __restrict__ dO, float* __restrict__ G, float* __restrict__ dQ, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    __shared__ float lds_g[WAVES][32];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
-    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
-    const int rn = cnt * 32;
-    const size_t hb = (size_t)bh * L * D;
-    const float* Vth = Vt + hb;
-    const float* Prow = P + (size_t)bh * nnz + offs[I * 32] + (size_t)li * rn + 4 * h;
-
-    float go[D / 2];
-    load_rows<D>(dO + hb, I * 32, li, h, go);
-
-    float g = 0.f;
-    for (int t = w; t < cnt; t += WAVES) {
-        const int J = tcol[t0 + t];
-        float vt[D / 2];
-        load_cols<D>(Vth, L, J * 32, li, h, vt);
-        f32x16 dp = mma_feat<D>(vt, go);  // dp[r] = dO_i . v_j
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            float4 pv = *reinterpret_cast<const float4*>(Prow + t * 32 + 8 * q4);
-            g = fmaf(dp[4 * q4], pv.x, g);
-            g = fmaf(dp[4 * q4 + 1], pv.y, g);
-            g = fmaf(dp[4 * q4 + 2], pv.z, g);
-            g = fmaf(dp[4 * q4 + 3], pv.w, g);
-        }
-    }
-    g += __shfl_xor(g, 32, 64);
-    if (WAVES > 1) {
-        if (h == 0) lds_g[w][li] = g;
-        __syncthreads();
-        g = 0.f;
-#pragma unroll
-        for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
-    }
-    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = g;
-
-    f32x16 acc[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) acc[c] = (f32x16){0};
-    for (int t = w; t < cnt; t += WAVES) {
-        const int J = tcol[t0 + t];
-        float vt[D / 2];
-        load_cols<D>(Vth, L, J * 32, li, h, vt);
-        f32x16 dp = mma_feat<D>(vt, go);
-        float ds[16];
-#pragma unroll
-        for (int q4 = 0; q4 < 4; ++q4) {
-            float4 pv = *reinterpret_cast<const float4*>(Prow + t * 32 + 8 * q4);
-            ds[4 * q4] = (dp[4 * q4] * pv.x - pv.x * g) * scale;
-            ds[4 * q4 + 1] = (dp[4 * q4 + 1] * pv.y - pv.y * g) * scale;
-            ds[4 * q4 + 2] = (dp[4 * q4 + 2] * pv.z - pv.z * g) * scale;
-            ds[4 * q4 + 3] = (dp[4 * q4 + 3] * pv.w - pv.w * g) * scale;
-        }
-        mma_tile<D>(ds, K + hb, J * 32, li, h, acc);
-    }
-    reduce_store<D, WAVES>(acc, dQ + hb, I * 32, w, li, h, lds);
-}
-
-// Backward, column pass, one work-group per (head, block column): dK_J = sum_I dS_IJ^T Q_I,
-// dV_J = sum_I P_IJ^T dO_I, walking the transposed tile index.
-template <int D, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void tile_bwd_col_kernel(
-    const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
-    const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
-    const int* __restrict__ trp, const int* __restrict__ tcp, const int* __restrict__ tcrow,
-    const int* __restrict__ tcord, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, J = item % nbr;
-    const int w = threadIdx.x >> 6, l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
-    const size_t hb = (size_t)bh * L * D;
-    const float* Ph = P + (size_t)bh * nnz;
-    const float* Gh = G + (size_t)bh * L;
-
-    float vt[D / 2];
-    load_cols<D>(Vt + hb, L, J * 32, li, h, vt);
-
-    f32x16 ak[D / 32], av[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) {
-        ak[c] = (f32x16){0};
-        av[c] = (f32x16){0};
-    }
-    for (int e = w; e < cnt; e += WAVES) {
-        const int I = tcrow[e0 + e], ord = tcord[e0 + e];
-        const int rn = (trp[I + 1] - trp[I]) * 32;
-        float go[D / 2];
-        load_rows<D>(dO + hb, I * 32, li, h, go);
-        f32x16 dp = mma_feat<D>(go, vt);  // dp[r] = dO_i . v_j, i = I*32+acc_row(r,h), j = J*32+li
-        const float* pt = Ph + offs[I * 32] + ord * 32 + li;
-        float p[16], ds[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int ir = acc_row(r, h);
-            p[r] = pt[(size_t)ir * rn];
-            const float g = Gh[I * 32 + ir];
-            ds[r] = (dp[r] * p[r] - p[r] * g) * scale;
-        }
-        mma_tile<D>(ds, Q + hb, I * 32, li, h, ak);
-        mma_tile<D>(p, dO + hb, I * 32, li, h, av);
-    }
-    reduce_store<D, WAVES>(ak, dK + hb, J * 32, w, li, h, lds);
-    if (WAVES > 1) __syncthreads();
-    reduce_store<D, WAVES>(av, dV + hb, J * 32, w, li, h, lds);
-}
-
-// =================================================================================================
 // host side
 // =================================================================================================
 struct PatternIndex {
@@ -460,6 +251,19 @@ struct SparseAttn {
     float scale;
     PatternIndex pat;
     float* ws_rowsum = nullptr;  // [NB][L]   g of the backward (tile path)
+    // Copies of O kept by the forward of the tile path, keyed by the Attn (P) buffer that forward
+    // filled: a backward that is handed the same P pointer gets its row sums g_i = dO_i . O_i from the
+    // copy in one cheap step instead of a sweep over all tiles.  The key is sound because a forward that
+    // overwrites a P buffer also overwrites the copy filed under it; an unknown P pointer simply takes the
+    // two-sweep kernel.
+    static constexpr int O_SLOTS = 4;
+    struct OSlot {
+        const float* key = nullptr;
+        float* buf = nullptr;
+        uint64_t stamp = 0;
+    } oslot[O_SLOTS];
+    uint64_t ostamp = 0;
+    bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
     int last_path = 0;
     bool force_element = false;
@@ -506,6 +310,8 @@ void sparse_destroy(void* h) {
     a->pat.release();
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
+    for (auto& sl : a->oslot)
+        if (sl.buf) (void)hipFree(sl.buf);
     a->hdr.magic = 0;
     delete a;
 }
@@ -656,10 +462,42 @@ static bool ensure_ws(float** p, size_t count) {
     return SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * count));
 }
 
+// Slot of the O copy for the forward that fills P buffer `key` (least recently used slot on a miss).
+static float* ocache_for_forward(SparseAttn* a, const float* key) {
+    if (!a->use_ocache) return nullptr;
+    SparseAttn::OSlot* pick = nullptr;
+    for (auto& sl : a->oslot)
+        if (sl.key == key) pick = &sl;
+    if (!pick) {
+        pick = &a->oslot[0];
+        for (auto& sl : a->oslot)
+            if (sl.stamp < pick->stamp) pick = &sl;
+    }
+    if (!pick->buf && hipMalloc((void**)&pick->buf, sizeof(float) * (size_t)a->NB * a->L * a->d) != hipSuccess) {
+        (void)hipGetLastError();  // no copy: the backward falls back to the two-sweep kernel
+        pick->buf = nullptr;
+        pick->key = nullptr;
+        return nullptr;
+    }
+    pick->key = key;
+    pick->stamp = ++a->ostamp;
+    return pick->buf;
+}
+static const float* ocache_for_backward(SparseAttn* a, const float* key) {
+    if (!a->use_ocache) return nullptr;
+    for (auto& sl : a->oslot)
+        if (sl.key == key && sl.buf) return sl.buf;
+    return nullptr;
+}
+
 static int pick_waves(const PatternIndex& pi, int nbr, bool by_col) {
     // average tiles per strip decides how many wavefronts share one strip
     const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
     (void)by_col;
+    if (const char* e = getenv("SPION_TILE_WAVES")) {
+        const int v = atoi(e);
+        if (v == 1 || v == 2 || v == 4) return v;
+    }
     if (avg <= 1) return 1;
     if (avg <= 3) return 2;
     return 4;
@@ -672,9 +510,18 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
     const int wv = pick_waves(pi, nbr, false);
+    float* ocache = ocache_for_forward(a, P);
+    // logit tiles stay in registers when every wavefront's share of the longest block row fits
+    constexpr int MAXT = D == 32 ? 8 : 4;
 #define SPION_LAUNCH(W)                                                                                             \
-    hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V, pen, P, O,    \
-                       pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale)
+    do {                                                                                                            \
+        if (pi.max_row_tiles <= W * MAXT)                                                                           \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V, \
+                               pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);      \
+        else                                                                                                        \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V,    \
+                               pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);      \
+    } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
     else SPION_LAUNCH(4);
@@ -688,11 +535,17 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
     const int wv = pick_waves(pi, nbr, false);
+    const float* ocache = ocache_for_backward(a, P);
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
-        if (a->bwd_passes & 1)                                                                                      \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P, dO,     \
-                               a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);       \
+        if ((a->bwd_passes & 1) && ocache)                                                                          \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,   \
+                               dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
+                               a->scale);                                                                           \
+        else if (a->bwd_passes & 1)                                                                                 \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,  \
+                               dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
+                               a->scale);                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
                                a->ws_rowsum, dK, dV, pi.d_trp, pi.d_tcp, pi.d_tcrow, pi.d_tcord, offs, a->L, nbr,   \
@@ -820,6 +673,12 @@ int sparse_last_path(void* h) {
 void sparse_set_bwd_passes(void* h, int mask) {
     SparseAttn* a = as_sparse(h, "spion_set_backward_passes");
     if (a) a->bwd_passes = mask & 3;
+}
+void sparse_use_ocache(void* h, int on) {
+    SparseAttn* a = as_sparse(h, "spion_use_output_cache");
+    if (!a) return;
+    a->use_ocache = on != 0;
+    for (auto& sl : a->oslot) sl.key = nullptr;
 }
 void sparse_force_element(void* h, int on) {
     SparseAttn* a = as_sparse(h, "spion_force_element_path");

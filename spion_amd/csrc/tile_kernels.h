@@ -1,0 +1,474 @@
+// MFMA tile kernels of the sparse path (forward, backward row pass, backward column pass).
+//
+// What shapes these kernels (measured on MI355X): an fp32 MFMA and ordinary vector-ALU instructions
+// do not overlap on a SIMD -- every VALU instruction adds its ~4-5 cycles (v_exp_f32 ~13) to the 64 cycles
+// of each v_mfma_f32_32x32x2_f32 -- while memory instructions issue for free.  So the kernels
+//   * do all addressing in scalar registers: buffer loads/stores with a per-head resource, one lane
+//     offset computed once per kernel and a scalar byte offset per tile;
+//   * fold constants into the MFMA chain instead of touching every element afterwards: the row maximum
+//     (forward) or the softmax row sum g (backward) enters as the chain's initial accumulator, the
+//     1/sqrt(d)*log2(e) factor is folded into Q once per work-group, the 1/sqrt(d) of the gradients is
+//     applied once to the 32 x d result instead of to every tile;
+//   * software-pipeline each wavefront's tile list (operands of the next tile are requested before the
+//     current MFMA chain starts).
+#pragma once
+#include "tile_ops.h"
+
+namespace spion {
+
+#define SPION_TILE_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2)))
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+// Raw buffer resource over [p, p + bytes): out-of-range loads return 0, stores are dropped.
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
+    const unsigned n = bytes > 0xfffffff0ull ? 0xfffffff0u : (unsigned)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)n, 0x00020000);
+}
+__device__ __forceinline__ float ld1(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ f32x4 ld4(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ void st4(rsrc_t r, int voff, int soff, f32x4 v) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
+}
+
+// Operand over the head dimension from a row-major [.][D] head slice: D/2 consecutive floats per lane.
+// voff = ((lane%32)*D + (lane/32)*(D/2))*4 bytes, soff = byte offset of the tile's first row.
+template <int D>
+__device__ __forceinline__ void ldr_rows(rsrc_t r, int voff, int soff, float (&x)[D / 2]) {
+#pragma unroll
+    for (int q = 0; q < D / 8; ++q) {
+        f32x4 v = ld4(r, voff, soff + 16 * q);
+        x[4 * q + 0] = v.x;
+        x[4 * q + 1] = v.y;
+        x[4 * q + 2] = v.z;
+        x[4 * q + 3] = v.w;
+    }
+}
+// Same operand from a feature-major [D][L] head slice.  voff = ((lane/32)*(D/2)*L + lane%32)*4,
+// soff = byte offset of the tile's first column.
+template <int D>
+__device__ __forceinline__ void ldr_cols(rsrc_t r, int L, int voff, int soff, float (&x)[D / 2]) {
+#pragma unroll
+    for (int s = 0; s < D / 2; ++s) x[s] = ld1(r, voff, soff + s * L * 4);
+}
+// B operand of a product over a tile's 32 rows from a row-major [.][D] head slice: slot (s, h) = tile row
+// acc_row(s, h).  voff = (4*(lane/32)*D + lane%32)*4, soff = byte offset of the tile's first row.
+template <int D>
+__device__ __forceinline__ void ldr_tile_b(rsrc_t r, int voff, int soff, float (&x)[D / 32][16]) {
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[c][s] = ld1(r, voff, soff + ((8 * (s >> 2) + (s & 3)) * D + c * 32) * 4);
+}
+// 16 floats per lane laid out as 4 groups of 4 consecutive floats 8 apart (accumulator rows of one lane).
+__device__ __forceinline__ void ldr_4x4(rsrc_t r, int voff, int soff, float (&x)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        f32x4 v = ld4(r, voff, soff + 32 * g);
+        x[4 * g + 0] = v.x;
+        x[4 * g + 1] = v.y;
+        x[4 * g + 2] = v.z;
+        x[4 * g + 3] = v.w;
+    }
+}
+__device__ __forceinline__ void str_4x4(rsrc_t r, int voff, int soff, const float (&x)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) st4(r, voff, soff + 32 * g, (f32x4){x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]});
+}
+
+// acc = init + A.B over the head dimension (chain of D/2 MFMA).
+template <int D>
+__device__ __forceinline__ f32x16 mma_feat_init(const float (&a)[D / 2], const float (&b)[D / 2], f32x16 init) {
+    f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], init, 0, 0, 0);
+#pragma unroll
+    for (int s = 1; s < D / 2; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+    return acc;
+}
+template <int D>
+__device__ __forceinline__ void mma_b(const float (&w)[16], const float (&x)[D / 32][16], f32x16 (&out)[D / 32]) {
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+        for (int s = 0; s < 16; ++s) out[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(w[s], x[c][s], out[c], 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 splat16(float v) {
+    return (f32x16){v, v, v, v, v, v, v, v, v, v, v, v, v, v, v, v};
+}
+__device__ __forceinline__ float max16(const f32x16& s, float m) {
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) m = fmaxf(fmaxf(s[r], s[r + 1]), m);
+    return m;
+}
+
+// Merge per-lane (max, sum-of-exp2) pairs of a row: the two half-waves, then the waves of the work-group.
+template <int WAVES>
+__device__ __forceinline__ void merge_max_sum(float& m, float& z, int w, int h, int li, float (*lds_m)[32],
+                                              float (*lds_z)[32]) {
+    float m2 = __shfl_xor(m, 32, 64), z2 = __shfl_xor(z, 32, 64);
+    float M = fmaxf(m, m2);
+    z = z * __builtin_amdgcn_exp2f(m - M) + z2 * __builtin_amdgcn_exp2f(m2 - M);
+    m = M;
+    if (WAVES > 1) {
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
+        float Mx = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+        m = Mx;
+        z = Z;
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward, one work-group per (head, block row).  Logits are kept in the log2 domain:
+// s' = (q.k) * log2(e)/sqrt(d) (- penalty*log2(e)), P = exp2(s' - m') / Z.
+//
+// MAXT > 0: every wavefront keeps the logit tiles of its share of the block row in registers (at most
+// MAXT tiles), so each tile costs one QK^T chain and one PV chain.  MAXT == 0: two sweeps, the second
+// recomputing the logits (any row length).  Ocache (optional): second copy of O for the backward.
+// -------------------------------------------------------------------------------------------------
+template <int D, int WAVES, bool MASK, int MAXT>
+SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
+    const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
+    const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
+    const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
+    int NB, int nnz, float scale) {
+    constexpr int KH = D / 2;
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int rn = cnt * 32;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(Kt + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int p_base = offs[I * 32] * 4;
+    const int p_voff = (li * rn + 4 * h) * 4;
+    const int col_voff = (h * KH * L + li) * 4;
+    const int b_voff = (4 * h * D + li) * 4;
+    const int m_voff = 16 * h;
+    const float c2 = scale * LOG2E;
+
+    float q[KH];
+    ldr_rows<D>(rQ, (li * D + h * KH) * 4, I * 32 * D * 4, q);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) q[s] *= c2;
+
+    // initial accumulator of a logit chain: minus the key penalties of the tile, in the log2 domain
+    auto chain_init = [&](int J) -> f32x16 {
+        if (!MASK) return splat16(0.f);
+        float pj[16];
+        ldr_4x4(rM, m_voff, J * 128, pj);
+        f32x16 v;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = -LOG2E * pj[r];
+        return v;
+    };
+
+    float m = MASK ? 0.f : -100.f * LOG2E, z = 0.f;
+    f32x16 o[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
+
+    if constexpr (MAXT > 0) {
+        const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
+        f32x16 S[MAXT];
+        float kbuf[2][KH];
+        if (nu > 0) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, kbuf[0]);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                const int t = w + u * WAVES;
+                if (u + 1 < nu) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kbuf[(u + 1) & 1]);
+                S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(tcol[t0 + t]));
+                m = max16(S[u], m);
+            }
+        }
+        {   // row maximum over half-waves and waves
+            m = fmaxf(m, __shfl_xor(m, 32, 64));
+            if (WAVES > 1) {
+                if (h == 0) lds_m[w][li] = m;
+                __syncthreads();
+#pragma unroll
+                for (int ww = 0; ww < WAVES; ++ww) m = fmaxf(m, lds_m[ww][li]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float e = __builtin_amdgcn_exp2f(S[u][r] - m);
+                    S[u][r] = e;
+                    z += e;
+                }
+            }
+        }
+        z += __shfl_xor(z, 32, 64);
+        if (WAVES > 1) {
+            if (h == 0) lds_z[w][li] = z;
+            __syncthreads();
+            z = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < WAVES; ++ww) z += lds_z[ww][li];
+        }
+        z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
+        const float rinv = 1.0f / z;  // +inf denominator -> 0 -> P = 0, as in the reference
+
+        float vbuf[2][D / 32][16];
+        if (nu > 0) ldr_tile_b<D>(rV, b_voff, tcol[t0 + w] * 32 * D * 4, vbuf[0]);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                const int t = w + u * WAVES;
+                if (u + 1 < nu) ldr_tile_b<D>(rV, b_voff, tcol[t0 + t + WAVES] * 32 * D * 4, vbuf[(u + 1) & 1]);
+                float p[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                str_4x4(rP, p_voff, p_base + t * 128, p);
+                mma_b<D>(p, vbuf[u & 1], o);
+            }
+        }
+    } else {
+        // ---- sweep 1: online row maximum and denominator -------------------------------------------
+        {
+            auto body = [&](float (&kc)[KH], float (&kn)[KH], int t) {
+                if (t + WAVES < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kn);
+                f32x16 s = mma_feat_init<D>(kc, q, chain_init(tcol[t0 + t]));
+                const float tm = max16(s, m);
+                float zz = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) zz += __builtin_amdgcn_exp2f(s[r] - tm);
+                z = z * __builtin_amdgcn_exp2f(m - tm) + zz;
+                m = tm;
+            };
+            float ka[KH], kb[KH];
+            if (w < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, ka);
+            for (int t = w; t < cnt; t += 2 * WAVES) {
+                body(ka, kb, t);
+                if (t + WAVES < cnt) body(kb, ka, t + WAVES);
+            }
+        }
+        merge_max_sum<WAVES>(m, z, w, h, li, lds_m, lds_z);
+        z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
+        const float rinv = 1.0f / z;
+        // ---- sweep 2: logits again (minus the row maximum, folded into the chain), P, O ------------
+        {
+            auto body = [&](float (&kc)[KH], float (&kn)[KH], int t) {
+                const int J = tcol[t0 + t];
+                float vb[D / 32][16];
+                ldr_tile_b<D>(rV, b_voff, J * 32 * D * 4, vb);
+                if (t + WAVES < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kn);
+                f32x16 init = chain_init(J);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] -= m;
+                f32x16 s = mma_feat_init<D>(kc, q, init);
+                float p[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
+                str_4x4(rP, p_voff, p_base + t * 128, p);
+                mma_b<D>(p, vb, o);
+            };
+            float ka[KH], kb[KH];
+            if (w < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, ka);
+            for (int t = w; t < cnt; t += 2 * WAVES) {
+                body(ka, kb, t);
+                if (t + WAVES < cnt) body(kb, ka, t + WAVES);
+            }
+        }
+    }
+    if (Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);
+    else reduce_store<D, WAVES>(o, O + hb, I * 32, w, li, h, lds);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, row pass.  HAVE_O: the handle kept O of the matching forward, so g_i = dO_i . O_i is known up
+// front; otherwise a first sweep accumulates g_i = sum_j dP_ij P_ij.  Main sweep per tile:
+// dP^T - g = V_J.dO_I^T chain started from -g, dS' = (dP - g)*P, dQ += dS'.K_J; the 1/sqrt(d) is applied to
+// the 32 x d result.  G receives -g for the column pass.
+// -------------------------------------------------------------------------------------------------
+template <int D, int WAVES, bool HAVE_O>
+SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
+    const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
+    const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
+    float* __restrict__ dQ, const int* __restrict__ trp, const int* __restrict__ tcol,
+    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    constexpr int KH = D / 2;
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    __shared__ float lds_g[WAVES][32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int rn = cnt * 32;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
+    const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
+    const int p_base = offs[I * 32] * 4;
+    const int p_voff = (li * rn + 4 * h) * 4;
+    const int col_voff = (h * KH * L + li) * 4;
+    const int b_voff = (4 * h * D + li) * 4;
+    const int r_voff = (li * D + h * KH) * 4;
+
+    float go[KH];
+    ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, go);
+
+    float g = 0.f;
+    if (HAVE_O) {
+        float oo[KH];
+        ldr_rows<D>(make_rsrc(Ocache + hb, hbytes), r_voff, I * 32 * D * 4, oo);
+#pragma unroll
+        for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
+        g += __shfl_xor(g, 32, 64);
+    } else {
+        auto body = [&](float (&vc)[KH], float (&vn)[KH], int t) {
+            float pv[16];
+            ldr_4x4(rP, p_voff, p_base + t * 128, pv);
+            if (t + WAVES < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + t + WAVES] * 128, vn);
+            f32x16 dp = mma_feat_init<D>(vc, go, splat16(0.f));
+#pragma unroll
+            for (int r = 0; r < 16; ++r) g = fmaf(dp[r], pv[r], g);
+        };
+        float va[KH], vb[KH];
+        if (w < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + w] * 128, va);
+        for (int t = w; t < cnt; t += 2 * WAVES) {
+            body(va, vb, t);
+            if (t + WAVES < cnt) body(vb, va, t + WAVES);
+        }
+        g += __shfl_xor(g, 32, 64);
+        if (WAVES > 1) {
+            if (h == 0) lds_g[w][li] = g;
+            __syncthreads();
+            g = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
+        }
+    }
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;
+    const f32x16 gneg = splat16(-g);
+
+    f32x16 acc[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
+    {
+        auto body = [&](float (&vc)[KH], float (&vn)[KH], int t) {
+            const int J = tcol[t0 + t];
+            float pv[16], kb[D / 32][16];
+            ldr_4x4(rP, p_voff, p_base + t * 128, pv);
+            ldr_tile_b<D>(rK, b_voff, J * 32 * D * 4, kb);
+            if (t + WAVES < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + t + WAVES] * 128, vn);
+            f32x16 dp = mma_feat_init<D>(vc, go, gneg);  // dp[r] = dO_i . v_j - g_i
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pv[r];
+            mma_b<D>(ds, kb, acc);
+        };
+        float va[KH], vb[KH];
+        if (w < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + w] * 128, va);
+        for (int t = w; t < cnt; t += 2 * WAVES) {
+            body(va, vb, t);
+            if (t + WAVES < cnt) body(vb, va, t + WAVES);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
+    reduce_store<D, WAVES>(acc, dQ + hb, I * 32, w, li, h, lds);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, column pass, one work-group per (head, block column): dK_J = sum_I dS_IJ^T Q_I,
+// dV_J = sum_I P_IJ^T dO_I over the transposed tile index; dP - g is recomputed per tile by a chain
+// started from the stored -g, the 1/sqrt(d) of dK is applied to the 32 x d result.
+// -------------------------------------------------------------------------------------------------
+template <int D, int WAVES>
+SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
+    const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
+    const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
+    const int* __restrict__ trp, const int* __restrict__ tcp, const int* __restrict__ tcrow,
+    const int* __restrict__ tcord, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    constexpr int KH = D / 2;
+    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
+    const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
+    const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
+    const int b_voff = (4 * h * D + li) * 4;
+    const int r_voff = (li * D + h * KH) * 4;
+
+    float vt[KH];
+    ldr_cols<D>(rV, L, (h * KH * L + li) * 4, J * 128, vt);
+
+    f32x16 ak[D / 32], av[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        ak[c] = splat16(0.f);
+        av[c] = splat16(0.f);
+    }
+    struct Pre {  // what is fetched one tile ahead
+        float go[KH];
+        float p[16];
+        float gneg[16];
+    };
+    auto fetch = [&](Pre& x, int e) {
+        const int I = tcrow[e0 + e], ord = tcord[e0 + e];
+        const int rn = (trp[I + 1] - trp[I]) * 32;
+        ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
+        const int pv = (4 * h * rn + li) * 4;
+        const int ps = (offs[I * 32] + ord * 32) * 4;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) x.p[r] = ld1(rP, pv, ps + (8 * (r >> 2) + (r & 3)) * rn * 4);
+        ldr_4x4(rG, 16 * h, I * 128, x.gneg);
+    };
+    auto body = [&](Pre& c, Pre& n, int e) {
+        const int I = tcrow[e0 + e];
+        float qb[D / 32][16], ob[D / 32][16];
+        ldr_tile_b<D>(rQ, b_voff, I * 32 * D * 4, qb);
+        ldr_tile_b<D>(rdO, b_voff, I * 32 * D * 4, ob);
+        if (e + WAVES < cnt) fetch(n, e + WAVES);
+        f32x16 init;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
+        f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dp[r] = dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
+        mma_b<D>(ds, qb, ak);
+        mma_b<D>(c.p, ob, av);
+    };
+    Pre a, b;
+    if (w < cnt) fetch(a, w);
+    for (int e = w; e < cnt; e += 2 * WAVES) {
+        body(a, b, e);
+        if (e + WAVES < cnt) body(b, a, e + WAVES);
+    }
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
+    reduce_store<D, WAVES>(ak, dK + hb, J * 32, w, li, h, lds);
+    if (WAVES > 1) __syncthreads();
+    reduce_store<D, WAVES>(av, dV + hb, J * 32, w, li, h, lds);
+}
+
+}  // namespace spion

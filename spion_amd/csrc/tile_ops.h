@@ -148,4 +148,34 @@ __device__ __forceinline__ void reduce_store(f32x16 (&acc)[D / 32], float* __res
         }
 }
 
+// Like reduce_store (row-major form), but the reduced tile goes to two arrays.
+template <int D, int WAVES>
+__device__ __forceinline__ void reduce_store2(f32x16 (&acc)[D / 32], float* __restrict__ out, float* __restrict__ out2,
+                                              int row0, int w, int li, int h, float* __restrict__ lds) {
+    constexpr int NC = D / 32;
+    const int l = h * 32 + li;
+    if (WAVES > 1) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) lds[((w * NC + c) * 16 + r) * 64 + l] = acc[c][r];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            if (WAVES > 1 && (r % WAVES) != w) continue;
+            float s = acc[c][r];
+            if (WAVES > 1) {
+                s = 0.f;
+#pragma unroll
+                for (int ww = 0; ww < WAVES; ++ww) s += lds[((ww * NC + c) * 16 + r) * 64 + l];
+            }
+            const size_t a = (size_t)(row0 + acc_row(r, h)) * D + c * 32 + li;
+            out[a] = s;
+            out2[a] = s;
+        }
+}
+
 }  // namespace spion

@@ -305,3 +305,33 @@ def test_inconsistent_csr_is_reported_not_launched():
     with pytest.raises(_lib.SpionLibraryError, match="do not match"):
         abi.forward(Q, K, V)
     abi.close()
+
+
+# ---------------------------------------------------------------------------------- output cache of the tile path
+def test_backward_row_sums_with_and_without_output_cache():
+    """The backward gets its row sums either from the handle's copy of O (P pointer known) or from an extra
+    sweep (unknown P pointer, copies switched off).  Two forwards in flight (siamese use) must not mix."""
+    from spion_amd import _lib
+    from tests.abi_utils import oracle_fwd_bwd
+
+    L, bs, d, NB = 256, 32, 32, 3
+    mat = _random_block_mask(L // bs, 0.35, seed=77)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    QA, KA, VA, dOA = _inputs(NB, L, d, seed=20)
+    QB, KB, VB, dOB = _inputs(NB, L, d, seed=21)
+    refA = oracle_fwd_bwd(QA, KA, VA, dOA, sm, off, col)
+    refB = oracle_fwd_bwd(QB, KB, VB, dOB, sm, off, col)
+    OA, PA = abi.forward(QA, KA, VA)
+    OB, PB = abi.forward(QB, KB, VB)          # second forward before the first backward
+    gA = abi.backward(QA, KA, VA, PA, dOA)    # copy of O filed under PA
+    gB = abi.backward(QB, KB, VB, PB, dOB)
+    gA2 = abi.backward(QA, KA, VA, PA.clone(), dOA)   # unknown pointer -> two-sweep kernel
+    _lib.core().spion_use_output_cache(abi.handle, 0)
+    OA3, PA3 = abi.forward(QA, KA, VA)
+    gA3 = abi.backward(QA, KA, VA, PA3, dOA)
+    for got, ref, tag in ((gA, refA, "A cached"), (gB, refB, "B cached"), (gA2, refA, "A clone"), (gA3, refA, "A off")):
+        for name, t in zip(("dQ", "dK", "dV"), got):
+            assert_close(t.cpu().numpy(), ref[name], what=f"{tag} {name}")
+    abi.close()
