@@ -236,7 +236,8 @@ struct PatternIndex {
     int ntiles = 0;
     int max_row_tiles = 0, max_col_tiles = 0;
     int* d_blob = nullptr;  // one allocation holding every array below
-    int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr, *d_tcrow = nullptr, *d_tcord = nullptr;
+    int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
+    int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     void release() {
         if (d_blob) (void)hipFree(d_blob);
@@ -386,10 +387,10 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         while (blob.size() % 4) blob.push_back(0);
         return o;
     };
-    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcrow = 0, o_tcord = 0, o_ccp = 0, o_crow = 0, o_cpos = 0;
+    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0;
     if (tiled) {
         const int nt = (int)tcol.size();
-        std::vector<int> tcp(nbr + 1, 0), tcrow(std::max(nt, 1)), tcord(std::max(nt, 1));
+        std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
         for (int t = 0; t < nt; ++t) tcp[tcol[t] + 1]++;
         for (int J = 0; J < nbr; ++J) tcp[J + 1] += tcp[J];
         std::vector<int> fill(tcp.begin(), tcp.end() - 1);
@@ -398,8 +399,9 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             mr = std::max(mr, trp[I + 1] - trp[I]);
             for (int t = trp[I]; t < trp[I + 1]; ++t) {
                 int e = fill[tcol[t]]++;
-                tcrow[e] = I;
-                tcord[e] = t - trp[I];
+                tcdesc[4 * (size_t)e + 0] = I;
+                tcdesc[4 * (size_t)e + 1] = off[I * 32] + (t - trp[I]) * 32;
+                tcdesc[4 * (size_t)e + 2] = (trp[I + 1] - trp[I]) * 32;
             }
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
@@ -407,8 +409,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         o_trp = append(trp);
         o_tcol = append(tcol);
         o_tcp = append(tcp);
-        o_tcrow = append(tcrow);
-        o_tcord = append(tcord);
+        o_tcdesc = append(tcdesc);
         pi.ntiles = nt;
         pi.max_row_tiles = mr;
         pi.max_col_tiles = mc;
@@ -436,8 +437,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_trp = pi.d_blob + o_trp;
         pi.d_tcol = pi.d_blob + o_tcol;
         pi.d_tcp = pi.d_blob + o_tcp;
-        pi.d_tcrow = pi.d_blob + o_tcrow;
-        pi.d_tcord = pi.d_blob + o_tcord;
+        pi.d_tcdesc = pi.d_blob + o_tcdesc;
     } else {
         pi.d_ccp = pi.d_blob + o_ccp;
         pi.d_crow = pi.d_blob + o_crow;
@@ -490,16 +490,25 @@ static const float* ocache_for_backward(SparseAttn* a, const float* key) {
     return nullptr;
 }
 
-static int pick_waves(const PatternIndex& pi, int nbr, bool by_col) {
-    // average tiles per strip decides how many wavefronts share one strip
-    const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
-    (void)by_col;
-    if (const char* e = getenv("SPION_TILE_WAVES")) {
+// Wavefronts per strip (block row or block column).  Forward: enough waves that each one's share of the
+// longest block row stays in registers (8 logit tiles at d = 32, 4 at d = 64).  Backward: one wave per strip
+// -- no cross-wave merge and the longest software pipeline -- unless strips are long and the launch is
+// too small to fill the 1024 SIMDs with single-wave work-groups.
+static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool forward) {
+    if (const char* e = getenv(forward ? "SPION_TILE_WAVES_FWD" : "SPION_TILE_WAVES_BWD")) {
         const int v = atoi(e);
         if (v == 1 || v == 2 || v == 4) return v;
     }
-    if (avg <= 1) return 1;
-    if (avg <= 3) return 2;
+    const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
+    if (forward) {
+        const int maxt = a->d == 32 ? 8 : 4;
+        if (pi.max_row_tiles <= maxt && avg <= 2) return 1;
+        if (pi.max_row_tiles <= 2 * maxt && avg <= 4) return 2;
+        return 4;
+    }
+    const long long strips = (long long)nbr * a->NB;
+    if (strips >= 2048 || avg <= 2) return 1;
+    if (strips >= 1024 || avg <= 4) return 2;
     return 4;
 }
 
@@ -509,7 +518,7 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
-    const int wv = pick_waves(pi, nbr, false);
+    const int wv = pick_waves(a, pi, nbr, true);
     float* ocache = ocache_for_forward(a, P);
     // logit tiles stay in registers when every wavefront's share of the longest block row fits
     constexpr int MAXT = D == 32 ? 8 : 4;
@@ -534,7 +543,7 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
-    const int wv = pick_waves(pi, nbr, false);
+    const int wv = pick_waves(a, pi, nbr, false);
     const float* ocache = ocache_for_backward(a, P);
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
@@ -548,7 +557,7 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
                                a->scale);                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
-                               a->ws_rowsum, dK, dV, pi.d_trp, pi.d_tcp, pi.d_tcrow, pi.d_tcord, offs, a->L, nbr,   \
+                               a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr,                          \
                                a->NB, nnz, a->scale);                                                               \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);

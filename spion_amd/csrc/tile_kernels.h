@@ -10,13 +10,19 @@
 //     1/sqrt(d)*log2(e) factor is folded into Q once per work-group, the 1/sqrt(d) of the gradients is
 //     applied once to the 32 x d result instead of to every tile;
 //   * software-pipeline each wavefront's tile list (operands of the next tile are requested before the
-//     current MFMA chain starts).
+//     current MFMA chain starts).  Loads are never issued under a branch between a load and its use: the
+//     compiler's s_waitcnt insertion merges conditional paths conservatively and would otherwise wait for
+//     the loads just issued.  When there is no next tile the current one is simply requested again.
+//     A wavefront's tiles are processed in pairs inside the loop (two register sets, no copies) and an odd
+//     last tile after it: a prefetch whose only consumer sits in a conditional block would be sunk into
+//     that block by the compiler, next to its use.
 #pragma once
 #include "tile_ops.h"
 
 namespace spion {
 
-#define SPION_TILE_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2)))
+#define SPION_TILE_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2, 2)))
+#define SPION_TILE_KERNEL3(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
@@ -135,6 +141,27 @@ __device__ __forceinline__ void merge_max_sum(float& m, float& z, int w, int h, 
     }
 }
 
+// Software-pipelined walk over the tiles first, first+step, ... (n of them) of one wavefront.
+//   fetch(X, i)   requests everything tile #i (0-based position in this wavefront's list) needs into X;
+//   compute(X, i) consumes it.  Positions past the end are clamped by the callers' fetch (valid, redundant).
+template <class Pre, class Fetch, class Compute>
+__device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch, Compute compute) {
+    if (n <= 0) return;
+    fetch(a, 0);
+    int i = 0;
+    for (; i + 1 < n; i += 2) {
+        fetch(b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(a, i);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(a, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (i < n) compute(a, i);
+}
+
 // -------------------------------------------------------------------------------------------------
 // Forward, one work-group per (head, block row).  Logits are kept in the log2 domain:
 // s' = (q.k) * log2(e)/sqrt(d) (- penalty*log2(e)), P = exp2(s' - m') / Z.
@@ -193,13 +220,15 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
         f32x16 S[MAXT];
         float kbuf[2][KH];
-        if (nu > 0) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, kbuf[0]);
+        int Js[MAXT];  // tile ids of this wavefront, fetched up front (scalar loads, one wait)
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) Js[u] = u < nu ? tcol[t0 + w + u * WAVES] : 0;
+        if (nu > 0) ldr_cols<D>(rK, L, col_voff, Js[0] * 128, kbuf[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
-                const int t = w + u * WAVES;
-                if (u + 1 < nu) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kbuf[(u + 1) & 1]);
-                S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(tcol[t0 + t]));
+                if (u + 1 < MAXT) ldr_cols<D>(rK, L, col_voff, Js[u + 1 < MAXT ? u + 1 : u] * 128, kbuf[(u + 1) & 1]);
+                S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(Js[u]));
                 m = max16(S[u], m);
             }
         }
@@ -235,12 +264,12 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         const float rinv = 1.0f / z;  // +inf denominator -> 0 -> P = 0, as in the reference
 
         float vbuf[2][D / 32][16];
-        if (nu > 0) ldr_tile_b<D>(rV, b_voff, tcol[t0 + w] * 32 * D * 4, vbuf[0]);
+        if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * D * 4, vbuf[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int t = w + u * WAVES;
-                if (u + 1 < nu) ldr_tile_b<D>(rV, b_voff, tcol[t0 + t + WAVES] * 32 * D * 4, vbuf[(u + 1) & 1]);
+                if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, vbuf[(u + 1) & 1]);
                 float p[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
@@ -250,50 +279,61 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         }
     } else {
         // ---- sweep 1: online row maximum and denominator -------------------------------------------
+        const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
+        struct PreK {
+            float k[KH];
+            float pj[16];  // key penalties of the tile (MASK only)
+        };
+        auto fetch_k = [&](PreK& x, int i) {
+            const int J = tcol[t0 + w + min(i, nu - 1) * WAVES];
+            ldr_cols<D>(rK, L, col_voff, J * 128, x.k);
+            if constexpr (MASK) ldr_4x4(rM, m_voff, J * 128, x.pj);
+        };
+        auto init_of = [&](const PreK& x, float shift) -> f32x16 {
+            f32x16 v;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                if constexpr (MASK) v[r] = -LOG2E * x.pj[r] - shift;
+                else v[r] = -shift;
+            }
+            return v;
+        };
         {
-            auto body = [&](float (&kc)[KH], float (&kn)[KH], int t) {
-                if (t + WAVES < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kn);
-                f32x16 s = mma_feat_init<D>(kc, q, chain_init(tcol[t0 + t]));
+            PreK ka, kb;
+            tile_pipeline(nu, ka, kb, fetch_k, [&](PreK& c, int) {
+                f32x16 s = mma_feat_init<D>(c.k, q, init_of(c, 0.f));
                 const float tm = max16(s, m);
                 float zz = 0.f;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) zz += __builtin_amdgcn_exp2f(s[r] - tm);
                 z = z * __builtin_amdgcn_exp2f(m - tm) + zz;
                 m = tm;
-            };
-            float ka[KH], kb[KH];
-            if (w < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, ka);
-            for (int t = w; t < cnt; t += 2 * WAVES) {
-                body(ka, kb, t);
-                if (t + WAVES < cnt) body(kb, ka, t + WAVES);
-            }
+            });
         }
         merge_max_sum<WAVES>(m, z, w, h, li, lds_m, lds_z);
         z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
         const float rinv = 1.0f / z;
         // ---- sweep 2: logits again (minus the row maximum, folded into the chain), P, O ------------
         {
-            auto body = [&](float (&kc)[KH], float (&kn)[KH], int t) {
-                const int J = tcol[t0 + t];
+            struct PreKV {
+                PreK k;
                 float vb[D / 32][16];
-                ldr_tile_b<D>(rV, b_voff, J * 32 * D * 4, vb);
-                if (t + WAVES < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + t + WAVES] * 128, kn);
-                f32x16 init = chain_init(J);
-#pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] -= m;
-                f32x16 s = mma_feat_init<D>(kc, q, init);
-                float p[16];
-#pragma unroll
-                for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
-                str_4x4(rP, p_voff, p_base + t * 128, p);
-                mma_b<D>(p, vb, o);
             };
-            float ka[KH], kb[KH];
-            if (w < cnt) ldr_cols<D>(rK, L, col_voff, tcol[t0 + w] * 128, ka);
-            for (int t = w; t < cnt; t += 2 * WAVES) {
-                body(ka, kb, t);
-                if (t + WAVES < cnt) body(kb, ka, t + WAVES);
-            }
+            PreKV xa, xb;
+            tile_pipeline(
+                nu, xa, xb,
+                [&](PreKV& x, int i) {
+                    fetch_k(x.k, i);
+                    ldr_tile_b<D>(rV, b_voff, tcol[t0 + w + min(i, nu - 1) * WAVES] * 32 * D * 4, x.vb);
+                },
+                [&](PreKV& c, int i) {
+                    f32x16 s = mma_feat_init<D>(c.k.k, q, init_of(c.k, m));
+                    float p[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
+                    str_4x4(rP, p_voff, p_base + (w + i * WAVES) * 128, p);
+                    mma_b<D>(p, c.vb, o);
+                });
         }
     }
     if (Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);
@@ -320,6 +360,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
+    const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
     const rsrc_t rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
@@ -340,20 +381,23 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
         for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
         g += __shfl_xor(g, 32, 64);
     } else {
-        auto body = [&](float (&vc)[KH], float (&vn)[KH], int t) {
+        struct PreG {
+            float vt[KH];
             float pv[16];
-            ldr_4x4(rP, p_voff, p_base + t * 128, pv);
-            if (t + WAVES < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + t + WAVES] * 128, vn);
-            f32x16 dp = mma_feat_init<D>(vc, go, splat16(0.f));
-#pragma unroll
-            for (int r = 0; r < 16; ++r) g = fmaf(dp[r], pv[r], g);
         };
-        float va[KH], vb[KH];
-        if (w < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + w] * 128, va);
-        for (int t = w; t < cnt; t += 2 * WAVES) {
-            body(va, vb, t);
-            if (t + WAVES < cnt) body(vb, va, t + WAVES);
-        }
+        PreG xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](PreG& x, int i) {
+                const int t = w + min(i, nu - 1) * WAVES;
+                ldr_cols<D>(rV, L, col_voff, tcol[t0 + t] * 128, x.vt);
+                ldr_4x4(rP, p_voff, p_base + t * 128, x.pv);
+            },
+            [&](PreG& c, int) {
+                f32x16 dp = mma_feat_init<D>(c.vt, go, splat16(0.f));
+#pragma unroll
+                for (int r = 0; r < 16; ++r) g = fmaf(dp[r], c.pv[r], g);
+            });
         g += __shfl_xor(g, 32, 64);
         if (WAVES > 1) {
             if (h == 0) lds_g[w][li] = g;
@@ -370,24 +414,35 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
     {
-        auto body = [&](float (&vc)[KH], float (&vn)[KH], int t) {
-            const int J = tcol[t0 + t];
-            float pv[16], kb[D / 32][16];
-            ldr_4x4(rP, p_voff, p_base + t * 128, pv);
-            ldr_tile_b<D>(rK, b_voff, J * 32 * D * 4, kb);
-            if (t + WAVES < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + t + WAVES] * 128, vn);
-            f32x16 dp = mma_feat_init<D>(vc, go, gneg);  // dp[r] = dO_i . v_j - g_i
-            float ds[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pv[r];
-            mma_b<D>(ds, kb, acc);
+        // One tile ahead: V^T operand, P tile and (d = 32) the K operand of the second product; for d = 64
+        // that operand would not fit in registers and is requested when the tile's first chain starts.
+        constexpr bool DEEP = D == 32;
+        struct Pre {
+            float vt[KH];
+            float pv[16];
+            float kb[DEEP ? D / 32 : 1][16];
+            int J;
         };
-        float va[KH], vb[KH];
-        if (w < cnt) ldr_cols<D>(rV, L, col_voff, tcol[t0 + w] * 128, va);
-        for (int t = w; t < cnt; t += 2 * WAVES) {
-            body(va, vb, t);
-            if (t + WAVES < cnt) body(vb, va, t + WAVES);
-        }
+        Pre xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](Pre& x, int i) {
+                const int t = w + min(i, nu - 1) * WAVES;
+                x.J = tcol[t0 + t];
+                ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
+                ldr_4x4(rP, p_voff, p_base + t * 128, x.pv);
+                if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * D * 4, x.kb);
+            },
+            [&](Pre& c, int) {
+                float kb2[D / 32][16];
+                if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * D * 4, kb2);
+                f32x16 dp = mma_feat_init<D>(c.vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
+                float ds[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.pv[r];
+                if constexpr (DEEP) mma_b<D>(ds, c.kb, acc);
+                else mma_b<D>(ds, kb2, acc);
+            });
     }
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
@@ -403,8 +458,7 @@ template <int D, int WAVES>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
-    const int* __restrict__ trp, const int* __restrict__ tcp, const int* __restrict__ tcrow,
-    const int* __restrict__ tcord, const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale) {
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
@@ -427,43 +481,58 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
         ak[c] = splat16(0.f);
         av[c] = splat16(0.f);
     }
-    struct Pre {  // what is fetched one tile ahead
+    // Per tile of the transposed index: {block row I, offset of the tile in this head's P, row stride}.
+    const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
+    // One tile ahead: dO rows, P tile, -g and (d = 32) the Q and dO operands of the second products; for
+    // d = 64 those would not fit in registers and are requested when the tile's first chain starts.
+    constexpr bool DEEP = D == 32;
+    struct Pre {
         float go[KH];
         float p[16];
         float gneg[16];
+        float qb[DEEP ? D / 32 : 1][16];
+        float ob[DEEP ? D / 32 : 1][16];
+        int I;
     };
-    auto fetch = [&](Pre& x, int e) {
-        const int I = tcrow[e0 + e], ord = tcord[e0 + e];
-        const int rn = (trp[I + 1] - trp[I]) * 32;
-        ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
-        const int pv = (4 * h * rn + li) * 4;
-        const int ps = (offs[I * 32] + ord * 32) * 4;
+    const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int4 d = desc[w + min(i, nu - 1) * WAVES];
+            const int I = d.x, rn = d.z;
+            x.I = I;
+            ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
+            const int pv = (4 * h * rn + li) * 4;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) x.p[r] = ld1(rP, pv, ps + (8 * (r >> 2) + (r & 3)) * rn * 4);
-        ldr_4x4(rG, 16 * h, I * 128, x.gneg);
-    };
-    auto body = [&](Pre& c, Pre& n, int e) {
-        const int I = tcrow[e0 + e];
-        float qb[D / 32][16], ob[D / 32][16];
-        ldr_tile_b<D>(rQ, b_voff, I * 32 * D * 4, qb);
-        ldr_tile_b<D>(rdO, b_voff, I * 32 * D * 4, ob);
-        if (e + WAVES < cnt) fetch(n, e + WAVES);
-        f32x16 init;
+            for (int r = 0; r < 16; ++r) x.p[r] = ld1(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
+            ldr_4x4(rG, 16 * h, I * 128, x.gneg);
+            if constexpr (DEEP) {
+                ldr_tile_b<D>(rQ, b_voff, I * 32 * D * 4, x.qb);
+                ldr_tile_b<D>(rdO, b_voff, I * 32 * D * 4, x.ob);
+            }
+        },
+        [&](Pre& c, int) {
+            float qb2[D / 32][16], ob2[D / 32][16];
+            if constexpr (!DEEP) {
+                ldr_tile_b<D>(rQ, b_voff, c.I * 32 * D * 4, qb2);
+                ldr_tile_b<D>(rdO, b_voff, c.I * 32 * D * 4, ob2);
+            }
+            f32x16 init;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
-        f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dp[r] = dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
-        float ds[16];
+            for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
+            f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+            float ds[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
-        mma_b<D>(ds, qb, ak);
-        mma_b<D>(c.p, ob, av);
-    };
-    Pre a, b;
-    if (w < cnt) fetch(a, w);
-    for (int e = w; e < cnt; e += 2 * WAVES) {
-        body(a, b, e);
-        if (e + WAVES < cnt) body(b, a, e + WAVES);
-    }
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
+            if constexpr (DEEP) {
+                mma_b<D>(ds, c.qb, ak);
+                mma_b<D>(c.p, c.ob, av);
+            } else {
+                mma_b<D>(ds, qb2, ak);
+                mma_b<D>(c.p, ob2, av);
+            }
+        });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
     reduce_store<D, WAVES>(ak, dK + hb, J * 32, w, li, h, lds);
