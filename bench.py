@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config4]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config2|config4|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -63,6 +63,14 @@ def build_workload(name):
         B, H, L, d, bs = 32, 2, 4096, 32, 1
         mat = None
         scale = 1.0
+    elif name == "config5_fp32":
+        # shape of the scale-up configuration (L=16384, d=64, 64x64 blocks, band of 4 + global row/column
+        # + 1 % random blocks), run through the fp32 path: the bf16 variant is not built
+        B, H, L, d, bs = 4, 8, 16384, 64, 64
+        mat = workloads.band_random_block_mask(L // bs, 2, extra_frac=0.01, seed=1)
+        mat[0, :] = 1.0
+        mat[:, 0] = 1.0
+        scale = 1.0 / 8.0
     else:
         raise SystemExit(f"unknown workload {name}")
     wl = dict(name=name, B=B, H=H, L=L, d=d, bs=bs, mat=mat, scale=scale)
@@ -86,6 +94,8 @@ def cpu_baseline(wl, budget_s=20.0):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     H, L, d = wl["H"], wl["L"], wl["d"]
+    if L > 8192:
+        H = 1  # an [H, L, L] fp32 buffer per head is 1 GiB at L = 16384: one head is the bounded sample
     rows = osa.csr_row_index(wl["offsets"])
     pat = torch.zeros(L, L)
     pat[torch.from_numpy(rows), torch.from_numpy(wl["columns"].astype(np.int64))] = 1.0
@@ -117,6 +127,52 @@ def cpu_baseline(wl, budget_s=20.0):
                        f"algorithmic 12*n*d FLOPs (dense FLOPs actually executed: {12.0 * L * L * d * H * n:.3e})")
 
 
+def bench_pattern_discovery(args, dev):
+    """Configuration 2: two 1024x1024 score maps -> 31x31 diagonal filter, 32x32 pooling, q = 0.90, path walk.
+    HBM-bound: 4*L*L bytes read per map.  CPU baseline: the oracle's PyTorch-CPU route on the same maps."""
+    import spion_amd
+    from oracle import pattern as op
+    from spion_amd import workloads
+
+    L, bs, q, n_maps = 1024, 32, 0.90, 2
+    maps_cpu = workloads.score_maps_config2(n_maps, L, 32, seed=0)
+    maps = maps_cpu.to(dev)
+
+    def step():
+        return spion_amd.discover_block_masks(maps, bs, mode="conv_ff", threshold=q)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    t_evt = _event_ms(step, max(10, args.steps))
+    bytes_read = 4.0 * L * L * n_maps
+    t1 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t1 < 10.0:
+        for i in range(n_maps):
+            op.generate_mask_conv_ff(maps_cpu[i].numpy(), bs, q, route="torch")
+        reps += 1
+    cpu_ms = 1e3 * (time.perf_counter() - t1) / reps
+    return {
+        "metric": "pattern discovery (conv filter + block pool + quantile + path walk), maps per second, 1 GPU",
+        "value": n_maps / (ms_step / 1e3), "unit": "maps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic (seeded softmax(QK^T) maps with a diagonal band boost)",
+        "config": {"workload": f"config2: {n_maps} score maps {L}x{L}, 31x31 diagonal filter, {bs}x{bs} pooling, q={q}"},
+        "roofline": {"bound": "hbm", "kernel": "conv_pool_kernel + threshold_walk_kernel", "achieved": bytes_read / t_evt / 1e6,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": bytes_read / t_evt / 1e6 / PEAK_HBM_GBS, "traffic": None,
+                     "event_ms": t_evt},
+        "cpu_baseline": {"value": n_maps / (cpu_ms / 1e3), "unit": "maps/s", "cores": min(os.cpu_count() or 1, torch.get_num_threads()),
+                         "kind": "port", "sample": f"the same {n_maps} maps, {reps} repetitions of the PyTorch-CPU route "
+                                                   "(F.conv2d, avg_pool2d, quantile) plus the iterative walk"},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -145,6 +201,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.workload == "config2":
+        print(json.dumps(bench_pattern_discovery(args, dev)))
+        return
 
     wl = build_workload(args.workload)
     B, H, L, d, bs, nnz = wl["B"], wl["H"], wl["L"], wl["d"], wl["bs"], wl["nnz"]

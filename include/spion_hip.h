@@ -166,6 +166,10 @@ void spion_set_backward_passes(void* handle, int mask);
  * row sums with one more sweep over the tiles); default on. */
 void spion_use_output_cache(void* handle, int on);
 
+/* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
+ * attention entry points take.  Returns 0 on success. */
+int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream);
+
 const char* spion_version(void);
 
 #ifdef __cplusplus

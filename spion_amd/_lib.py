@@ -62,6 +62,8 @@ def core() -> ctypes.CDLL:
     lib.spion_set_backward_passes.restype = None
     lib.spion_use_output_cache.argtypes = [_P, c_int]
     lib.spion_use_output_cache.restype = None
+    lib.spion_transpose_last2.argtypes = [_P, _P, c_int, c_int, c_int, _P]
+    lib.spion_transpose_last2.restype = c_int
     lib.spion_version.restype = c_char_p
     lib.spion_version.argtypes = []
     lib.spion_pattern_generate.argtypes = [_P, c_int, c_int, c_int, c_int, c_int, c_double, _P, _P, _P, _P]
@@ -86,6 +88,22 @@ def core() -> ctypes.CDLL:
         getattr(lib, f"spion_{fam}_destroy").restype = None
     lib._spion_typed = True
     return lib
+
+
+def transpose_last2(x):
+    """[..., R, C] fp32 CUDA tensor -> new contiguous [..., C, R] tensor (the library's tiled transpose)."""
+    x = x.contiguous()
+    R, C = x.shape[-2], x.shape[-1]
+    batch = x.numel() // (R * C) if x.numel() else 0
+    out = torch.empty(x.shape[:-2] + (C, R), dtype=torch.float32, device=x.device)
+    if batch == 0:
+        return out
+    if batch > 65535:
+        return x.transpose(-1, -2).contiguous()
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    if core().spion_transpose_last2(x.data_ptr(), out.data_ptr(), batch, R, C, stream) != 0:
+        check_error("spion_transpose_last2")
+    return out
 
 
 def check_error(where: str = "") -> None:

@@ -29,7 +29,7 @@ class _BlockAttnFunction(torch.autograd.Function):
             )
         dev = query.device
         q = query.contiguous()
-        kt = key.permute(0, 1, 3, 2).contiguous()  # the ABI takes K transposed in the forward
+        kt = _lib.transpose_last2(key)  # the ABI takes K transposed in the forward
         v = value.contiguous()
         p_flat = torch.empty(nb_ * idx.nnz, dtype=torch.float32, device=dev)
         out = torch.empty((m.batch_size, m.num_heads, L, d), dtype=torch.float32, device=dev)
@@ -44,6 +44,7 @@ class _BlockAttnFunction(torch.autograd.Function):
                                     idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
         _lib.check_error("attn_forward")
         ctx.save_for_backward(q, key, value, p_flat, idx.offsets, idx.columns, idx.sum_mat)
+        ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
         ctx.nnz = idx.nnz
         if m.with_mask:
@@ -58,7 +59,9 @@ class _BlockAttnFunction(torch.autograd.Function):
         dev = q.device
         n_total = m.num_batches * ctx.nnz
         k = key.contiguous()
-        vt = value.permute(0, 1, 3, 2).contiguous()  # the ABI takes V transposed in the backward
+        vt = _lib.transpose_last2(value)  # the ABI takes V transposed in the backward
+        if grad_output is None:  # only the probabilities were used downstream: their gradient is ignored
+            grad_output = torch.zeros(m.batch_size, m.num_heads, m.seq_len, m.emb_dim, dtype=torch.float32, device=dev)
         go = grad_output.contiguous()
         scratch_dp = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
         scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)

@@ -21,9 +21,9 @@ class _DenseAttnFunction(torch.autograd.Function):
         if tuple(query.shape) != (B, H, L, d):
             raise ValueError(f"query shape {tuple(query.shape)} does not match the handle ({B}, {H}, {L}, {d})")
         dev = query.device
-        qt = query.permute(0, 1, 3, 2).contiguous()  # [B,H,d,L]
+        qt = _lib.transpose_last2(query)  # [B,H,d,L]
         k = key.contiguous()
-        vt = value.permute(0, 1, 3, 2).contiguous()
+        vt = _lib.transpose_last2(value)
         attn = torch.empty((B, H, L, L), dtype=torch.float32, device=dev)  # memory [key][query]
         out_t = torch.empty((B, H, d, L), dtype=torch.float32, device=dev)
         if m.with_mask:
@@ -35,6 +35,7 @@ class _DenseAttnFunction(torch.autograd.Function):
                                     out_t.data_ptr())
         _lib.check_error("attn_forward")
         ctx.save_for_backward(qt, key, value, attn)
+        ctx.set_materialize_grads(False)  # the gradient of the returned map is ignored (as in the reference)
         ctx.module = m
         return out_t.permute(0, 1, 3, 2), attn.permute(0, 1, 3, 2)
 
@@ -44,9 +45,11 @@ class _DenseAttnFunction(torch.autograd.Function):
         qt, key, value, attn = ctx.saved_tensors
         B, H, L, d = m.batch_size, m.num_heads, m.seq_len, m.emb_dim
         dev = qt.device
-        kt = key.permute(0, 1, 3, 2).contiguous()
+        kt = _lib.transpose_last2(key)
         v = value.contiguous()
-        got = grad_output.permute(0, 1, 3, 2).contiguous()
+        if grad_output is None:  # only the returned map was used downstream: its gradient is ignored
+            grad_output = torch.zeros(B, H, L, d, dtype=torch.float32, device=dev)
+        got = _lib.transpose_last2(grad_output)
         dq_t = torch.empty((B, H, d, L), dtype=torch.float32, device=dev)
         dk_t = torch.empty((B, H, d, L), dtype=torch.float32, device=dev)
         dv_t = torch.empty((B, H, d, L), dtype=torch.float32, device=dev)

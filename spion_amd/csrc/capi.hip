@@ -33,6 +33,7 @@ int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
 void sparse_use_ocache(void*, int);
+int transpose_last2(const float*, float*, int, int, int, hipStream_t);
 void* dense_init(int, int, int, bool);
 void dense_destroy(void*);
 void dense_forward(void*, const float*, const float*, const float*, const float*, float*, float*, bool);
@@ -146,6 +147,9 @@ int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
 void spion_use_output_cache(void* h, int on) { sparse_use_ocache(h, on); }
+int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
+    return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));
+}
 const char* spion_version(void) { return "spion_hip 0.1 (gfx950)"; }
 
 }  // extern "C"

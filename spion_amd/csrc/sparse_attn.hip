@@ -507,6 +507,8 @@ static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool
         return 4;
     }
     const long long strips = (long long)nbr * a->NB;
+    // a few very long strips (global rows / columns) would leave one wave working alone at the end
+    if (std::max(pi.max_row_tiles, pi.max_col_tiles) > 8 * avg + 16) return 4;
     if (strips >= 2048 || avg <= 2) return 1;
     if (strips >= 1024 || avg <= 4) return 2;
     return 4;
@@ -669,6 +671,31 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         default: launch_elem_bwd<128>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
     }
     check_launch("elem_bwd kernels");
+}
+
+// [batch][rows][cols] -> [batch][cols][rows], fp32.  Used by the host modules for the K^T / V^T operands
+// the ABI asks for (models/attention_blockcuda.py:48,80 do it with permute + copy).
+__global__ __launch_bounds__(256) void transpose_last2_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                              int rows, int cols) {
+    __shared__ float tile[64][65];
+    const size_t base = (size_t)blockIdx.z * rows * cols;
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+    for (int r = ty; r < 64; r += 4)
+        if (r0 + r < rows && c0 + tx < cols) tile[r][tx] = in[base + (size_t)(r0 + r) * cols + c0 + tx];
+    __syncthreads();
+    for (int c = ty; c < 64; c += 4)
+        if (c0 + c < cols && r0 + tx < rows) out[base + (size_t)(c0 + c) * rows + r0 + tx] = tile[tx][c];
+}
+
+int transpose_last2(const float* in, float* out, int batch, int rows, int cols, hipStream_t stream) {
+    if (!in || !out || batch <= 0 || rows <= 0 || cols <= 0 || batch > 65535) {
+        set_error("spion_transpose_last2: bad arguments");
+        return 1;
+    }
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64, batch);
+    hipLaunchKernelGGL(transpose_last2_kernel, grid, dim3(256), 0, stream, in, out, rows, cols);
+    return check_launch("transpose_last2_kernel") ? 0 : 1;
 }
 
 void sparse_invalidate(void* h) {

@@ -162,6 +162,31 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
     if (i < n) compute(a, i);
 }
 
+// Same walk with three register sets: everything is requested two tiles ahead.
+template <class Pre, class Fetch, class Compute>
+__device__ __forceinline__ void tile_pipeline3(int n, Pre& a, Pre& b, Pre& c, Fetch fetch, Compute compute) {
+    if (n <= 0) return;
+    fetch(a, 0);
+    fetch(b, 1);
+    int i = 0;
+    for (; i + 2 < n; i += 3) {
+        fetch(c, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(a, i);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(a, i + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(b, i + 4);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(c, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (i < n) compute(a, i);
+    if (i + 1 < n) compute(b, i + 1);
+}
+
 // -------------------------------------------------------------------------------------------------
 // Forward, one work-group per (head, block row).  Logits are kept in the log2 domain:
 // s' = (q.k) * log2(e)/sqrt(d) (- penalty*log2(e)), P = exp2(s' - m') / Z.
@@ -423,9 +448,12 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             float kb[DEEP ? D / 32 : 1][16];
             int J;
         };
-        Pre xa, xb;
-        tile_pipeline(
-            nu, xa, xb,
+        Pre xa, xb, xc;
+        auto run = [&](auto fetch, auto compute) {
+            (void)xc;  // a third register set (two tiles of lead) was measured and brings nothing
+            tile_pipeline(nu, xa, xb, fetch, compute);
+        };
+        run(
             [&](Pre& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
                 x.J = tcol[t0 + t];
