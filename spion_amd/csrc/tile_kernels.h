@@ -9,6 +9,10 @@
 //     (forward) or the softmax row sum g (backward) enters as the chain's initial accumulator, the
 //     1/sqrt(d)*log2(e) factor is folded into Q once per work-group, the 1/sqrt(d) of the gradients is
 //     applied once to the 32 x d result instead of to every tile;
+//   * keep the per-CU vector-memory pipeline (TA/TCP tag lookups, the next bottleneck after the ALUs)
+//     lean: a P tile, whose MFMA layout gives every lane 16-byte pieces of its own row (64 distinct
+//     pieces per instruction), is read and written with one full 128-byte row per half-wave instead and
+//     transposed through a wave-private LDS tile; LDS instructions do not compete with the MFMAs either;
 //   * software-pipeline each wavefront's tile list (operands of the next tile are requested before the
 //     current MFMA chain starts).  Loads are never issued under a branch between a load and its use: the
 //     compiler's s_waitcnt insertion merges conditional paths conservatively and would otherwise wait for
@@ -92,6 +96,62 @@ __device__ __forceinline__ void str_4x4(rsrc_t r, int voff, int soff, const floa
     for (int g = 0; g < 4; ++g) st4(r, voff, soff + 32 * g, (f32x4){x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]});
 }
 
+__device__ __forceinline__ void st1(rsrc_t r, int voff, int soff, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v), r, voff, soff, 0);
+}
+
+// A 32 x 32 tile in the two register layouts a wavefront can hold it in:
+//   "row owner": lane (li, h) holds M[li][acc_row(r, h)], r = 0..15  (the accumulator of M^T; A operand)
+//   "col owner": lane (li, h) holds M[acc_row(r, h)][li]             (the accumulator of M; one full row per
+//                                                                     half-wave and register: coalesced in memory)
+// Global memory is touched in the col-owner layout; the wave-private LDS tile T (row stride TS floats)
+// converts between the two.  Same-wave LDS accesses complete in order, so no barrier is involved.
+constexpr int TS = 36;
+// col-owner tile of a row-major array whose rows are `ld` floats apart: 16 b32 accesses.
+// voff = (4*(lane/32)*ld + lane%32)*4, soff = byte offset of the tile's first element.
+__device__ __forceinline__ void ldr_tile_cols(rsrc_t r, int voff, int soff, int ld, float (&x)[16]) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) x[q] = ld1(r, voff, soff + (8 * (q >> 2) + (q & 3)) * ld * 4);
+}
+__device__ __forceinline__ void str_tile_cols(rsrc_t r, int voff, int soff, int ld, const float (&x)[16]) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) st1(r, voff, soff + (8 * (q >> 2) + (q & 3)) * ld * 4, x[q]);
+}
+__device__ __forceinline__ void lds_put_cols(float* T, int li, int h, const float (&x)[16], int col0 = 0) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) T[acc_row(q, h) * TS + col0 + li] = x[q];
+}
+__device__ __forceinline__ void lds_get_cols(const float* T, int li, int h, float (&x)[16]) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) x[q] = T[acc_row(q, h) * TS + li];
+}
+__device__ __forceinline__ void lds_put_rows(float* T, int li, int h, const float (&x)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<f32x4*>(T + li * TS + 8 * g + 4 * h) = (f32x4){x[4 * g], x[4 * g + 1], x[4 * g + 2], x[4 * g + 3]};
+}
+__device__ __forceinline__ void lds_get_rows(const float* T, int li, int h, float (&x)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(T + li * TS + 8 * g + 4 * h);
+        x[4 * g + 0] = v.x;
+        x[4 * g + 1] = v.y;
+        x[4 * g + 2] = v.z;
+        x[4 * g + 3] = v.w;
+    }
+}
+// operand over 32 features of row li: x[s] = T[li][16*h + s]
+__device__ __forceinline__ void lds_get_feat32(const float* T, int li, int h, float (&x)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(T + li * TS + 16 * h + 4 * g);
+        x[4 * g + 0] = v.x;
+        x[4 * g + 1] = v.y;
+        x[4 * g + 2] = v.z;
+        x[4 * g + 3] = v.w;
+    }
+}
+
 // acc = init + A.B over the head dimension (chain of D/2 MFMA).
 template <int D>
 __device__ __forceinline__ f32x16 mma_feat_init(const float (&a)[D / 2], const float (&b)[D / 2], f32x16 init) {
@@ -162,31 +222,6 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
     if (i < n) compute(a, i);
 }
 
-// Same walk with three register sets: everything is requested two tiles ahead.
-template <class Pre, class Fetch, class Compute>
-__device__ __forceinline__ void tile_pipeline3(int n, Pre& a, Pre& b, Pre& c, Fetch fetch, Compute compute) {
-    if (n <= 0) return;
-    fetch(a, 0);
-    fetch(b, 1);
-    int i = 0;
-    for (; i + 2 < n; i += 3) {
-        fetch(c, i + 2);
-        __builtin_amdgcn_sched_barrier(0);
-        compute(a, i);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(a, i + 3);
-        __builtin_amdgcn_sched_barrier(0);
-        compute(b, i + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(b, i + 4);
-        __builtin_amdgcn_sched_barrier(0);
-        compute(c, i + 2);
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    if (i < n) compute(a, i);
-    if (i + 1 < n) compute(b, i + 1);
-}
-
 // -------------------------------------------------------------------------------------------------
 // Forward, one work-group per (head, block row).  Logits are kept in the log2 domain:
 // s' = (q.k) * log2(e)/sqrt(d) (- penalty*log2(e)), P = exp2(s' - m') / Z.
@@ -204,6 +239,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -214,10 +250,18 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int p_base = offs[I * 32] * 4;
-    const int p_voff = (li * rn + 4 * h) * 4;
+    const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
     const int b_voff = (4 * h * D + li) * 4;
     const int m_voff = 16 * h;
+    float* T = lds_t[w];
+    // P tile t of this block row: transpose to the col-owner layout and store full rows
+    auto store_p = [&](const float (&p)[16], int t) {
+        float pc[16];
+        lds_put_rows(T, li, h, p);
+        lds_get_cols(T, li, h, pc);
+        str_tile_cols(rP, pc_voff, p_base + t * 128, rn, pc);
+    };
     const float c2 = scale * LOG2E;
 
     float q[KH];
@@ -298,7 +342,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                 float p[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
-                str_4x4(rP, p_voff, p_base + t * 128, p);
+                store_p(p, t);
                 mma_b<D>(p, vbuf[u & 1], o);
             }
         }
@@ -356,7 +400,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                     float p[16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
-                    str_4x4(rP, p_voff, p_base + (w + i * WAVES) * 128, p);
+                    store_p(p, w + i * WAVES);
                     mma_b<D>(p, c.vb, o);
                 });
         }
@@ -380,6 +424,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_g[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -390,10 +435,16 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const rsrc_t rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const int p_base = offs[I * 32] * 4;
-    const int p_voff = (li * rn + 4 * h) * 4;
+    const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
     const int b_voff = (4 * h * D + li) * 4;
     const int r_voff = (li * D + h * KH) * 4;
+    float* T = lds_t[w];
+    // P tile as loaded (col owner) -> row-owner layout, the one dP^T comes in
+    auto p_rows = [&](const float (&pc)[16], float (&pr)[16]) {
+        lds_put_cols(T, li, h, pc);
+        lds_get_rows(T, li, h, pr);
+    };
 
     float go[KH];
     ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, go);
@@ -416,12 +467,14 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             [&](PreG& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
                 ldr_cols<D>(rV, L, col_voff, tcol[t0 + t] * 128, x.vt);
-                ldr_4x4(rP, p_voff, p_base + t * 128, x.pv);
+                ldr_tile_cols(rP, pc_voff, p_base + t * 128, rn, x.pv);
             },
             [&](PreG& c, int) {
+                float pr[16];
+                p_rows(c.pv, pr);
                 f32x16 dp = mma_feat_init<D>(c.vt, go, splat16(0.f));
 #pragma unroll
-                for (int r = 0; r < 16; ++r) g = fmaf(dp[r], c.pv[r], g);
+                for (int r = 0; r < 16; ++r) g = fmaf(dp[r], pr[r], g);
             });
         g += __shfl_xor(g, 32, 64);
         if (WAVES > 1) {
@@ -448,26 +501,25 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             float kb[DEEP ? D / 32 : 1][16];
             int J;
         };
-        Pre xa, xb, xc;
-        auto run = [&](auto fetch, auto compute) {
-            (void)xc;  // a third register set (two tiles of lead) was measured and brings nothing
-            tile_pipeline(nu, xa, xb, fetch, compute);
-        };
-        run(
+        Pre xa, xb;  // a third register set (two tiles of lead) was measured and brings nothing
+        tile_pipeline(
+            nu, xa, xb,
             [&](Pre& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
                 x.J = tcol[t0 + t];
                 ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
-                ldr_4x4(rP, p_voff, p_base + t * 128, x.pv);
+                ldr_tile_cols(rP, pc_voff, p_base + t * 128, rn, x.pv);
                 if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * D * 4, x.kb);
             },
             [&](Pre& c, int) {
                 float kb2[D / 32][16];
                 if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * D * 4, kb2);
+                float pr[16];
+                p_rows(c.pv, pr);
                 f32x16 dp = mma_feat_init<D>(c.vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.pv[r];
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
                 if constexpr (DEEP) mma_b<D>(ds, c.kb, acc);
                 else mma_b<D>(ds, kb2, acc);
             });
@@ -489,6 +541,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale) {
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, J = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -511,11 +564,14 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     }
     // Per tile of the transposed index: {block row I, offset of the tile in this head's P, row stride}.
     const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
-    // One tile ahead: dO rows, P tile, -g and (d = 32) the Q and dO operands of the second products; for
-    // d = 64 those would not fit in registers and are requested when the tile's first chain starts.
+    // One tile ahead: P tile, -g and, for d = 32, the Q and dO operands of the second products; the dO tile
+    // is then loaded once (one full row per half-wave) and its other layout, the A operand of the dP chain,
+    // comes out of a wave-private LDS transpose.  For d = 64 the operands of the second products would not
+    // fit in registers: they are requested when the tile's first chain starts and the dO rows separately.
     constexpr bool DEEP = D == 32;
+    float* T = lds_t[w];
     struct Pre {
-        float go[KH];
+        float go[DEEP ? 1 : KH];
         float p[16];
         float gneg[16];
         float qb[DEEP ? D / 32 : 1][16];
@@ -530,7 +586,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
             const int4 d = desc[w + min(i, nu - 1) * WAVES];
             const int I = d.x, rn = d.z;
             x.I = I;
-            ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
+            if constexpr (!DEEP) ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
             const int pv = (4 * h * rn + li) * 4;
 #pragma unroll
             for (int r = 0; r < 16; ++r) x.p[r] = ld1(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
@@ -549,7 +605,15 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
             f32x16 init;
 #pragma unroll
             for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
-            f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+            f32x16 dp;  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+            if constexpr (DEEP) {
+                float go[KH];
+                lds_put_cols(T, li, h, c.ob[0]);
+                lds_get_feat32(T, li, h, go);
+                dp = mma_feat_init<D>(go, vt, init);
+            } else {
+                dp = mma_feat_init<D>(c.go, vt, init);
+            }
             float ds[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
