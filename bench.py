@@ -173,6 +173,67 @@ def bench_pattern_discovery(args, dev):
     }
 
 
+def bench_encoder_step(args, dev):
+    """Configuration 3: one training step (forward, backward, AdamW update) of the 2-layer sparse encoder,
+    batch 256, L=1024, d_model 64, FFN 128, H=2, d_head 32, masks discovered from the model's own dense phase.
+    The model around the attention layers is plain torch.nn (tests/encoder_harness.py)."""
+    import spion_amd
+    from tests import encoder_harness as eh
+
+    torch.manual_seed(0)
+    cfg = eh.model_config(L=1024, batch=256, block_size=32, key_mask=False, threshold=0.90)
+    ids, mask, labels = eh.synthetic_batch(cfg, seed=1, device=dev)
+    model = eh.EncoderForSC(cfg, spion_amd.Attention).to(dev)
+    with torch.no_grad():
+        _, attn_lst = model(ids, mask, labels, None, is_attn=True)
+    mat_lst = spion_amd.generate_pattern_conv_ff(attn_lst, cfg)
+    density = [float(m.mean()) for m in mat_lst[0]]
+    del attn_lst
+    torch.cuda.empty_cache()
+    for layer in model.layers:
+        layer.mha.reconstruct_for_blocksparse(cfg)
+    opt = eh.make_optimizer(model)
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        loss, _ = model(ids, mask, labels, mat_lst)
+        loss.mean().backward()
+        opt.step()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # attention share: the two layers' C-ABI kernels, from HIP events around a forward+backward of one layer's
+    # attention core at the same shape
+    B, H, L, d = cfg["batch_size"], cfg["num_head"], cfg["max_seq_len"], cfg["head_dim"]
+    core_mod = model.layers[0].mha.block_attn
+    q, k, v, do = (torch.randn(B, H, L, d, device=dev) for _ in range(4))
+    for t in (q, k, v):
+        t.requires_grad_()
+
+    def attn_only():
+        out, _ = core_mod(q, k, v, mask, mat_lst[0][0])
+        out.backward(do)
+
+    t_attn = _event_ms(attn_only, max(10, args.steps))
+    return {
+        "metric": "2-layer sparse encoder training step (fwd+bwd+AdamW), samples per second, 1 GPU",
+        "value": B / (ms_step / 1e3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (uniform token ids, uniform labels, random-init weights)",
+        "config": {"workload": f"config3: 2-layer encoder step, batch {B}, L={L}, d_model 64, FFN 128, H={H}, d_head {d}, "
+                               f"block {cfg['block_size']}, discovered block densities {[round(x, 3) for x in density]}"},
+        "attention_core_ms_per_layer": t_attn,
+        "attention_share_of_step": 2.0 * t_attn / ms_step,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -204,6 +265,9 @@ def main():
 
     if args.workload == "config2":
         print(json.dumps(bench_pattern_discovery(args, dev)))
+        return
+    if args.workload == "config3":
+        print(json.dumps(bench_encoder_step(args, dev)))
         return
 
     wl = build_workload(args.workload)
