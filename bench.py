@@ -47,6 +47,27 @@ def _event_ms(fn, iters, warm=3):
     return start.elapsed_time(end) / iters
 
 
+def _profiled_traffic_bytes(kernel):
+    """HBM bytes per launch of ``kernel`` on the north-star workload as measured with rocprofv3 --pmc
+    (FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size): the 'HBM MiB/launch' column of the
+    committed summary profiles/north_star_tile_kernels.txt.  None if the summary has no such row."""
+    path = os.path.join(ROOT, "profiles", "north_star_tile_kernels.txt")
+    try:
+        in_table = False
+        for line in open(path):
+            if line.startswith("kernel") and "HBM MiB/launch" in line:
+                in_table = True
+                continue
+            if in_table:
+                if not line.strip():
+                    break
+                if line.startswith(kernel):
+                    return float(line.split()[-1]) * 1048576.0
+    except OSError:
+        pass
+    return None
+
+
 def build_workload(name):
     from spion_amd import workloads
     from spion_amd.csr import block_mask_to_csr_host
@@ -365,6 +386,8 @@ def main():
         roof = dict(bound="hbm", kernel=dom, achieved=share / dom_ms / 1e6, peak=PEAK_HBM_GBS, unit="GB/s",
                     traffic=None)
     roof["frac"] = roof["achieved"] / roof["peak"]
+    if wl["name"] == "north_star":
+        roof["traffic"] = _profiled_traffic_bytes(dom)
     roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
 
     result = {

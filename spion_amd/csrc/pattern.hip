@@ -13,6 +13,7 @@ namespace spion {
 
 constexpr int POOL_THREADS = 256;
 constexpr int WALK_THREADS = 1024;
+constexpr int POOLED_LDS = 8192;  // block grids up to 90 x 90 are walked from LDS
 
 // pooled[I][J] = (1/bs^2) sum_{i in I, j in J} sum_{t=-hk..hk} A[i+t][j+t]  (zero outside the map).
 // Regrouped per source element A[p][q]: its weight is the number of shifts t that land in the block.
@@ -90,11 +91,18 @@ __global__ __launch_bounds__(WALK_THREADS) void threshold_walk_kernel(const floa
     __shared__ int sh[2];
     __shared__ int s_cnt;
     __shared__ uint32_t s_min;
+    __shared__ float s_pooled[POOLED_LDS];
     const int map = blockIdx.x, N = nb * nb;
     const float* pooled = pooled_all + (size_t)map * N;
     float* mat = mat_all + (size_t)map * N;
 
     for (int i = threadIdx.x; i < N; i += blockDim.x) mat[i] = 0.f;
+    if (N <= POOLED_LDS) {
+        // the select passes and the walkers' dependent neighbour reads then stay in LDS
+        for (int i = threadIdx.x; i < N; i += blockDim.x) s_pooled[i] = pooled[i];
+        __syncthreads();
+        pooled = s_pooled;
+    }
 
     if (mode == SPION_PATTERN_FLOOD) {
         // torch.quantile, linear interpolation, every step in fp32 (main_conv_ff.py:268)
