@@ -78,6 +78,31 @@ void spion_blockmask_attn_backward(void* handle, const float* Q, const float* K,
 void spion_blockmask_destroy(void* handle);
 
 /* ------------------------------------------------------------------------------------------------
+ * Sparse attention on bf16 tensors (scale-up shapes).  No counterpart in the reference, which is fp32 only;
+ * the arithmetic is that of models/block_attn.cu:33-130 (with Mask: models/block_attn_mask.cu:88-173) on
+ * bf16 inputs with fp32 accumulation and softmax.  Like the reference's key-mask module
+ * (models/attention_blockcuda_mask.py:61, which returns 0 for the map) it does not hand out the probabilities:
+ * they are never written to memory, the backward recomputes them.
+ *   Q, K, V, Out, dO, dQ, dK, dV: bf16, row-major [NB][L][d] (no transposed operands), d = 32 or 64;
+ *   Mask: NULL, or the additive key penalty [NB][L] fp32 of the block-mask family;
+ *   Lse [NB][L] fp32: written by the forward (row maximum + log2 of the softmax denominator, log2 domain),
+ *     to be handed back to the backward together with Out;
+ *   the pattern must be a union of aligned 32x32 tiles (any block mask with block size 32, 64, ...).
+ * ---------------------------------------------------------------------------------------------- */
+void* spion_block_bf16_init(int emb_dim, int seq_len, int num_batches, int block_size);
+
+void spion_block_bf16_attn_forward(void* handle, const void* Q, const void* K, const void* V, const float* Mask,
+                                   void* Out, float* Lse,
+                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+void spion_block_bf16_attn_backward(void* handle, const void* Q, const void* K, const void* V, const float* Mask,
+                                    const void* Out, const float* Lse, const void* dO,
+                                    void* dQ, void* dK, void* dV,
+                                    const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
+void spion_block_bf16_destroy(void* handle);
+
+/* ------------------------------------------------------------------------------------------------
  * Dense-phase attention (produces the full probability map that feeds pattern discovery).
  * Replaces models/attn.cu:265-280.  Operands follow the reference's column-major convention:
  *   forward : Qt [NB][d][L], K [NB][L][d], Vt [NB][d][L];

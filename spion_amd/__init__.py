@@ -9,6 +9,7 @@ from .attention_cuda import CUDAAttention
 from .attention_cuda_mask import CUDAMaskAttention
 from .attention_blockcuda import CUDABlockAttention
 from .attention_blockcuda_mask import CUDABlockMaskAttention
+from .attention_blockbf16 import BlockAttentionBF16
 from .pattern import (
     discover_block_masks,
     generate_pattern_conv,
@@ -24,6 +25,7 @@ __all__ = [
     "CUDAMaskAttention",
     "CUDABlockAttention",
     "CUDABlockMaskAttention",
+    "BlockAttentionBF16",
     "discover_block_masks",
     "generate_pattern_conv",
     "generate_pattern_conv_ff",

@@ -77,6 +77,14 @@ def core() -> ctypes.CDLL:
         getattr(lib, f"spion_{fam}_attn_backward").restype = None
         getattr(lib, f"spion_{fam}_destroy").argtypes = [_P]
         getattr(lib, f"spion_{fam}_destroy").restype = None
+    lib.spion_block_bf16_init.argtypes = [c_int, c_int, c_int, c_int]
+    lib.spion_block_bf16_init.restype = _P
+    lib.spion_block_bf16_attn_forward.argtypes = [_P] * 10 + [c_int]
+    lib.spion_block_bf16_attn_forward.restype = None
+    lib.spion_block_bf16_attn_backward.argtypes = [_P] * 14 + [c_int]
+    lib.spion_block_bf16_attn_backward.restype = None
+    lib.spion_block_bf16_destroy.argtypes = [_P]
+    lib.spion_block_bf16_destroy.restype = None
     for fam, extra in (("dense", 0), ("densemask", 1)):
         getattr(lib, f"spion_{fam}_init").argtypes = [c_int, c_int, c_int]
         getattr(lib, f"spion_{fam}_init").restype = _P

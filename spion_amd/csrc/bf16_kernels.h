@@ -1,0 +1,482 @@
+// bf16 tile kernels of the sparse path (scale-up configuration: bf16 tensors, fp32 accumulation and softmax).
+//
+// No counterpart in the reference (fp32 only); the semantics are those of models/block_attn.cu:33-130 (and
+// the key-penalty variant models/block_attn_mask.cu:88-173) with the probabilities never written to memory:
+// the forward stores one fp32 number per row, lse2_i = m_i + log2(Z_i) in the log2 domain, and both
+// backward passes recompute P_ij = exp2(s_ij*log2(e)/sqrt(d) - lse2_i) from Q and K.
+//
+// All tensors are row-major [head][L][D] bf16.  Every contraction is a chain of v_mfma_f32_32x32x16_bf16
+// (lane l supplies 8 consecutive k-slots of row l%32 for both operands, half-wave l/32 the second 8; the
+// fp32 accumulator layout is the one of every 32x32 MFMA: register r of lane l is row acc_row(r, l/32),
+// column l%32).  Which feature / tile row a k-slot stands for is free as long as both operands agree:
+//   * products over the head dimension: lane (row, h) holds features h*D/2 .. h*D/2+D/2-1 of its row, D/2
+//     consecutive bf16 of a row-major row (D/16 instructions);
+//   * products over a tile's 32 keys or queries: slot e of instruction t in half h is tile row
+//     16t + 8(e/4) + 4h + e%4 = acc_row(8t+e, h), so the accumulator of the first product, converted to
+//     bf16, is the B operand of the second one register for register.  The A operand (the tile of K, V, Q or
+//     dO seen feature-major) comes from the row-major tile the first product already loaded: it is written
+//     to a wave-private LDS tile and read back with the transposing LDS read of gfx950.
+// Queries are the lane index of every row-pass accumulator (S^T, dP^T, O^T, dQ^T), so row statistics are
+// lane scalars; keys are the lane index in the column pass.
+//
+// Work-groups have four wavefronts and take one entry of a host-built list: four short strips (one per
+// wavefront, no barriers) or one long strip (a global row or column) walked by the four wavefronts together.
+#pragma once
+#include "tile_kernels.h"
+
+namespace spion {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int BF16_WAVES = 4;
+constexpr float BF16_LAZY = 8.f;  // the running row maximum is raised only when a tile exceeds it by 2^8
+
+template <int D>
+__device__ __forceinline__ void ldb_rows(rsrc_t r, int voff, int soff, bf16x8 (&x)[D / 16]) {
+#pragma unroll
+    for (int t = 0; t < D / 16; ++t)
+        x[t] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff + 16 * t, 0));
+}
+
+template <int D>
+__device__ __forceinline__ f32x16 mma_feat_bf16(const bf16x8 (&a)[D / 16], const bf16x8 (&b)[D / 16], f32x16 init) {
+    f32x16 acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[0], b[0], init, 0, 0, 0);
+#pragma unroll
+    for (int t = 1; t < D / 16; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[t], b[t], acc, 0, 0, 0);
+    return acc;
+}
+
+// out[c] (features 32c.. x lanes) += X_tile^T . W^T, W given as accumulator-layout values packed to bf16
+template <int D>
+__device__ __forceinline__ void mma_tile_bf16(const bf16x8 (&xt)[D / 32][2], const bf16x8 (&wb)[2], f32x16 (&out)[D / 32]) {
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) out[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xt[c][t], wb[t], out[c], 0, 0, 0);
+}
+
+__device__ __forceinline__ void pack16(const float (&p)[16], bf16x8 (&pb)[2]) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) pb[t][e] = (__bf16)p[8 * t + e];
+}
+
+// Wave-private LDS tile of 32 row-major rows of D bf16, rows RS bytes apart.
+template <int D>
+struct LdsTile {
+    static constexpr int RS = D * 2 + 32;
+    static constexpr int BYTES = 32 * RS;
+    // lane (row li, half h) stores the D/2 features it holds as a head-dimension operand
+    static __device__ __forceinline__ void put_rows(char* T, int li, int h, const bf16x8 (&x)[D / 16]) {
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) *reinterpret_cast<u32x4*>(T + li * RS + h * D + 16 * t) = __builtin_bit_cast(u32x4, x[t]);
+    }
+    // The transposing read works on groups of 16 lanes: lane j of a group points at 4 consecutive bf16,
+    // and lane 4a+b receives element b of the pieces of lanes a, 4+a, 8+a, 12+a.  With lane j pointing at
+    // row R + j/4, features F + 4(j%4) .., lane 4a+b gets rows R..R+3 of feature F + 4a + b.
+    // lane_base: byte offset of this lane's piece for R = 4h, F = 16*((l/16)%2).
+    static __device__ __forceinline__ int lane_base(int l) {
+        const int h = l >> 5, gm = (l >> 4) & 1, j = l & 15;
+        return (4 * h + (j >> 2)) * RS + (16 * gm + 4 * (j & 3)) * 2;
+    }
+    static __device__ __forceinline__ void get_tile_t(const char* T, int base, bf16x8 (&xt)[D / 32][2]) {
+        typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + base + (16 * t) * RS + c * 64));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + base + (16 * t + 8) * RS + c * 64));
+                xt[c][t] = __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1,
+                                                   2, 3, 4, 5, 6, 7);
+            }
+    }
+};
+
+// x of the lower and of the upper half-wave lane with the same lane%32, by v_permlane32_swap (exchanges the
+// upper half of its first operand with the lower half of its second).  Written as inline assembly with two
+// read-write operands: they must be different registers for the exchange to mean anything.
+__device__ __forceinline__ void half_swap(float x, float& lo, float& hi) {
+    float a = x, b = x;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lo = a;  // {x of lanes 0-31, x of lanes 0-31}
+    hi = b;  // {x of lanes 32-63, x of lanes 32-63}
+}
+__device__ __forceinline__ float half_swap_max(float x) {
+    float lo, hi;
+    half_swap(x, lo, hi);
+    return fmaxf(lo, hi);
+}
+__device__ __forceinline__ float half_swap_sum(float x) {
+    float lo, hi;
+    half_swap(x, lo, hi);
+    return lo + hi;
+}
+
+// Sum the per-wave partial results of a cooperative strip (coop) and store the 32 x D result as bf16 rows.
+// acc[c][r] of lane (li, h): row li, feature 32c + acc_row(r, h).
+template <int D>
+__device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO, int row0, bool coop, int w, int li, int h,
+                                                float* lds) {
+    const int l = li + 32 * h;
+    if (coop) {
+        if (w > 0) {
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) lds[(((w - 1) * (D / 32) + c) * 16 + r) * 64 + l] = acc[c][r];
+        }
+        __syncthreads();
+        if (w > 0) return;
+#pragma unroll
+        for (int ww = 0; ww < BF16_WAVES - 1; ++ww)
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[c][r] += lds[((ww * (D / 32) + c) * 16 + r) * 64 + l];
+    }
+    const int voff = (li * D + 4 * h) * 2;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            bf16x4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = (__bf16)acc[c][4 * g + e];
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rO, voff, row0 * D * 2 + (32 * c + 8 * g) * 2, 0);
+        }
+}
+
+// Work-group entry: strip of each wavefront (-1: none); the four wavefronts share a strip iff the first two
+// entries are equal.
+struct StripAssign {
+    int strip, rank, step;
+    bool coop;
+};
+__device__ __forceinline__ StripAssign strip_of_wave(const int* __restrict__ wg_list, int g, int w) {
+    const int4 e = reinterpret_cast<const int4*>(wg_list)[g];
+    StripAssign s;
+    s.coop = e.x == e.y;
+    s.strip = w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w;
+    s.rank = s.coop ? w : 0;
+    s.step = s.coop ? BF16_WAVES : 1;
+    return s;
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward: one sweep per block row with a lazily raised running maximum.
+// -------------------------------------------------------------------------------------------------
+template <int D, bool MASK>
+SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    typedef LdsTile<D> LT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][LT::BYTES];
+    __shared__ float lds_m[BF16_WAVES][32], lds_z[BF16_WAVES][32];
+    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
+    if (sa.strip < 0) return;  // only in entries of independent strips: no barrier is skipped
+    const int I = sa.strip;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rO = make_rsrc(O + hb, hbytes);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int r_voff = li * D * 2 + h * D;
+    char* T = lds_t[w];
+    const int tbase = LT::lane_base(l);
+    const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+
+    bf16x8 q[D / 16];
+    ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, q);
+
+    // Floor of the running maximum (the reference's max(-100, .) / max(0, .), models/block_attn.cu:52): any
+    // value gives the same probabilities; 2^-100 keeps (L - n) * 2^-m finite in fp32 for empty rows.
+    float m = MASK ? 0.f : -100.f, z = 0.f;
+    f32x16 o[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
+
+    struct Pre {
+        bf16x8 k[D / 16], v[D / 16];
+        float pj[MASK ? 16 : 1];
+    };
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
+            ldb_rows<D>(rK, r_voff, J * 32 * D * 2, x.k);
+            ldb_rows<D>(rV, r_voff, J * 32 * D * 2, x.v);
+            if constexpr (MASK) {
+                float pj[16];
+                ldr_4x4(rM, 16 * h, J * 128, pj);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
+            }
+        },
+        [&](Pre& c, int) {
+            LT::put_rows(T, li, h, c.v);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
+            }
+            const f32x16 s = mma_feat_bf16<D>(c.k, q, init);  // S^T: register = key, lane = query
+            const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
+            if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
+                const float mn = t2 > m + BF16_LAZY ? t2 : m;
+                const float f = __builtin_amdgcn_exp2f(m - mn);
+                z *= f;
+#pragma unroll
+                for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
+                m = mn;
+            }
+            float p[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
+                z += p[r];
+            }
+            bf16x8 pb[2];
+            pack16(p, pb);
+            bf16x8 vt[D / 32][2];
+            LT::get_tile_t(T, tbase, vt);
+            mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
+        });
+    z = half_swap_sum(z);
+    if (sa.coop) {
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
+        float M = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < BF16_WAVES; ++ww) M = fmaxf(M, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < BF16_WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - M);
+        const float f = __builtin_amdgcn_exp2f(m - M);
+#pragma unroll
+        for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
+        m = M;
+        z = Z;
+    }
+    const int off_pattern = L - cnt * 32;
+    if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);  // models/block_attn.cu:74
+    const float rinv = 1.0f / z;
+#pragma unroll
+    for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
+    if (sa.rank == 0 && h == 0) Lse[(size_t)bh * L + I * 32 + li] = m + __builtin_amdgcn_logf(z);
+    store_rows_bf16<D>(o, rO, I * 32, sa.coop, w, li, h, lds_o);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, row pass: g_i = dO_i . O_i, P and dP recomputed per tile, dS' = P*(dP - g), dQ += dS'.K_J;
+// the 1/sqrt(d) is applied to the 32 x d result.  Gneg receives -g for the column pass.
+// -------------------------------------------------------------------------------------------------
+template <int D, bool MASK>
+SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
+    const float* __restrict__ pen, float* __restrict__ Gneg, __bf16* __restrict__ dQ, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    typedef LdsTile<D> LT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][LT::BYTES];
+    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
+    if (sa.strip < 0) return;
+    const int I = sa.strip;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rO = make_rsrc(O + hb, hbytes), rdQ = make_rsrc(dQ + hb, hbytes);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int r_voff = li * D * 2 + h * D;
+    char* T = lds_t[w];
+    const int tbase = LT::lane_base(l);
+    const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+
+    bf16x8 q[D / 16], go[D / 16];
+    ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, q);
+    ldb_rows<D>(rdO, r_voff, I * 32 * D * 2, go);
+    float g = 0.f;
+    {
+        bf16x8 oo[D / 16];
+        ldb_rows<D>(rO, r_voff, I * 32 * D * 2, oo);
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) g = fmaf((float)go[t][e], (float)oo[t][e], g);
+        g = half_swap_sum(g);
+    }
+    const float lse = Lse[(size_t)bh * L + I * 32 + li];
+    if (sa.rank == 0 && h == 0) Gneg[(size_t)bh * L + I * 32 + li] = -g;
+    const f32x16 gneg = splat16(-g);
+
+    f32x16 acc[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
+    struct Pre {
+        bf16x8 k[D / 16], v[D / 16];
+        float pj[MASK ? 16 : 1];
+    };
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
+            ldb_rows<D>(rK, r_voff, J * 32 * D * 2, x.k);
+            ldb_rows<D>(rV, r_voff, J * 32 * D * 2, x.v);
+            if constexpr (MASK) {
+                float pj[16];
+                ldr_4x4(rM, 16 * h, J * 128, pj);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
+            }
+        },
+        [&](Pre& c, int) {
+            LT::put_rows(T, li, h, c.k);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
+            }
+            const f32x16 s = mma_feat_bf16<D>(c.k, q, init);
+            const f32x16 dp = mma_feat_bf16<D>(c.v, go, gneg);  // dO_i . v_j - g_i
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
+            bf16x8 dsb[2];
+            pack16(ds, dsb);
+            bf16x8 kt[D / 32][2];
+            LT::get_tile_t(T, tbase, kt);
+            mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
+        });
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
+    store_rows_bf16<D>(acc, rdQ, I * 32, sa.coop, w, li, h, lds_o);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
+// -------------------------------------------------------------------------------------------------
+template <int D, bool MASK>
+SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const __bf16* __restrict__ dO, const float* __restrict__ Lse, const float* __restrict__ Gneg,
+    const float* __restrict__ pen, __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcp,
+    const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    typedef LdsTile<D> LT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
+    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
+    if (sa.strip < 0) return;
+    const int J = sa.strip;
+    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
+    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rdK = make_rsrc(dK + hb, hbytes), rdV = make_rsrc(dV + hb, hbytes);
+    const rsrc_t rL = make_rsrc(Lse + (size_t)bh * L, (size_t)L * 4), rG = make_rsrc(Gneg + (size_t)bh * L, (size_t)L * 4);
+    const int r_voff = li * D * 2 + h * D;
+    char* Tq = lds_t[w][0];
+    char* Tg = lds_t[w][1];
+    const int tbase = LT::lane_base(l);
+    const float c2 = scale * LOG2E;
+
+    bf16x8 k[D / 16], v[D / 16];
+    ldb_rows<D>(rK, r_voff, J * 32 * D * 2, k);
+    ldb_rows<D>(rV, r_voff, J * 32 * D * 2, v);
+    f32x16 sinit = splat16(0.f);
+    if constexpr (MASK) sinit = splat16(-pen[(size_t)bh * L + J * 32 + li] / scale);
+
+    f32x16 ak[D / 32], av[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        ak[c] = splat16(0.f);
+        av[c] = splat16(0.f);
+    }
+    const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
+    // One tile ahead: the Q and dO rows and, for d = 32, the row statistics of the tile's queries; for d = 64
+    // those would not fit in registers next to two operand sets and are requested when the tile's first
+    // chain starts.
+    constexpr bool DEEP = D == 32;
+    struct Pre {
+        bf16x8 q[D / 16], go[D / 16];
+        float lse[DEEP ? 16 : 1], gneg[DEEP ? 16 : 1];
+        int I;
+    };
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int I = desc[sa.rank + min(i, nu - 1) * sa.step].x;
+            x.I = I;
+            ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, x.q);
+            ldb_rows<D>(rdO, r_voff, I * 32 * D * 2, x.go);
+            if constexpr (DEEP) {
+                ldr_4x4(rL, 16 * h, I * 128, x.lse);
+                ldr_4x4(rG, 16 * h, I * 128, x.gneg);
+            }
+        },
+        [&](Pre& c, int) {
+            float lse[16], gn[16];
+            if constexpr (DEEP) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    lse[r] = c.lse[r];
+                    gn[r] = c.gneg[r];
+                }
+            } else {
+                ldr_4x4(rG, 16 * h, c.I * 128, gn);
+                ldr_4x4(rL, 16 * h, c.I * 128, lse);
+            }
+            LT::put_rows(Tq, li, h, c.q);
+            LT::put_rows(Tg, li, h, c.go);
+            const f32x16 s = mma_feat_bf16<D>(c.q, k, sinit);  // S: register = query, lane = key
+            f32x16 ginit;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
+            const f32x16 dp = mma_feat_bf16<D>(c.go, v, ginit);  // dO_i . v_j - g_i
+            float p[16], ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse[r]));
+                ds[r] = p[r] * dp[r];
+            }
+            bf16x8 pb[2], dsb[2];
+            pack16(p, pb);
+            pack16(ds, dsb);
+            bf16x8 qt[D / 32][2], gt[D / 32][2];
+            LT::get_tile_t(Tq, tbase, qt);
+            LT::get_tile_t(Tg, tbase, gt);
+            mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
+            mma_tile_bf16<D>(gt, pb, av);   // dV^T
+        });
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
+    store_rows_bf16<D>(ak, rdK, J * 32, sa.coop, w, li, h, lds_o);
+    if (sa.coop) __syncthreads();
+    store_rows_bf16<D>(av, rdV, J * 32, sa.coop, w, li, h, lds_o);
+}
+
+}  // namespace spion

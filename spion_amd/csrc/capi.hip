@@ -33,6 +33,11 @@ int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
 void sparse_use_ocache(void*, int);
+void* sparse_bf16_init(int, int, int, int);
+void sparse_bf16_forward(void*, const void*, const void*, const void*, const float*, void*, float*, const int*,
+                         const int*, int);
+void sparse_bf16_backward(void*, const void*, const void*, const void*, const float*, const void*, const float*,
+                          const void*, void*, void*, void*, const int*, const int*, int);
 int transpose_last2(const float*, float*, int, int, int, hipStream_t);
 void* dense_init(int, int, int, bool);
 void dense_destroy(void*);
@@ -46,6 +51,23 @@ int pattern_generate(const float*, int, int, int, int, int, double, float*, floa
 using namespace spion;
 
 extern "C" {
+
+// ---- sparse, bf16 tensors (no reference counterpart) ---------------------------------------------
+void* spion_block_bf16_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    return sparse_bf16_init(emb_dim, seq_len, num_batches, block_size);
+}
+void spion_block_bf16_attn_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
+                                   float* Lse, const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_bf16_forward(h, Q, K, V, Mask, Out, Lse, Offsets, Columns, nnz);
+}
+void spion_block_bf16_attn_backward(void* h, const void* Q, const void* K, const void* V, const float* Mask,
+                                    const void* Out, const float* Lse, const void* dO, void* dQ, void* dK, void* dV,
+                                    const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_bf16_backward(h, Q, K, V, Mask, Out, Lse, dO, dQ, dK, dV, Offsets, Columns, nnz);
+}
+void spion_block_bf16_destroy(void* h) { sparse_destroy(h); }
 
 // ---- sparse, no key mask -----------------------------------------------------------------------
 void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size) {

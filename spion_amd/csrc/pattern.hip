@@ -64,14 +64,26 @@ __device__ uint32_t block_select(const float* __restrict__ v, int N, int rank, i
             if ((k & mask) == prefix) atomicAdd(&hist[(k >> shift) & 255u], 1);
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
-            int c = 0, b = 0;
-            for (; b < 255; ++b) {
-                if (c + hist[b] > rem) break;
-                c += hist[b];
+        if (threadIdx.x < 64) {
+            // first wavefront: lane l owns bins 4l..4l+3; the bin whose cumulative count first exceeds rem
+            const int l = threadIdx.x;
+            const int h0 = hist[4 * l], h1 = hist[4 * l + 1], h2 = hist[4 * l + 2], h3 = hist[4 * l + 3];
+            const int own = h0 + h1 + h2 + h3;
+            int incl = own;
+            for (int o = 1; o < 64; o <<= 1) {
+                const int up = __shfl_up(incl, o, 64);
+                if (l >= o) incl += up;
             }
-            sh[0] = b;
-            sh[1] = rem - c;
+            int c = incl - own;
+            const bool last = (l == 63);
+            if ((c <= rem && rem < incl) || (last && rem >= incl)) {
+                int b = 4 * l;
+                if (c + h0 <= rem) { c += h0; ++b;
+                    if (c + h1 <= rem) { c += h1; ++b;
+                        if (c + h2 <= rem) { c += h2; ++b; } } }
+                sh[0] = b;
+                sh[1] = rem - c;
+            }
         }
         __syncthreads();
         prefix |= (uint32_t)sh[0] << shift;
@@ -163,20 +175,31 @@ __global__ __launch_bounds__(WALK_THREADS) void threshold_walk_kernel(const floa
             const uint32_t kk = block_select(pooled, N, N - k, hist, sh);  // k-th largest
             if (threadIdx.x == 0) s_cnt = 0;
             __syncthreads();
-            int c = 0;
-            for (int i = threadIdx.x; i < N; i += blockDim.x)
-                if (float_key(pooled[i]) > kk) {
+            if (threadIdx.x == 0) s_min = 0u;  // number of blocks equal to the k-th largest
+            __syncthreads();
+            int c = 0, ties = 0;
+            for (int i = threadIdx.x; i < N; i += blockDim.x) {
+                const uint32_t key = float_key(pooled[i]);
+                if (key > kk) {
                     mat[i] = 1.f;
                     ++c;
+                } else if (key == kk) {
+                    ++ties;
                 }
+            }
             atomicAdd(&s_cnt, c);
+            atomicAdd(&s_min, (uint32_t)ties);
             __syncthreads();
-            if (threadIdx.x == 0) {
-                int need = k - s_cnt;
-                for (int i = 0; i < N && need > 0; ++i)
+            const int need = k - s_cnt;
+            if (need >= (int)s_min) {  // the usual case (one such block): every tie is selected
+                for (int i = threadIdx.x; i < N; i += blockDim.x)
+                    if (float_key(pooled[i]) == kk) mat[i] = 1.f;
+            } else if (threadIdx.x == 0) {
+                int left = need;
+                for (int i = 0; i < N && left > 0; ++i)
                     if (float_key(pooled[i]) == kk) {
                         mat[i] = 1.f;
-                        --need;
+                        --left;
                     }
             }
             if (threadIdx.x == 0 && thresh_out) thresh_out[map] = key_float(kk);

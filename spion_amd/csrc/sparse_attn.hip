@@ -14,6 +14,7 @@
 // the softmax denominator counts every off-pattern key with logit 0.
 #include "common.h"
 #include "tile_kernels.h"
+#include "bf16_kernels.h"
 #include "../../include/spion_hip.h"
 
 #include <algorithm>
@@ -239,6 +240,9 @@ struct PatternIndex {
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
+    // work-group lists of the bf16 kernels (four strip ids per work-group) over block rows / block columns
+    int *d_wg_row = nullptr, *d_wg_col = nullptr;
+    int n_wg_row = 0, n_wg_col = 0;
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -267,6 +271,7 @@ struct SparseAttn {
     bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
     int last_path = 0;
+    bool is_bf16 = false;  // handle of the bf16 family: tile patterns only, P is never materialised
     bool force_element = false;
     int bwd_passes = 3;  // bit 0: row pass (g, dQ), bit 1: column pass (dK, dV); profiling only
 };
@@ -315,6 +320,25 @@ void sparse_destroy(void* h) {
         if (sl.buf) (void)hipFree(sl.buf);
     a->hdr.magic = 0;
     delete a;
+}
+
+// Work-group list of the bf16 kernels: strips sorted by length (longest first, so the tail of the launch is
+// made of short ones); a strip much longer than the average (a global row or column) is walked by the four
+// wavefronts of a work-group together, the others are dealt four to a work-group, one per wavefront.
+static std::vector<int> build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles) {
+    std::vector<int> order(nstrips);
+    for (int i = 0; i < nstrips; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(),
+                     [&](int a, int b) { return ptr[a + 1] - ptr[a] > ptr[b + 1] - ptr[b]; });
+    const int avg = nstrips ? (ntiles + nstrips - 1) / nstrips : 0;
+    const int long_len = std::max(4 * avg + 8, 32);
+    std::vector<int> wg;
+    int i = 0;
+    for (; i < nstrips && ptr[order[i] + 1] - ptr[order[i]] > long_len; ++i)
+        for (int w = 0; w < 4; ++w) wg.push_back(order[i]);
+    for (; i < nstrips; i += 4)
+        for (int w = 0; w < 4; ++w) wg.push_back(i + w < nstrips ? order[i + w] : -1);
+    return wg;
 }
 
 // Copy the index to the host once, validate it, detect the tile structure and build the transposed
@@ -387,7 +411,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         while (blob.size() % 4) blob.push_back(0);
         return o;
     };
-    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0;
+    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -405,6 +429,11 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             }
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
+        const std::vector<int> wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
+        pi.n_wg_row = (int)wgr.size() / 4;
+        pi.n_wg_col = (int)wgc.size() / 4;
+        o_wgr = append(wgr);
+        o_wgc = append(wgc);
         if (tcol.empty()) tcol.push_back(0);
         o_trp = append(trp);
         o_tcol = append(tcol);
@@ -438,6 +467,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcol = pi.d_blob + o_tcol;
         pi.d_tcp = pi.d_blob + o_tcp;
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
+        pi.d_wg_row = pi.d_blob + o_wgr;
+        pi.d_wg_col = pi.d_blob + o_wgc;
     } else {
         pi.d_ccp = pi.d_blob + o_ccp;
         pi.d_crow = pi.d_blob + o_crow;
@@ -605,8 +636,8 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
                     float* Out, const int* Offsets, const int* Columns, int nnz, bool mask_entry) {
     SparseAttn* a = as_sparse(h, "attn_forward");
     if (!a) return;
-    if (a->has_mask != mask_entry) {
-        set_error("attn_forward: handle was created by the %s init", a->has_mask ? "mask" : "no-mask");
+    if (a->has_mask != mask_entry || a->is_bf16) {
+        set_error("attn_forward: handle was created by the %s init", a->is_bf16 ? "bf16" : a->has_mask ? "mask" : "no-mask");
         return;
     }
     if (!Q || !Kt || !V || !Attn || !Out || !Offsets || (nnz > 0 && !Columns) || (mask_entry && !Mask)) {
@@ -644,6 +675,10 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
     SparseAttn* a = as_sparse(h, "attn_backward");
     if (!a) return;
     (void)dP;
+    if (a->is_bf16) {
+        set_error("attn_backward: handle was created by the bf16 init");
+        return;
+    }
     if (!Q || !K || !Vt || !P || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
         set_error("attn_backward: null pointer argument");
         return;
@@ -671,6 +706,104 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         default: launch_elem_bwd<128>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
     }
     check_launch("elem_bwd kernels");
+}
+
+// =================================================================================================
+// bf16 family: row-major bf16 Q, K, V, dO, O and gradients; fp32 row statistics; tile patterns only
+// =================================================================================================
+void* sparse_bf16_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    if (emb_dim != 32 && emb_dim != 64) {
+        set_error("bf16 init: emb_dim %d unsupported (32 or 64)", emb_dim);
+        return nullptr;
+    }
+    if (seq_len <= 0 || seq_len % 32) {
+        set_error("bf16 init: seq_len %d must be a positive multiple of 32", seq_len);
+        return nullptr;
+    }
+    SparseAttn* a = static_cast<SparseAttn*>(sparse_init(emb_dim, seq_len, num_batches, block_size, false));
+    if (a) a->is_bf16 = true;
+    return a;
+}
+
+static SparseAttn* as_bf16(void* h, const char* who, const int* Offsets, const int* Columns, int nnz) {
+    SparseAttn* a = as_sparse(h, who);
+    if (!a) return nullptr;
+    if (!a->is_bf16) {
+        set_error("%s: handle was not created by the bf16 init", who);
+        return nullptr;
+    }
+    if (!ensure_pattern(a, Offsets, Columns, nnz)) return nullptr;
+    if (!a->pat.tiled) {
+        set_error("%s: the bf16 path needs a pattern made of aligned 32x32 tiles (block masks of block size 32, 64, ...)",
+                  who);
+        return nullptr;
+    }
+    return a;
+}
+
+void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out, float* Lse,
+                         const int* Offsets, const int* Columns, int nnz) {
+    if (!Q || !K || !V || !Out || !Lse || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("bf16 attn_forward: null pointer argument");
+        return;
+    }
+    SparseAttn* a = as_bf16(h, "bf16 attn_forward", Offsets, Columns, nnz);
+    if (!a) return;
+    const PatternIndex& pi = a->pat;
+    a->last_path = 1;
+    const dim3 grid(pi.n_wg_row * a->NB), block(64 * BF16_WAVES);
+    const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
+    __bf16* o = static_cast<__bf16*>(Out);
+#define SPION_LAUNCH(DD, MM)                                                                                         \
+    hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse, pi.d_trp,    \
+                       pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale)
+    if (a->d == 32) {
+        if (Mask) SPION_LAUNCH(32, true);
+        else SPION_LAUNCH(32, false);
+    } else {
+        if (Mask) SPION_LAUNCH(64, true);
+        else SPION_LAUNCH(64, false);
+    }
+#undef SPION_LAUNCH
+    check_launch("bf16_fwd_kernel");
+}
+
+void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, const float* Mask, const void* Out,
+                          const float* Lse, const void* dO, void* dQ, void* dK, void* dV, const int* Offsets,
+                          const int* Columns, int nnz) {
+    if (!Q || !K || !V || !Out || !Lse || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("bf16 attn_backward: null pointer argument");
+        return;
+    }
+    SparseAttn* a = as_bf16(h, "bf16 attn_backward", Offsets, Columns, nnz);
+    if (!a) return;
+    const PatternIndex& pi = a->pat;
+    a->last_path = 1;
+    if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+    const dim3 grid_r(pi.n_wg_row * a->NB), grid_c(pi.n_wg_col * a->NB), block(64 * BF16_WAVES);
+    const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
+    const __bf16 *o = static_cast<const __bf16*>(Out), *go = static_cast<const __bf16*>(dO);
+    __bf16 *dq = static_cast<__bf16*>(dQ), *dk = static_cast<__bf16*>(dK), *dv = static_cast<__bf16*>(dV);
+#define SPION_LAUNCH(DD, MM)                                                                                          \
+    do {                                                                                                              \
+        if (a->bwd_passes & 1)                                                                                        \
+            hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o, Lse,   \
+                               Mask, a->ws_rowsum, dq, pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB,    \
+                               a->scale);                                                                             \
+        if (a->bwd_passes & 2)                                                                                        \
+            hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM>), grid_c, block, 0, a->hdr.stream, q, k, v, go, Lse,      \
+                               a->ws_rowsum, Mask, dk, dv, pi.d_tcp, pi.d_tcdesc, pi.d_wg_col, pi.n_wg_col, a->L,     \
+                               a->NB, a->scale);                                                                      \
+    } while (0)
+    if (a->d == 32) {
+        if (Mask) SPION_LAUNCH(32, true);
+        else SPION_LAUNCH(32, false);
+    } else {
+        if (Mask) SPION_LAUNCH(64, true);
+        else SPION_LAUNCH(64, false);
+    }
+#undef SPION_LAUNCH
+    check_launch("bf16_bwd kernels");
 }
 
 // [batch][rows][cols] -> [batch][cols][rows], fp32.  Used by the host modules for the K^T / V^T operands

@@ -38,6 +38,14 @@ def north_star_mask(block_size: int = 32) -> np.ndarray:
     return band_random_block_mask(4096 // block_size, 1, density=0.10, seed=1)
 
 
+def config5_mask() -> np.ndarray:
+    """L=16384, 64x64 blocks: diagonal band, one global block row and column, 1 % random blocks (about 3.7 %)."""
+    mat = band_random_block_mask(256, 2, extra_frac=0.01, seed=1)
+    mat[0, :] = 1.0
+    mat[:, 0] = 1.0
+    return mat
+
+
 def window_random_csr(L: int, window: int, per_row: int, seed: int = 3):
     """Element-sparse pattern: columns [i-window, i+window] plus uniform random columns up to
     ``per_row`` entries in every row (sorted, unique).  Returns (sum_mat, offsets, columns) int32."""

@@ -1,0 +1,262 @@
+"""Parity of the bf16 sparse-attention kernels with the float64 oracle, through the C ABI (GPU box only).
+
+The oracle runs on the bf16-rounded inputs in float64.  Tolerance for the bf16 outputs and gradients, 1e-2
+relative, read for tensors whose every element carries the 2^-9 rounding of the bf16 result itself (measured
+relative L2 error of a correct kernel: 2.3e-3) and whose gradients cancel (dS = P (dP - g)):
+  * relative error in the L2 norm <= 1e-2, and
+  * no element further from the oracle than 1e-2 * (|ref| + max|ref|).
+The fp32 row statistic the forward hands to the backward must agree within 1e-3 absolute (measured 1e-6).
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sparse_attention as osa
+from spion_amd import BlockAttentionBF16, _lib, workloads
+from tests.abi_utils import SparseABI
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL_BF16 = 1e-2
+LOG2E = 1.4426950408889634
+
+
+def assert_close_bf16(got, ref, what=""):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    assert got.shape == ref.shape, (what, got.shape, ref.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite values"
+    err = np.abs(got - ref)
+    rel_l2 = float(np.sqrt((err * err).sum() / max((ref * ref).sum(), 1e-300)))
+    assert rel_l2 <= REL_TOL_BF16, f"{what}: relative L2 error {rel_l2:.3e}"
+    tol = REL_TOL_BF16 * (np.abs(ref) + np.abs(ref).max())
+    bad = err > tol
+    if bad.any():
+        idx = np.unravel_index(np.argmax(err - tol), err.shape)
+        raise AssertionError(f"{what}: {int(bad.sum())}/{bad.size} outside tolerance; worst at {idx}: "
+                             f"got {got[idx]!r}, ref {ref[idx]!r}")
+    return rel_l2
+
+
+class BF16ABI:
+    def __init__(self, d, L, NB, block_size):
+        self.lib = _lib.core()
+        self.d, self.L, self.NB = d, L, NB
+        self.handle = self.lib.spion_block_bf16_init(d, L, NB, block_size)
+        _lib.check_error("spion_block_bf16_init")
+        assert self.handle
+
+    def close(self):
+        self.lib.spion_block_bf16_destroy(self.handle)
+        self.handle = None
+
+    def set_pattern(self, sum_mat, offsets, columns):
+        dev = "cuda"
+        self.np_pattern = (np.asarray(sum_mat), np.asarray(offsets), np.asarray(columns))
+        self.sum_mat = torch.from_numpy(np.ascontiguousarray(sum_mat)).to(dev)
+        self.offsets = torch.from_numpy(np.ascontiguousarray(offsets)).to(dev)
+        cols = np.ascontiguousarray(columns) if len(columns) else np.zeros(1, np.int32)
+        self.columns = torch.from_numpy(cols).to(dev)
+        self.nnz = int(offsets[-1])
+
+    def forward(self, Q, K, V, pen=None):
+        O = torch.full((self.NB, self.L, self.d), float("nan"), dtype=torch.bfloat16, device="cuda")
+        lse = torch.full((self.NB, self.L), float("nan"), dtype=torch.float32, device="cuda")
+        self.lib.spion_block_bf16_attn_forward(self.handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                               pen.data_ptr() if pen is not None else None, O.data_ptr(),
+                                               lse.data_ptr(), self.offsets.data_ptr(), self.columns.data_ptr(),
+                                               self.sum_mat.data_ptr(), self.nnz)
+        _lib.check_error("bf16 forward")
+        return O, lse
+
+    def backward(self, Q, K, V, O, lse, dO, pen=None):
+        dQ, dK, dV = (torch.full((self.NB, self.L, self.d), float("nan"), dtype=torch.bfloat16, device="cuda")
+                      for _ in range(3))
+        self.lib.spion_block_bf16_attn_backward(self.handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(),
+                                                pen.data_ptr() if pen is not None else None, O.data_ptr(),
+                                                lse.data_ptr(), dO.data_ptr(), dQ.data_ptr(), dK.data_ptr(),
+                                                dV.data_ptr(), self.offsets.data_ptr(), self.columns.data_ptr(),
+                                                self.sum_mat.data_ptr(), self.nnz)
+        _lib.check_error("bf16 backward")
+        return dQ, dK, dV
+
+
+def _bf16_inputs(NB, L, d, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return tuple((torch.randn(NB, L, d, generator=g) * s).to(torch.bfloat16).cuda() for s in (scale, scale, 1.0, 1.0))
+
+
+def _oracle(Q, K, V, dO, sum_mat, offsets, columns, pen=None):
+    f = lambda t: t.detach().float().cpu().numpy().astype(np.float64)
+    q, k, v, do = f(Q), f(K), f(V), f(dO)
+    penn = None if pen is None else pen.detach().cpu().numpy().astype(np.float64)
+    O, P = osa.csr_attention_forward(q, k, v, offsets, columns, sum_mat, penn)
+    dQ, dK, dV, _ = osa.csr_attention_backward(q, k, v, P, do, offsets, columns)
+    # row statistic: log2 of the softmax denominator with the row maximum folded in
+    NB, L, d = q.shape
+    rows = osa.csr_row_index(offsets)
+    cols = np.asarray(columns[: int(offsets[-1])], dtype=np.int64)
+    lse = np.zeros((NB, L))
+    for b in range(NB):
+        val = np.einsum("nd,nd->n", q[b][rows], k[b][cols]) * float(np.float32(1) / np.sqrt(np.float32(d)))
+        if penn is not None:
+            val = val - penn[b][cols]
+        big = np.full(L, 0.0 if penn is not None else -100.0)
+        np.maximum.at(big, rows, val)
+        z = np.zeros(L)
+        np.add.at(z, rows, np.exp(val - big[rows]))
+        z += (L - np.asarray(sum_mat)) * np.exp(-big)
+        lse[b] = (big + np.log(z)) * LOG2E
+    return dict(O=O, dQ=dQ, dK=dK, dV=dV, lse=lse)
+
+
+def _run_and_check(abi, Q, K, V, dO, pen=None, tag=""):
+    sm, off, col = abi.np_pattern
+    ref = _oracle(Q, K, V, dO, sm, off, col, pen)
+    O, lse = abi.forward(Q, K, V, pen)
+    dQ, dK, dV = abi.backward(Q, K, V, O, lse, dO, pen)
+    torch.cuda.synchronize()
+    got_lse = lse.cpu().numpy().astype(np.float64)
+    assert np.isfinite(got_lse).all(), f"{tag}: lse not finite"
+    assert np.max(np.abs(got_lse - ref["lse"])) < 1e-3, f"{tag}: lse off by {np.max(np.abs(got_lse - ref['lse']))}"
+    for name, t in (("O", O), ("dQ", dQ), ("dK", dK), ("dV", dV)):
+        assert_close_bf16(t.float().cpu().numpy(), ref[name], f"{tag} {name}")
+
+
+def _mask(nb, p, seed, global_block=False, empty_row=None, empty_col=None):
+    rng = np.random.default_rng(seed)
+    mat = (rng.random((nb, nb)) < p).astype(np.float32)
+    mat[np.arange(nb), np.arange(nb)] = 1
+    if global_block:
+        mat[0, :] = 1
+        mat[:, 0] = 1
+    if empty_row is not None:
+        mat[empty_row, :] = 0
+    if empty_col is not None:
+        mat[:, empty_col] = 0
+    return mat
+
+
+@pytest.mark.parametrize(
+    "L,bs,d,NB,p,glob",
+    [
+        (128, 32, 32, 3, 0.30, False),
+        (256, 32, 64, 2, 0.40, False),
+        (256, 64, 64, 2, 0.40, False),   # 64x64 blocks = 2x2 tiles
+        (512, 128, 32, 1, 0.50, False),
+        (2048, 32, 32, 1, 0.04, True),   # a global row and column: strips walked by four wavefronts together
+        (2048, 64, 64, 1, 0.06, True),
+    ],
+)
+def test_bf16_matches_oracle(L, bs, d, NB, p, glob):
+    mat = _mask(L // bs, p, seed=L + bs + d, global_block=glob)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=1, scale=1.2)
+    _run_and_check(abi, Q, K, V, dO, tag=f"bf16 L={L} bs={bs} d={d}")
+    abi.close()
+
+
+def test_bf16_empty_block_row_and_column_and_large_logits():
+    L, bs, d, NB = 256, 32, 32, 2
+    mat = _mask(L // bs, 0.4, seed=5, empty_row=2, empty_col=5)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=2, scale=4.0)  # logits of +-50 and more: exercises the running maximum
+    _run_and_check(abi, Q, K, V, dO, tag="bf16 empty strips, large logits")
+    abi.close()
+
+
+@pytest.mark.parametrize("d", [32, 64])
+def test_bf16_with_key_mask(d):
+    L, bs, NB = 256, 32, 4
+    mat = _mask(L // bs, 0.5, seed=7)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=3)
+    valid = torch.tensor([256, 200, 131, 64])
+    key_mask = (torch.arange(L)[None, :] < valid[:, None]).float()
+    pen = (1e6 * (1.0 - key_mask)).contiguous().cuda()
+    _run_and_check(abi, Q, K, V, dO, pen, tag=f"bf16 key mask d={d}")
+    O, _ = abi.forward(Q, K, V, pen)
+    assert torch.isfinite(O.float()).all()
+    abi.close()
+
+
+def test_bf16_rejects_element_patterns_and_fp32_handles():
+    L, d, NB = 128, 32, 1
+    sm, off, col = workloads.window_random_csr(L, 4, 12, seed=3)
+    abi = BF16ABI(d, L, NB, 1)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=4)
+    with pytest.raises(_lib.SpionLibraryError, match="32x32 tiles"):
+        abi.forward(Q, K, V)
+    abi.close()
+    fp32 = SparseABI(d, L, NB, 32, with_mask=False)
+    abi2 = BF16ABI(d, L, NB, 32)
+    abi2.set_pattern(sm, off, col)
+    good = abi2.handle
+    abi2.handle = fp32.handle
+    with pytest.raises(_lib.SpionLibraryError, match="bf16 init"):
+        abi2.forward(Q, K, V)
+    abi2.handle = good
+    abi2.close()
+    fp32.close()
+
+
+def test_bf16_module_autograd_matches_dense_statement():
+    B, H, L, d, bs = 2, 2, 256, 64, 64
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    mat = torch.from_numpy(_mask(L // bs, 0.5, seed=9)).cuda()
+    g = torch.Generator().manual_seed(11)
+    q, k, v, do = ((torch.randn(B, H, L, d, generator=g) * s).to(torch.bfloat16).cuda() for s in (1.0, 1.0, 1.0, 1.0))
+    for t in (q, k, v):
+        t.requires_grad_()
+    mod = BlockAttentionBF16(cfg)
+    out, zero = mod(q, k, v, torch.ones(B, L, device="cuda"), mat)
+    assert zero == 0 and out.dtype == torch.bfloat16
+    out.backward(do)
+    qr, kr, vr = (t.detach().double().cpu().requires_grad_() for t in (q, k, v))
+    pattern = mat.cpu().double().repeat_interleave(bs, 0).repeat_interleave(bs, 1)
+    ref, _ = osa.dense_masked_attention(qr, kr, vr, pattern, None)
+    ref.backward(do.double().cpu())
+    assert_close_bf16(out.detach().float().cpu().numpy(), ref.detach().numpy(), "module out")
+    for name, a, b in (("dq", q, qr), ("dk", k, kr), ("dv", v, vr)):
+        assert_close_bf16(a.grad.float().cpu().numpy(), b.grad.numpy(), f"module {name}")
+
+
+def test_bf16_scale_up_shape_agrees_with_fp32_path():
+    """Config 5 at full size (B=4, H=8, L=16384, d=64, 64x64 blocks, band + global row/column + 1 % random):
+    too large for the CPU oracle, so the bf16 kernels are compared with the fp32 tile kernels (themselves
+    checked against the oracle at smaller sizes) on the same bf16-rounded inputs."""
+    B, H, L, d, bs = 4, 8, 16384, 64, 64
+    NB = B * H
+    mat = workloads.config5_mask()
+    from spion_amd.csr import block_mask_to_csr_host
+    sm, off, col = block_mask_to_csr_host(mat, bs)
+    g = torch.Generator().manual_seed(0)
+    Q, K, V, dO = ((torch.randn(NB, L, d, generator=g) * s).to(torch.bfloat16).cuda() for s in (1.0, 1.0, 1.0, 1.0))
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    O, lse = abi.forward(Q, K, V)
+    dQ, dK, dV = abi.backward(Q, K, V, O, lse, dO)
+    torch.cuda.synchronize()
+    ref = SparseABI(d, L, NB, bs, with_mask=False)
+    ref.set_pattern(sm, off, col)
+    Qf, Kf, Vf, dOf = (t.float() for t in (Q, K, V, dO))
+    Or, P = ref.forward(Qf, Kf, Vf)
+    dQr, dKr, dVr = ref.backward(Qf, Kf, Vf, P, dOf)
+    torch.cuda.synchronize()
+    del P
+    for name, a, b in (("O", O, Or), ("dQ", dQ, dQr), ("dK", dK, dKr), ("dV", dV, dVr)):
+        a = a.float()
+        assert torch.isfinite(a).all(), name
+        rel_l2 = ((a - b).pow(2).sum() / b.pow(2).sum()).sqrt().item()
+        assert rel_l2 <= REL_TOL_BF16, f"{name}: relative L2 error {rel_l2:.3e}"
+        excess = ((a - b).abs() - REL_TOL_BF16 * (b.abs() + b.abs().max())).max().item()
+        assert excess <= 0, f"{name}: exceeds the element tolerance by {excess}"
+    abi.close()
+    ref.close()

@@ -56,6 +56,24 @@ def test_pattern_config2_bit_exact_against_both_routes():
         assert np.array_equal(mat[i].astype(np.int8), m32)
 
 
+@pytest.mark.parametrize("density", [0.2, 0.45, 0.8])
+def test_pattern_topk_with_ties(density):
+    """Maps of few exact levels (multiples of 1/4): pooled values are exact in both routes and tie massively, so
+    the k-th largest value is shared by many blocks and the lower-flat-index rule decides."""
+    L, bs = 512, 32
+    g = torch.Generator().manual_seed(11)
+    levels = torch.randint(0, 3, (2, L // 64, L // 64), generator=g).float() / 4
+    maps = levels.repeat_interleave(64, 1).repeat_interleave(64, 2).contiguous()
+    mat, pooled, _ = discover_block_masks(maps.cuda(), bs, mode="conv", density=density, return_aux=True)
+    mat, pooled = mat.cpu().numpy(), pooled.cpu().numpy()
+    for i in range(2):
+        ref, ref_pooled, k = op.generate_mask_conv(maps[i].numpy(), bs, density)
+        assert np.array_equal(pooled[i], ref_pooled)
+        kth = np.sort(ref_pooled.ravel())[::-1][k - 1]
+        assert (ref_pooled == kth).sum() > 1
+        assert np.array_equal(mat[i].astype(np.int8), ref)
+
+
 def test_pattern_topk_and_generators():
     L, bs = 256, 32
     g = torch.Generator().manual_seed(3)
