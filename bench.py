@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config2|config4|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -30,6 +30,7 @@ if ROOT not in sys.path:
 
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+PEAK_BF16_MFMA_TFLOPS = 2500.0
 
 
 def _event_ms(fn, iters, warm=3):
@@ -85,12 +86,10 @@ def build_workload(name):
         mat = None
         scale = 1.0
     elif name == "config5_fp32":
-        # shape of the scale-up configuration (L=16384, d=64, 64x64 blocks, band of 4 + global row/column
-        # + 1 % random blocks), run through the fp32 path: the bf16 variant is not built
+        # shape of the scale-up configuration (L=16384, d=64, 64x64 blocks, band + global row/column
+        # + 1 % random blocks) run through the fp32 path, for comparison with the bf16 one ("config5")
         B, H, L, d, bs = 4, 8, 16384, 64, 64
-        mat = workloads.band_random_block_mask(L // bs, 2, extra_frac=0.01, seed=1)
-        mat[0, :] = 1.0
-        mat[:, 0] = 1.0
+        mat = workloads.config5_mask()
         scale = 1.0 / 8.0
     else:
         raise SystemExit(f"unknown workload {name}")
@@ -255,6 +254,106 @@ def bench_encoder_step(args, dev):
     }
 
 
+def bench_bf16_scale_up(args, dev):
+    """Configuration 5: bf16 tensors, fp32 accumulation and softmax, B=4, H=8, L=16384, d=64, 64x64 blocks (band +
+    one global block row and column + 1 % random blocks), Q, K, V ~ N(0,1)/8.  A step is forward + backward of the
+    ``BlockAttentionBF16`` module.  The probabilities are never written to memory, so the algorithmic bytes are the
+    eleven [NB, L, d] bf16 tensors plus the fp32 row statistics; the roofline is HBM (ridge of bf16 MFMA: 310 flop/B,
+    this workload: 12*n*d / (22*L*d) = 268 flop/B)."""
+    import spion_amd
+    from spion_amd import _lib, workloads
+    from spion_amd.csr import block_mask_to_csr_host
+
+    B, H, L, d, bs = 4, 8, 16384, 64, 64
+    NB = B * H
+    mat_np = workloads.config5_mask()
+    _, off, _ = block_mask_to_csr_host(mat_np, bs)
+    nnz = int(off[-1])
+    mat = torch.from_numpy(mat_np).to(dev)
+    q, k, v, do = (t.to(torch.bfloat16) for t in workloads.qkv(B, H, L, d, scale=1.0 / 8.0, seed=0, device=dev))
+    for t in (q, k, v):
+        t.requires_grad_()
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    module = spion_amd.BlockAttentionBF16(cfg)
+    ones = torch.ones(B, L, device=dev)
+
+    def step():
+        for t in (q, k, v):
+            t.grad = None
+        out, _ = module(q, k, v, ones, mat)
+        out.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    core = _lib.core()
+    idx = module.csr_cache.get(mat, bs)
+    Q, K, V, dO = (t.detach().reshape(NB, L, d).contiguous() for t in (q, k, v, do))
+    O, dQ, dK, dV = (torch.empty_like(Q) for _ in range(4))
+    lse = torch.empty(NB, L, device=dev)
+    tail = (idx.offsets.data_ptr(), idx.columns.data_ptr(), idx.sum_mat.data_ptr(), nnz)
+
+    def fwd():
+        core.spion_block_bf16_attn_forward(module.attn_handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(), None,
+                                           O.data_ptr(), lse.data_ptr(), *tail)
+
+    def bwd():
+        core.spion_block_bf16_attn_backward(module.attn_handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(), None,
+                                            O.data_ptr(), lse.data_ptr(), dO.data_ptr(), dQ.data_ptr(), dK.data_ptr(),
+                                            dV.data_ptr(), *tail)
+
+    it = max(10, args.steps)
+    t_fwd = _event_ms(fwd, it)
+    t_bwd = _event_ms(bwd, it)
+    core.spion_set_backward_passes(module.attn_handle, 1)
+    t_row = _event_ms(bwd, it)
+    core.spion_set_backward_passes(module.attn_handle, 2)
+    t_col = _event_ms(bwd, it)
+    core.spion_set_backward_passes(module.attn_handle, 3)
+    _lib.check_error("bench bf16 kernels")
+
+    alg_flops = workloads.sparse_flops(nnz, d, NB)
+    tensor = 2.0 * L * d * NB  # one [NB, L, d] bf16 tensor
+    stat = 4.0 * L * NB        # one [NB, L] fp32 row statistic
+    # forward: read Q, K, V, write O, lse; row pass: read Q, K, V, dO, O, lse, write dQ, -g; column pass: read
+    # Q, K, V, dO, lse, -g, write dK, dV
+    kbytes = {"bf16_fwd_kernel": 4 * tensor + stat, "bf16_bwd_row_kernel": 6 * tensor + 2 * stat,
+              "bf16_bwd_col_kernel": 6 * tensor + 2 * stat}
+    alg_bytes = 11 * tensor + 2 * stat  # each tensor once (11 of them) plus the statistic written and read back
+    kernels = dict(zip(kbytes, (t_fwd, t_row, t_col)))
+    dom = max(kernels, key=kernels.get)
+    roof = dict(bound="hbm", kernel=dom, achieved=kbytes[dom] / kernels[dom] / 1e6, peak=PEAK_HBM_GBS, unit="GB/s",
+                traffic=None)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
+    roof["mfma_frac_of_bf16_peak"] = (alg_flops / 3.0) / kernels[dom] / 1e9 / PEAK_BF16_MFMA_TFLOPS
+    result = {
+        "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
+        "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1)/8 tensors rounded to bf16, seeded block mask)",
+        "config": {"workload": f"config5: bf16 sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, block {bs}, "
+                               f"nnz/head={nnz}, block density={round(float(mat_np.mean()), 4)}",
+                   "kernel_path": "mfma-bf16-tile"},
+        "abi_ms": {"attn_forward": round(t_fwd, 4), "attn_backward": round(t_bwd, 4),
+                   "fwd_plus_bwd": round(t_fwd + t_bwd, 4)},
+        "abi_effective_tflops": alg_flops / (t_fwd + t_bwd) / 1e9,
+        "abi_effective_hbm_gbs": alg_bytes / (t_fwd + t_bwd) / 1e6,
+        "algorithmic": {"gflop": alg_flops / 1e9, "mbytes": alg_bytes / 1e6},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        wl = build_workload("config5_fp32")
+        result["cpu_baseline"] = cpu_baseline(wl)
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -289,6 +388,9 @@ def main():
         return
     if args.workload == "config3":
         print(json.dumps(bench_encoder_step(args, dev)))
+        return
+    if args.workload == "config5":
+        print(json.dumps(bench_bf16_scale_up(args, dev)))
         return
 
     wl = build_workload(args.workload)
