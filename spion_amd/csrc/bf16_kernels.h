@@ -14,8 +14,10 @@
 //   * products over a tile's 32 keys or queries: slot e of instruction t in half h is tile row
 //     16t + 8(e/4) + 4h + e%4 = acc_row(8t+e, h), so the accumulator of the first product, converted to
 //     bf16, is the B operand of the second one register for register.  The A operand (the tile of K, V, Q or
-//     dO seen feature-major) comes from the row-major tile the first product already loaded: it is written
-//     to a wave-private LDS tile and read back with the transposing LDS read of gfx950.
+//     dO seen feature-major) is read from the tile's wave-private LDS copy with the transposing LDS read
+//     of gfx950.
+// Tiles travel global memory -> registers (consecutive addresses across the wavefront, one tile ahead) ->
+// wave-private LDS tile -> operand layouts; same-wave LDS accesses complete in order, so no barrier is involved.
 // Queries are the lane index of every row-pass accumulator (S^T, dP^T, O^T, dQ^T), so row statistics are
 // lane scalars; keys are the lane index in the column pass.
 //
@@ -40,6 +42,16 @@ __device__ __forceinline__ void ldb_rows(rsrc_t r, int voff, int soff, bf16x8 (&
 #pragma unroll
     for (int t = 0; t < D / 16; ++t)
         x[t] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff + 16 * t, 0));
+}
+
+// A 32 x D bf16 tile of a row-major head slice is 64*D consecutive bytes.  Loaded as D/16 instructions in which
+// the 64 lanes read 1 KB of consecutive addresses: 8 cache lines per instruction.  (Reading it directly in the
+// operand layout -- every lane 16 bytes of its own row -- costs one tag lookup per lane and was measured to
+// keep the texture path busy 84 % of the time.)  Lane l, instruction i holds 16-byte piece 64i + l of the tile.
+template <int D>
+__device__ __forceinline__ void ldb_tile(rsrc_t r, int l16, int soff, u32x4 (&raw)[D / 16]) {
+#pragma unroll
+    for (int i = 0; i < D / 16; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(r, l16, soff + 1024 * i, 0);
 }
 
 template <int D>
@@ -75,6 +87,19 @@ struct LdsTile {
     static __device__ __forceinline__ void put_rows(char* T, int li, int h, const bf16x8 (&x)[D / 16]) {
 #pragma unroll
         for (int t = 0; t < D / 16; ++t) *reinterpret_cast<u32x4*>(T + li * RS + h * D + 16 * t) = __builtin_bit_cast(u32x4, x[t]);
+    }
+    // the tile as loaded by ldb_tile: piece 64i + l is row (64i + l) / (D/8), 16-byte column (64i + l) % (D/8)
+    static __device__ __forceinline__ void put_raw(char* T, int l, const u32x4 (&raw)[D / 16]) {
+        constexpr int CPR = D / 8;
+#pragma unroll
+        for (int i = 0; i < D / 16; ++i)
+            *reinterpret_cast<u32x4*>(T + ((64 * i) / CPR + l / CPR) * RS + (l % CPR) * 16) = raw[i];
+    }
+    // head-dimension operand of lane (row li, half h): features h*D/2 ..
+    static __device__ __forceinline__ void get_rows(const char* T, int li, int h, bf16x8 (&x)[D / 16]) {
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t)
+            x[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(T + li * RS + h * D + 16 * t));
     }
     // The transposing read works on groups of 16 lanes: lane j of a group points at 4 consecutive bf16,
     // and lane 4a+b receives element b of the pieces of lanes a, 4+a, 8+a, 12+a.  With lane j pointing at
@@ -177,7 +202,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
     const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
     typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][LT::BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     __shared__ float lds_m[BF16_WAVES][32], lds_z[BF16_WAVES][32];
     __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
@@ -193,7 +218,8 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
     const rsrc_t rO = make_rsrc(O + hb, hbytes);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int r_voff = li * D * 2 + h * D;
-    char* T = lds_t[w];
+    char* Tk = lds_t[w][0];
+    char* Tv = lds_t[w][1];
     const int tbase = LT::lane_base(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
@@ -208,7 +234,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
     for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
 
     struct Pre {
-        bf16x8 k[D / 16], v[D / 16];
+        u32x4 k[D / 16], v[D / 16];
         float pj[MASK ? 16 : 1];
     };
     Pre xa, xb;
@@ -216,8 +242,8 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_rows<D>(rK, r_voff, J * 32 * D * 2, x.k);
-            ldb_rows<D>(rV, r_voff, J * 32 * D * 2, x.v);
+            ldb_tile<D>(rK, l * 16, J * 32 * D * 2, x.k);
+            ldb_tile<D>(rV, l * 16, J * 32 * D * 2, x.v);
             if constexpr (MASK) {
                 float pj[16];
                 ldr_4x4(rM, 16 * h, J * 128, pj);
@@ -226,13 +252,16 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
             }
         },
         [&](Pre& c, int) {
-            LT::put_rows(T, li, h, c.v);
+            LT::put_raw(Tk, l, c.k);
+            LT::put_raw(Tv, l, c.v);
+            bf16x8 kr[D / 16];
+            LT::get_rows(Tk, li, h, kr);
             f32x16 init = splat16(0.f);
             if constexpr (MASK) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
             }
-            const f32x16 s = mma_feat_bf16<D>(c.k, q, init);  // S^T: register = key, lane = query
+            const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
             const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
             if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
                 const float mn = t2 > m + BF16_LAZY ? t2 : m;
@@ -251,7 +280,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
             bf16x8 pb[2];
             pack16(p, pb);
             bf16x8 vt[D / 32][2];
-            LT::get_tile_t(T, tbase, vt);
+            LT::get_tile_t(Tv, tbase, vt);
             mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
         });
     z = half_swap_sum(z);
@@ -293,7 +322,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
     const float* __restrict__ pen, float* __restrict__ Gneg, __bf16* __restrict__ dQ, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
     typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][LT::BYTES];
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
@@ -308,7 +337,8 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
     const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rO = make_rsrc(O + hb, hbytes), rdQ = make_rsrc(dQ + hb, hbytes);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int r_voff = li * D * 2 + h * D;
-    char* T = lds_t[w];
+    char* Tk = lds_t[w][0];
+    char* Tv = lds_t[w][1];
     const int tbase = LT::lane_base(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
@@ -333,7 +363,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
     struct Pre {
-        bf16x8 k[D / 16], v[D / 16];
+        u32x4 k[D / 16], v[D / 16];
         float pj[MASK ? 16 : 1];
     };
     Pre xa, xb;
@@ -341,8 +371,8 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_rows<D>(rK, r_voff, J * 32 * D * 2, x.k);
-            ldb_rows<D>(rV, r_voff, J * 32 * D * 2, x.v);
+            ldb_tile<D>(rK, l * 16, J * 32 * D * 2, x.k);
+            ldb_tile<D>(rV, l * 16, J * 32 * D * 2, x.v);
             if constexpr (MASK) {
                 float pj[16];
                 ldr_4x4(rM, 16 * h, J * 128, pj);
@@ -351,21 +381,25 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
             }
         },
         [&](Pre& c, int) {
-            LT::put_rows(T, li, h, c.k);
+            LT::put_raw(Tk, l, c.k);
+            LT::put_raw(Tv, l, c.v);
+            bf16x8 kr[D / 16], vr[D / 16];
+            LT::get_rows(Tk, li, h, kr);
+            LT::get_rows(Tv, li, h, vr);
             f32x16 init = splat16(0.f);
             if constexpr (MASK) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
             }
-            const f32x16 s = mma_feat_bf16<D>(c.k, q, init);
-            const f32x16 dp = mma_feat_bf16<D>(c.v, go, gneg);  // dO_i . v_j - g_i
+            const f32x16 s = mma_feat_bf16<D>(kr, q, init);
+            const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
             float ds[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
             bf16x8 dsb[2];
             pack16(ds, dsb);
             bf16x8 kt[D / 32][2];
-            LT::get_tile_t(T, tbase, kt);
+            LT::get_tile_t(Tk, tbase, kt);
             mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
         });
 #pragma unroll
@@ -421,7 +455,7 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
     // chain starts.
     constexpr bool DEEP = D == 32;
     struct Pre {
-        bf16x8 q[D / 16], go[D / 16];
+        u32x4 q[D / 16], go[D / 16];
         float lse[DEEP ? 16 : 1], gneg[DEEP ? 16 : 1];
         int I;
     };
@@ -431,8 +465,8 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
         [&](Pre& x, int i) {
             const int I = desc[sa.rank + min(i, nu - 1) * sa.step].x;
             x.I = I;
-            ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, x.q);
-            ldb_rows<D>(rdO, r_voff, I * 32 * D * 2, x.go);
+            ldb_tile<D>(rQ, l * 16, I * 32 * D * 2, x.q);
+            ldb_tile<D>(rdO, l * 16, I * 32 * D * 2, x.go);
             if constexpr (DEEP) {
                 ldr_4x4(rL, 16 * h, I * 128, x.lse);
                 ldr_4x4(rG, 16 * h, I * 128, x.gneg);
@@ -450,13 +484,16 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
                 ldr_4x4(rG, 16 * h, c.I * 128, gn);
                 ldr_4x4(rL, 16 * h, c.I * 128, lse);
             }
-            LT::put_rows(Tq, li, h, c.q);
-            LT::put_rows(Tg, li, h, c.go);
-            const f32x16 s = mma_feat_bf16<D>(c.q, k, sinit);  // S: register = query, lane = key
+            LT::put_raw(Tq, l, c.q);
+            LT::put_raw(Tg, l, c.go);
+            bf16x8 qr[D / 16], gr[D / 16];
+            LT::get_rows(Tq, li, h, qr);
+            LT::get_rows(Tg, li, h, gr);
+            const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
             f32x16 ginit;
 #pragma unroll
             for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
-            const f32x16 dp = mma_feat_bf16<D>(c.go, v, ginit);  // dO_i . v_j - g_i
+            const f32x16 dp = mma_feat_bf16<D>(gr, v, ginit);  // dO_i . v_j - g_i
             float p[16], ds[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
