@@ -463,6 +463,7 @@ def main():
     it = max(10, args.steps)
     t_fwd = _event_ms(fwd, it)
     t_bwd = _event_ms(bwd, it)
+    t_seq = _event_ms(lambda: (fwd(), bwd()), it)  # the order a training step runs them in (cache state differs)
     core.spion_set_backward_passes(handle, 1)
     t_row = _event_ms(bwd, it)
     core.spion_set_backward_passes(handle, 2)
@@ -510,7 +511,7 @@ def main():
                                f"{wl['block_density'] if wl['block_density'] is None else round(wl['block_density'], 4)}",
                    "kernel_path": {1: "mfma-tile", 2: "element"}[path]},
         "abi_ms": {"attn_forward": round(t_fwd, 4), "attn_backward": round(t_bwd, 4),
-                   "fwd_plus_bwd": round(t_fwd + t_bwd, 4)},
+                   "fwd_plus_bwd": round(t_fwd + t_bwd, 4), "fwd_then_bwd_sequence": round(t_seq, 4)},
         "abi_effective_tflops": alg_flops / (t_fwd + t_bwd) / 1e9,
         "abi_fraction_of_fp32_mfma_peak": alg_flops / (t_fwd + t_bwd) / 1e9 / PEAK_FP32_MFMA_TFLOPS,
         "abi_effective_hbm_gbs": alg_bytes / (t_fwd + t_bwd) / 1e6,

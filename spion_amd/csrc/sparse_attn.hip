@@ -821,10 +821,40 @@ __global__ __launch_bounds__(256) void transpose_last2_kernel(const float* __res
         if (c0 + c < cols && r0 + tx < rows) out[base + (size_t)(c0 + c) * rows + r0 + tx] = tile[tx][c];
 }
 
+// Same for narrow matrices (cols = 32 or 64, the head dimension) with rows a multiple of 256: a work-group
+// moves 256 rows, reading 16 bytes per thread and writing 1 KB runs of each output row.
+template <int COLS>
+__global__ __launch_bounds__(256) void transpose_narrow_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                               int rows) {
+    __shared__ float tile[256][COLS + 1];
+    const size_t base = (size_t)blockIdx.y * rows * COLS;
+    const int r0 = blockIdx.x * 256, t = threadIdx.x;
+    const float4* src = reinterpret_cast<const float4*>(in + base + (size_t)r0 * COLS);
+#pragma unroll
+    for (int k = 0; k < COLS / 4; ++k) {
+        const int e = t + 256 * k;  // float4 index inside the 256 x COLS slab
+        const float4 v = src[e];
+        const int r = e / (COLS / 4), c = (e % (COLS / 4)) * 4;
+        tile[r][c] = v.x;
+        tile[r][c + 1] = v.y;
+        tile[r][c + 2] = v.z;
+        tile[r][c + 3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int c = 0; c < COLS; ++c) out[base + (size_t)c * rows + r0 + t] = tile[t][c];
+}
+
 int transpose_last2(const float* in, float* out, int batch, int rows, int cols, hipStream_t stream) {
     if (!in || !out || batch <= 0 || rows <= 0 || cols <= 0 || batch > 65535) {
         set_error("spion_transpose_last2: bad arguments");
         return 1;
+    }
+    if ((cols == 32 || cols == 64) && rows % 256 == 0) {
+        const dim3 grid(rows / 256, batch);
+        if (cols == 32) hipLaunchKernelGGL(transpose_narrow_kernel<32>, grid, dim3(256), 0, stream, in, out, rows);
+        else hipLaunchKernelGGL(transpose_narrow_kernel<64>, grid, dim3(256), 0, stream, in, out, rows);
+        return check_launch("transpose_narrow_kernel") ? 0 : 1;
     }
     dim3 grid((cols + 63) / 64, (rows + 63) / 64, batch);
     hipLaunchKernelGGL(transpose_last2_kernel, grid, dim3(256), 0, stream, in, out, rows, cols);

@@ -152,6 +152,35 @@ __device__ __forceinline__ void lds_get_feat32(const float* T, int li, int h, fl
     }
 }
 
+// "Linear" access to a 32 x 32 fp32 tile whose rows are `ld` floats apart: four 16-byte instructions in which
+// lane l, instruction i touch row 8i + l/8, columns 4(l%8) .. +3 -- eight full 128-byte rows per instruction.
+// The texture path spends about as long on a 4-byte-per-lane instruction as on half a 16-byte-per-lane one
+// (measured: ~16 vs ~32 cycles per wavefront instruction), so a tile fetched this way costs half the
+// 16 single-float instructions of the operand layouts; the operand layouts are then read from a wave-private
+// LDS copy of the tile.
+__device__ __forceinline__ int lin_voff(int l, int ld) { return ((l >> 3) * ld + 4 * (l & 7)) * 4; }
+__device__ __forceinline__ void ldr_tile_lin(rsrc_t r, int voff, int soff, int ld, f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = ld4(r, voff, soff + 32 * i * ld);
+}
+__device__ __forceinline__ void str_tile_lin(rsrc_t r, int voff, int soff, int ld, const f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st4(r, voff, soff + 32 * i * ld, raw[i]);
+}
+__device__ __forceinline__ void lds_put_lin(float* T, int l, const f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(T + (8 * i + (l >> 3)) * TS + 4 * (l & 7)) = raw[i];
+}
+__device__ __forceinline__ void lds_get_lin(const float* T, int l, f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const f32x4*>(T + (8 * i + (l >> 3)) * TS + 4 * (l & 7));
+}
+// operand over 32 features from a feature-major tile T[feature][row]: x[s] = T[16h + s][li]
+__device__ __forceinline__ void lds_get_featcols32(const float* T, int li, int h, float (&x)[16]) {
+#pragma unroll
+    for (int s = 0; s < 16; ++s) x[s] = T[(16 * h + s) * TS + li];
+}
+
 // acc = init + A.B over the head dimension (chain of D/2 MFMA).
 template <int D>
 __device__ __forceinline__ f32x16 mma_feat_init(const float (&a)[D / 2], const float (&b)[D / 2], f32x16 init) {
@@ -424,8 +453,9 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_g[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 ? 3 : 1) * 32 * TS];
+    // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
+    const int item = nbr * NB - 1 - xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
@@ -491,7 +521,42 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     f32x16 acc[D / 32];
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
-    {
+    if constexpr (D == 32) {
+        // One tile ahead: the V^T tile, the P tile and the K tile, each fetched linearly (12 instructions a
+        // tile instead of 48) and turned into operands through wave-private LDS copies.
+        struct Pre {
+            f32x4 vt[4], pv[4], kb[4];
+        };
+        float* Tv = T;
+        float* Tp = T + 32 * TS;
+        float* Tk = T + 64 * TS;
+        const int vl = lin_voff(l, L), pl = lin_voff(l, rn), kl = lin_voff(l, D);
+        Pre xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](Pre& x, int i) {
+                const int t = w + min(i, nu - 1) * WAVES;
+                const int J = tcol[t0 + t];
+                ldr_tile_lin(rV, vl, J * 128, L, x.vt);
+                ldr_tile_lin(rP, pl, p_base + t * 128, rn, x.pv);
+                ldr_tile_lin(rK, kl, J * 32 * D * 4, D, x.kb);
+            },
+            [&](Pre& c, int) {
+                lds_put_lin(Tv, l, c.vt);
+                lds_put_lin(Tp, l, c.pv);
+                lds_put_lin(Tk, l, c.kb);
+                float vt[16], pr[16];
+                lds_get_featcols32(Tv, li, h, vt);
+                lds_get_rows(Tp, li, h, pr);
+                f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
+                float ds[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
+                float kb[1][16];
+                lds_get_cols(Tk, li, h, kb[0]);
+                mma_b<D>(ds, kb, acc);
+            });
+    } else {
         // One tile ahead: V^T operand, P tile and (d = 32) the K operand of the second product; for d = 64
         // that operand would not fit in registers and is requested when the tile's first chain starts.
         constexpr bool DEEP = D == 32;

@@ -335,3 +335,11 @@ def test_backward_row_sums_with_and_without_output_cache():
         for name, t in zip(("dQ", "dK", "dV"), got):
             assert_close(t.cpu().numpy(), ref[name], what=f"{tag} {name}")
     abi.close()
+
+
+@pytest.mark.parametrize("shape", [(3, 512, 32), (2, 256, 64), (2, 100, 32), (1, 70, 45), (4, 2, 1024, 32)])
+def test_library_transpose_is_exact(shape):
+    from spion_amd import _lib
+    x = torch.randn(*shape, device="cuda")
+    got = _lib.transpose_last2(x)
+    assert got.is_contiguous() and torch.equal(got, x.transpose(-1, -2).contiguous())
