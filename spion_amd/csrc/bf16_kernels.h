@@ -254,8 +254,12 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
         [&](Pre& c, int) {
             LT::put_raw(Tk, l, c.k);
             LT::put_raw(Tv, l, c.v);
-            bf16x8 kr[D / 16];
+            // every LDS read is issued before the first chain starts (the compiler would otherwise sink each
+            // one next to its use and wait for it there)
+            bf16x8 kr[D / 16], vt[D / 32][2];
             LT::get_rows(Tk, li, h, kr);
+            LT::get_tile_t(Tv, tbase, vt);
+            __builtin_amdgcn_sched_barrier(0);
             f32x16 init = splat16(0.f);
             if constexpr (MASK) {
 #pragma unroll
@@ -279,8 +283,6 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
             }
             bf16x8 pb[2];
             pack16(p, pb);
-            bf16x8 vt[D / 32][2];
-            LT::get_tile_t(Tv, tbase, vt);
             mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
         });
     z = half_swap_sum(z);
@@ -383,9 +385,11 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
         [&](Pre& c, int) {
             LT::put_raw(Tk, l, c.k);
             LT::put_raw(Tv, l, c.v);
-            bf16x8 kr[D / 16], vr[D / 16];
+            bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
             LT::get_rows(Tk, li, h, kr);
             LT::get_rows(Tv, li, h, vr);
+            LT::get_tile_t(Tk, tbase, kt);
+            __builtin_amdgcn_sched_barrier(0);
             f32x16 init = splat16(0.f);
             if constexpr (MASK) {
 #pragma unroll
@@ -398,8 +402,6 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
             for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
             bf16x8 dsb[2];
             pack16(ds, dsb);
-            bf16x8 kt[D / 32][2];
-            LT::get_tile_t(Tk, tbase, kt);
             mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
         });
 #pragma unroll
@@ -486,9 +488,14 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
             }
             LT::put_raw(Tq, l, c.q);
             LT::put_raw(Tg, l, c.go);
-            bf16x8 qr[D / 16], gr[D / 16];
+            bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
             LT::get_rows(Tq, li, h, qr);
             LT::get_rows(Tg, li, h, gr);
+            if constexpr (DEEP) {
+                LT::get_tile_t(Tq, tbase, qt);
+                LT::get_tile_t(Tg, tbase, gt);
+            }
+            __builtin_amdgcn_sched_barrier(0);
             const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
             f32x16 ginit;
 #pragma unroll
@@ -503,9 +510,10 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
             bf16x8 pb[2], dsb[2];
             pack16(p, pb);
             pack16(ds, dsb);
-            bf16x8 qt[D / 32][2], gt[D / 32][2];
-            LT::get_tile_t(Tq, tbase, qt);
-            LT::get_tile_t(Tg, tbase, gt);
+            if constexpr (!DEEP) {  // d = 64: no registers to hold them across the chains
+                LT::get_tile_t(Tq, tbase, qt);
+                LT::get_tile_t(Tg, tbase, gt);
+            }
             mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
             mma_tile_bf16<D>(gt, pb, av);   // dV^T
         });

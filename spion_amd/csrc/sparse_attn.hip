@@ -430,6 +430,17 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
         const std::vector<int> wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
+        // Behind each pointer array: the strips sorted by length, longest first (the order the fp32 kernels
+        // walk a head in, so that the launch does not end on a long strip).
+        auto append_order = [&](std::vector<int>& ptr) {
+            std::vector<int> order(nbr);
+            for (int i = 0; i < nbr; ++i) order[i] = i;
+            std::stable_sort(order.begin(), order.end(),
+                             [&](int x, int y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
+            ptr.insert(ptr.end(), order.begin(), order.end());
+        };
+        append_order(trp);
+        append_order(tcp);
         pi.n_wg_row = (int)wgr.size() / 4;
         pi.n_wg_col = (int)wgc.size() / 4;
         o_wgr = append(wgr);

@@ -270,7 +270,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
+    const int bh = item / nbr, I = trp[nbr + 1 + item % nbr];  // strips of a head, longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
@@ -455,8 +455,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     __shared__ float lds_g[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 ? 3 : 1) * 32 * TS];
     // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
-    const int item = nbr * NB - 1 - xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = NB - 1 - item / nbr, I = trp[nbr + 1 + item % nbr];  // strips of a head, longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
@@ -545,15 +545,17 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 lds_put_lin(Tv, l, c.vt);
                 lds_put_lin(Tp, l, c.pv);
                 lds_put_lin(Tk, l, c.kb);
-                float vt[16], pr[16];
+                // every LDS read is issued before the first chain starts (left to itself the compiler sinks
+                // each read next to the MFMA that uses it and waits for it there)
+                float vt[16], pr[16], kb[1][16];
                 lds_get_featcols32(Tv, li, h, vt);
                 lds_get_rows(Tp, li, h, pr);
+                lds_get_cols(Tk, li, h, kb[0]);
+                __builtin_amdgcn_sched_barrier(0);
                 f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
-                float kb[1][16];
-                lds_get_cols(Tk, li, h, kb[0]);
                 mma_b<D>(ds, kb, acc);
             });
     } else {
@@ -608,7 +610,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, J = item % nbr;
+    const int bh = item / nbr, J = tcp[nbr + 1 + item % nbr];  // strips of a head, longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
