@@ -243,6 +243,7 @@ struct PatternIndex {
     // work-group lists of the bf16 kernels (four strip ids per work-group) over block rows / block columns
     int *d_wg_row = nullptr, *d_wg_col = nullptr;
     int n_wg_row = 0, n_wg_col = 0;
+    std::vector<int> row_len_desc;  // host copy: tiles per block row, longest first
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -441,6 +442,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         };
         append_order(trp);
         append_order(tcp);
+        pi.row_len_desc.resize(nbr);
+        for (int i = 0; i < nbr; ++i) pi.row_len_desc[i] = trp[trp[nbr + 1 + i] + 1] - trp[trp[nbr + 1 + i]];
         pi.n_wg_row = (int)wgr.size() / 4;
         pi.n_wg_col = (int)wgc.size() / 4;
         o_wgr = append(wgr);
@@ -561,23 +564,31 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
                             float* O, const int* offs, int nnz) {
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
-    const dim3 grid(nbr * a->NB);
-    const int wv = pick_waves(a, pi, nbr, true);
     float* ocache = ocache_for_forward(a, P);
-    // logit tiles stay in registers when every wavefront's share of the longest block row fits
+    // Logit tiles stay in registers when every wavefront's share of a block row fits (MAXT tiles).  Block rows
+    // are launched by length class -- up to MAXT tiles with one wavefront per row, up to 2 MAXT with two, up
+    // to 4 MAXT with four -- so that short rows do not pay for four nearly idle wavefronts and their merges.
     constexpr int MAXT = D == 32 ? 8 : 4;
-#define SPION_LAUNCH(W)                                                                                             \
-    do {                                                                                                            \
-        if (pi.max_row_tiles <= W * MAXT)                                                                           \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V, \
-                               pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);      \
-        else                                                                                                        \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Kt, V,    \
-                               pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale);      \
-    } while (0)
-    if (wv == 1) SPION_LAUNCH(1);
-    else if (wv == 2) SPION_LAUNCH(2);
-    else SPION_LAUNCH(4);
+#define SPION_LAUNCH(W, MT, S0, NS)                                                                                  \
+    hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MT>), dim3((NS) * a->NB), dim3(64 * W), 0, a->hdr.stream, Q, Kt, \
+                       V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale, S0, NS)
+    const int forced = getenv("SPION_TILE_WAVES_FWD") ? atoi(getenv("SPION_TILE_WAVES_FWD")) : 0;
+    if (pi.max_row_tiles > 4 * MAXT || forced) {  // rows too long for registers: two sweeps for every row
+        const int wv = forced == 1 || forced == 2 || forced == 4 ? forced : pick_waves(a, pi, nbr, true);
+        if (wv == 1) SPION_LAUNCH(1, 0, 0, nbr);
+        else if (wv == 2) SPION_LAUNCH(2, 0, 0, nbr);
+        else SPION_LAUNCH(4, 0, 0, nbr);
+    } else {
+        int n4 = 0, n2 = 0;  // pi.row_len_desc: lengths of the block rows, longest first
+        for (int len : pi.row_len_desc) {
+            if (len > 2 * MAXT) ++n4;
+            else if (len > MAXT) ++n2;
+        }
+        const int n1 = nbr - n4 - n2;
+        if (n4) SPION_LAUNCH(4, MAXT, 0, n4);
+        if (n2) SPION_LAUNCH(2, MAXT, n4, n2);
+        if (n1) SPION_LAUNCH(1, MAXT, n4 + n2, n1);
+    }
 #undef SPION_LAUNCH
 }
 

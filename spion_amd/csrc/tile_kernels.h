@@ -264,13 +264,14 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
     const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
-    int NB, int nnz, float scale) {
+    int NB, int nnz, float scale, int s0, int ns) {
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = trp[nbr + 1 + item % nbr];  // strips of a head, longest first
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 && MAXT > 0 ? 2 : 1) * 32 * TS];
+    // this launch covers strips s0 .. s0+ns-1 of the longest-first order of every head
+    const int item = xcd_remap(blockIdx.x, ns * NB);
+    const int bh = item / ns, I = trp[nbr + 1 + s0 + item % ns];
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
@@ -317,28 +318,46 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     if constexpr (MAXT > 0) {
         const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
         f32x16 S[MAXT];
-        float kbuf[2][KH];
         int Js[MAXT];  // tile ids of this wavefront, fetched up front (scalar loads, one wait)
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) Js[u] = u < nu ? tcol[t0 + w + u * WAVES] : 0;
-        if (nu > 0) ldr_cols<D>(rK, L, col_voff, Js[0] * 128, kbuf[0]);
+        // d = 32: K^T, V and P tiles move as four 16-byte instructions each (linear layout) and change layout
+        // in wave-private LDS tiles: a quarter of the vector-memory instructions, which keeps the wavefront
+        // clear of the 63 outstanding instructions it may have (loads and stores share that counter).
+        constexpr bool LIN = D == 32;
+        float* Tx = T + 32 * TS;  // K^T tile, later V tile (LIN only)
+        const int klin = lin_voff(l, L), vlin = lin_voff(l, D), plin = lin_voff(l, rn);
+        if constexpr (LIN) {
+            f32x4 kraw[2][4];
+            if (nu > 0) ldr_tile_lin(rK, klin, Js[0] * 128, L, kraw[0]);
 #pragma unroll
-        for (int u = 0; u < MAXT; ++u) {
-            if (u < nu) {
-                if (u + 1 < MAXT) ldr_cols<D>(rK, L, col_voff, Js[u + 1 < MAXT ? u + 1 : u] * 128, kbuf[(u + 1) & 1]);
-                S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(Js[u]));
-                m = max16(S[u], m);
+            for (int u = 0; u < MAXT; ++u) {
+                if (u < nu) {
+                    if (u + 1 < MAXT) ldr_tile_lin(rK, klin, Js[u + 1 < MAXT ? u + 1 : u] * 128, L, kraw[(u + 1) & 1]);
+                    lds_put_lin(Tx, l, kraw[u & 1]);
+                    float kf[KH];
+                    lds_get_featcols32(Tx, li, h, kf);
+                    __builtin_amdgcn_sched_barrier(0);
+                    S[u] = mma_feat_init<D>(kf, q, chain_init(Js[u]));
+                    m = max16(S[u], m);
+                }
+            }
+        } else {
+            float kbuf[2][KH];
+            if (nu > 0) ldr_cols<D>(rK, L, col_voff, Js[0] * 128, kbuf[0]);
+#pragma unroll
+            for (int u = 0; u < MAXT; ++u) {
+                if (u < nu) {
+                    if (u + 1 < MAXT) ldr_cols<D>(rK, L, col_voff, Js[u + 1 < MAXT ? u + 1 : u] * 128, kbuf[(u + 1) & 1]);
+                    S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(Js[u]));
+                    m = max16(S[u], m);
+                }
             }
         }
-        {   // row maximum over half-waves and waves
-            m = fmaxf(m, __shfl_xor(m, 32, 64));
-            if (WAVES > 1) {
-                if (h == 0) lds_m[w][li] = m;
-                __syncthreads();
-#pragma unroll
-                for (int ww = 0; ww < WAVES; ++ww) m = fmaxf(m, lds_m[ww][li]);
-            }
-        }
+        // Exponentials relative to this wavefront's own maximum; one merge of (maximum, sum) pairs over the
+        // half-waves and wavefronts then gives the row's maximum M and denominator, and the probabilities
+        // are the exponentials times 2^(m - M) / Z.
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
@@ -350,29 +369,62 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                 }
             }
         }
+        const float m_own = m;
         z += __shfl_xor(z, 32, 64);
         if (WAVES > 1) {
-            if (h == 0) lds_z[w][li] = z;
+            if (h == 0) {
+                lds_m[w][li] = m;
+                lds_z[w][li] = z;
+            }
             __syncthreads();
-            z = 0.f;
+            float Mx = lds_m[0][li];
 #pragma unroll
-            for (int ww = 0; ww < WAVES; ++ww) z += lds_z[ww][li];
+            for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+            float Z = 0.f;
+#pragma unroll
+            for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+            m = Mx;
+            z = Z;
         }
         z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
-        const float rinv = 1.0f / z;  // +inf denominator -> 0 -> P = 0, as in the reference
+        // +inf denominator -> 0 -> P = 0, as in the reference
+        const float rinv = __builtin_amdgcn_exp2f(m_own - m) * (1.0f / z);
 
-        float vbuf[2][D / 32][16];
-        if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * D * 4, vbuf[0]);
+        if constexpr (LIN) {
+            f32x4 vraw[2][4];
+            if (nu > 0) ldr_tile_lin(rV, vlin, Js[0] * 32 * D * 4, D, vraw[0]);
 #pragma unroll
-        for (int u = 0; u < MAXT; ++u) {
-            if (u < nu) {
-                const int t = w + u * WAVES;
-                if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, vbuf[(u + 1) & 1]);
-                float p[16];
+            for (int u = 0; u < MAXT; ++u) {
+                if (u < nu) {
+                    const int t = w + u * WAVES;
+                    if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, D, vraw[(u + 1) & 1]);
+                    lds_put_lin(Tx, l, vraw[u & 1]);
+                    float p[16], vb[1][16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
-                store_p(p, t);
-                mma_b<D>(p, vbuf[u & 1], o);
+                    for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                    lds_put_rows(T, li, h, p);
+                    lds_get_cols(Tx, li, h, vb[0]);
+                    f32x4 pl[4];
+                    lds_get_lin(T, l, pl);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mma_b<D>(p, vb, o);
+                    str_tile_lin(rP, plin, p_base + t * 128, rn, pl);
+                }
+            }
+        } else {
+            float vbuf[2][D / 32][16];
+            if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * D * 4, vbuf[0]);
+#pragma unroll
+            for (int u = 0; u < MAXT; ++u) {
+                if (u < nu) {
+                    const int t = w + u * WAVES;
+                    if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, vbuf[(u + 1) & 1]);
+                    float p[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                    store_p(p, t);
+                    mma_b<D>(p, vbuf[u & 1], o);
+                }
             }
         }
     } else {
