@@ -63,6 +63,50 @@ __device__ __forceinline__ float row_dot(const float* __restrict__ a, const floa
     return s;
 }
 
+// Dot products of one vector a (the same for all lanes) with up to 64 gathered rows X[row_l], one result per
+// lane.  The rows are fetched LPR lanes to a row -- one or two cache lines per instruction instead of the 64 a
+// lane-per-row gather touches -- into a wave-private LDS tile (row stride D + 4 floats), from which every lane
+// then reads its own row.  D <= 64.
+template <int D>
+struct GatherDot {
+    static constexpr int LPR = D >= 64 ? 64 : D;
+    static constexpr int G = 64 / LPR;
+    static constexpr int CPL = D / LPR;
+    static constexpr int RS = D + 4;
+    static constexpr int FLOATS = 64 * RS;
+    static __device__ __forceinline__ float run(float* T, const float* __restrict__ a, const float* __restrict__ X,
+                                                int row_l, int nk, int lane) {
+        const int grp = lane / LPR, cl = lane % LPR;
+        constexpr int UN = 8;
+        for (int kb = 0; kb < nk; kb += UN * G) {
+            float x[UN][CPL];
+#pragma unroll
+            for (int j = 0; j < UN; ++j) {
+                const int rr = __shfl(row_l, (kb + j * G + grp) & 63, 64);
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) x[j][c] = X[(size_t)rr * D + cl + c * LPR];
+            }
+#pragma unroll
+            for (int j = 0; j < UN; ++j)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) T[((kb + j * G + grp) & 63) * RS + cl + c * LPR] = x[j][c];
+        }
+        // same-wave LDS accesses complete in order: no barrier
+        const float4* t4 = reinterpret_cast<const float4*>(T + lane * RS);
+        const float4* a4 = reinterpret_cast<const float4*>(a);
+        float s = 0.f;
+#pragma unroll
+        for (int t = 0; t < D / 4; ++t) {
+            const float4 x = t4[t], y = a4[t];
+            s = fmaf(x.x, y.x, s);
+            s = fmaf(x.y, y.y, s);
+            s = fmaf(x.z, y.z, s);
+            s = fmaf(x.w, y.w, s);
+        }
+        return s;
+    }
+};
+
 // acc[c] += sum_k w_k * X[col_k][c] over the entries of one CSR row, the entries being held one per
 // lane in chunks of 64 (w_l, col_l); LPR lanes cover one X row, 64/LPR entries are processed at once.
 template <int D>
@@ -79,13 +123,29 @@ struct RowAcc {
         const int grp = lane / LPR, cl = lane % LPR;
         // Uniform trip count: every lane takes part in every shuffle.  Slots past nk carry w = 0
         // and row 0 (set by the caller), so they add nothing.
-        for (int kb = 0; kb < nk; kb += G) {
-            const int kk = kb + grp;
-            float w = __shfl(w_l, kk, 64);
-            int rr = __shfl(row_l, kk, 64);
-            const float* xr = X + (size_t)rr * D + cl;
+        // Eight gathers are in flight per lane before the first one is consumed: the loop is bound by the
+        // latency of the gathered rows, not by their volume.
+        constexpr int UN = 8;
+        for (int kb = 0; kb < nk; kb += UN * G) {
+            float w[UN];
+            const float* xr[UN];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) acc[c] = fmaf(w, xr[c * LPR], acc[c]);
+            for (int j = 0; j < UN; ++j) {
+                const int kk = kb + j * G + grp;  // < 64 + UN*G: shuffles wrap, slots past nk are zero weights
+                w[j] = __shfl(w_l, kk & 63, 64);
+                const int rr = __shfl(row_l, kk & 63, 64);
+                if (kb + j * G >= 64) w[j] = 0.f;
+                xr[j] = X + (size_t)rr * D + cl;
+            }
+            float x[UN][CPL];
+#pragma unroll
+            for (int j = 0; j < UN; ++j)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) x[j][c] = xr[j][c * LPR];
+#pragma unroll
+            for (int j = 0; j < UN; ++j)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) acc[c] = fmaf(w[j], x[j][c], acc[c]);
         }
     }
     __device__ __forceinline__ void finish(float* __restrict__ out_row, int lane) {
@@ -165,10 +225,25 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
     const int* cj = cols + r0;
 
     float g = 0.f;
-    for (int k = lane; k < cnt; k += 64) {
-        float t = row_dot<D>(go, V + hb + (size_t)cj[k] * D) * p[k];
-        ds[k] = t;
-        g += t;
+    if constexpr (D <= 64) {
+        __shared__ __attribute__((aligned(16))) float lds_rows[ELEM_WAVES][GatherDot<D>::FLOATS];
+        float* T = lds_rows[threadIdx.x >> 6];
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + lane;
+            const int col = k < cnt ? cj[k] : 0;
+            const float dp = GatherDot<D>::run(T, go, V + hb, col, min(64, cnt - c0), lane);
+            if (k < cnt) {
+                const float t = dp * p[k];
+                ds[k] = t;
+                g += t;
+            }
+        }
+    } else {
+        for (int k = lane; k < cnt; k += 64) {
+            float t = row_dot<D>(go, V + hb + (size_t)cj[k] * D) * p[k];
+            ds[k] = t;
+            g += t;
+        }
     }
     g = wave_sum(g);
 
