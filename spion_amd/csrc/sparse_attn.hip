@@ -318,7 +318,7 @@ struct PatternIndex {
     // work-group lists of the bf16 kernels (four strip ids per work-group) over block rows / block columns
     int *d_wg_row = nullptr, *d_wg_col = nullptr;
     int n_wg_row = 0, n_wg_col = 0;
-    std::vector<int> row_len_desc;  // host copy: tiles per block row, longest first
+    std::vector<int> row_len_desc;  // host copy: tiles per block row in the order the kernels walk them
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -398,16 +398,22 @@ void sparse_destroy(void* h) {
     delete a;
 }
 
-// Work-group list of the bf16 kernels: strips sorted by length (longest first, so the tail of the launch is
-// made of short ones); a strip much longer than the average (a global row or column) is walked by the four
-// wavefronts of a work-group together, the others are dealt four to a work-group, one per wavefront.
+// A strip counts as long (a global row or column) when it has more tiles than this.
+static int long_strip_threshold(int nstrips, int ntiles) {
+    const int avg = nstrips ? (ntiles + nstrips - 1) / nstrips : 0;
+    return std::max(4 * avg + 8, 32);
+}
+
+// Work-group list of the bf16 kernels: long strips first, each walked by the four wavefronts of a work-group
+// together; the others in index order (neighbouring strips of a banded pattern share K/V tiles in the caches),
+// four to a work-group, one per wavefront.
 static std::vector<int> build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles) {
     std::vector<int> order(nstrips);
     for (int i = 0; i < nstrips; ++i) order[i] = i;
-    std::stable_sort(order.begin(), order.end(),
-                     [&](int a, int b) { return ptr[a + 1] - ptr[a] > ptr[b + 1] - ptr[b]; });
-    const int avg = nstrips ? (ntiles + nstrips - 1) / nstrips : 0;
-    const int long_len = std::max(4 * avg + 8, 32);
+    const int long_len = long_strip_threshold(nstrips, ntiles);
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
+        return (ptr[a + 1] - ptr[a] > long_len) > (ptr[b + 1] - ptr[b] > long_len);
+    });
     std::vector<int> wg;
     int i = 0;
     for (; i < nstrips && ptr[order[i] + 1] - ptr[order[i]] > long_len; ++i)
@@ -506,17 +512,24 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
         const std::vector<int> wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
-        // Behind each pointer array: the strips sorted by length, longest first (the order the fp32 kernels
-        // walk a head in, so that the launch does not end on a long strip).
-        auto append_order = [&](std::vector<int>& ptr) {
+        // Behind each pointer array: the order the fp32 kernels walk the strips of a head in.  Strips are
+        // bucketed by length class -- rows: the forward's classes (more than 2 MAXT tiles, more than MAXT, the
+        // rest; it launches them separately); columns: long ones, the rest -- so that long strips start first,
+        // and keep their index order inside a bucket (neighbouring strips share K/V tiles in the caches).
+        const int maxt = a->d == 32 ? 8 : 4, long_len = long_strip_threshold(nbr, nt);
+        auto append_order = [&](std::vector<int>& ptr, bool rows) {
             std::vector<int> order(nbr);
             for (int i = 0; i < nbr; ++i) order[i] = i;
-            std::stable_sort(order.begin(), order.end(),
-                             [&](int x, int y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
+            auto bucket = [&](int i) {
+                const int len = ptr[i + 1] - ptr[i];
+                if (rows) return len > 2 * maxt ? 0 : len > maxt ? 1 : 2;
+                return len > long_len ? 0 : 1;
+            };
+            std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return bucket(x) < bucket(y); });
             ptr.insert(ptr.end(), order.begin(), order.end());
         };
-        append_order(trp);
-        append_order(tcp);
+        append_order(trp, true);
+        append_order(tcp, false);
         pi.row_len_desc.resize(nbr);
         for (int i = 0; i < nbr; ++i) pi.row_len_desc[i] = trp[trp[nbr + 1 + i] + 1] - trp[trp[nbr + 1 + i]];
         pi.n_wg_row = (int)wgr.size() / 4;
@@ -654,7 +667,7 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
         else if (wv == 2) SPION_LAUNCH(2, 0, 0, nbr);
         else SPION_LAUNCH(4, 0, 0, nbr);
     } else {
-        int n4 = 0, n2 = 0;  // pi.row_len_desc: lengths of the block rows, longest first
+        int n4 = 0, n2 = 0;  // pi.row_len_desc: lengths of the block rows, bucketed by these classes
         for (int len : pi.row_len_desc) {
             if (len > 2 * MAXT) ++n4;
             else if (len > MAXT) ++n2;

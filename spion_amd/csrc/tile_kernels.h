@@ -627,14 +627,15 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 const int t = w + min(i, nu - 1) * WAVES;
                 x.J = tcol[t0 + t];
                 ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
-                ldr_tile_cols(rP, pc_voff, p_base + t * 128, rn, x.pv);
+                // the P tile straight in the layout dP^T comes in (every lane pieces of its own row): measured
+                // twice as fast here as full rows plus an LDS transpose, which costs this path its registers
+                ldr_4x4(rP, (li * rn + 4 * h) * 4, p_base + t * 128, x.pv);
                 if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * D * 4, x.kb);
             },
             [&](Pre& c, int) {
                 float kb2[D / 32][16];
                 if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * D * 4, kb2);
-                float pr[16];
-                p_rows(c.pv, pr);
+                const float (&pr)[16] = c.pv;
                 f32x16 dp = mma_feat_init<D>(c.vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
 #pragma unroll
