@@ -318,7 +318,6 @@ struct PatternIndex {
     // work-group lists of the bf16 kernels (four strip ids per work-group) over block rows / block columns
     int *d_wg_row = nullptr, *d_wg_col = nullptr;
     int n_wg_row = 0, n_wg_col = 0;
-    std::vector<int> row_len_desc;  // host copy: tiles per block row in the order the kernels walk them
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -513,8 +512,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
         const std::vector<int> wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
         // Behind each pointer array: the order the fp32 kernels walk the strips of a head in.  Strips are
-        // bucketed by length class -- rows: the forward's classes (more than 2 MAXT tiles, more than MAXT, the
-        // rest; it launches them separately); columns: long ones, the rest -- so that long strips start first,
+        // bucketed by length class -- rows: more than 2 MAXT tiles of the forward's register budget, more than
+        // MAXT, the rest; columns: long ones, the rest -- so that long strips start first,
         // and keep their index order inside a bucket (neighbouring strips share K/V tiles in the caches).
         const int maxt = a->d == 32 ? 8 : 4, long_len = long_strip_threshold(nbr, nt);
         auto append_order = [&](std::vector<int>& ptr, bool rows) {
@@ -530,8 +529,6 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         };
         append_order(trp, true);
         append_order(tcp, false);
-        pi.row_len_desc.resize(nbr);
-        for (int i = 0; i < nbr; ++i) pi.row_len_desc[i] = trp[trp[nbr + 1 + i] + 1] - trp[trp[nbr + 1 + i]];
         pi.n_wg_row = (int)wgr.size() / 4;
         pi.n_wg_col = (int)wgc.size() / 4;
         o_wgr = append(wgr);
@@ -628,10 +625,6 @@ static const float* ocache_for_backward(SparseAttn* a, const float* key) {
 // -- no cross-wave merge and the longest software pipeline -- unless strips are long and the launch is
 // too small to fill the 1024 SIMDs with single-wave work-groups.
 static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool forward) {
-    if (const char* e = getenv(forward ? "SPION_TILE_WAVES_FWD" : "SPION_TILE_WAVES_BWD")) {
-        const int v = atoi(e);
-        if (v == 1 || v == 2 || v == 4) return v;
-    }
     const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
     if (forward) {
         const int maxt = a->d == 32 ? 8 : 4;
@@ -653,30 +646,25 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     float* ocache = ocache_for_forward(a, P);
-    // Logit tiles stay in registers when every wavefront's share of a block row fits (MAXT tiles).  Block rows
-    // are launched by length class -- up to MAXT tiles with one wavefront per row, up to 2 MAXT with two, up
-    // to 4 MAXT with four -- so that short rows do not pay for four nearly idle wavefronts and their merges.
+    // Logit tiles stay in registers when every wavefront's share of the longest block row fits (MAXT tiles);
+    // otherwise two sweeps.  (Launching the block rows by length class with 1, 2 and 4 wavefronts per row was
+    // measured and brings nothing over four wavefronts for all.)
     constexpr int MAXT = D == 32 ? 8 : 4;
-#define SPION_LAUNCH(W, MT, S0, NS)                                                                                  \
-    hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MT>), dim3((NS) * a->NB), dim3(64 * W), 0, a->hdr.stream, Q, Kt, \
-                       V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz, a->scale, S0, NS)
-    const int forced = getenv("SPION_TILE_WAVES_FWD") ? atoi(getenv("SPION_TILE_WAVES_FWD")) : 0;
-    if (pi.max_row_tiles > 4 * MAXT || forced) {  // rows too long for registers: two sweeps for every row
-        const int wv = forced == 1 || forced == 2 || forced == 4 ? forced : pick_waves(a, pi, nbr, true);
-        if (wv == 1) SPION_LAUNCH(1, 0, 0, nbr);
-        else if (wv == 2) SPION_LAUNCH(2, 0, 0, nbr);
-        else SPION_LAUNCH(4, 0, 0, nbr);
-    } else {
-        int n4 = 0, n2 = 0;  // pi.row_len_desc: lengths of the block rows, bucketed by these classes
-        for (int len : pi.row_len_desc) {
-            if (len > 2 * MAXT) ++n4;
-            else if (len > MAXT) ++n2;
-        }
-        const int n1 = nbr - n4 - n2;
-        if (n4) SPION_LAUNCH(4, MAXT, 0, n4);
-        if (n2) SPION_LAUNCH(2, MAXT, n4, n2);
-        if (n1) SPION_LAUNCH(1, MAXT, n4 + n2, n1);
-    }
+    const int wv = pick_waves(a, pi, nbr, true);
+#define SPION_LAUNCH(W)                                                                                              \
+    do {                                                                                                             \
+        if (pi.max_row_tiles <= W * MAXT)                                                                            \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT>), dim3(nbr * a->NB), dim3(64 * W), 0,              \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
+                               a->NB, nnz, a->scale, 0, nbr);                                                        \
+        else                                                                                                         \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0>), dim3(nbr * a->NB), dim3(64 * W), 0, a->hdr.stream,  \
+                               Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,        \
+                               a->scale, 0, nbr);                                                                    \
+    } while (0)
+    if (wv == 1) SPION_LAUNCH(1);
+    else if (wv == 2) SPION_LAUNCH(2);
+    else SPION_LAUNCH(4);
 #undef SPION_LAUNCH
 }
 
