@@ -40,7 +40,7 @@ def build_csr_from_block_mask(mat: np.ndarray, block_size: int):
     while sum_mat sums the values; the two agree for 0/1 masks, which is all
     the reference produces.
 
-    Pinned by: brute-force double loop in tests (tests/test_oracle_csr.py).
+    Pinned by: brute-force double loop in tests (tests/test_oracle_sparse.py).
     """
     mat = np.asarray(mat)
     nb = mat.shape[0]

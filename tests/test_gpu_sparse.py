@@ -100,6 +100,35 @@ def test_tile_path_with_key_mask(d):
     abi.close()
 
 
+@pytest.mark.parametrize("L,d,with_mask", [(2048, 32, False), (2048, 32, True), (1024, 64, False), (1024, 64, True)])
+def test_tile_path_global_row_and_column(L, d, with_mask):
+    """A block row and a block column that span the whole sequence: rows too long for the register-resident
+    forward (two-sweep kernel), long strips walked by several wavefronts in the backward passes, and the
+    one-pass backward without the kept copy of O."""
+    from spion_amd import _lib
+    bs, B, H = 32, 1, 2
+    NB, nb = B * H, L // bs
+    mat = _random_block_mask(nb, 0.04, seed=L + d)
+    mat[0, :] = 1
+    mat[:, 0] = 1
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=12, scale=1.3)
+    pen = None
+    if with_mask:
+        key_mask = np.ones((B, L), np.float32)
+        key_mask[0, L - 301:] = 0
+        pen = torch.from_numpy(osa.key_penalty_from_mask(key_mask, H)).cuda()
+    got, ref = run_and_check(abi, Q, K, V, dO, penalty=pen, tag=f"global row/column L={L} d={d}")
+    assert abi.last_path() == 1
+    _lib.core().spion_use_output_cache(abi.handle, 0)  # backward must find g by its own sweep now
+    dQ, dK, dV = abi.backward(Q, K, V, got["P"], dO)
+    for name, t in (("dQ", dQ), ("dK", dK), ("dV", dV)):
+        assert_close(t.cpu().numpy(), ref[name], what=f"global row/column, no O copy: {name}")
+    abi.close()
+
+
 def test_row_sum_invariant_large_logits_and_guard():
     # logits of +-30: exp range exercised; every row still obeys sum P = 1 - (L-n) e^{-m} / Z
     L, bs, d, NB = 128, 32, 32, 2
