@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|config1|config2|config3|config4|config5|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bf16|config1|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -254,8 +254,8 @@ def bench_encoder_step(args, dev):
     }
 
 
-def bench_bf16_scale_up(args, dev):
-    """Configuration 5: bf16 tensors, fp32 accumulation and softmax, B=4, H=8, L=16384, d=64, 64x64 blocks (band +
+def bench_bf16_scale_up(args, dev, shape="config5"):
+    """Configuration 5 (``shape="north_star"``: the north-star shape and mask with bf16 tensors instead): bf16 tensors, fp32 accumulation and softmax, B=4, H=8, L=16384, d=64, 64x64 blocks (band +
     one global block row and column + 1 % random blocks), Q, K, V ~ N(0,1)/8.  A step is forward + backward of the
     ``BlockAttentionBF16`` module.  The probabilities are never written to memory, so the algorithmic bytes are the
     eleven [NB, L, d] bf16 tensors plus the fp32 row statistics; the roofline is HBM (ridge of bf16 MFMA: 310 flop/B,
@@ -264,13 +264,17 @@ def bench_bf16_scale_up(args, dev):
     from spion_amd import _lib, workloads
     from spion_amd.csr import block_mask_to_csr_host
 
-    B, H, L, d, bs = 4, 8, 16384, 64, 64
+    if shape == "north_star":
+        B, H, L, d, bs, in_scale = 32, 2, 4096, 32, 32, 1.0
+        mat_np = workloads.north_star_mask(bs)
+    else:
+        B, H, L, d, bs, in_scale = 4, 8, 16384, 64, 64, 1.0 / 8.0
+        mat_np = workloads.config5_mask()
     NB = B * H
-    mat_np = workloads.config5_mask()
     _, off, _ = block_mask_to_csr_host(mat_np, bs)
     nnz = int(off[-1])
     mat = torch.from_numpy(mat_np).to(dev)
-    q, k, v, do = (t.to(torch.bfloat16) for t in workloads.qkv(B, H, L, d, scale=1.0 / 8.0, seed=0, device=dev))
+    q, k, v, do = (t.to(torch.bfloat16) for t in workloads.qkv(B, H, L, d, scale=in_scale, seed=0, device=dev))
     for t in (q, k, v):
         t.requires_grad_()
     cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
@@ -337,8 +341,8 @@ def bench_bf16_scale_up(args, dev):
         "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic (seeded N(0,1)/8 tensors rounded to bf16, seeded block mask)",
-        "config": {"workload": f"config5: bf16 sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, block {bs}, "
+        "data": f"synthetic (seeded N(0,1)*{in_scale:g} tensors rounded to bf16, seeded block mask)",
+        "config": {"workload": f"{shape}{'_bf16' if shape != 'config5' else ''}: bf16 sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, block {bs}, "
                                f"nnz/head={nnz}, block density={round(float(mat_np.mean()), 4)}",
                    "kernel_path": "mfma-bf16-tile"},
         "abi_ms": {"attn_forward": round(t_fwd, 4), "attn_backward": round(t_bwd, 4),
@@ -349,7 +353,7 @@ def bench_bf16_scale_up(args, dev):
         "roofline": roof,
     }
     if not args.no_cpu_baseline:
-        wl = build_workload("config5_fp32")
+        wl = build_workload("config5_fp32" if shape == "config5" else "north_star")
         result["cpu_baseline"] = cpu_baseline(wl)
     return result
 
@@ -391,6 +395,9 @@ def main():
         return
     if args.workload == "config5":
         print(json.dumps(bench_bf16_scale_up(args, dev)))
+        return
+    if args.workload == "north_star_bf16":
+        print(json.dumps(bench_bf16_scale_up(args, dev, "north_star")))
         return
 
     wl = build_workload(args.workload)
