@@ -10,6 +10,7 @@ from .attention_cuda_mask import CUDAMaskAttention
 from .attention_blockcuda import CUDABlockAttention
 from .attention_blockcuda_mask import CUDABlockMaskAttention
 from .attention_blockbf16 import BlockAttentionBF16
+from .masks import TransitionDetector, load_mask_list, save_mask_list, stack_for_replicas
 from .pattern import (
     discover_block_masks,
     generate_pattern_conv,
@@ -26,6 +27,10 @@ __all__ = [
     "CUDABlockAttention",
     "CUDABlockMaskAttention",
     "BlockAttentionBF16",
+    "TransitionDetector",
+    "load_mask_list",
+    "save_mask_list",
+    "stack_for_replicas",
     "discover_block_masks",
     "generate_pattern_conv",
     "generate_pattern_conv_ff",

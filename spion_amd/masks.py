@@ -1,0 +1,98 @@
+"""Block-mask persistence and the dense-to-sparse transition test of the training drivers.
+
+* ``save_mask_list`` / ``load_mask_list``: the ``[4, layers, nb, nb]`` float32 tensor of block masks in the file
+  format the reference writes and reads (a plain ``pickle.dump`` of the tensor, main_conv_ff.py:301-306,
+  main_inference.py:164-166), so masks discovered by either side load into the other.  Loading goes through a
+  restricted unpickler: only the handful of callables a pickled tensor needs are resolved, and the storage bytes
+  are decoded with ``torch.load(..., weights_only=True)``; anything else in the file raises.
+* ``TransitionDetector``: the test that ends the dense phase (main_conv_ff.py:211-242).  After every evaluation
+  the head/batch-averaged score map of each layer is compared with the previous one; the Frobenius distance of
+  consecutive maps is itself compared with the previous distance, and once it changed by less than 15 % (after
+  truncation to an integer percentage) in every layer the pattern is considered settled.
+"""
+from __future__ import annotations
+
+import io
+import pickle
+
+import torch
+
+
+def stack_for_replicas(layer_masks, replicas: int = 4) -> torch.Tensor:
+    """[layers][nb, nb] masks -> [replicas, layers, nb, nb] (main_conv_ff.py:298-299: one copy per GPU replica)."""
+    m = torch.stack([torch.as_tensor(x, dtype=torch.float32) for x in layer_masks], 0)
+    return torch.stack([m] * replicas, 0)
+
+
+def save_mask_list(mat_lst: torch.Tensor, path: str) -> None:
+    if mat_lst.dim() != 4 or mat_lst.shape[-1] != mat_lst.shape[-2]:
+        raise ValueError(f"expected [replicas, layers, nb, nb], got {tuple(mat_lst.shape)}")
+    with open(path, "wb") as f:
+        pickle.dump(mat_lst.detach().to(torch.float32).cpu().contiguous(), f, pickle.HIGHEST_PROTOCOL)
+
+
+def _storage_from_bytes(b: bytes):
+    return torch.load(io.BytesIO(b), weights_only=True)
+
+
+class _TensorOnlyUnpickler(pickle.Unpickler):
+    _ALLOWED = {
+        ("torch._utils", "_rebuild_tensor_v2"),
+        ("torch._utils", "_rebuild_tensor"),
+        ("collections", "OrderedDict"),
+        ("torch", "FloatStorage"),
+        ("torch", "device"),
+    }
+
+    def find_class(self, module, name):
+        if (module, name) == ("torch.storage", "_load_from_bytes"):
+            return _storage_from_bytes
+        if (module, name) in self._ALLOWED:
+            return super().find_class(module, name)
+        raise pickle.UnpicklingError(f"mask file refers to {module}.{name}: not a plain float tensor")
+
+
+def load_mask_list(path: str, device=None) -> torch.Tensor:
+    with open(path, "rb") as f:
+        obj = _TensorOnlyUnpickler(f).load()
+    if not isinstance(obj, torch.Tensor) or obj.dim() != 4 or obj.shape[-1] != obj.shape[-2]:
+        raise ValueError("mask file does not hold a [replicas, layers, nb, nb] tensor")
+    obj = obj.to(torch.float32)
+    return obj.to(device) if device is not None else obj
+
+
+class TransitionDetector:
+    """``update(attn_lst)`` after each evaluation; returns True from the call on which every layer's change of
+    distance fell below ``percent`` (main_conv_ff.py:211-242).  ``attn_lst[l]`` is the layer's averaged score map."""
+
+    def __init__(self, num_layers: int, percent: int = 15):
+        self.num_layers = num_layers
+        self.percent = percent
+        self.before_attn: list = []
+        self.before_distance: list = []
+        self.diff: list = []
+        self.transition = False
+
+    def update(self, attn_lst) -> bool:
+        if self.transition:
+            return True
+        cur = [attn_lst[l].detach() for l in range(self.num_layers)]
+        if not self.before_attn:  # first evaluation: nothing to compare with
+            self.before_attn = cur
+            return False
+        dist = [torch.sqrt(torch.sum(torch.pow(self.before_attn[l] - cur[l], 2))) for l in range(self.num_layers)]
+        if not self.before_distance:  # second evaluation: first distance, no change yet; the reference map stays
+            self.before_distance = dist
+            self.diff = [0.0] * self.num_layers
+            return False
+        settled = 0
+        for l in range(self.num_layers):
+            self.diff[l] = float((abs(dist[l] - self.before_distance[l]) / self.before_distance[l]) * 100)
+            self.before_distance[l] = dist[l]
+            if int(self.diff[l]) < self.percent:
+                settled += 1
+        if settled == self.num_layers:
+            self.transition = True
+        else:
+            self.before_attn = cur
+        return self.transition
