@@ -452,42 +452,34 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
         av[c] = splat16(0.f);
     }
     const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
-    // One tile ahead: the Q and dO rows and, for d = 32, the row statistics of the tile's queries; for d = 64
-    // those would not fit in registers next to two operand sets and are requested when the tile's first
-    // chain starts.
+    // One tile ahead: the Q and dO tiles and the two row statistics of the tile's 32 queries, one query per lane
+    // (two 4-byte instructions; fetching each lane's 16 values directly would take eight 16-byte ones, as
+    // costly on the vector-memory path as the two tiles).  The statistics reach the accumulator layout
+    // (register r = query acc_row(r, h)) through a small wave-private LDS array.
     constexpr bool DEEP = D == 32;
+    __shared__ __attribute__((aligned(16))) float lds_stat[BF16_WAVES][2][32];
+    float* St = &lds_stat[w][0][0];
     struct Pre {
         u32x4 q[D / 16], go[D / 16];
-        float lse[DEEP ? 16 : 1], gneg[DEEP ? 16 : 1];
-        int I;
+        float lse, gneg;
     };
     Pre xa, xb;
     tile_pipeline(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int I = desc[sa.rank + min(i, nu - 1) * sa.step].x;
-            x.I = I;
             ldb_tile<D>(rQ, l * 16, I * 32 * D * 2, x.q);
             ldb_tile<D>(rdO, l * 16, I * 32 * D * 2, x.go);
-            if constexpr (DEEP) {
-                ldr_4x4(rL, 16 * h, I * 128, x.lse);
-                ldr_4x4(rG, 16 * h, I * 128, x.gneg);
-            }
+            x.lse = ld1(rL, li * 4, I * 128);
+            x.gneg = ld1(rG, li * 4, I * 128);
         },
         [&](Pre& c, int) {
-            float lse[16], gn[16];
-            if constexpr (DEEP) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    lse[r] = c.lse[r];
-                    gn[r] = c.gneg[r];
-                }
-            } else {
-                ldr_4x4(rG, 16 * h, c.I * 128, gn);
-                ldr_4x4(rL, 16 * h, c.I * 128, lse);
-            }
+            St[l] = h ? c.gneg : c.lse;  // lanes 0-31: lse of query li, lanes 32-63: -g of query li
             LT::put_raw(Tq, l, c.q);
             LT::put_raw(Tg, l, c.go);
+            float lse[16], gn[16];
+            lds_get_rows(St, 0, h, lse);      // lse[r] = St[acc_row(r, h)]
+            lds_get_rows(St + 32, 0, h, gn);  // gn[r]  = St[32 + acc_row(r, h)]
             bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
             LT::get_rows(Tq, li, h, qr);
             LT::get_rows(Tg, li, h, gr);
