@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bf16|config1|config2|config3|config4|config5|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bf16|dense_phase|config1|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -358,6 +358,88 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
     return result
 
 
+def bench_dense_phase(args, dev):
+    """Dense-phase attention (the phase that feeds pattern discovery) at configuration 3's layer shape: B=256, H=2,
+    L=1024, d=32, fp32, forward + backward of the ``CUDAAttention`` module, which materialises the full
+    [B, H, L, L] probability map (2.1 GB) as the reference does.  FLOPs 12*L*L*d*NB; MFMA-bound."""
+    import spion_amd
+    from oracle import sparse_attention as osa
+    from spion_amd import _lib, workloads
+    from spion_amd.attention import Attention
+
+    B, H, L, d = 256, 2, 1024, 32
+    NB = B * H
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
+    cpp = Attention._cuda_compile_module()
+    handle = cpp.init(d, L, NB)
+    _lib.check_error("init")
+    module = spion_amd.CUDAAttention(cfg, cpp, handle)
+    q, k, v, do = workloads.qkv(B, H, L, d, scale=1.0, seed=0, device=dev)
+    for t in (q, k, v):
+        t.requires_grad_()
+    ones = torch.ones(B, L, device=dev)
+
+    def step():
+        for t in (q, k, v):
+            t.grad = None
+        out, _ = module(q, k, v, ones)
+        out.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # forward kernel alone at the C ABI (operands in the layouts it takes: Qt, Vt feature-major)
+    Qt = _lib.transpose_last2(q.detach().reshape(NB, L, d))
+    Vt = _lib.transpose_last2(v.detach().reshape(NB, L, d))
+    K = k.detach().reshape(NB, L, d).contiguous()
+    attn = torch.empty(NB, L, L, device=dev)
+    out_t = torch.empty(NB, d, L, device=dev)
+    t_fwd = _event_ms(lambda: cpp.attn_forward(handle, Qt.data_ptr(), K.data_ptr(), Vt.data_ptr(), attn.data_ptr(),
+                                               out_t.data_ptr()), max(10, args.steps // 4))
+    _lib.check_error("dense forward")
+    alg_flops = 12.0 * L * L * d * NB
+    roof = dict(bound="mfma", kernel="dense_fwd_kernel", achieved=alg_flops / 3.0 / t_fwd / 1e9,
+                peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s", traffic=None)
+    roof["frac"] = roof["achieved"] / roof["peak"]
+    roof["kernel_ms"] = {"dense_fwd_kernel": round(t_fwd, 4)}
+    result = {
+        "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
+        "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (seeded N(0,1) tensors)",
+        "config": {"workload": f"dense_phase: softmax attention fwd+bwd with the full probability map, B={B} H={H} L={L} d={d}"},
+        "algorithmic": {"gflop": alg_flops / 1e9, "map_gbytes": 4.0 * NB * L * L / 1e9},
+        "roofline": roof,
+    }
+    if not args.no_cpu_baseline:
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        qc, kc, vc, doc = workloads.qkv(1, H, L, d, scale=1.0, seed=0)
+        for t in (qc, kc, vc):
+            t.requires_grad_()
+        pat = torch.ones(L, L)
+        n, t1 = 0, time.perf_counter()
+        while time.perf_counter() - t1 < 10.0:
+            for t in (qc, kc, vc):
+                t.grad = None
+            o, _ = osa.dense_masked_attention(qc, kc, vc, pat, None)
+            o.backward(doc)
+            n += 1
+        el = time.perf_counter() - t1
+        result["cpu_baseline"] = dict(value=12.0 * L * L * d * H * n / el / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                                      ms_per_sample=1e3 * el / n,
+                                      sample=f"{n} repetitions of one sample (H={H}, L={L}, d={d}): dense softmax attention "
+                                             "forward + autograd backward in PyTorch fp32 (the oracle's dense statement; its "
+                                             "off-pattern term vanishes on a full pattern)")
+    return result
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,6 +477,9 @@ def main():
         return
     if args.workload == "config5":
         print(json.dumps(bench_bf16_scale_up(args, dev)))
+        return
+    if args.workload == "dense_phase":
+        print(json.dumps(bench_dense_phase(args, dev)))
         return
     if args.workload == "north_star_bf16":
         print(json.dumps(bench_bf16_scale_up(args, dev, "north_star")))
