@@ -163,9 +163,13 @@ __device__ __forceinline__ void ldr_tile_lin(rsrc_t r, int voff, int soff, int l
 #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = ld4(r, voff, soff + 32 * i * ld);
 }
+// Non-temporal: the P stream of the forward (written once, far larger than the caches) is kept from displacing
+// the K/V tiles in L2; measured -11 % on the forward kernel, -1.3 % on the whole step.
 __device__ __forceinline__ void str_tile_lin(rsrc_t r, int voff, int soff, int ld, const f32x4 (&raw)[4]) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) st4(r, voff, soff + 32 * i * ld, raw[i]);
+    for (int i = 0; i < 4; ++i)
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, raw[i]), r, voff, soff + 32 * i * ld, 2);
 }
 __device__ __forceinline__ void lds_put_lin(float* T, int l, const f32x4 (&raw)[4]) {
 #pragma unroll
