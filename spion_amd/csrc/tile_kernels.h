@@ -46,6 +46,14 @@ __device__ __forceinline__ float ld1(rsrc_t r, int voff, int soff) {
 __device__ __forceinline__ f32x4 ld4(rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
+// Non-temporal forms for the P stream (read or written once per pass, far larger than the caches): P then
+// does not displace the K/V/Q/dO tiles in L2.  Measured on the north star: -4 % on the whole step.
+__device__ __forceinline__ float ld1_nt(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 2));
+}
+__device__ __forceinline__ f32x4 ld4_nt(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2));
+}
 __device__ __forceinline__ void st4(rsrc_t r, int voff, int soff, f32x4 v) {
     typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
@@ -594,7 +602,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 const int t = w + min(i, nu - 1) * WAVES;
                 const int J = tcol[t0 + t];
                 ldr_tile_lin(rV, vl, J * 128, L, x.vt);
-                ldr_tile_lin(rP, pl, p_base + t * 128, rn, x.pv);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) x.pv[i] = ld4_nt(rP, pl, p_base + t * 128 + 32 * i * rn);
                 ldr_tile_lin(rK, kl, J * 32 * D * 4, D, x.kb);
             },
             [&](Pre& c, int) {
@@ -713,7 +722,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
             if constexpr (!DEEP) ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
             const int pv = (4 * h * rn + li) * 4;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) x.p[r] = ld1(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
+            for (int r = 0; r < 16; ++r) x.p[r] = ld1_nt(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
             ldr_4x4(rG, 16 * h, I * 128, x.gneg);
             if constexpr (DEEP) {
                 ldr_tile_b<D>(rQ, b_voff, I * 32 * D * 4, x.qb);
