@@ -123,7 +123,8 @@ __device__ __forceinline__ void ldr_tile_cols(rsrc_t r, int voff, int soff, int 
 }
 __device__ __forceinline__ void str_tile_cols(rsrc_t r, int voff, int soff, int ld, const float (&x)[16]) {
 #pragma unroll
-    for (int q = 0; q < 16; ++q) st1(r, voff, soff + (8 * (q >> 2) + (q & 3)) * ld * 4, x[q]);
+    for (int q = 0; q < 16; ++q)  // only P tiles are written this way: non-temporal
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, x[q]), r, voff, soff + (8 * (q >> 2) + (q & 3)) * ld * 4, 2);
 }
 __device__ __forceinline__ void lds_put_cols(float* T, int li, int h, const float (&x)[16], int col0 = 0) {
 #pragma unroll
@@ -642,6 +643,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
                 // the P tile straight in the layout dP^T comes in (every lane pieces of its own row): measured
                 // twice as fast here as full rows plus an LDS transpose, which costs this path its registers
+                // (not non-temporal: a lane reads its 128-byte row in four instructions)
                 ldr_4x4(rP, (li * rn + 4 * h) * 4, p_base + t * 128, x.pv);
                 if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * D * 4, x.kb);
             },
