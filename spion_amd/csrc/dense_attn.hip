@@ -19,8 +19,8 @@ constexpr int DENSE_WAVES = 4;
 template <int D, bool MASK>
 __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
-    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, int L, int nbr, int NB,
-    float scale) {
+    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
+    int L, int nbr, int NB, float scale) {
     constexpr int WAVES = DENSE_WAVES;
     __shared__ float lds[WAVES * (D / 32) * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
@@ -86,19 +86,25 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
             float v = s[r] * scale;
             if (MASK) v -= penh[J * 32 + acc_row(r, h)];
             p[r] = __expf(v - m) * rinv;
-            Ah[(size_t)(J * 32 + acc_row(r, h)) * L] = p[r];
+            // the map is written once and is far larger than the caches: non-temporal
+            __builtin_nontemporal_store(p[r], &Ah[(size_t)(J * 32 + acc_row(r, h)) * L]);
         }
         mma_tile_t<D>(p, Vt + hb, L, J * 32, li, h, o);
     }
     reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+    if (OutCopy) {  // kept by the handle for the backward's row sums
+        __syncthreads();
+        reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+    }
 }
 
 // Row pass: g_i = sum_j dP_ij P_ij (kept in G), dS = (dP*P - P*g)*scale, dQ^T = K^T-tiles . dS^T.
-template <int D>
+// HAVE_O: the handle kept Out of the forward that filled this map, so g_i = dO_i . O_i needs no sweep.
+template <int D, bool HAVE_O>
 __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_row_kernel(
     const float* __restrict__ Kt, const float* __restrict__ V, const float* __restrict__ Attn,
-    const float* __restrict__ dOt, float* __restrict__ G, float* __restrict__ dQ, int L, int nbr, int NB,
-    float scale) {
+    const float* __restrict__ dOt, const float* __restrict__ OutCopy, float* __restrict__ G,
+    float* __restrict__ dQ, int L, int nbr, int NB, float scale) {
     constexpr int WAVES = DENSE_WAVES;
     __shared__ float lds[WAVES * (D / 32) * 16 * 64];
     __shared__ float lds_g[WAVES][32];
@@ -112,19 +118,27 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_row_kernel(
     load_cols<D>(dOt + hb, L, I * 32, li, h, go);
 
     float g = 0.f;
-    for (int J = w; J < nbr; J += WAVES) {
-        float v[D / 2];
-        load_rows<D>(V + hb, J * 32, li, h, v);
-        f32x16 dp = mma_feat<D>(v, go);
+    if (HAVE_O) {
+        float oo[D / 2];
+        load_cols<D>(OutCopy + hb, L, I * 32, li, h, oo);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) g = fmaf(dp[r], Ah[(size_t)(J * 32 + acc_row(r, h)) * L], g);
+        for (int s = 0; s < D / 2; ++s) g = fmaf(go[s], oo[s], g);
+        g += __shfl_xor(g, 32, 64);
+    } else {
+        for (int J = w; J < nbr; J += WAVES) {
+            float v[D / 2];
+            load_rows<D>(V + hb, J * 32, li, h, v);
+            f32x16 dp = mma_feat<D>(v, go);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) g = fmaf(dp[r], Ah[(size_t)(J * 32 + acc_row(r, h)) * L], g);
+        }
+        g += __shfl_xor(g, 32, 64);
+        if (h == 0) lds_g[w][li] = g;
+        __syncthreads();
+        g = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
     }
-    g += __shfl_xor(g, 32, 64);
-    if (h == 0) lds_g[w][li] = g;
-    __syncthreads();
-    g = 0.f;
-#pragma unroll
-    for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
     if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = g;
 
     f32x16 acc[D / 32];
@@ -137,7 +151,8 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_row_kernel(
         float ds[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float p = Ah[(size_t)(J * 32 + acc_row(r, h)) * L];
+            const float p = HAVE_O ? __builtin_nontemporal_load(&Ah[(size_t)(J * 32 + acc_row(r, h)) * L])
+                                   : Ah[(size_t)(J * 32 + acc_row(r, h)) * L];
             ds[r] = (dp[r] * p - p * g) * scale;
         }
         mma_tile_t<D>(ds, Kt + hb, L, J * 32, li, h, acc);
@@ -202,6 +217,10 @@ struct DenseAttn {
     bool has_mask;
     float scale;
     float* ws_rowsum = nullptr;  // [NB][L]
+    // Copy of Out kept by the forward, filed under the map (Attn) it filled: a backward handed the same map
+    // takes its row sums g_i = dO_i . O_i from it instead of a sweep over the whole map.
+    float* ws_out = nullptr;      // [NB][d][L]
+    const float* out_key = nullptr;
 };
 
 static DenseAttn* as_dense(void* h, const char* who) {
@@ -238,6 +257,7 @@ void dense_destroy(void* h) {
     DenseAttn* a = as_dense(h, "destroy");
     if (!a) return;
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
+    if (a->ws_out) (void)hipFree(a->ws_out);
     a->hdr.magic = 0;
     delete a;
 }
@@ -247,12 +267,17 @@ static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, cons
                              float* Attn, float* Out) {
     const int nbr = a->L / 32;
     dim3 grid(nbr * a->NB), block(64 * DENSE_WAVES);
+    if (!a->ws_out && hipMalloc((void**)&a->ws_out, sizeof(float) * (size_t)a->NB * a->L * a->d) != hipSuccess) {
+        (void)hipGetLastError();  // no copy: the backward sweeps the map for its row sums
+        a->ws_out = nullptr;
+    }
+    a->out_key = a->ws_out ? Attn : nullptr;
     if (a->has_mask)
         hipLaunchKernelGGL((dense_fwd_kernel<D, true>), grid, block, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
-                           a->L, nbr, a->NB, a->scale);
+                           a->ws_out, a->L, nbr, a->NB, a->scale);
     else
         hipLaunchKernelGGL((dense_fwd_kernel<D, false>), grid, block, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
-                           a->L, nbr, a->NB, a->scale);
+                           a->ws_out, a->L, nbr, a->NB, a->scale);
 }
 
 template <int D>
@@ -260,8 +285,12 @@ static void dense_bwd_launch(DenseAttn* a, const float* Qt, const float* Kt, con
                              const float* dOt, float* dQ, float* dK, float* dV) {
     const int nbr = a->L / 32;
     dim3 grid(nbr * a->NB), block(64 * DENSE_WAVES);
-    hipLaunchKernelGGL((dense_bwd_row_kernel<D>), grid, block, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_rowsum, dQ, a->L,
-                       nbr, a->NB, a->scale);
+    if (a->out_key == P && a->ws_out)
+        hipLaunchKernelGGL((dense_bwd_row_kernel<D, true>), grid, block, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_out,
+                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale);
+    else
+        hipLaunchKernelGGL((dense_bwd_row_kernel<D, false>), grid, block, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_out,
+                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale);
     hipLaunchKernelGGL((dense_bwd_col_kernel<D>), grid, block, 0, a->hdr.stream, Qt, V, P, dOt, a->ws_rowsum, dK, dV,
                        a->L, nbr, a->NB, a->scale);
 }

@@ -12,8 +12,10 @@ from tests.abi_utils import assert_close
 pytestmark = pytest.mark.gpu
 
 
-def _run_dense(d, L, NB, Q, K, V, dO, pen=None):
-    """Drive attn.so / attn_mask.so with the reference's operand layouts (models/attention_cuda.py:18-74)."""
+def _run_dense(d, L, NB, Q, K, V, dO, pen=None, moved_map=False):
+    """Drive attn.so / attn_mask.so with the reference's operand layouts (models/attention_cuda.py:18-74).
+    ``moved_map``: hand the backward a copy of the map at another address, so that it cannot use the copy of Out
+    the forward filed under the original one and must sweep the map for its row sums."""
     lib = Attention._cuda_mask_compile_module() if pen is not None else Attention._cuda_compile_module()
     h = lib.init(d, L, NB)
     _lib.check_error("init")
@@ -27,6 +29,8 @@ def _run_dense(d, L, NB, Q, K, V, dO, pen=None):
     lib.attn_forward(*args, attn.data_ptr(), out_t.data_ptr())
     _lib.check_error("attn_forward")
     dq, dk, dv = (torch.full((NB, d, L), nan, device="cuda") for _ in range(3))
+    if moved_map:
+        attn = attn.clone()
     lib.attn_backward(h, Qt.data_ptr(), Kt.data_ptr(), V.data_ptr(), attn.data_ptr(), dOt.data_ptr(), None, None,
                       None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr())
     _lib.check_error("attn_backward")
@@ -58,6 +62,18 @@ def test_dense_matches_oracle(L, d, NB, with_mask):
     assert_close(got["P"].sum(-1), np.ones((NB, L)), what="rows of P sum to one")
     if with_mask:
         assert (got["P"][0][:, 130:] == 0).all() and (got["P"][2][:, 33:] == 0).all()
+
+
+def test_dense_backward_without_the_kept_output():
+    L, d, NB = 256, 32, 2
+    g = torch.Generator().manual_seed(5)
+    Q, K, V, dO = (torch.randn(NB, L, d, generator=g).cuda() for _ in range(4))
+    got = _run_dense(d, L, NB, Q, K, V, dO, moved_map=True)
+    f = lambda t: t.cpu().numpy().astype(np.float64)
+    O, P = oda.dense_attention_forward(f(Q), f(K), f(V), None)
+    dQ, dK, dV = oda.dense_attention_backward(f(Q), f(K), f(V), P, f(dO))
+    for name, ref in (("dQ", dQ), ("dK", dK), ("dV", dV)):
+        assert_close(got[name], ref, what=f"dense, map at another address: {name}")
 
 
 @pytest.mark.parametrize("with_mask", [False, True])
