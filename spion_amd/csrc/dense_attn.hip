@@ -7,7 +7,7 @@
 // One work-group owns 32 queries (forward, row pass) or 32 keys (column pass) of one head and walks all
 // L/32 tiles of the other dimension with v_mfma_f32_32x32x2_f32; see tile_ops.h for the register layout.
 #include "common.h"
-#include "tile_ops.h"
+#include "tile_kernels.h"
 #include "../../include/spion_hip.h"
 
 #include <cmath>
@@ -93,6 +93,128 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
     }
     reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
     if (OutCopy) {  // kept by the handle for the backward's row sums
+        __syncthreads();
+        reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+    }
+}
+
+// Forward for d = 32 and L <= 1024 (at most 32 key tiles per query strip): the register-resident scheme of the
+// sparse forward (tile_kernels.h) on the dense layouts.  Each of the four wavefronts keeps the logit tiles of its
+// share of the strip (at most 8) in registers, so a tile costs one QK^T chain and one PV chain instead of the
+// two-sweep kernel's three; K, V^T and map tiles move as four 16-byte instructions each and change layout in
+// wave-private LDS tiles; the map is written non-temporally.
+template <bool MASK>
+SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
+    const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
+    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
+    int L, int nbr, int NB, float scale) {
+    constexpr int D = 32, KH = 16, WAVES = 4, MAXT = 8;
+    __shared__ float lds[WAVES * 16 * 64];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][2 * 32 * TS];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w+4, ... of this wavefront
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes);
+    const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    float* T = lds_t[w];         // map tile on its way to memory
+    float* Tx = T + 32 * TS;     // K tile, later V^T tile
+    const int klin = lin_voff(l, D), vlin = lin_voff(l, L);
+    const float c2 = scale * LOG2E;
+
+    float q[KH];
+    ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) q[s] *= c2;
+    auto chain_init = [&](int J) -> f32x16 {  // minus the key penalties of the tile, log2 domain
+        if (!MASK) return splat16(0.f);
+        float pj[16];
+        ldr_4x4(rM, 16 * h, J * 128, pj);
+        f32x16 v;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) v[r] = -LOG2E * pj[r];
+        return v;
+    };
+
+    float m = -10.f * LOG2E, z = 0.f;  // models/attn.cu:17
+    f32x16 S[MAXT];
+    {
+        f32x4 kraw[2][4];
+        if (nu > 0) ldr_tile_lin(rK, klin, w * 32 * D * 4, D, kraw[0]);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                const int J = w + u * WAVES;
+                if (u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * D * 4, D, kraw[(u + 1) & 1]);
+                lds_put_lin(Tx, l, kraw[u & 1]);
+                float kf[KH];
+                lds_get_feat32(Tx, li, h, kf);
+                __builtin_amdgcn_sched_barrier(0);
+                S[u] = mma_feat_init<D>(kf, q, chain_init(J));  // S^T: register = key, lane = query
+                m = max16(S[u], m);
+            }
+        }
+    }
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u < nu) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = __builtin_amdgcn_exp2f(S[u][r] - m);
+                S[u][r] = e;
+                z += e;
+            }
+        }
+    }
+    const float m_own = m;
+    z += __shfl_xor(z, 32, 64);
+    {
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
+        float Mx = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+        m = Mx;
+        z = Z;
+    }
+    const float rinv = __builtin_amdgcn_exp2f(m_own - m) * (1.0f / z);
+
+    f32x16 o[1] = {splat16(0.f)};  // O^T: register = feature, lane = query
+    {
+        f32x4 vraw[2][4];
+        if (nu > 0) ldr_tile_lin(rV, vlin, w * 128, L, vraw[0]);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                const int J = w + u * WAVES;
+                if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * 128, L, vraw[(u + 1) & 1]);
+                lds_put_lin(Tx, l, vraw[u & 1]);
+                float p[16], vb[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                lds_put_cols(T, li, h, p);        // T[key][query]: the map is stored key-major
+                lds_get_rows(Tx, li, h, vb);      // vb[s] = V[key acc_row(s, h)][feature li]
+                f32x4 pl[4];
+                lds_get_lin(T, l, pl);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
+                str_tile_lin(rA, vlin, (J * 32 * L + I * 32) * 4, L, pl);
+            }
+        }
+    }
+    reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+    if (OutCopy) {
         __syncthreads();
         reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
     }
@@ -272,6 +394,16 @@ static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, cons
         a->ws_out = nullptr;
     }
     a->out_key = a->ws_out ? Attn : nullptr;
+    if (D == 32 && nbr <= 32) {
+        const dim3 block4(64 * 4);
+        if (a->has_mask)
+            hipLaunchKernelGGL(dense_fwd_reg_kernel<true>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
+                               a->ws_out, a->L, nbr, a->NB, a->scale);
+        else
+            hipLaunchKernelGGL(dense_fwd_reg_kernel<false>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
+                               a->ws_out, a->L, nbr, a->NB, a->scale);
+        return;
+    }
     if (a->has_mask)
         hipLaunchKernelGGL((dense_fwd_kernel<D, true>), grid, block, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
                            a->ws_out, a->L, nbr, a->NB, a->scale);
