@@ -261,7 +261,7 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_row_kernel(
 #pragma unroll
         for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
     }
-    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = g;
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;  // the column passes start their chains from it
 
     f32x16 acc[D / 32];
 #pragma unroll
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_col_kernel(
         }
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float g = Gh[I * 32 + acc_row(r, h)];
+            const float g = -Gh[I * 32 + acc_row(r, h)];
             ds[r] = (dp[r] * p[r] - p[r] * g) * scale;
         }
         mma_tile_t<D>(ds, Qt + hb, L, I * 32, li, h, ak);
@@ -330,6 +330,147 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_col_kernel(
     reduce_store<D, WAVES, true>(ak, dK + hb, J * 32, w, li, h, lds, L);
     __syncthreads();
     reduce_store<D, WAVES, true>(av, dV + hb, J * 32, w, li, h, lds, L);
+}
+
+// Backward passes for d = 32 with the kept copy of Out: the schedule of the sparse tile kernels (tile_kernels.h)
+// on the dense layouts.  Every operand tile -- V, K^T, Q^T, dO^T and the key-major map tile -- is fetched as four
+// 16-byte instructions one tile ahead and turned into MFMA operands through wave-private LDS copies; -g enters as
+// the initial accumulator of the dP chain; the 1/sqrt(d) is applied to the 32 x d results.
+template <int WAVES>
+SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
+    const float* __restrict__ Kt, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dOt, const float* __restrict__ OutCopy, float* __restrict__ G,
+    float* __restrict__ dQ, int L, int nbr, int NB, float scale) {
+    constexpr int D = 32, KH = 16;
+    __shared__ float lds[WAVES * 16 * 64];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS];
+    // last head first: the tail of the map is what the memory-side cache still holds after the forward
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = NB - 1 - item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rK = make_rsrc(Kt + hb, hbytes), rV = make_rsrc(V + hb, hbytes), rdO = make_rsrc(dOt + hb, hbytes);
+    const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    float* Tv = lds_t[w];
+    float* Tp = Tv + 32 * TS;
+    float* Tk = Tv + 64 * TS;
+
+    float go[KH], oo[KH];
+    ldr_cols<D>(rdO, L, (h * KH * L + li) * 4, I * 128, go);
+    ldr_cols<D>(make_rsrc(OutCopy + hb, hbytes), L, (h * KH * L + li) * 4, I * 128, oo);
+    float g = 0.f;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
+    g += __shfl_xor(g, 32, 64);
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;
+    const f32x16 gneg = splat16(-g);
+
+    f32x16 acc = splat16(0.f);  // dQ^T: register = feature, lane = query
+    struct Pre {
+        f32x4 v[4], p[4], k[4];
+    };
+    const int vl = lin_voff(l, D), ll = lin_voff(l, L);
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int J = w + min(i, nu - 1) * WAVES;
+            ldr_tile_lin(rV, vl, J * 32 * D * 4, D, x.v);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
+            ldr_tile_lin(rK, ll, J * 128, L, x.k);
+        },
+        [&](Pre& c, int) {
+            lds_put_lin(Tv, l, c.v);
+            lds_put_lin(Tp, l, c.p);
+            lds_put_lin(Tk, l, c.k);
+            float vt[16], pr[16], kb[16];
+            lds_get_feat32(Tv, li, h, vt);  // V[key li][feature 16h + s]
+            lds_get_cols(Tp, li, h, pr);    // P[query li][key acc_row(r, h)]
+            lds_get_rows(Tk, li, h, kb);    // K^T[feature li][key acc_row(s, h)]
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // register = key, lane = query: dO_i . v_j - g_i
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(kb[s], ds[s], acc, 0, 0, 0);
+        });
+    f32x16 out[1] = {acc * scale};
+    reduce_store<D, WAVES, true>(out, dQ + hb, I * 32, w, li, h, lds, L);
+}
+
+template <int WAVES>
+SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
+    const float* __restrict__ Qt, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dOt, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
+    int L, int nbr, int NB, float scale) {
+    constexpr int D = 32, KH = 16;
+    __shared__ float lds[WAVES * 16 * 64];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS + 32];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rV = make_rsrc(V + hb, hbytes), rdO = make_rsrc(dOt + hb, hbytes);
+    const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
+    float* To = lds_t[w];
+    float* Tp = To + 32 * TS;
+    float* Tq = To + 64 * TS;
+    float* Tg = To + 96 * TS;
+
+    float v[KH];
+    ldr_rows<D>(rV, (li * D + h * KH) * 4, J * 32 * D * 4, v);
+
+    f32x16 ak = splat16(0.f), av = splat16(0.f);  // dK^T, dV^T: register = feature, lane = key
+    struct Pre {
+        f32x4 o[4], p[4], q[4];
+        float gneg;  // of query li; spread over the registers of dP through LDS
+    };
+    const int ll = lin_voff(l, L);
+    Pre xa, xb;
+    tile_pipeline(
+        nu, xa, xb,
+        [&](Pre& x, int i) {
+            const int I = w + min(i, nu - 1) * WAVES;
+            ldr_tile_lin(rdO, ll, I * 128, L, x.o);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
+            ldr_tile_lin(rQ, ll, I * 128, L, x.q);
+            x.gneg = ld1(rG, li * 4, I * 128);
+        },
+        [&](Pre& c, int) {
+            lds_put_lin(To, l, c.o);
+            lds_put_lin(Tp, l, c.p);
+            lds_put_lin(Tq, l, c.q);
+            Tg[li] = c.gneg;
+            float go[16], ob[16], p[16], qb[16], gn[16];
+            lds_get_rows(Tg, 0, h, gn);         // -g[query acc_row(r, h)]
+            lds_get_featcols32(To, li, h, go);  // dO[query li][feature 16h + s]
+            lds_get_rows(Tp, li, h, p);         // P[query acc_row(r, h)][key li]
+            lds_get_rows(Tq, li, h, qb);        // Q^T[feature li][query acc_row(s, h)]
+            lds_get_rows(To, li, h, ob);        // dO^T[feature li][query acc_row(s, h)]
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 init;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) init[r] = gn[r];
+            f32x16 dp = mma_feat_init<D>(go, v, init);  // register = query, lane = key
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * p[r];
+#pragma unroll
+            for (int s = 0; s < 16; ++s) ak = __builtin_amdgcn_mfma_f32_32x32x2f32(qb[s], ds[s], ak, 0, 0, 0);
+#pragma unroll
+            for (int s = 0; s < 16; ++s) av = __builtin_amdgcn_mfma_f32_32x32x2f32(ob[s], p[s], av, 0, 0, 0);
+        });
+    f32x16 out[1] = {ak * scale};
+    reduce_store<D, WAVES, true>(out, dK + hb, J * 32, w, li, h, lds, L);
+    __syncthreads();
+    out[0] = av;
+    reduce_store<D, WAVES, true>(out, dV + hb, J * 32, w, li, h, lds, L);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -417,6 +558,15 @@ static void dense_bwd_launch(DenseAttn* a, const float* Qt, const float* Kt, con
                              const float* dOt, float* dQ, float* dK, float* dV) {
     const int nbr = a->L / 32;
     dim3 grid(nbr * a->NB), block(64 * DENSE_WAVES);
+    // 32-bit byte offsets into one head's map: L*L*4 < 2^31
+    if (D == 32 && a->L <= 16384 && a->out_key == P && a->ws_out) {
+        const dim3 block4(64 * 4);
+        hipLaunchKernelGGL(dense_bwd_row32_kernel<4>, grid, block4, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_out,
+                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale);
+        hipLaunchKernelGGL(dense_bwd_col32_kernel<4>, grid, block4, 0, a->hdr.stream, Qt, V, P, dOt, a->ws_rowsum, dK,
+                           dV, a->L, nbr, a->NB, a->scale);
+        return;
+    }
     if (a->out_key == P && a->ws_out)
         hipLaunchKernelGGL((dense_bwd_row_kernel<D, true>), grid, block, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_out,
                            a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale);
