@@ -22,7 +22,10 @@
 // lane scalars; keys are the lane index in the column pass.
 //
 // Work-groups have four wavefronts and take one entry of a host-built list: four short strips (one per
-// wavefront, no barriers) or one long strip (a global row or column) walked by the four wavefronts together.
+// wavefront, no barriers) or one chunk of a long strip (a global row or column) walked by the four wavefronts
+// together.  A long strip is cut into chunks of about the work of an ordinary work-group, so that it does not
+// outlast the rest of the launch; every chunk leaves fp32 partial results in a workspace slot and a small
+// merge kernel combines the slots of a strip.
 #pragma once
 #include "tile_kernels.h"
 
@@ -35,6 +38,10 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BF16_WAVES = 4;
+// These kernels are bound by the latency of each wavefront's chain load -> LDS -> MFMA -> exp -> MFMA rather than
+// by any one unit, so they run at the highest occupancy their registers allow (OCC wavefronts per SIMD).
+#define SPION_BF16_KERNEL(OCC) \
+    __global__ __launch_bounds__(64 * BF16_WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 constexpr float BF16_LAZY = 8.f;  // the running row maximum is raised only when a tile exceeds it by 2^8
 
 template <int D>
@@ -145,11 +152,14 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 
 // Sum the per-wave partial results of a cooperative strip (coop) and store the 32 x D result as bf16 rows.
 // acc[c][r] of lane (li, h): row li, feature 32c + acc_row(r, h).
+// part (chunk of a long strip only): the work-group's sum goes there as fp32, register (c, r) of lane l at
+// [(16c + r)*64 + l], instead of to the tensor.
 template <int D>
 __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO, int row0, bool coop, int w, int li, int h,
-                                                float* lds) {
+                                                float* lds, float* part = nullptr) {
     const int l = li + 32 * h;
     if (coop) {
+        __syncthreads();  // lds is the memory of the wave-private tiles: every wavefront is done with them
         if (w > 0) {
 #pragma unroll
             for (int c = 0; c < D / 32; ++c)
@@ -164,6 +174,13 @@ __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO
             for (int c = 0; c < D / 32; ++c)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[c][r] += lds[((ww * (D / 32) + c) * 16 + r) * 64 + l];
+        if (part) {
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) part[(16 * c + r) * 64 + l] = acc[c][r];
+            return;
+        }
     }
     const int voff = (li * D + 4 * h) * 2;
 #pragma unroll
@@ -177,42 +194,52 @@ __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO
         }
 }
 
-// Work-group entry: strip of each wavefront (-1: none); the four wavefronts share a strip iff the first two
-// entries are equal.
+// Work-group entry {a, b, c, d}.  a != b: strips a, b, c, d, one per wavefront (-1: none).  a == b: the four
+// wavefronts walk chunk c of long strip a together (tiles c*chunk .. of the strip, `chunk` a launch parameter) and
+// leave their sum in workspace slot d.
 struct StripAssign {
-    int strip, rank, step;
+    int strip, rank, step, chunk_id, slot;
     bool coop;
 };
 __device__ __forceinline__ StripAssign strip_of_wave(const int* __restrict__ wg_list, int g, int w) {
     const int4 e = reinterpret_cast<const int4*>(wg_list)[g];
     StripAssign s;
     s.coop = e.x == e.y;
-    s.strip = w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w;
+    s.strip = s.coop ? e.x : (w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w);
     s.rank = s.coop ? w : 0;
     s.step = s.coop ? BF16_WAVES : 1;
+    s.chunk_id = s.coop ? e.z : 0;
+    s.slot = s.coop ? e.w : -1;
     return s;
 }
+// floats per workspace slot: two 32 x D results (the column pass has dK and dV) and 64 row statistics
+template <int D>
+constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
 
 // -------------------------------------------------------------------------------------------------
 // Forward: one sweep per block row with a lazily raised running maximum.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK>
-SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
+SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : (MASK ? 2 : 3)) void bf16_fwd_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
+    float* __restrict__ Part, int n_slots, int chunk) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     __shared__ float lds_m[BF16_WAVES][32], lds_z[BF16_WAVES][32];
-    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
     if (sa.strip < 0) return;  // only in entries of independent strips: no barrier is skipped
     const int I = sa.strip;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
+    const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
     const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
     const rsrc_t rO = make_rsrc(O + hb, hbytes);
@@ -304,7 +331,15 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
         m = M;
         z = Z;
     }
-    const int off_pattern = L - cnt * 32;
+    if (part) {  // chunk of a long strip: unnormalised sums relative to m; the merge kernel finishes the rows
+        if (w == 0 && h == 0) {
+            part[2 * 32 * D + li] = m;
+            part[2 * 32 * D + 32 + li] = z;
+        }
+        store_rows_bf16<D>(o, rO, I * 32, true, w, li, h, lds_o, part);
+        return;
+    }
+    const int off_pattern = L - cnt_all * 32;
     if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);  // models/block_attn.cu:74
     const float rinv = 1.0f / z;
 #pragma unroll
@@ -318,22 +353,26 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_fwd_kernel(
 // the 1/sqrt(d) is applied to the 32 x d result.  Gneg receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK>
-SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
+SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
     const float* __restrict__ pen, float* __restrict__ Gneg, __bf16* __restrict__ dQ, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
+    float* __restrict__ Part, int n_slots, int chunk) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
     if (sa.strip < 0) return;
     const int I = sa.strip;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
+    const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
     const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
     const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rO = make_rsrc(O + hb, hbytes), rdQ = make_rsrc(dQ + hb, hbytes);
@@ -406,29 +445,33 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_row_kernel(
         });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
-    store_rows_bf16<D>(acc, rdQ, I * 32, sa.coop, w, li, h, lds_o);
+    store_rows_bf16<D>(acc, rdQ, I * 32, sa.coop, w, li, h, lds_o, part);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK>
-SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
+SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const float* __restrict__ Lse, const float* __restrict__ Gneg,
     const float* __restrict__ pen, __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcp,
-    const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale) {
+    const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
+    float* __restrict__ Part, int n_slots, int chunk) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    __shared__ float lds_o[(BF16_WAVES - 1) * (D / 32) * 16 * 64];
+    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
     if (sa.strip < 0) return;
     const int J = sa.strip;
-    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
+    const int cnt_all = tcp[J + 1] - tcp[J], tb = sa.chunk_id * chunk;
+    const int e0 = tcp[J] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
+    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
     const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
     const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rdK = make_rsrc(dK + hb, hbytes), rdV = make_rsrc(dV + hb, hbytes);
@@ -511,9 +554,99 @@ SPION_TILE_KERNEL(BF16_WAVES) void bf16_bwd_col_kernel(
         });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
-    store_rows_bf16<D>(ak, rdK, J * 32, sa.coop, w, li, h, lds_o);
+    store_rows_bf16<D>(ak, rdK, J * 32, sa.coop, w, li, h, lds_o, part);
     if (sa.coop) __syncthreads();
-    store_rows_bf16<D>(av, rdV, J * 32, sa.coop, w, li, h, lds_o);
+    store_rows_bf16<D>(av, rdV, J * 32, sa.coop, w, li, h, lds_o, part ? part + 32 * D : nullptr);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Merge of the chunks of long strips.  desc[k] = {strip, first slot, number of chunks, tiles of the strip};
+// one work-group per (head, long strip, 256 elements of the 32 x D result), one element per thread, the loads of
+// up to eight chunks in flight at a time.  Element e of a slot is register (c, r) = (e / 1024, e / 64 % 16) of lane
+// l = e % 64: row l % 32 of the strip, feature 32c + acc_row(r, l / 32).
+// -------------------------------------------------------------------------------------------------
+template <int D>
+__global__ __launch_bounds__(256) void bf16_merge_fwd_kernel(const float* __restrict__ Part, const int* __restrict__ desc,
+                                                             int n_long, int n_slots, __bf16* __restrict__ O,
+                                                             float* __restrict__ Lse, int L) {
+    constexpr int PSZ = bf16_slot_floats<D>(), EB = 32 * D / 256;
+    const int eb = blockIdx.x % EB, item = blockIdx.x / EB;
+    const int bh = item / n_long;
+    const int4 d = reinterpret_cast<const int4*>(desc)[item % n_long];
+    const float* p0 = Part + ((size_t)bh * n_slots + d.y) * PSZ;
+    const float* st = p0 + 2 * 32 * D;  // {m[32], z[32]} of chunk 0
+    __shared__ float sm[32], sr[32];
+    const int t = threadIdx.x;
+    if (t < 32) {
+        float M = -3.0e38f;
+        for (int c0 = 0; c0 < d.z; c0 += 8) {
+            float mm[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) mm[k] = st[(size_t)min(c0 + k, d.z - 1) * PSZ + t];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) M = fmaxf(M, mm[k]);
+        }
+        float Z = 0.f;
+        for (int c0 = 0; c0 < d.z; c0 += 8) {
+            float mm[8], zz[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                mm[k] = st[(size_t)min(c0 + k, d.z - 1) * PSZ + t];
+                zz[k] = st[(size_t)min(c0 + k, d.z - 1) * PSZ + 32 + t];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (c0 + k < d.z) Z += zz[k] * __builtin_amdgcn_exp2f(mm[k] - M);
+        }
+        const int off_pattern = L - d.w * 32;
+        if (off_pattern > 0) Z += (float)off_pattern * __builtin_amdgcn_exp2f(-M);  // models/block_attn.cu:74
+        sm[t] = M;
+        sr[t] = 1.0f / Z;
+        if (eb == 0) Lse[(size_t)bh * L + d.x * 32 + t] = M + __builtin_amdgcn_logf(Z);
+    }
+    __syncthreads();
+    const int e = eb * 256 + t;
+    const int l = e & 63, r = (e >> 6) & 15, c = e >> 10, row = l & 31;
+    float v = 0.f;
+    for (int c0 = 0; c0 < d.z; c0 += 8) {
+        float x[8], mm[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            x[k] = p0[(size_t)min(c0 + k, d.z - 1) * PSZ + e];
+            mm[k] = st[(size_t)min(c0 + k, d.z - 1) * PSZ + row];
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (c0 + k < d.z) v += x[k] * __builtin_amdgcn_exp2f(mm[k] - sm[row]);
+    }
+    O[((size_t)bh * L + d.x * 32 + row) * D + 32 * c + acc_row(r, l >> 5)] = (__bf16)(v * sr[row]);
+}
+
+// Plain sums (backward): out0 from the first 32 x D block of the slots, out1 (column pass: dV; grid twice as
+// large) from the second.
+template <int D>
+__global__ __launch_bounds__(256) void bf16_merge_sum_kernel(const float* __restrict__ Part, const int* __restrict__ desc,
+                                                             int n_long, int n_slots, __bf16* __restrict__ out0,
+                                                             __bf16* __restrict__ out1, int L) {
+    constexpr int PSZ = bf16_slot_floats<D>();
+    const int EB = (out1 ? 2 : 1) * 32 * D / 256;
+    const int eb = blockIdx.x % EB, item = blockIdx.x / EB;
+    const int bh = item / n_long;
+    const int4 d = reinterpret_cast<const int4*>(desc)[item % n_long];
+    const float* p0 = Part + ((size_t)bh * n_slots + d.y) * PSZ;
+    const int e = eb * 256 + threadIdx.x;
+    const int which = e / (32 * D), ee = e % (32 * D);
+    const int l = ee & 63, r = (ee >> 6) & 15, c = ee >> 10, row = l & 31;
+    float v = 0.f;
+    for (int c0 = 0; c0 < d.z; c0 += 8) {
+        float x[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) x[k] = p0[(size_t)min(c0 + k, d.z - 1) * PSZ + e];
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (c0 + k < d.z) v += x[k];
+    }
+    (which ? out1 : out0)[((size_t)bh * L + d.x * 32 + row) * D + 32 * c + acc_row(r, l >> 5)] = (__bf16)v;
 }
 
 }  // namespace spion

@@ -315,9 +315,12 @@ struct PatternIndex {
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
-    // work-group lists of the bf16 kernels (four strip ids per work-group) over block rows / block columns
+    // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
+    // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
     int *d_wg_row = nullptr, *d_wg_col = nullptr;
     int n_wg_row = 0, n_wg_col = 0;
+    int chunk_row = 1, chunk_col = 1, slots_row = 0, slots_col = 0, n_long_row = 0, n_long_col = 0;
+    int *d_long_row = nullptr, *d_long_col = nullptr;
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -345,6 +348,8 @@ struct SparseAttn {
     uint64_t ostamp = 0;
     bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
+    float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
+    size_t ws_part_floats = 0;
     int last_path = 0;
     bool is_bf16 = false;  // handle of the bf16 family: tile patterns only, P is never materialised
     bool force_element = false;
@@ -373,6 +378,10 @@ void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, boo
         set_error("init: emb_dim %d unsupported (16, 32, 64 or 128)", emb_dim);
         return nullptr;
     }
+    if ((long long)emb_dim * seq_len >= (1LL << 29)) {  // 32-bit byte offsets into one head's [L][d] slice
+        set_error("init: seq_len %d x emb_dim %d too large (one head's slice must stay under 2 GiB)", seq_len, emb_dim);
+        return nullptr;
+    }
     SparseAttn* a = new SparseAttn();
     a->hdr.magic = KIND_SPARSE;
     a->hdr.stream = nullptr;
@@ -391,6 +400,7 @@ void sparse_destroy(void* h) {
     a->pat.release();
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
+    if (a->ws_part) (void)hipFree(a->ws_part);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
     a->hdr.magic = 0;
@@ -403,23 +413,34 @@ static int long_strip_threshold(int nstrips, int ntiles) {
     return std::max(4 * avg + 8, 32);
 }
 
-// Work-group list of the bf16 kernels: long strips first, each walked by the four wavefronts of a work-group
-// together; the others in index order (neighbouring strips of a banded pattern share K/V tiles in the caches),
-// four to a work-group, one per wavefront.
-static std::vector<int> build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles) {
-    std::vector<int> order(nstrips);
-    for (int i = 0; i < nstrips; ++i) order[i] = i;
+// Work-group list of the bf16 kernels: the chunks of long strips first, each walked by the four wavefronts of a
+// work-group together; the other strips in index order (neighbouring strips of a banded pattern share K/V tiles
+// in the caches), four to a work-group, one per wavefront.  A chunk has about the tiles of an ordinary
+// work-group, so no work-group outlasts the others by much.
+struct WgList {
+    std::vector<int> wg;     // four ints per work-group
+    std::vector<int> longs;  // {strip, first slot, chunks, tiles} per long strip
+    int chunk = 1, slots = 0;
+};
+static WgList build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles) {
+    WgList out;
     const int long_len = long_strip_threshold(nstrips, ntiles);
-    std::stable_sort(order.begin(), order.end(), [&](int a, int b) {
-        return (ptr[a + 1] - ptr[a] > long_len) > (ptr[b + 1] - ptr[b] > long_len);
-    });
-    std::vector<int> wg;
-    int i = 0;
-    for (; i < nstrips && ptr[order[i] + 1] - ptr[order[i]] > long_len; ++i)
-        for (int w = 0; w < 4; ++w) wg.push_back(order[i]);
-    for (; i < nstrips; i += 4)
-        for (int w = 0; w < 4; ++w) wg.push_back(i + w < nstrips ? order[i + w] : -1);
-    return wg;
+    out.chunk = long_len;
+    std::vector<int> rest;
+    for (int i = 0; i < nstrips; ++i) {
+        const int cnt = ptr[i + 1] - ptr[i];
+        if (cnt <= long_len) {
+            rest.push_back(i);
+            continue;
+        }
+        const int chunks = (cnt + out.chunk - 1) / out.chunk;
+        out.longs.insert(out.longs.end(), {i, out.slots, chunks, cnt});
+        for (int c = 0; c < chunks; ++c) out.wg.insert(out.wg.end(), {i, i, c, out.slots + c});
+        out.slots += chunks;
+    }
+    for (size_t i = 0; i < rest.size(); i += 4)
+        for (size_t w = 0; w < 4; ++w) out.wg.push_back(i + w < rest.size() ? rest[i + w] : -1);
+    return out;
 }
 
 // Copy the index to the host once, validate it, detect the tile structure and build the transposed
@@ -430,6 +451,10 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
     const int L = a->L;
     if (nnz < 0) {
         set_error("pattern: nnz %d is negative", nnz);
+        return false;
+    }
+    if (nnz >= (1 << 29)) {  // the kernels address one head's map with 32-bit byte offsets
+        set_error("pattern: nnz %d too large (one head's map must stay under 2 GiB)", nnz);
         return false;
     }
     std::vector<int> off(L + 1), col((size_t)nnz);
@@ -493,6 +518,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         return o;
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
+    size_t o_lgr = 0, o_lgc = 0;
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -510,7 +536,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             }
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
-        const std::vector<int> wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
+        const WgList wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
         // Behind each pointer array: the order the fp32 kernels walk the strips of a head in.  Strips are
         // bucketed by length class -- rows: more than 2 MAXT tiles of the forward's register budget, more than
         // MAXT, the rest; columns: long ones, the rest -- so that long strips start first,
@@ -529,10 +555,18 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         };
         append_order(trp, true);
         append_order(tcp, false);
-        pi.n_wg_row = (int)wgr.size() / 4;
-        pi.n_wg_col = (int)wgc.size() / 4;
-        o_wgr = append(wgr);
-        o_wgc = append(wgc);
+        pi.n_wg_row = (int)wgr.wg.size() / 4;
+        pi.n_wg_col = (int)wgc.wg.size() / 4;
+        pi.chunk_row = wgr.chunk;
+        pi.chunk_col = wgc.chunk;
+        pi.slots_row = wgr.slots;
+        pi.slots_col = wgc.slots;
+        pi.n_long_row = (int)wgr.longs.size() / 4;
+        pi.n_long_col = (int)wgc.longs.size() / 4;
+        o_wgr = append(wgr.wg);
+        o_wgc = append(wgc.wg);
+        o_lgr = append(wgr.longs);
+        o_lgc = append(wgc.longs);
         if (tcol.empty()) tcol.push_back(0);
         o_trp = append(trp);
         o_tcol = append(tcol);
@@ -568,6 +602,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
         pi.d_wg_row = pi.d_blob + o_wgr;
         pi.d_wg_col = pi.d_blob + o_wgc;
+        pi.d_long_row = pi.d_blob + o_lgr;
+        pi.d_long_col = pi.d_blob + o_lgc;
     } else {
         pi.d_ccp = pi.d_blob + o_ccp;
         pi.d_crow = pi.d_blob + o_crow;
@@ -839,6 +875,21 @@ static SparseAttn* as_bf16(void* h, const char* who, const int* Offsets, const i
     return a;
 }
 
+// Workspace for the partial results of long strips: grows to the largest pattern seen.
+static bool ensure_part_ws(SparseAttn* a, int slots) {
+    const size_t need = (size_t)a->NB * slots * (a->d == 32 ? bf16_slot_floats<32>() : bf16_slot_floats<64>());
+    if (need <= a->ws_part_floats) return true;
+    if (a->ws_part) {
+        if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
+        (void)hipFree(a->ws_part);
+        a->ws_part = nullptr;
+        a->ws_part_floats = 0;
+    }
+    if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_part, sizeof(float) * need))) return false;
+    a->ws_part_floats = need;
+    return true;
+}
+
 void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out, float* Lse,
                          const int* Offsets, const int* Columns, int nnz) {
     if (!Q || !K || !V || !Out || !Lse || !Offsets || (nnz > 0 && !Columns)) {
@@ -849,12 +900,19 @@ void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, c
     if (!a) return;
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
-    const dim3 grid(pi.n_wg_row * a->NB), block(64 * BF16_WAVES);
+    if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
+    const dim3 grid(pi.n_wg_row * a->NB), block(64 * BF16_WAVES), grid_m(pi.n_long_row * a->NB * (32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
     __bf16* o = static_cast<__bf16*>(Out);
 #define SPION_LAUNCH(DD, MM)                                                                                         \
-    hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse, pi.d_trp,    \
-                       pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale)
+    do {                                                                                                             \
+        hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,          \
+                           pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,         \
+                           pi.slots_row, pi.chunk_row);                                                              \
+        if (pi.n_long_row)                                                                                           \
+            hipLaunchKernelGGL((bf16_merge_fwd_kernel<DD>), grid_m, dim3(256), 0, a->hdr.stream, a->ws_part,         \
+                               pi.d_long_row, pi.n_long_row, pi.slots_row, o, Lse, a->L);                            \
+    } while (0)
     if (a->d == 32) {
         if (Mask) SPION_LAUNCH(32, true);
         else SPION_LAUNCH(32, false);
@@ -878,20 +936,30 @@ void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, 
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+    if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
     const dim3 grid_r(pi.n_wg_row * a->NB), grid_c(pi.n_wg_col * a->NB), block(64 * BF16_WAVES);
+    const dim3 grid_mr(pi.n_long_row * a->NB * (32 * a->d / 256)), grid_mc(pi.n_long_col * a->NB * (2 * 32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
     const __bf16 *o = static_cast<const __bf16*>(Out), *go = static_cast<const __bf16*>(dO);
     __bf16 *dq = static_cast<__bf16*>(dQ), *dk = static_cast<__bf16*>(dK), *dv = static_cast<__bf16*>(dV);
 #define SPION_LAUNCH(DD, MM)                                                                                          \
     do {                                                                                                              \
-        if (a->bwd_passes & 1)                                                                                        \
+        if (a->bwd_passes & 1) {                                                                                      \
             hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o, Lse,   \
                                Mask, a->ws_rowsum, dq, pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB,    \
-                               a->scale);                                                                             \
-        if (a->bwd_passes & 2)                                                                                        \
+                               a->scale, a->ws_part, pi.slots_row, pi.chunk_row);                                     \
+            if (pi.n_long_row)                                                                                        \
+                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD>), grid_mr, dim3(256), 0, a->hdr.stream, a->ws_part,     \
+                                   pi.d_long_row, pi.n_long_row, pi.slots_row, dq, (__bf16*)nullptr, a->L);           \
+        }                                                                                                             \
+        if (a->bwd_passes & 2) {                                                                                      \
             hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM>), grid_c, block, 0, a->hdr.stream, q, k, v, go, Lse,      \
                                a->ws_rowsum, Mask, dk, dv, pi.d_tcp, pi.d_tcdesc, pi.d_wg_col, pi.n_wg_col, a->L,     \
-                               a->NB, a->scale);                                                                      \
+                               a->NB, a->scale, a->ws_part, pi.slots_col, pi.chunk_col);                              \
+            if (pi.n_long_col)                                                                                        \
+                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD>), grid_mc, dim3(256), 0, a->hdr.stream, a->ws_part,     \
+                                   pi.d_long_col, pi.n_long_col, pi.slots_col, dk, dv, a->L);                         \
+        }                                                                                                             \
     } while (0)
     if (a->d == 32) {
         if (Mask) SPION_LAUNCH(32, true);

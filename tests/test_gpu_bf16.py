@@ -186,6 +186,23 @@ def test_bf16_with_key_mask(d):
     abi.close()
 
 
+@pytest.mark.parametrize("d", [32, 64])
+def test_bf16_long_strips_with_key_mask_and_large_logits(d):
+    """A global block row and column are cut into chunks whose partial results a merge kernel combines: the
+    chunks of a row see different maxima (logits of +-40) and some lie wholly behind the key mask."""
+    L, bs, NB = 2048, 32, 2
+    mat = _mask(L // bs, 0.04, seed=11, global_block=True)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=4, scale=3.0)
+    valid = torch.tensor([2048, 1000])
+    key_mask = (torch.arange(L)[None, :] < valid[:, None]).float()
+    pen = (1e6 * (1.0 - key_mask)).contiguous().cuda()
+    _run_and_check(abi, Q, K, V, dO, pen, tag=f"bf16 long strips, key mask d={d}")
+    abi.close()
+
+
 def test_bf16_rejects_element_patterns_and_fp32_handles():
     L, d, NB = 128, 32, 1
     sm, off, col = workloads.window_random_csr(L, 4, 12, seed=3)
