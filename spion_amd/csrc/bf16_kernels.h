@@ -38,8 +38,8 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int BF16_WAVES = 4;
-// These kernels are bound by the latency of each wavefront's chain load -> LDS -> MFMA -> exp -> MFMA rather than
-// by any one unit, so they run at the highest occupancy their registers allow (OCC wavefronts per SIMD).
+// OCC wavefronts per SIMD: what the registers of each variant allow without spilling (measured: going from two to
+// three or four changes little, the kernels are bound by the instruction mix of a tile, not by latency).
 #define SPION_BF16_KERNEL(OCC) \
     __global__ __launch_bounds__(64 * BF16_WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 constexpr float BF16_LAZY = 8.f;  // the running row maximum is raised only when a tile exceeds it by 2^8
@@ -220,7 +220,7 @@ constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
 // Forward: one sweep per block row with a lazily raised running maximum.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK>
-SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : (MASK ? 2 : 3)) void bf16_fwd_kernel(
+SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
