@@ -404,11 +404,22 @@ def bench_dense_phase(args, dev):
     t_fwd = _event_ms(lambda: cpp.attn_forward(handle, Qt.data_ptr(), K.data_ptr(), Vt.data_ptr(), attn.data_ptr(),
                                                out_t.data_ptr()), max(10, args.steps // 4))
     _lib.check_error("dense forward")
+    # the two backward kernels together (operands: Qt, Kt, V, the map, dOt)
+    Kt = _lib.transpose_last2(k.detach().reshape(NB, L, d))
+    V = v.detach().reshape(NB, L, d).contiguous()
+    dOt = _lib.transpose_last2(do.reshape(NB, L, d))
+    dq, dk, dv = (torch.empty(NB, d, L, device=dev) for _ in range(3))
+    t_bwd = _event_ms(lambda: cpp.attn_backward(handle, Qt.data_ptr(), Kt.data_ptr(), V.data_ptr(), attn.data_ptr(),
+                                                dOt.data_ptr(), None, None, None, dq.data_ptr(), dk.data_ptr(),
+                                                dv.data_ptr()), max(10, args.steps // 4))
+    _lib.check_error("dense backward")
     alg_flops = 12.0 * L * L * d * NB
-    roof = dict(bound="mfma", kernel="dense_fwd_kernel", achieved=alg_flops / 3.0 / t_fwd / 1e9,
+    roof = dict(bound="mfma", kernel="dense_fwd_reg_kernel", achieved=alg_flops / 3.0 / t_fwd / 1e9,
                 peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s", traffic=None)
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["kernel_ms"] = {"dense_fwd_kernel": round(t_fwd, 4)}
+    roof["kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd, 4),
+                         "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd, 4)}
+    roof["backward_frac"] = alg_flops * 2.0 / 3.0 / t_bwd / 1e9 / PEAK_FP32_MFMA_TFLOPS
     result = {
         "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
