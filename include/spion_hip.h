@@ -160,6 +160,19 @@ int spion_pattern_generate(const float* Score, int n_maps, int seq_len, int bloc
                            float* Mat, float* Pooled, float* Thresh, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Score map of a layer for pattern discovery: the mean of the dense phase's probability maps over the
+ * batch and then over the heads -- models/model_transformer.py:136-137
+ * (attn_lst.append(torch.mean(torch.mean(attn, dim=0), dim=0))) -- in one pass over the maps.
+ *   Attn [batch][heads][seq_len][seq_len] fp32 device memory.  key_major != 0: every map is stored
+ *        keys x queries, the layout the dense attn_forward writes (models/attention_cuda.py:30-44 hands
+ *        it out as a permuted view); key_major == 0: queries x keys.
+ *   Mean [seq_len][seq_len] out, queries x keys: the Score input of spion_pattern_generate.
+ * seq_len must be a multiple of 32.  Returns 0 on success.
+ * ---------------------------------------------------------------------------------------------- */
+int spion_score_map_mean(const float* Attn, int batch, int heads, int seq_len, int key_major,
+                         float* Mean, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Additions with no counterpart in the reference (which reports no errors at all).
  * ---------------------------------------------------------------------------------------------- */
 

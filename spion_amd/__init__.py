@@ -16,6 +16,7 @@ from .pattern import (
     generate_pattern_conv,
     generate_pattern_conv_ff,
     generate_pattern_ff,
+    mean_score_map,
 )
 
 __all__ = [
@@ -35,4 +36,5 @@ __all__ = [
     "generate_pattern_conv",
     "generate_pattern_conv_ff",
     "generate_pattern_ff",
+    "mean_score_map",
 ]

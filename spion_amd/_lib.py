@@ -68,6 +68,8 @@ def core() -> ctypes.CDLL:
     lib.spion_version.argtypes = []
     lib.spion_pattern_generate.argtypes = [_P, c_int, c_int, c_int, c_int, c_int, c_double, _P, _P, _P, _P]
     lib.spion_pattern_generate.restype = c_int
+    lib.spion_score_map_mean.argtypes = [_P, c_int, c_int, c_int, c_int, _P, _P]
+    lib.spion_score_map_mean.restype = c_int
     for fam, extra in (("block", 0), ("blockmask", 1)):
         getattr(lib, f"spion_{fam}_init").argtypes = [c_int, c_int, c_int, c_int]
         getattr(lib, f"spion_{fam}_init").restype = _P

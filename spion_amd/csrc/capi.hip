@@ -45,6 +45,7 @@ void dense_forward(void*, const float*, const float*, const float*, const float*
 void dense_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
                     float*);
 int pattern_generate(const float*, int, int, int, int, int, double, float*, float*, float*, hipStream_t);
+int score_map_mean(const float*, int, int, int, int, float*, hipStream_t);
 
 }  // namespace spion
 
@@ -143,6 +144,11 @@ int spion_pattern_generate(const float* Score, int n_maps, int seq_len, int bloc
                            double param, float* Mat, float* Pooled, float* Thresh, void* stream) {
     return pattern_generate(Score, n_maps, seq_len, block_size, conv_ksize, mode, param, Mat, Pooled, Thresh,
                             static_cast<hipStream_t>(stream));
+}
+
+int spion_score_map_mean(const float* Attn, int batch, int heads, int seq_len, int key_major, float* Mean,
+                         void* stream) {
+    return score_map_mean(Attn, batch, heads, seq_len, key_major, Mean, static_cast<hipStream_t>(stream));
 }
 
 // ---- additions -----------------------------------------------------------------------------------

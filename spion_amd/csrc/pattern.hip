@@ -213,6 +213,61 @@ static std::mutex g_ws_mutex;
 static float* g_pool_ws = nullptr;
 static size_t g_pool_ws_count = 0;
 
+// Mean of the dense phase's probability maps over the batch, then over the heads
+// (models/model_transformer.py:136-137: torch.mean(torch.mean(attn, dim=0), dim=0)), read once at HBM rate.
+// A is [batch][heads][L][L]; KEY_MAJOR: the maps are stored keys x queries (what the dense kernels write, the
+// reference's column-major map) and the mean is written queries x keys, transposed through LDS.
+template <bool KEY_MAJOR>
+__global__ __launch_bounds__(256) void score_map_mean_kernel(const float* __restrict__ A, int batch, int heads, int L,
+                                                             float* __restrict__ Mean) {
+    __shared__ float tile[32][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
+    const size_t map = (size_t)L * L;
+    const float* a = A + (size_t)(r0 + ty) * L + c0 + tx;
+    float hs[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < heads; ++h) {
+        float bs[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* ah = a + (size_t)h * map;
+#pragma unroll 4
+        for (int b = 0; b < batch; ++b) {  // 16 loads in flight per thread (measured: 32 are slower)
+            const float* ab = ah + (size_t)b * heads * map;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bs[j] += __builtin_nontemporal_load(ab + (size_t)8 * j * L);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) hs[j] += bs[j] / (float)batch;
+    }
+    if (KEY_MAJOR) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) tile[ty + 8 * j][tx] = hs[j] / (float)heads;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Mean[(size_t)(c0 + ty + 8 * j) * L + r0 + tx] = tile[tx][ty + 8 * j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) Mean[(size_t)(r0 + ty + 8 * j) * L + c0 + tx] = hs[j] / (float)heads;
+    }
+}
+
+int score_map_mean(const float* Attn, int batch, int heads, int L, int key_major, float* Mean, hipStream_t stream) {
+    if (!Attn || !Mean || batch <= 0 || heads <= 0 || L <= 0 || L % 32) {
+        set_error("spion_score_map_mean: need Attn, Mean, batch > 0, heads > 0 and seq_len a positive multiple of 32 "
+                  "(got %d, %d, %d)", batch, heads, L);
+        return 1;
+    }
+    if (L / 32 > 65535) {
+        set_error("spion_score_map_mean: seq_len %d too large", L);
+        return 1;
+    }
+    const dim3 grid(L / 32, L / 32), block(256);
+    if (key_major)
+        hipLaunchKernelGGL(score_map_mean_kernel<true>, grid, block, 0, stream, Attn, batch, heads, L, Mean);
+    else
+        hipLaunchKernelGGL(score_map_mean_kernel<false>, grid, block, 0, stream, Attn, batch, heads, L, Mean);
+    return SPION_HIP_OK(hipGetLastError()) ? 0 : 1;
+}
+
 int pattern_generate(const float* Score, int n_maps, int L, int bs, int ksize, int mode, double param, float* Mat,
                      float* Pooled, float* Thresh, hipStream_t stream) {
     if (!Score || !Mat) {

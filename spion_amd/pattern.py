@@ -58,6 +58,29 @@ def discover_block_masks(score_maps: torch.Tensor, block_size: int, *, mode: str
     return (mat, pooled, thresh) if return_aux else mat
 
 
+def mean_score_map(attn: torch.Tensor) -> torch.Tensor:
+    """attn [B, H, L, L] (fp32, on the GPU) -> [L, L], ``torch.mean(torch.mean(attn, dim=0), dim=0)``
+    (models/model_transformer.py:136-137) in one pass of a HIP kernel.  Takes the permuted view the dense modules
+    return (maps stored keys x queries) as it is, without a copy; any other layout is made contiguous first."""
+    if attn.dim() != 4 or attn.shape[-1] != attn.shape[-2]:
+        raise ValueError(f"expected [B, H, L, L], got {tuple(attn.shape)}")
+    if not attn.is_cuda:
+        raise _lib.SpionLibraryError("mean_score_map runs on the GPU only; got a CPU tensor")
+    B, H, L, _ = attn.shape
+    x = attn.detach()
+    if x.dtype != torch.float32:
+        x = x.float()
+    key_major = x.stride() == (H * L * L, L * L, 1, L) and L > 1
+    if not key_major:
+        x = x.contiguous()
+    out = torch.empty((L, L), dtype=torch.float32, device=x.device)
+    stream = torch.cuda.current_stream(x.device).cuda_stream
+    if _lib.core().spion_score_map_mean(x.data_ptr(), B, H, L, int(key_major), out.data_ptr(), stream) != 0:
+        _lib.check_error("spion_score_map_mean")
+        raise _lib.SpionLibraryError("spion_score_map_mean failed")
+    return out
+
+
 def _stack_layers(attn_lst, model_config):
     L = model_config["max_seq_len"]
     # the reference keeps the first L rows of each gathered map (main_conv_ff.py:255)

@@ -60,6 +60,9 @@ def test_init_validation_and_error_slot():
     assert core.spion_pattern_generate(None, 1, 64, 32, 31, 0, 0.9, None, None, None, None) != 0
     with pytest.raises(_lib.SpionLibraryError, match="null"):
         _lib.check_error()
+    assert core.spion_score_map_mean(None, 2, 2, 64, 1, None, None) != 0
+    with pytest.raises(_lib.SpionLibraryError, match="spion_score_map_mean"):
+        _lib.check_error()
 
 
 def test_modules_refuse_to_run_without_library_handle():

@@ -89,3 +89,30 @@ def test_pattern_topk_and_generators():
         assert ml.shape == (4, 2, L // bs, L // bs) and ml.dtype == torch.float32
         assert torch.equal(ml[0], ml[3]) and set(ml.unique().tolist()) <= {0.0, 1.0}
         assert (torch.diagonal(ml[0], dim1=-2, dim2=-1) == 1).all()
+
+
+@pytest.mark.parametrize("B,H,L", [(3, 2, 64), (5, 3, 128), (64, 2, 1024)])
+def test_mean_score_map_matches_torch(B, H, L):
+    """Batch-then-head mean of the maps (models/model_transformer.py:136-137), for the key-major memory the dense
+    modules hand out as a permuted view and for plain contiguous maps."""
+    import spion_amd
+
+    g = torch.Generator().manual_seed(B * L)
+    base = torch.rand(B, H, L, L, generator=g).cuda()
+    view = base.permute(0, 1, 3, 2)            # [B, H, Lq, Lk] over keys x queries memory
+    for attn in (view, base):
+        ref = torch.mean(torch.mean(attn.double(), dim=0), dim=0)
+        got = spion_amd.mean_score_map(attn)
+        assert got.shape == (L, L) and got.is_contiguous()
+        assert torch.max(torch.abs(got.double() - ref)).item() < 1e-6
+    # the view the dense module returns is taken without a copy
+    cfg = dict(head_dim=32, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
+    if L <= 128:
+        from spion_amd.attention import Attention
+        cpp = Attention._cuda_compile_module()
+        mod = spion_amd.CUDAAttention(cfg, cpp, cpp.init(32, L, B * H))
+        q, k, v = (torch.randn(B, H, L, 32, generator=g).cuda() for _ in range(3))
+        _, p = mod(q, k, v, torch.ones(B, L).cuda())
+        assert p.stride() == (H * L * L, L * L, 1, L)
+        ref = torch.mean(torch.mean(p.double(), dim=0), dim=0)
+        assert torch.max(torch.abs(spion_amd.mean_score_map(p).double() - ref)).item() < 1e-6
