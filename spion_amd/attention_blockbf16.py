@@ -21,6 +21,7 @@ class _BlockBF16Function(torch.autograd.Function):
     @staticmethod
     def forward(ctx, query, key, value, mask, mat, module):
         m = module
+        _lib.use_current_stream(m, query.device)
         idx = m.csr_cache.get(mat, m.block_size)
         shape = (m.batch_size, m.num_heads, m.seq_len, m.emb_dim)
         if tuple(query.shape) != shape or tuple(key.shape) != shape or tuple(value.shape) != shape:
@@ -46,6 +47,7 @@ class _BlockBF16Function(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output):
         m = ctx.module
+        _lib.use_current_stream(m, ctx.saved_tensors[0].device)
         q, k, v, out, lse, offsets, columns, sum_mat = ctx.saved_tensors
         go = grad_output.to(torch.bfloat16).contiguous()
         dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(q)

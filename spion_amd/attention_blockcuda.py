@@ -20,6 +20,7 @@ class _BlockAttnFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, query, key, value, mask, mat, module):
         m = module
+        _lib.use_current_stream(m, query.device)
         idx = m.csr_cache.get(mat, m.block_size)
         nb_, L, d = m.num_batches, m.seq_len, m.emb_dim
         if tuple(query.shape) != (m.batch_size, m.num_heads, L, d):
@@ -55,6 +56,7 @@ class _BlockAttnFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output, grad_weight):
         m = ctx.module
+        _lib.use_current_stream(m, ctx.saved_tensors[0].device)
         q, key, value, p_flat, offsets, columns, sum_mat = ctx.saved_tensors
         dev = q.device
         n_total = m.num_batches * ctx.nnz

@@ -17,6 +17,7 @@ class _DenseAttnFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, query, key, value, mask, module):
         m = module
+        _lib.use_current_stream(m, query.device)
         B, H, L, d = m.batch_size, m.num_heads, m.seq_len, m.emb_dim
         if tuple(query.shape) != (B, H, L, d):
             raise ValueError(f"query shape {tuple(query.shape)} does not match the handle ({B}, {H}, {L}, {d})")
@@ -42,6 +43,7 @@ class _DenseAttnFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_output, grad_weights):
         m = ctx.module
+        _lib.use_current_stream(m, ctx.saved_tensors[0].device)
         qt, key, value, attn = ctx.saved_tensors
         B, H, L, d = m.batch_size, m.num_heads, m.seq_len, m.emb_dim
         dev = qt.device

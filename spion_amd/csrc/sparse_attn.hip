@@ -639,11 +639,22 @@ static float* ocache_for_forward(SparseAttn* a, const float* key) {
         for (auto& sl : a->oslot)
             if (sl.stamp < pick->stamp) pick = &sl;
     }
-    if (!pick->buf && hipMalloc((void**)&pick->buf, sizeof(float) * (size_t)a->NB * a->L * a->d) != hipSuccess) {
-        (void)hipGetLastError();  // no copy: the backward falls back to the two-sweep kernel
-        pick->buf = nullptr;
-        pick->key = nullptr;
-        return nullptr;
+    if (!pick->buf) {
+        // All slots are allocated on the first forward, so that later calls -- under HIP graph capture, where an
+        // allocation would invalidate the capture -- find a buffer whatever P pointer they are handed.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+        if (cap == hipStreamCaptureStatusNone)
+            for (auto& sl : a->oslot)
+                if (!sl.buf && hipMalloc((void**)&sl.buf, sizeof(float) * (size_t)a->NB * a->L * a->d) != hipSuccess) {
+                    (void)hipGetLastError();
+                    sl.buf = nullptr;
+                    break;
+                }
+        if (!pick->buf) {  // no copy: the backward falls back to the two-sweep kernel
+            pick->key = nullptr;
+            return nullptr;
+        }
     }
     pick->key = key;
     pick->stamp = ++a->ostamp;

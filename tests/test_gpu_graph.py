@@ -1,0 +1,83 @@
+"""The modules under HIP graph capture: a whole forward + backward step recorded once and replayed must give, on
+every replay, bit for bit what the eager step gives -- with eager work and synchronisations between the replays."""
+import numpy as np
+import pytest
+import torch
+
+import spion_amd
+from spion_amd import workloads
+from spion_amd.attention import Attention
+
+pytestmark = pytest.mark.gpu
+
+
+def _capture_step(module, args, q, k, v, do):
+    """Warm up on a side stream (first calls analyse the pattern and allocate the library's workspaces, which a
+    capture must not do), then record one step."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            for t in (q, k, v):
+                t.grad = None
+            out = module(q, k, v, *args)[0]
+            out.backward(do)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for t in (q, k, v):
+        t.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = module(q, k, v, *args)[0]
+        out.backward(do)
+    return graph, out, [t.grad for t in (q, k, v)]  # the tensors every replay writes
+
+
+def _eager_step(module, args, q, k, v, do):
+    for t in (q, k, v):
+        t.grad = None
+    out = module(q, k, v, *args)[0]
+    out.backward(do)
+    return out.detach().clone(), [t.grad.clone() for t in (q, k, v)]
+
+
+@pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16"])
+def test_whole_step_graph_replays_match_eager(kind):
+    B, H, L, d, bs = 2, 2, 256, 32, 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    mat = torch.from_numpy(workloads.band_random_block_mask(L // bs, 1, extra_frac=0.1, seed=3)).cuda()
+    key_mask = torch.ones(B, L)
+    key_mask[1, 200:] = 0
+    key_mask = key_mask.cuda()
+    if kind == "block":
+        cpp = Attention._blockcuda_compile_module()
+        module, args = spion_amd.CUDABlockAttention(cfg, cpp, cpp.init(d, L, B * H, bs)), (key_mask, mat)
+    elif kind == "blockmask":
+        cpp = Attention._blockcuda_mask_compile_module()
+        module, args = spion_amd.CUDABlockMaskAttention(cfg, cpp, cpp.init(d, L, B * H, bs)), (key_mask, mat)
+    elif kind == "dense":
+        cpp = Attention._cuda_compile_module()
+        module, args = spion_amd.CUDAAttention(cfg, cpp, cpp.init(d, L, B * H)), (key_mask,)
+    else:
+        module, args = spion_amd.BlockAttentionBF16(cfg), (key_mask, mat)
+    dtype = torch.bfloat16 if kind == "bf16" else torch.float32
+    q, k, v, do = (t.to(dtype) for t in workloads.qkv(B, H, L, d, seed=11, device="cuda"))
+    for t in (q, k, v):
+        t.requires_grad_()
+    ref_out, ref_grads = _eager_step(module, args, q, k, v, do)
+    graph, out, static_grads = _capture_step(module, args, q, k, v, do)
+    for replay in range(4):
+        out.detach().zero_()
+        for g in static_grads:
+            g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref_out), f"{kind}: output of replay {replay} differs from the eager step"
+        for name, g, r in zip("qkv", static_grads, ref_grads):
+            assert torch.equal(g, r), f"{kind}: d{name} of replay {replay} differs from the eager step"
+        # eager work of the same module (same handle, other buffers) between the replays
+        e_out, e_grads = _eager_step(module, args, q, k, v, do)
+        assert torch.equal(e_out, ref_out)
+        for g, r in zip(e_grads, ref_grads):
+            assert torch.equal(g, r)
+    assert np.isfinite(ref_out.float().cpu().numpy()).all()
