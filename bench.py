@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_bf16|dense_phase|config1|config2|config3|config4|config5|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_bf16|dense_phase|config1|config1_b256|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -78,8 +78,9 @@ def build_workload(name):
         B, H, L, d, bs = 32, 2, 4096, 32, 64 if name == "north_star_bs64" else 32
         mat = workloads.north_star_mask(bs)
         scale = 1.0
-    elif name == "config1":
-        B, H, L, d, bs = 8, 2, 1024, 32, 32
+    elif name in ("config1", "config1_b256"):
+        # b256: the same layer at the batch size the reference trains its L = 1024 tasks with (config.py:60)
+        B, H, L, d, bs = 256 if name == "config1_b256" else 8, 2, 1024, 32, 32
         mat = workloads.config1_mask()
         scale = 1.0 / np.sqrt(32.0)
     elif name == "config4":
