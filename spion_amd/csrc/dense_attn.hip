@@ -220,6 +220,152 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     }
 }
 
+// Forward for d = 32 and any L: two sweeps over the key tiles of a query strip, four wavefronts sharing the strip.
+// Sweep 1 keeps a running maximum and sum of exponentials per wavefront (merged over the work-group afterwards);
+// sweep 2 recomputes the logits with -M folded into the chain's initial accumulator, writes the map and
+// accumulates O^T.  Tiles are fetched linearly one tile ahead and re-laid out in wave-private LDS tiles, as in
+// the kernels above.  48 MFMA per tile against the 32 of the register-resident kernel, which is why that one is
+// used whenever a strip's logits fit in the registers of four wavefronts.
+template <bool MASK>
+SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
+    const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
+    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
+    int L, int nbr, int NB, float scale) {
+    constexpr int D = 32, KH = 16, WAVES = 4;
+    __shared__ float lds[WAVES * 16 * 64];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
+    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes);
+    const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    float* T = lds_t[w];          // map tile on its way to memory
+    float* Tk = T + 32 * TS;
+    float* Tv = T + 64 * TS;
+    const int klin = lin_voff(l, D), vlin = lin_voff(l, L);
+    const float c2 = scale * LOG2E;
+
+    float q[KH];
+    ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) q[s] *= c2;
+
+    struct Pre1 {
+        f32x4 k[4];
+        float pj[MASK ? 16 : 1];
+    };
+    struct Pre2 {
+        f32x4 k[4], v[4];
+        float pj[MASK ? 16 : 1];
+    };
+    auto penalties = [&](float (&pj)[MASK ? 16 : 1], int J) {
+        if constexpr (MASK) {
+            float t[16];
+            ldr_4x4(rM, 16 * h, J * 128, t);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pj[r] = t[r];
+        }
+    };
+
+    // ---- sweep 1: running maximum and sum over this wavefront's tiles (log2 domain) ----------------
+    float m = -10.f * LOG2E, z = 0.f;  // models/attn.cu:17
+    {
+        Pre1 xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](Pre1& x, int i) {
+                const int J = w + min(i, nu - 1) * WAVES;
+                ldr_tile_lin(rK, klin, J * 32 * D * 4, D, x.k);
+                penalties(x.pj, J);
+            },
+            [&](Pre1& c, int) {
+                lds_put_lin(Tk, l, c.k);
+                float kf[KH];
+                lds_get_feat32(Tk, li, h, kf);
+                __builtin_amdgcn_sched_barrier(0);
+                f32x16 init = splat16(0.f);
+                if constexpr (MASK) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) init[r] = -LOG2E * c.pj[r];
+                }
+                const f32x16 S = mma_feat_init<D>(kf, q, init);  // register = key, lane = query
+                const float mn = max16(S, m);
+                z *= __builtin_amdgcn_exp2f(m - mn);
+                m = mn;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) z += __builtin_amdgcn_exp2f(S[r] - m);
+            });
+    }
+    {   // the two half-waves, then the four wavefronts
+        const float mo = __shfl_xor(m, 32, 64), zo = __shfl_xor(z, 32, 64);
+        const float mn = fmaxf(m, mo);
+        z = z * __builtin_amdgcn_exp2f(m - mn) + zo * __builtin_amdgcn_exp2f(mo - mn);
+        m = mn;
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
+        float Mx = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+        m = Mx;
+        z = Z;
+    }
+    const float rinv = 1.0f / z;
+    const f32x16 minus_m = splat16(-m);
+
+    // ---- sweep 2: probabilities, map tiles and O^T --------------------------------------------------
+    f32x16 o[1] = {splat16(0.f)};  // O^T: register = feature, lane = query
+    {
+        Pre2 xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](Pre2& x, int i) {
+                const int J = w + min(i, nu - 1) * WAVES;
+                ldr_tile_lin(rK, klin, J * 32 * D * 4, D, x.k);
+                ldr_tile_lin(rV, vlin, J * 128, L, x.v);
+                penalties(x.pj, J);
+            },
+            [&](Pre2& c, int i) {
+                const int J = w + i * WAVES;
+                lds_put_lin(Tk, l, c.k);
+                lds_put_lin(Tv, l, c.v);
+                float kf[KH], vb[16];
+                lds_get_feat32(Tk, li, h, kf);
+                lds_get_rows(Tv, li, h, vb);  // V[key acc_row(s, h)][feature li]
+                __builtin_amdgcn_sched_barrier(0);
+                f32x16 init = minus_m;
+                if constexpr (MASK) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) init[r] -= LOG2E * c.pj[r];
+                }
+                const f32x16 S = mma_feat_init<D>(kf, q, init);  // logits minus the row maximum
+                float p[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(S[r]) * rinv;
+                lds_put_cols(T, li, h, p);  // T[key][query]: the map is stored key-major
+                f32x4 pl[4];
+                lds_get_lin(T, l, pl);
+#pragma unroll
+                for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
+                str_tile_lin(rA, vlin, (J * 32 * L + I * 32) * 4, L, pl);
+            });
+    }
+    reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+    if (OutCopy) {
+        __syncthreads();
+        reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+    }
+}
+
 // Row pass: g_i = sum_j dP_ij P_ij (kept in G), dS = (dP*P - P*g)*scale, dQ^T = K^T-tiles . dS^T.
 // HAVE_O: the handle kept Out of the forward that filled this map, so g_i = dO_i . O_i needs no sweep.
 template <int D, bool HAVE_O>
@@ -543,6 +689,16 @@ static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, cons
         else
             hipLaunchKernelGGL(dense_fwd_reg_kernel<false>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
                                a->ws_out, a->L, nbr, a->NB, a->scale);
+        return;
+    }
+    if (D == 32 && a->L <= 16384) {  // 32-bit byte offsets into one head's map: L*L*4 < 2^31
+        const dim3 block4(64 * 4);
+        if (a->has_mask)
+            hipLaunchKernelGGL(dense_fwd_sweep32_kernel<true>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn,
+                               Out, a->ws_out, a->L, nbr, a->NB, a->scale);
+        else
+            hipLaunchKernelGGL(dense_fwd_sweep32_kernel<false>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn,
+                               Out, a->ws_out, a->L, nbr, a->NB, a->scale);
         return;
     }
     if (a->has_mask)

@@ -42,7 +42,7 @@ def _run_dense(d, L, NB, Q, K, V, dO, pen=None, moved_map=False):
 
 @pytest.mark.parametrize("L,d,NB,with_mask", [(128, 32, 3, False), (256, 64, 2, False), (256, 32, 4, True),
                                               (1024, 32, 2, False), (96, 32, 2, False), (160, 32, 4, True),
-                                              (992, 32, 2, False), (1024, 32, 4, True), (1056, 32, 2, False)])
+                                              (992, 32, 2, False), (1024, 32, 4, True), (1056, 32, 2, False), (1088, 32, 4, True), (2048, 32, 2, False)])
 def test_dense_matches_oracle(L, d, NB, with_mask):
     g = torch.Generator().manual_seed(L + d)
     Q, K, V, dO = (torch.randn(NB, L, d, generator=g).cuda() for _ in range(4))
