@@ -39,6 +39,11 @@ def _random_block_mask(nb, p, seed, empty_row=None, empty_col=None):
         (256, 64, 32, 2, 0.40),   # 64x64 blocks = 2x2 tiles
         (256, 32, 64, 2, 0.50),   # head dim 64
         (512, 128, 64, 1, 0.50),
+        # launches of 2048 block rows and more take the fewest wavefronts that keep a row's logits in registers
+        (256, 32, 32, 256, 0.50),   # 2048 rows of at most 8 tiles  -> 1 wavefront, register-resident
+        (512, 32, 32, 128, 0.60),   # 2048 rows of up to 16 tiles   -> 2 wavefronts
+        (256, 32, 32, 160, 0.50),   # 1280 rows                     -> at least 2 wavefronts
+        (256, 32, 64, 256, 0.40),   # head dim 64: 4 tiles per wavefront
     ],
 )
 def test_tile_path_matches_oracle(L, bs, d, NB, p):
