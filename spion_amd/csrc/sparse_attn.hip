@@ -64,14 +64,13 @@ __device__ __forceinline__ float row_dot(const float* __restrict__ a, const floa
 }
 
 // Dot products of one vector a (the same for all lanes) with up to 64 gathered rows X[row_l], one result per
-// lane.  The rows are fetched LPR lanes to a row -- one or two cache lines per instruction instead of the 64 a
-// lane-per-row gather touches -- into a wave-private LDS tile (row stride D + 4 floats), from which every lane
-// then reads its own row.  D <= 64.
+// lane.  The rows are fetched D/4 lanes to a row, 16 bytes per lane -- 256/D rows per instruction instead of the
+// 64 cache lines a lane-per-row gather touches -- into a wave-private LDS tile (row stride D + 4 floats), from
+// which every lane then reads its own row.  D <= 64.
 template <int D>
 struct GatherDot {
-    static constexpr int LPR = D >= 64 ? 64 : D;
-    static constexpr int G = 64 / LPR;
-    static constexpr int CPL = D / LPR;
+    static constexpr int LPR = D / 4;   // 16 bytes per lane
+    static constexpr int G = 64 / LPR;  // rows per load instruction
     static constexpr int RS = D + 4;
     static constexpr int FLOATS = 64 * RS;
     static __device__ __forceinline__ float run(float* T, const float* __restrict__ a, const float* __restrict__ X,
@@ -79,17 +78,15 @@ struct GatherDot {
         const int grp = lane / LPR, cl = lane % LPR;
         constexpr int UN = 8;
         for (int kb = 0; kb < nk; kb += UN * G) {
-            float x[UN][CPL];
+            float4 x[UN];
 #pragma unroll
             for (int j = 0; j < UN; ++j) {
                 const int rr = __shfl(row_l, (kb + j * G + grp) & 63, 64);
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) x[j][c] = X[(size_t)rr * D + cl + c * LPR];
+                x[j] = reinterpret_cast<const float4*>(X + (size_t)rr * D)[cl];
             }
 #pragma unroll
             for (int j = 0; j < UN; ++j)
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) T[((kb + j * G + grp) & 63) * RS + cl + c * LPR] = x[j][c];
+                *reinterpret_cast<float4*>(T + ((kb + j * G + grp) & 63) * RS + 4 * cl) = x[j];
         }
         // same-wave LDS accesses complete in order: no barrier
         const float4* t4 = reinterpret_cast<const float4*>(T + lane * RS);
@@ -107,64 +104,13 @@ struct GatherDot {
     }
 };
 
-// acc[c] += sum_k w_k * X[col_k][c] over the entries of one CSR row, the entries being held one per
-// lane in chunks of 64 (w_l, col_l); LPR lanes cover one X row, 64/LPR entries are processed at once.
-template <int D>
-struct RowAcc {
-    static constexpr int LPR = D >= 64 ? 64 : D;
-    static constexpr int G = 64 / LPR;
-    static constexpr int CPL = D / LPR;
-    float acc[CPL];
-    __device__ __forceinline__ void clear() {
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
-    }
-    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int lane) {
-        const int grp = lane / LPR, cl = lane % LPR;
-        // Uniform trip count: every lane takes part in every shuffle.  Slots past nk carry w = 0
-        // and row 0 (set by the caller), so they add nothing.
-        // Eight gathers are in flight per lane before the first one is consumed: the loop is bound by the
-        // latency of the gathered rows, not by their volume.
-        constexpr int UN = 8;
-        for (int kb = 0; kb < nk; kb += UN * G) {
-            float w[UN];
-            const float* xr[UN];
-#pragma unroll
-            for (int j = 0; j < UN; ++j) {
-                const int kk = kb + j * G + grp;  // < 64 + UN*G: shuffles wrap, slots past nk are zero weights
-                w[j] = __shfl(w_l, kk & 63, 64);
-                const int rr = __shfl(row_l, kk & 63, 64);
-                if (kb + j * G >= 64) w[j] = 0.f;
-                xr[j] = X + (size_t)rr * D + cl;
-            }
-            float x[UN][CPL];
-#pragma unroll
-            for (int j = 0; j < UN; ++j)
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) x[j][c] = xr[j][c * LPR];
-#pragma unroll
-            for (int j = 0; j < UN; ++j)
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) acc[c] = fmaf(w[j], x[j][c], acc[c]);
-        }
-    }
-    __device__ __forceinline__ void finish(float* __restrict__ out_row, int lane) {
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-            float a = acc[c];
-#pragma unroll
-            for (int o = LPR; o < 64; o <<= 1) a += __shfl_xor(a, o, 64);
-            if (lane < LPR) out_row[lane + c * LPR] = a;
-        }
-    }
-};
-
-// The same with VEC floats per lane: D/VEC lanes cover one X row and 64*VEC/D entries are processed per load
-// instruction.  With 16-byte loads the backward passes of configuration 4 are faster (row pass 1.47 -> 1.19 ms,
-// column pass 1.22 -> 1.17 ms) and the forward slower (1.28 -> 1.61 ms; 1.49 ms with 8-byte loads), so the
-// forward keeps the four-byte form above.
+// acc += sum_k w_k * X[col_k][:] over the entries of one CSR row, the entries being held one per lane in chunks
+// of 64 (w_l, col_l).  VEC floats per lane: D/VEC lanes cover one X row and 64*VEC/D entries are processed per load
+// instruction.  16-byte loads (eight entries per instruction at d = 32) because the vector-memory path charges per
+// instruction and per row touched, not per byte: with four-byte loads, 32 lanes to a row, configuration 4 took
+// 3.98 ms instead of 3.21 ms.
 template <int D, int VEC = 4>
-struct RowAccV {
+struct RowAcc {
     typedef float vec_t __attribute__((ext_vector_type(VEC)));
     static constexpr int LPR = D / VEC;
     static constexpr int G = 64 / LPR;
@@ -222,12 +168,27 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
     const int* cj = cols + r0;
 
     float m = MASK ? 0.f : -100.f;
-    for (int k = lane; k < cnt; k += 64) {
-        int col = cj[k];
-        float v = row_dot<D>(q, K + hb + (size_t)col * D) * scale;
-        if (MASK) v -= pen[(size_t)bh * L + col];
-        p[k] = v;
-        m = fmaxf(m, v);
+    if constexpr (D <= 64) {
+        __shared__ __attribute__((aligned(16))) float lds_rows[ELEM_WAVES][GatherDot<D>::FLOATS];
+        float* T = lds_rows[threadIdx.x >> 6];
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + lane;
+            const int col = k < cnt ? cj[k] : 0;
+            float v = GatherDot<D>::run(T, q, K + hb, col, min(64, cnt - c0), lane) * scale;
+            if (k < cnt) {
+                if (MASK) v -= pen[(size_t)bh * L + col];
+                p[k] = v;
+                m = fmaxf(m, v);
+            }
+        }
+    } else {
+        for (int k = lane; k < cnt; k += 64) {
+            int col = cj[k];
+            float v = row_dot<D>(q, K + hb + (size_t)col * D) * scale;
+            if (MASK) v -= pen[(size_t)bh * L + col];
+            p[k] = v;
+            m = fmaxf(m, v);
+        }
     }
     m = wave_max(m);
     float z = 0.f;
@@ -293,7 +254,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
     }
     g = wave_sum(g);
 
-    RowAccV<D, 4> acc;
+    RowAcc<D> acc;
     acc.clear();
     for (int c0 = 0; c0 < cnt; c0 += 64) {
         const int k = c0 + lane;
@@ -325,7 +286,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
     const float* p = P + (size_t)bh * nnz;
     const float* ds = dS + (size_t)bh * nnz;
 
-    RowAccV<D, 4> ak, av;
+    RowAcc<D> ak, av;
     ak.clear();
     av.clear();
     for (int c0 = 0; c0 < cnt; c0 += 64) {
