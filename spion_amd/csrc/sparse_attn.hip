@@ -158,7 +158,8 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
     const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
     const int lane = threadIdx.x & 63;
-    const long long wrow = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    // consecutive rows (which gather overlapping K/V rows and share lines of P) on the same XCD
+    const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * ELEM_WAVES + (threadIdx.x >> 6);
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = offs[row], cnt = offs[row + 1] - r0;
@@ -221,7 +222,8 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
     const float* __restrict__ dO, float* __restrict__ dS, float* __restrict__ dQ,
     const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
     const int lane = threadIdx.x & 63;
-    const long long wrow = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    // consecutive rows (which gather overlapping K/V rows and share lines of P) on the same XCD
+    const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * ELEM_WAVES + (threadIdx.x >> 6);
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = offs[row], cnt = offs[row + 1] - r0;
@@ -278,7 +280,9 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
     const int* __restrict__ colptr, const int* __restrict__ crow, const int* __restrict__ cpos, int L, int NB,
     int nnz) {
     const int lane = threadIdx.x & 63;
-    const long long wcol = (long long)blockIdx.x * ELEM_WAVES + (threadIdx.x >> 6);
+    // consecutive columns on the same XCD: the 32 columns whose entries in a row share a 128-byte line of P and
+    // dS then share it in one L2 instead of fetching it into eight
+    const long long wcol = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * ELEM_WAVES + (threadIdx.x >> 6);
     if (wcol >= (long long)NB * L) return;
     const int bh = (int)(wcol / L), col = (int)(wcol % L);
     const int c0p = colptr[col], cnt = colptr[col + 1] - c0p;
