@@ -142,7 +142,9 @@ void spion_densemask_destroy(void* handle);
  *
  *   Score  [n_maps][L][L]  head/batch-averaged probability maps (one per layer).
  *   Mat    [n_maps][nb][nb] out: 0.0 / 1.0 block masks, nb = L / block_size.
- *   Pooled [n_maps][nb][nb] out, optional (may be NULL): pooled filtered map, fp32.
+ *   Pooled [n_maps][nb][nb] out, optional (may be NULL): pooled filtered map, fp32.  With NULL the library
+ *                           uses one buffer of its own, shared by all such calls: callers that run
+ *                           discovery on several streams at once pass their own Pooled.
  *   Thresh [n_maps]         out, optional (may be NULL): the quantile threshold used.
  *   conv_ksize : odd size of the diagonal (identity) filter, 31 in the reference; 0 = no filter.
  *   mode       : SPION_PATTERN_FLOOD  -> param = quantile q in [0,1], greedy path walk from the

@@ -118,16 +118,9 @@ def transpose_last2(x):
 
 def use_current_stream(module, device) -> None:
     """Point the module's handle at torch's current stream on ``device`` (the reference runs on the legacy
-    default stream only).  Costs one ctypes call when the stream changes, nothing otherwise; what makes the
-    modules usable on side streams and under HIP graph capture."""
-    stream = torch.cuda.current_stream(device).cuda_stream
-    handle = module.attn_handle
-    if _handle_stream.get(handle, 0) != stream:
-        core().spion_set_stream(handle, stream)
-        _handle_stream[handle] = stream
-
-
-_handle_stream: dict = {}  # handle -> stream it was last pointed at (a new handle starts on the null stream)
+    default stream only): what makes the modules usable on side streams and under HIP graph capture.  One
+    ctypes call per forward / backward; not cached, since handles can be shared or their addresses reused."""
+    core().spion_set_stream(module.attn_handle, torch.cuda.current_stream(device).cuda_stream)
 
 
 def check_error(where: str = "") -> None:

@@ -296,9 +296,13 @@ int pattern_generate(const float* Score, int n_maps, int L, int bs, int ksize, i
         set_error("spion_pattern_generate: quantile %g outside [0, 1]", param);
         return 1;
     }
+    // Without a caller's Pooled buffer the pooled maps go to one buffer the library owns: such calls are
+    // serialised, and the buffer is reused by the next one as soon as this one has been enqueued -- callers that
+    // work on several streams at once pass their own Pooled.
     float* pooled = Pooled;
+    std::unique_lock<std::mutex> lock(g_ws_mutex, std::defer_lock);
     if (!pooled) {
-        std::lock_guard<std::mutex> lock(g_ws_mutex);
+        lock.lock();
         const size_t need = (size_t)n_maps * nb * nb;
         if (g_pool_ws_count < need) {
             if (g_pool_ws) (void)hipFree(g_pool_ws);
