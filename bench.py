@@ -568,6 +568,9 @@ def main():
     for t in (q, k, v):
         t.grad = None
     _lib.use_current_stream(module, dev)  # the capture left the handle on its own stream
+    # the module hands the forward's output to the backward itself; a caller of the reference's ABI cannot, so
+    # the timings below run with the library's kept copies of Out, as such a caller would
+    _lib.core().spion_use_output_cache(handle, 1)
 
     # ---- per-kernel times at the C ABI, HIP events on the library's stream -----------------------
     core = _lib.core()

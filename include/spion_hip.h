@@ -206,6 +206,16 @@ void spion_set_backward_passes(void* handle, int mask);
  * row sums with one more sweep over the tiles); default on. */
 void spion_use_output_cache(void* handle, int on);
 
+/* attn_backward of the two sparse families (spion_block_* and spion_blockmask_*) for callers that still hold
+ * the forward's output -- the reference's backward (models/block_attn.cu:558) is not handed it.  Out
+ * [NB][L][d] fp32: the row sums dO.Out come from it, so such callers can switch the kept copies off
+ * (spion_use_output_cache(handle, 0)) and save their memory and traffic.  All other arguments as in
+ * spion_block_attn_backward. */
+void spion_attn_backward_with_out(void* handle, const float* Q, const float* K, const float* Vt, const float* P,
+                                  const float* Out, const float* dO, float* dP, float* dS,
+                                  float* dQ, float* dK, float* dV,
+                                  const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
 /* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
  * attention entry points take.  Returns 0 on success. */
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream);

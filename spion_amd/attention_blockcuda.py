@@ -44,7 +44,7 @@ class _BlockAttnFunction(torch.autograd.Function):
                                     p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
                                     idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
         _lib.check_error("attn_forward")
-        ctx.save_for_backward(q, key, value, p_flat, idx.offsets, idx.columns, idx.sum_mat)
+        ctx.save_for_backward(q, key, value, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
         ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
         ctx.nnz = idx.nnz
@@ -57,7 +57,7 @@ class _BlockAttnFunction(torch.autograd.Function):
     def backward(ctx, grad_output, grad_weight):
         m = ctx.module
         _lib.use_current_stream(m, ctx.saved_tensors[0].device)
-        q, key, value, p_flat, offsets, columns, sum_mat = ctx.saved_tensors
+        q, key, value, p_flat, offsets, columns, sum_mat, out = ctx.saved_tensors
         dev = q.device
         n_total = m.num_batches * ctx.nnz
         k = key.contiguous()
@@ -65,16 +65,23 @@ class _BlockAttnFunction(torch.autograd.Function):
         if grad_output is None:  # only the probabilities were used downstream: their gradient is ignored
             grad_output = torch.zeros(m.batch_size, m.num_heads, m.seq_len, m.emb_dim, dtype=torch.float32, device=dev)
         go = grad_output.contiguous()
-        scratch_dp = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
-        scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
+        # The ABI's two [NB*nnz] scratch arguments (models/attention_blockcuda.py:83-84): the tile kernels use
+        # neither, the element kernels only dS -- nothing that size is allocated unless it is needed.
+        core = _lib.core()
+        scratch_ds = None
+        if core.spion_last_path(m.attn_handle) != 1:
+            scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
+        ds_ptr = scratch_ds.data_ptr() if scratch_ds is not None else None
         shape = (m.batch_size, m.num_heads, m.seq_len, m.emb_dim)
         dq = torch.empty(shape, dtype=torch.float32, device=dev)
         dk = torch.empty(shape, dtype=torch.float32, device=dev)
         dv = torch.empty(shape, dtype=torch.float32, device=dev)
-        m.attn_cpp.attn_backward(m.attn_handle, q.data_ptr(), k.data_ptr(), vt.data_ptr(), p_flat.data_ptr(),
-                                 go.data_ptr(), scratch_dp.data_ptr(), scratch_ds.data_ptr(), dq.data_ptr(),
-                                 dk.data_ptr(), dv.data_ptr(), offsets.data_ptr(), columns.data_ptr(),
-                                 sum_mat.data_ptr(), ctx.nnz)
+        # The reference's attn_backward (models/block_attn.cu:558) is not handed the forward's output; autograd
+        # still holds it here, so the library takes its softmax row sums from it and keeps no copy of its own.
+        core.spion_attn_backward_with_out(
+            m.attn_handle, q.data_ptr(), k.data_ptr(), vt.data_ptr(), p_flat.data_ptr(), out.data_ptr(),
+            go.data_ptr(), None, ds_ptr, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+            offsets.data_ptr(), columns.data_ptr(), sum_mat.data_ptr(), ctx.nnz)
         _lib.check_error("attn_backward")
         return dq, dk, dv, None, None, None
 
@@ -100,6 +107,7 @@ class _BlockAttentionBase(nn.Module):
         self.attn_handle = attn_handle
         self.csr_cache = CsrCache()
         self.attn_func = _BlockAttnFunction
+        _lib.core().spion_use_output_cache(attn_handle, 0)  # the backward is handed the output instead
 
 
 class CUDABlockAttention(_BlockAttentionBase):

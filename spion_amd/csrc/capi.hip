@@ -27,7 +27,7 @@ void sparse_destroy(void*);
 void sparse_forward(void*, const float*, const float*, const float*, const float*, float*, float*, const int*,
                     const int*, int, bool);
 void sparse_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
-                     float*, float*, float*, const int*, const int*, int);
+                     float*, float*, float*, const int*, const int*, int, const float*);
 void sparse_invalidate(void*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
@@ -83,7 +83,7 @@ void spion_block_attn_backward(void* h, const float* Q, const float* K, const fl
                                const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
                                const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz);
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr);
 }
 void spion_block_destroy(void* h) { sparse_destroy(h); }
 
@@ -101,7 +101,7 @@ void spion_blockmask_attn_backward(void* h, const float* Q, const float* K, cons
                                    const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
                                    const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz);
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr);
 }
 void spion_blockmask_destroy(void* h) { sparse_destroy(h); }
 
@@ -175,6 +175,12 @@ int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
 void spion_use_output_cache(void* h, int on) { sparse_use_ocache(h, on); }
+void spion_attn_backward_with_out(void* h, const float* Q, const float* K, const float* Vt, const float* P,
+                                  const float* Out, const float* dO, float* dP, float* dS, float* dQ, float* dK,
+                                  float* dV, const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, Out);
+}
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
     return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));
 }

@@ -734,12 +734,13 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 
 template <int D>
 static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
-                            const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz) {
+                            const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz,
+                            const float* Out) {
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
     const int wv = pick_waves(a, pi, nbr, false);
-    const float* ocache = ocache_for_backward(a, P);
+    const float* ocache = Out ? Out : ocache_for_backward(a, P);
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
@@ -831,9 +832,11 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
     check_launch("elem_fwd_kernel");
 }
 
+// Out (optional): the forward's output, for callers that still have it; the row sums g_i = dO_i . O_i then come
+// from it and no kept copy is looked up.
 void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P, const float* dO,
                      float* dP, float* dS, float* dQ, float* dK, float* dV, const int* Offsets, const int* Columns,
-                     int nnz) {
+                     int nnz, const float* Out) {
     SparseAttn* a = as_sparse(h, "attn_backward");
     if (!a) return;
     (void)dP;
@@ -849,8 +852,8 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
     if (a->pat.tiled) {
         a->last_path = 1;
         if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
-        if (a->d == 32) launch_tile_bwd<32>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz);
-        else launch_tile_bwd<64>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz);
+        if (a->d == 32) launch_tile_bwd<32>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
+        else launch_tile_bwd<64>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
         check_launch("tile_bwd kernels");
         return;
     }

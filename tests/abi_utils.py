@@ -81,6 +81,17 @@ class SparseABI:
         _lib.check_error("attn_backward")
         return dQ, dK, dV
 
+    def backward_with_out(self, Q, K, V, P, O, dO):
+        """The library's own backward entry for callers that still hold the forward's output; no scratch."""
+        Vt = V.transpose(1, 2).contiguous()
+        dQ, dK, dV = (torch.full((self.NB, self.L, self.d), float("nan"), device=self.dev) for _ in range(3))
+        _lib.core().spion_attn_backward_with_out(
+            self.handle, Q.data_ptr(), K.data_ptr(), Vt.data_ptr(), P.contiguous().data_ptr(), O.data_ptr(),
+            dO.data_ptr(), None, None, dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(), self.offsets.data_ptr(),
+            self.columns.data_ptr(), self.sum_mat.data_ptr(), self.nnz)
+        _lib.check_error("spion_attn_backward_with_out")
+        return dQ, dK, dV
+
     def last_path(self):
         return _lib.core().spion_last_path(self.handle)
 

@@ -365,7 +365,9 @@ def test_backward_row_sums_with_and_without_output_cache():
     _lib.core().spion_use_output_cache(abi.handle, 0)
     OA3, PA3 = abi.forward(QA, KA, VA)
     gA3 = abi.backward(QA, KA, VA, PA3, dOA)
-    for got, ref, tag in ((gA, refA, "A cached"), (gB, refB, "B cached"), (gA2, refA, "A clone"), (gA3, refA, "A off")):
+    gA4 = abi.backward_with_out(QA, KA, VA, PA3, OA3, dOA)   # no copies kept: the caller hands Out over
+    for got, ref, tag in ((gA, refA, "A cached"), (gB, refB, "B cached"), (gA2, refA, "A clone"), (gA3, refA, "A off"),
+                          (gA4, refA, "A with Out")):
         for name, t in zip(("dQ", "dK", "dV"), got):
             assert_close(t.cpu().numpy(), ref[name], what=f"{tag} {name}")
     abi.close()
