@@ -216,6 +216,22 @@ void spion_attn_backward_with_out(void* handle, const float* Q, const float* K, 
                                   float* dQ, float* dK, float* dV,
                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz);
 
+/* The sparse entry points for callers whose tensors are all row-major [NB][L][d] -- the layout the reference's
+ * modules start from before they make the transposed copies its ABI asks for
+ * (models/attention_blockcuda.py:48 key.permute(0,1,3,2), :80 value.permute(0,1,3,2)).  K (forward) and V
+ * (backward) are read as they are: no transposed copy is made by anyone (d = 32 and the element kernels; the
+ * d = 64 tile kernels make one internally).  Mask: NULL for a handle of spion_block_init, the [NB][L] penalty
+ * for a handle of spion_blockmask_init.  Out in the backward: the forward's output (may be NULL: the kept copy,
+ * or one more sweep, is used).  dS: scratch [NB][nnz], needed by the element kernels only (may be NULL for
+ * tile patterns). */
+void spion_attn_forward_rowmajor(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
+                                 float* Attn, float* Out,
+                                 const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+void spion_attn_backward_rowmajor(void* handle, const float* Q, const float* K, const float* V, const float* P,
+                                  const float* Out, const float* dO, float* dS,
+                                  float* dQ, float* dK, float* dV,
+                                  const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+
 /* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
  * attention entry points take.  Returns 0 on success. */
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream);

@@ -64,6 +64,10 @@ def core() -> ctypes.CDLL:
     lib.spion_use_output_cache.restype = None
     lib.spion_attn_backward_with_out.argtypes = [_P] * 15 + [c_int]
     lib.spion_attn_backward_with_out.restype = None
+    lib.spion_attn_forward_rowmajor.argtypes = [_P] * 10 + [c_int]
+    lib.spion_attn_forward_rowmajor.restype = None
+    lib.spion_attn_backward_rowmajor.argtypes = [_P] * 14 + [c_int]
+    lib.spion_attn_backward_rowmajor.restype = None
     lib.spion_transpose_last2.argtypes = [_P, _P, c_int, c_int, c_int, _P]
     lib.spion_transpose_last2.restype = c_int
     lib.spion_version.restype = c_char_p

@@ -17,6 +17,12 @@ from .csr import CsrCache
 
 
 class _BlockAttnFunction(torch.autograd.Function):
+    """The reference's function (models/attention_blockcuda.py:20-112) makes a transposed copy of K for the forward
+    and of V for the backward because its ABI takes them that way, and its backward is not handed the forward's
+    output.  Here every tensor stays row-major and autograd's saved ``out`` goes to the backward: the library's
+    row-major entry points (spion_attn_forward_rowmajor / spion_attn_backward_rowmajor) take them as they are.
+    ``attn_cpp`` (the drop-in with the reference's four symbols) is still what created the handle."""
+
     @staticmethod
     def forward(ctx, query, key, value, mask, mat, module):
         m = module
@@ -29,58 +35,48 @@ class _BlockAttnFunction(torch.autograd.Function):
                 f"({m.batch_size}, {m.num_heads}, {L}, {d})"
             )
         dev = query.device
-        q = query.contiguous()
-        kt = _lib.transpose_last2(key)  # the ABI takes K transposed in the forward
-        v = value.contiguous()
+        q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
         p_flat = torch.empty(nb_ * idx.nnz, dtype=torch.float32, device=dev)
         out = torch.empty((m.batch_size, m.num_heads, L, d), dtype=torch.float32, device=dev)
+        pen_ptr = None
         if m.with_mask:
             pen = (1e6 * (1.0 - mask.repeat(1, m.num_heads))).to(torch.float32).contiguous()  # [B, H*L]
-            m.attn_cpp.attn_forward(m.attn_handle, q.data_ptr(), kt.data_ptr(), v.data_ptr(), pen.data_ptr(),
-                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
-                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
-        else:
-            m.attn_cpp.attn_forward(m.attn_handle, q.data_ptr(), kt.data_ptr(), v.data_ptr(),
-                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
-                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
+            pen_ptr = pen.data_ptr()
+        _lib.core().spion_attn_forward_rowmajor(m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
+                                                p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
+                                                idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
         _lib.check_error("attn_forward")
-        ctx.save_for_backward(q, key, value, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
+        ctx.save_for_backward(q, k, v, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
         ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
         ctx.nnz = idx.nnz
         if m.with_mask:
             ctx.mark_non_differentiable(p_flat)
-            return out, p_flat
         return out, p_flat
 
     @staticmethod
     def backward(ctx, grad_output, grad_weight):
         m = ctx.module
         _lib.use_current_stream(m, ctx.saved_tensors[0].device)
-        q, key, value, p_flat, offsets, columns, sum_mat, out = ctx.saved_tensors
+        q, k, v, p_flat, offsets, columns, sum_mat, out = ctx.saved_tensors
         dev = q.device
         n_total = m.num_batches * ctx.nnz
-        k = key.contiguous()
-        vt = _lib.transpose_last2(value)  # the ABI takes V transposed in the backward
         if grad_output is None:  # only the probabilities were used downstream: their gradient is ignored
             grad_output = torch.zeros(m.batch_size, m.num_heads, m.seq_len, m.emb_dim, dtype=torch.float32, device=dev)
         go = grad_output.contiguous()
-        # The ABI's two [NB*nnz] scratch arguments (models/attention_blockcuda.py:83-84): the tile kernels use
-        # neither, the element kernels only dS -- nothing that size is allocated unless it is needed.
+        # Of the ABI's two [NB*nnz] scratch arguments (models/attention_blockcuda.py:83-84) the tile kernels use
+        # neither and the element kernels only dS: nothing that size is allocated unless it is needed.
         core = _lib.core()
         scratch_ds = None
         if core.spion_last_path(m.attn_handle) != 1:
             scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
-        ds_ptr = scratch_ds.data_ptr() if scratch_ds is not None else None
         shape = (m.batch_size, m.num_heads, m.seq_len, m.emb_dim)
         dq = torch.empty(shape, dtype=torch.float32, device=dev)
         dk = torch.empty(shape, dtype=torch.float32, device=dev)
         dv = torch.empty(shape, dtype=torch.float32, device=dev)
-        # The reference's attn_backward (models/block_attn.cu:558) is not handed the forward's output; autograd
-        # still holds it here, so the library takes its softmax row sums from it and keeps no copy of its own.
-        core.spion_attn_backward_with_out(
-            m.attn_handle, q.data_ptr(), k.data_ptr(), vt.data_ptr(), p_flat.data_ptr(), out.data_ptr(),
-            go.data_ptr(), None, ds_ptr, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+        core.spion_attn_backward_rowmajor(
+            m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), p_flat.data_ptr(), out.data_ptr(), go.data_ptr(),
+            scratch_ds.data_ptr() if scratch_ds is not None else None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
             offsets.data_ptr(), columns.data_ptr(), sum_mat.data_ptr(), ctx.nnz)
         _lib.check_error("attn_backward")
         return dq, dk, dv, None, None, None

@@ -25,9 +25,9 @@ bool error_pending() {
 void* sparse_init(int, int, int, int, bool);
 void sparse_destroy(void*);
 void sparse_forward(void*, const float*, const float*, const float*, const float*, float*, float*, const int*,
-                    const int*, int, bool);
+                    const int*, int, bool, bool);
 void sparse_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
-                     float*, float*, float*, const int*, const int*, int, const float*);
+                     float*, float*, float*, const int*, const int*, int, const float*, bool);
 void sparse_invalidate(void*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
@@ -77,13 +77,13 @@ void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size
 void spion_block_attn_forward(void* h, const float* Q, const float* Kt, const float* V, float* Attn, float* Out,
                               const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_forward(h, Q, Kt, V, nullptr, Attn, Out, Offsets, Columns, nnz, false);
+    sparse_forward(h, Q, Kt, V, nullptr, Attn, Out, Offsets, Columns, nnz, false, false);
 }
 void spion_block_attn_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P,
                                const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
                                const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr);
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr, false);
 }
 void spion_block_destroy(void* h) { sparse_destroy(h); }
 
@@ -95,13 +95,13 @@ void spion_blockmask_attn_forward(void* h, const float* Q, const float* Kt, cons
                                   float* Attn, float* Out, const int* Offsets, const int* Columns,
                                   const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_forward(h, Q, Kt, V, Mask, Attn, Out, Offsets, Columns, nnz, true);
+    sparse_forward(h, Q, Kt, V, Mask, Attn, Out, Offsets, Columns, nnz, true, false);
 }
 void spion_blockmask_attn_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P,
                                    const float* dO, float* dP, float* dS, float* dQ, float* dK, float* dV,
                                    const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr);
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, nullptr, false);
 }
 void spion_blockmask_destroy(void* h) { sparse_destroy(h); }
 
@@ -179,7 +179,19 @@ void spion_attn_backward_with_out(void* h, const float* Q, const float* K, const
                                   const float* Out, const float* dO, float* dP, float* dS, float* dQ, float* dK,
                                   float* dV, const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
-    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, Out);
+    sparse_backward(h, Q, K, Vt, P, dO, dP, dS, dQ, dK, dV, Offsets, Columns, nnz, Out, false);
+}
+void spion_attn_forward_rowmajor(void* h, const float* Q, const float* K, const float* V, const float* Mask,
+                                 float* Attn, float* Out, const int* Offsets, const int* Columns, const int* SumMat,
+                                 int nnz) {
+    (void)SumMat;
+    sparse_forward(h, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, Mask != nullptr, true);
+}
+void spion_attn_backward_rowmajor(void* h, const float* Q, const float* K, const float* V, const float* P,
+                                  const float* Out, const float* dO, float* dS, float* dQ, float* dK, float* dV,
+                                  const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_backward(h, Q, K, V, P, dO, nullptr, dS, dQ, dK, dV, Offsets, Columns, nnz, Out, true);
 }
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
     return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));

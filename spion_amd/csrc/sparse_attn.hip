@@ -639,6 +639,8 @@ static bool ensure_ws(float** p, size_t count) {
     return SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * count));
 }
 
+int transpose_last2(const float* in, float* out, int batch, int rows, int cols, hipStream_t stream);
+
 // Slot of the O copy for the forward that fills P buffer `key` (least recently used slot on a miss).
 static float* ocache_for_forward(SparseAttn* a, const float* key) {
     if (!a->use_ocache) return nullptr;
@@ -704,7 +706,7 @@ static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool
     return 4;
 }
 
-template <int D, bool MASK>
+template <int D, bool MASK, bool KROW>
 static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, const float* V, const float* pen, float* P,
                             float* O, const int* offs, int nnz) {
     const PatternIndex& pi = a->pat;
@@ -718,13 +720,13 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 #define SPION_LAUNCH(W)                                                                                              \
     do {                                                                                                             \
         if (pi.max_row_tiles <= W * MAXT)                                                                            \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT>), dim3(nbr * a->NB), dim3(64 * W), 0,              \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
                                a->NB, nnz, a->scale, 0, nbr);                                                        \
         else                                                                                                         \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0>), dim3(nbr * a->NB), dim3(64 * W), 0, a->hdr.stream,  \
-                               Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,        \
-                               a->scale, 0, nbr);                                                                    \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
+                               a->NB, nnz, a->scale, 0, nbr);                                                        \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
@@ -732,7 +734,7 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 #undef SPION_LAUNCH
 }
 
-template <int D>
+template <int D, bool VROW>
 static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
                             const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz,
                             const float* Out) {
@@ -744,15 +746,15 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,   \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,   \
                                dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
                                a->scale);                                                                           \
         else if (a->bwd_passes & 1)                                                                                 \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,  \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,  \
                                dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
                                a->scale);                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
-            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
+            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
                                a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr,                          \
                                a->NB, nnz, a->scale);                                                               \
     } while (0)
@@ -795,8 +797,9 @@ static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const
                            dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz);
 }
 
+// krow: Kt is K itself, row-major [NB][L][d], not the transposed copy of the reference's ABI.
 void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, const float* Mask, float* Attn,
-                    float* Out, const int* Offsets, const int* Columns, int nnz, bool mask_entry) {
+                    float* Out, const int* Offsets, const int* Columns, int nnz, bool mask_entry, bool krow) {
     SparseAttn* a = as_sparse(h, "attn_forward");
     if (!a) return;
     if (a->has_mask != mask_entry || a->is_bf16) {
@@ -811,32 +814,46 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
     if (a->pat.tiled) {
         a->last_path = 1;
         if (a->d == 32) {
-            if (a->has_mask) launch_tile_fwd<32, true>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
-            else launch_tile_fwd<32, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+            if (krow) {
+                if (a->has_mask) launch_tile_fwd<32, true, true>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
+                else launch_tile_fwd<32, false, true>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+            } else {
+                if (a->has_mask) launch_tile_fwd<32, true, false>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
+                else launch_tile_fwd<32, false, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+            }
         } else {
-            if (a->has_mask) launch_tile_fwd<64, true>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
-            else launch_tile_fwd<64, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
+            if (krow) {  // the d = 64 kernels read the transposed operand only: make it
+                if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+                if (transpose_last2(Kt, a->ws_trans, a->NB, a->L, a->d, a->hdr.stream) != 0) return;
+                Kt = a->ws_trans;
+            }
+            if (a->has_mask) launch_tile_fwd<64, true, false>(a, Q, Kt, V, Mask, Attn, Out, Offsets, nnz);
+            else launch_tile_fwd<64, false, false>(a, Q, Kt, V, nullptr, Attn, Out, Offsets, nnz);
         }
         check_launch("tile_fwd_kernel");
         return;
     }
     a->last_path = 2;
-    if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
-    launch_transpose(a, Kt, a->ws_trans);
+    const float* Krm = Kt;  // the element kernels read K row-major
+    if (!krow) {
+        if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+        launch_transpose(a, Kt, a->ws_trans);
+        Krm = a->ws_trans;
+    }
     switch (a->d) {
-        case 16: launch_elem_fwd<16>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
-        case 32: launch_elem_fwd<32>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
-        case 64: launch_elem_fwd<64>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
-        default: launch_elem_fwd<128>(a, Q, a->ws_trans, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        case 16: launch_elem_fwd<16>(a, Q, Krm, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        case 32: launch_elem_fwd<32>(a, Q, Krm, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        case 64: launch_elem_fwd<64>(a, Q, Krm, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
+        default: launch_elem_fwd<128>(a, Q, Krm, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
     }
     check_launch("elem_fwd_kernel");
 }
 
 // Out (optional): the forward's output, for callers that still have it; the row sums g_i = dO_i . O_i then come
-// from it and no kept copy is looked up.
+// from it and no kept copy is looked up.  vrow: Vt is V itself, row-major [NB][L][d].
 void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, const float* P, const float* dO,
                      float* dP, float* dS, float* dQ, float* dK, float* dV, const int* Offsets, const int* Columns,
-                     int nnz, const float* Out) {
+                     int nnz, const float* Out, bool vrow) {
     SparseAttn* a = as_sparse(h, "attn_backward");
     if (!a) return;
     (void)dP;
@@ -852,8 +869,17 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
     if (a->pat.tiled) {
         a->last_path = 1;
         if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
-        if (a->d == 32) launch_tile_bwd<32>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
-        else launch_tile_bwd<64>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
+        if (a->d == 32) {
+            if (vrow) launch_tile_bwd<32, true>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
+            else launch_tile_bwd<32, false>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
+        } else {
+            if (vrow) {
+                if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+                if (transpose_last2(Vt, a->ws_trans, a->NB, a->L, a->d, a->hdr.stream) != 0) return;
+                Vt = a->ws_trans;
+            }
+            launch_tile_bwd<64, false>(a, Q, K, Vt, P, dO, dQ, dK, dV, Offsets, nnz, Out);
+        }
         check_launch("tile_bwd kernels");
         return;
     }
@@ -862,13 +888,17 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         set_error("attn_backward: the element path needs the dS scratch buffer");
         return;
     }
-    if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
-    launch_transpose(a, Vt, a->ws_trans);
+    const float* Vrm = Vt;  // the element kernels read V row-major
+    if (!vrow) {
+        if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
+        launch_transpose(a, Vt, a->ws_trans);
+        Vrm = a->ws_trans;
+    }
     switch (a->d) {
-        case 16: launch_elem_bwd<16>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
-        case 32: launch_elem_bwd<32>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
-        case 64: launch_elem_bwd<64>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
-        default: launch_elem_bwd<128>(a, Q, K, a->ws_trans, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        case 16: launch_elem_bwd<16>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        case 32: launch_elem_bwd<32>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        case 64: launch_elem_bwd<64>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
+        default: launch_elem_bwd<128>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
     }
     check_launch("elem_bwd kernels");
 }

@@ -272,7 +272,9 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // MAXT tiles), so each tile costs one QK^T chain and one PV chain.  MAXT == 0: two sweeps, the second
 // recomputing the logits (any row length).  Ocache (optional): second copy of O for the backward.
 // -------------------------------------------------------------------------------------------------
-template <int D, int WAVES, bool MASK, int MAXT>
+// KROW: the K operand is row-major [NB][L][D] (what a caller has before it makes the transposed copy the
+// reference's ABI asks for) instead of feature-major [NB][D][L]; d = 32 only.
+template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false>
 SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
@@ -311,6 +313,11 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     ldr_rows<D>(rQ, (li * D + h * KH) * 4, I * 32 * D * 4, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
+    // operand over the head dimension of key tile J (lane = key, features h*D/2 ..)
+    auto load_kf = [&](int J, float (&x)[KH]) {
+        if constexpr (KROW) ldr_rows<D>(rK, (li * D + h * KH) * 4, J * 32 * D * 4, x);
+        else ldr_cols<D>(rK, L, col_voff, J * 128, x);
+    };
 
     // initial accumulator of a logit chain: minus the key penalties of the tile, in the log2 domain
     auto chain_init = [&](int J) -> f32x16 {
@@ -339,17 +346,21 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         // clear of the 63 outstanding instructions it may have (loads and stores share that counter).
         constexpr bool LIN = D == 32;
         float* Tx = T + 32 * TS;  // K^T tile, later V tile (LIN only)
-        const int klin = lin_voff(l, L), vlin = lin_voff(l, D), plin = lin_voff(l, rn);
+        // a K tile is 32 features x 32 keys with rows L floats apart, or (KROW) 32 keys x 32 features, contiguous
+        constexpr int KSTEP = KROW ? 32 * D * 4 : 128;
+        const int kld = KROW ? D : L;
+        const int klin = lin_voff(l, kld), vlin = lin_voff(l, D), plin = lin_voff(l, rn);
         if constexpr (LIN) {
             f32x4 kraw[2][4];
-            if (nu > 0) ldr_tile_lin(rK, klin, Js[0] * 128, L, kraw[0]);
+            if (nu > 0) ldr_tile_lin(rK, klin, Js[0] * KSTEP, kld, kraw[0]);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
-                    if (u + 1 < MAXT) ldr_tile_lin(rK, klin, Js[u + 1 < MAXT ? u + 1 : u] * 128, L, kraw[(u + 1) & 1]);
+                    if (u + 1 < MAXT) ldr_tile_lin(rK, klin, Js[u + 1 < MAXT ? u + 1 : u] * KSTEP, kld, kraw[(u + 1) & 1]);
                     lds_put_lin(Tx, l, kraw[u & 1]);
                     float kf[KH];
-                    lds_get_featcols32(Tx, li, h, kf);
+                    if constexpr (KROW) lds_get_feat32(Tx, li, h, kf);
+                    else lds_get_featcols32(Tx, li, h, kf);
                     __builtin_amdgcn_sched_barrier(0);
                     S[u] = mma_feat_init<D>(kf, q, chain_init(Js[u]));
                     m = max16(S[u], m);
@@ -357,11 +368,11 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
             }
         } else {
             float kbuf[2][KH];
-            if (nu > 0) ldr_cols<D>(rK, L, col_voff, Js[0] * 128, kbuf[0]);
+            if (nu > 0) load_kf(Js[0], kbuf[0]);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
-                    if (u + 1 < MAXT) ldr_cols<D>(rK, L, col_voff, Js[u + 1 < MAXT ? u + 1 : u] * 128, kbuf[(u + 1) & 1]);
+                    if (u + 1 < MAXT) load_kf(Js[u + 1 < MAXT ? u + 1 : u], kbuf[(u + 1) & 1]);
                     S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(Js[u]));
                     m = max16(S[u], m);
                 }
@@ -449,7 +460,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         };
         auto fetch_k = [&](PreK& x, int i) {
             const int J = tcol[t0 + w + min(i, nu - 1) * WAVES];
-            ldr_cols<D>(rK, L, col_voff, J * 128, x.k);
+            load_kf(J, x.k);
             if constexpr (MASK) ldr_4x4(rM, m_voff, J * 128, x.pj);
         };
         auto init_of = [&](const PreK& x, float shift) -> f32x16 {
@@ -509,12 +520,14 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
 // dP^T - g = V_J.dO_I^T chain started from -g, dS' = (dP - g)*P, dQ += dS'.K_J; the 1/sqrt(d) is applied to
 // the 32 x d result.  G receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------
-template <int D, int WAVES, bool HAVE_O>
+// VROW: the V operand is row-major [NB][L][D] instead of feature-major [NB][D][L]; d = 32 only.
+template <int D, int WAVES, bool HAVE_O, bool VROW = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
     float* __restrict__ dQ, const int* __restrict__ trp, const int* __restrict__ tcol,
     const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    static_assert(!VROW || D == 32, "row-major V operand: d = 32 only");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_g[WAVES][32];
@@ -561,7 +574,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             nu, xa, xb,
             [&](PreG& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
-                ldr_cols<D>(rV, L, col_voff, tcol[t0 + t] * 128, x.vt);
+                if constexpr (VROW) ldr_rows<D>(rV, r_voff, tcol[t0 + t] * 32 * D * 4, x.vt);
+                else ldr_cols<D>(rV, L, col_voff, tcol[t0 + t] * 128, x.vt);
                 ldr_tile_cols(rP, pc_voff, p_base + t * 128, rn, x.pv);
             },
             [&](PreG& c, int) {
@@ -595,14 +609,16 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
         float* Tv = T;
         float* Tp = T + 32 * TS;
         float* Tk = T + 64 * TS;
-        const int vl = lin_voff(l, L), pl = lin_voff(l, rn), kl = lin_voff(l, D);
+        constexpr int VSTEP = VROW ? 32 * D * 4 : 128;
+        const int vld = VROW ? D : L;
+        const int vl = lin_voff(l, vld), pl = lin_voff(l, rn), kl = lin_voff(l, D);
         Pre xa, xb;
         tile_pipeline(
             nu, xa, xb,
             [&](Pre& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
                 const int J = tcol[t0 + t];
-                ldr_tile_lin(rV, vl, J * 128, L, x.vt);
+                ldr_tile_lin(rV, vl, J * VSTEP, vld, x.vt);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) x.pv[i] = ld4_nt(rP, pl, p_base + t * 128 + 32 * i * rn);
                 ldr_tile_lin(rK, kl, J * 32 * D * 4, D, x.kb);
@@ -614,7 +630,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 // every LDS read is issued before the first chain starts (left to itself the compiler sinks
                 // each read next to the MFMA that uses it and waits for it there)
                 float vt[16], pr[16], kb[1][16];
-                lds_get_featcols32(Tv, li, h, vt);
+                if constexpr (VROW) lds_get_feat32(Tv, li, h, vt);
+                else lds_get_featcols32(Tv, li, h, vt);
                 lds_get_rows(Tp, li, h, pr);
                 lds_get_cols(Tk, li, h, kb[0]);
                 __builtin_amdgcn_sched_barrier(0);
@@ -669,7 +686,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
 // dV_J = sum_I P_IJ^T dO_I over the transposed tile index; dP - g is recomputed per tile by a chain
 // started from the stored -g, the 1/sqrt(d) of dK is applied to the 32 x d result.
 // -------------------------------------------------------------------------------------------------
-template <int D, int WAVES>
+// VROW: as in the row pass.
+template <int D, int WAVES, bool VROW = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
@@ -689,7 +707,8 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const int r_voff = (li * D + h * KH) * 4;
 
     float vt[KH];
-    ldr_cols<D>(rV, L, (h * KH * L + li) * 4, J * 128, vt);
+    if constexpr (VROW) ldr_rows<D>(rV, r_voff, J * 32 * D * 4, vt);
+    else ldr_cols<D>(rV, L, (h * KH * L + li) * 4, J * 128, vt);
 
     f32x16 ak[D / 32], av[D / 32];
 #pragma unroll

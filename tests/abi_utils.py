@@ -92,6 +92,28 @@ class SparseABI:
         _lib.check_error("spion_attn_backward_with_out")
         return dQ, dK, dV
 
+    def forward_rowmajor(self, Q, K, V, penalty=None):
+        """The library's entry for row-major K (no transposed copy).  Returns (O, P)."""
+        P = torch.full((self.NB * max(self.nnz, 1),), float("nan"), device=self.dev)
+        O = torch.full((self.NB, self.L, self.d), float("nan"), device=self.dev)
+        _lib.core().spion_attn_forward_rowmajor(
+            self.handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(), penalty.data_ptr() if penalty is not None else None,
+            P.data_ptr(), O.data_ptr(), self.offsets.data_ptr(), self.columns.data_ptr(), self.sum_mat.data_ptr(),
+            self.nnz)
+        _lib.check_error("spion_attn_forward_rowmajor")
+        return O, P[: self.NB * self.nnz].view(self.NB, self.nnz)
+
+    def backward_rowmajor(self, Q, K, V, P, O, dO):
+        """Row-major V, the forward's output handed over; dS scratch only where the element kernels need it."""
+        dS = torch.full((self.NB * max(self.nnz, 1),), float("nan"), device=self.dev)
+        dQ, dK, dV = (torch.full((self.NB, self.L, self.d), float("nan"), device=self.dev) for _ in range(3))
+        _lib.core().spion_attn_backward_rowmajor(
+            self.handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(), P.contiguous().data_ptr(),
+            O.data_ptr() if O is not None else None, dO.data_ptr(), dS.data_ptr(), dQ.data_ptr(), dK.data_ptr(),
+            dV.data_ptr(), self.offsets.data_ptr(), self.columns.data_ptr(), self.sum_mat.data_ptr(), self.nnz)
+        _lib.check_error("spion_attn_backward_rowmajor")
+        return dQ, dK, dV
+
     def last_path(self):
         return _lib.core().spion_last_path(self.handle)
 

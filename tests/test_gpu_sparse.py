@@ -8,7 +8,7 @@ import torch
 
 from oracle import sparse_attention as osa
 from spion_amd import workloads
-from tests.abi_utils import SparseABI, assert_close, run_and_check
+from tests.abi_utils import SparseABI, assert_close, oracle_fwd_bwd, run_and_check
 
 pytestmark = pytest.mark.gpu
 
@@ -370,6 +370,45 @@ def test_backward_row_sums_with_and_without_output_cache():
                           (gA4, refA, "A with Out")):
         for name, t in zip(("dQ", "dK", "dV"), got):
             assert_close(t.cpu().numpy(), ref[name], what=f"{tag} {name}")
+    abi.close()
+
+
+@pytest.mark.parametrize("kind,d,with_mask", [("tile", 32, False), ("tile", 32, True), ("tile", 64, False),
+                                              ("tile_rows", 32, False), ("element", 32, True), ("element", 128, False)])
+def test_rowmajor_entry_points_match_oracle(kind, d, with_mask):
+    """spion_attn_forward_rowmajor / spion_attn_backward_rowmajor: K and V as they are, Out handed to the backward
+    (and, once, withheld: the backward then finds the row sums itself).  "tile_rows": long rows, the two-sweep
+    forward; 2048 rows and more: one wavefront per row."""
+    NB = 3
+    if kind == "element":
+        L = 150
+        sm, off, col = _random_element_csr(L, 0.3, seed=d)
+        bs = 1
+    else:
+        L, bs = (2048, 32) if kind == "tile_rows" else (256, 32)
+        mat = _random_block_mask(L // bs, 0.3, seed=d + 1)
+        if kind == "tile_rows":
+            mat[3, :] = 1   # 64 tiles in one row: beyond what four wavefronts keep in registers
+            NB = 1
+        sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=31, scale=1.3)
+    pen = None
+    if with_mask:
+        valid = torch.tensor([L, L - 40, L // 2][:NB])
+        pen = (1e6 * (torch.arange(L)[None, :] >= valid[:, None]).float()).contiguous().cuda()
+    ref = oracle_fwd_bwd(Q, K, V, dO, sm, off, col, pen)
+    O, P = abi.forward_rowmajor(Q, K, V, pen)
+    grads = abi.backward_rowmajor(Q, K, V, P, O, dO)
+    grads_no_out = abi.backward_rowmajor(Q, K, V, P, None, dO)
+    torch.cuda.synchronize()
+    assert abi.last_path() == (2 if kind == "element" else 1)
+    assert_close(P.cpu().numpy(), ref["P"], what=f"{kind} d={d} P")
+    assert_close(O.cpu().numpy(), ref["O"], what=f"{kind} d={d} O")
+    for got, tag in ((grads, "with Out"), (grads_no_out, "without Out")):
+        for name, t in zip(("dQ", "dK", "dV"), got):
+            assert_close(t.cpu().numpy(), ref[name], what=f"{kind} d={d} {tag} {name}")
     abi.close()
 
 
