@@ -706,6 +706,15 @@ static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool
     return 4;
 }
 
+// Heads whose strips are interleaved in launch order (see item_to_head_strip): as many as share an XCD's slice of
+// the launch, at most 8 -- their K and V (2 * L * d floats a head) stay within reach of that XCD's L2.
+static int heads_per_group(const SparseAttn* a) {
+    // Two heads share a stretch of the launch order when every die's share of the heads is even: the long strips of
+    // both come first, so the last work groups of a die are short ones (north star shape: step 2 % shorter than
+    // with one head at a time; four heads give the same, eight lose it again to the L2's reach).
+    return a->NB % 16 == 0 ? 2 : 1;
+}
+
 template <int D, bool MASK, bool KROW>
 static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, const float* V, const float* pen, float* P,
                             float* O, const int* offs, int nnz) {
@@ -717,16 +726,17 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     // measured and brings nothing over four wavefronts for all.)
     constexpr int MAXT = D == 32 ? 8 : 4;
     const int wv = pick_waves(a, pi, nbr, true);
+    const int hc = heads_per_group(a);
 #define SPION_LAUNCH(W)                                                                                              \
     do {                                                                                                             \
         if (pi.max_row_tiles <= W * MAXT)                                                                            \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
-                               a->NB, nnz, a->scale, 0, nbr);                                                        \
+                               a->NB, nnz, a->scale, 0, nbr, hc);                                                        \
         else                                                                                                         \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
-                               a->NB, nnz, a->scale, 0, nbr);                                                        \
+                               a->NB, nnz, a->scale, 0, nbr, hc);                                                        \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
@@ -742,21 +752,22 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
     const int wv = pick_waves(a, pi, nbr, false);
+    const int hc = heads_per_group(a);
     const float* ocache = Out ? Out : ocache_for_backward(a, P);
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
             hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,   \
                                dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
-                               a->scale);                                                                           \
+                               a->scale, hc);                                                                       \
         else if (a->bwd_passes & 1)                                                                                 \
             hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,  \
                                dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
-                               a->scale);                                                                           \
+                               a->scale, hc);                                                                       \
         if (a->bwd_passes & 2)                                                                                      \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
                                a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr,                          \
-                               a->NB, nnz, a->scale);                                                               \
+                               a->NB, nnz, a->scale, hc);                                                           \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);

@@ -243,6 +243,17 @@ __device__ __forceinline__ void merge_max_sum(float& m, float& z, int w, int h, 
     }
 }
 
+// Work item -> (head, position in the strip order).  The heads are taken hc at a time; within such a group the
+// items walk the strip order (long strips first) with the group's heads innermost, so that all long strips of the
+// group start before any short one and the launch ends on short strips.  (Time stamps per work group on the north
+// star shape, backward row pass: a CU's eight wavefront slots are 88 % filled over the launch, 5 % of the launch is
+// the tail after the average CU's last work group ends, the dies end within 5 % of each other.)
+__device__ __forceinline__ void item_to_head_strip(int item, int nstrips, int hc, int& head, int& pos) {
+    const int per = nstrips * hc, g = item / per, r = item - g * per;
+    head = g * hc + r % hc;
+    pos = r / hc;
+}
+
 // Software-pipelined walk over the tiles first, first+step, ... (n of them) of one wavefront.
 //   fetch(X, i)   requests everything tile #i (0-based position in this wavefront's list) needs into X;
 //   compute(X, i) consumes it.  Positions past the end are clamped by the callers' fetch (valid, redundant).
@@ -279,14 +290,16 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
     const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
-    int NB, int nnz, float scale, int s0, int ns) {
+    int NB, int nnz, float scale, int s0, int ns, int hc) {
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 && MAXT > 0 ? 2 : 1) * 32 * TS];
     // this launch covers strips s0 .. s0+ns-1 of the longest-first order of every head
     const int item = xcd_remap(blockIdx.x, ns * NB);
-    const int bh = item / ns, I = trp[nbr + 1 + s0 + item % ns];
+    int bh, pos;
+    item_to_head_strip(item, ns, hc, bh, pos);
+    const int I = trp[nbr + 1 + s0 + pos];
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
@@ -526,7 +539,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
     float* __restrict__ dQ, const int* __restrict__ trp, const int* __restrict__ tcol,
-    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale) {
+    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale, int hc) {
     static_assert(!VROW || D == 32, "row-major V operand: d = 32 only");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
@@ -534,7 +547,10 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 ? 3 : 1) * 32 * TS];
     // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
     const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = NB - 1 - item / nbr, I = trp[nbr + 1 + item % nbr];  // strips of a head, longest first
+    int bh, pos;
+    item_to_head_strip(item, nbr, hc, bh, pos);
+    bh = NB - 1 - bh;
+    const int I = trp[nbr + 1 + pos];  // strips longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
@@ -691,12 +707,15 @@ template <int D, int WAVES, bool VROW = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
-    const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale) {
+    const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
+    int hc) {
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, J = tcp[nbr + 1 + item % nbr];  // strips of a head, longest first
+    int bh, pos;
+    item_to_head_strip(item, nbr, hc, bh, pos);
+    const int J = tcp[nbr + 1 + pos];  // strips longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
