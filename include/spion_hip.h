@@ -232,6 +232,33 @@ void spion_attn_backward_rowmajor(void* handle, const float* Q, const float* K, 
                                   float* dQ, float* dK, float* dV,
                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz);
 
+/* The same for heads that are views of other memory: the reference's layer produces Q, K and V as
+ * [B][L][H*d] projections and views them as [B][H][L][d] (models/attention.py:84-96 and split_heads :136-139),
+ * then copies each into a contiguous [NB][L][d] buffer before the call (models/attention_blockcuda.py:48,80;
+ * the output is copied back by combine_heads, models/attention.py:131-134).  These two entry points read and
+ * write such views in place.  Element (b, h, i, f) of a tensor lies batch_stride*b + head_stride*h +
+ * row_stride*i + f floats after its pointer; one layout for the inputs Q, K, V, one for Out and dO, one for
+ * the gradients dQ, dK, dV.  heads = H (num_batches of the handle = B*H, head index fastest).  Strides are
+ * multiples of 4 floats, pointers 16-byte aligned, seq_len * row_stride < 2^29.  Served by the tile kernels
+ * for emb_dim 32 (patterns of aligned 32x32 tiles); otherwise an error is recorded and the caller makes
+ * contiguous copies for the row-major entry points above.  Attn / P stay [NB][nnz] as everywhere.  The kept
+ * copies of Out are not used: the backward takes Out (required). */
+typedef struct spion_head_layout {
+    long long batch_stride;
+    int head_stride;
+    int row_stride;
+} spion_head_layout;
+void spion_attn_forward_strided(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
+                                float* Attn, float* Out,
+                                const int* Offsets, const int* Columns, const int* SumMat, int nnz,
+                                int heads, const spion_head_layout* in, const spion_head_layout* out);
+void spion_attn_backward_strided(void* handle, const float* Q, const float* K, const float* V, const float* P,
+                                 const float* Out, const float* dO,
+                                 float* dQ, float* dK, float* dV,
+                                 const int* Offsets, const int* Columns, const int* SumMat, int nnz,
+                                 int heads, const spion_head_layout* in, const spion_head_layout* out,
+                                 const spion_head_layout* grad);
+
 /* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
  * attention entry points take.  Returns 0 on success. */
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream);

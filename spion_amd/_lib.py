@@ -68,6 +68,10 @@ def core() -> ctypes.CDLL:
     lib.spion_attn_forward_rowmajor.restype = None
     lib.spion_attn_backward_rowmajor.argtypes = [_P] * 14 + [c_int]
     lib.spion_attn_backward_rowmajor.restype = None
+    lib.spion_attn_forward_strided.argtypes = [_P] * 10 + [c_int, c_int, _P, _P]
+    lib.spion_attn_forward_strided.restype = None
+    lib.spion_attn_backward_strided.argtypes = [_P] * 13 + [c_int, c_int, _P, _P, _P]
+    lib.spion_attn_backward_strided.restype = None
     lib.spion_transpose_last2.argtypes = [_P, _P, c_int, c_int, c_int, _P]
     lib.spion_transpose_last2.restype = c_int
     lib.spion_version.restype = c_char_p
@@ -120,6 +124,25 @@ def transpose_last2(x):
     if core().spion_transpose_last2(x.data_ptr(), out.data_ptr(), batch, R, C, stream) != 0:
         check_error("spion_transpose_last2")
     return out
+
+
+class HeadLayout(ctypes.Structure):
+    """``spion_head_layout``: where element (b, h, i, f) of a [B, H, L, d] view lies, in floats."""
+
+    _fields_ = [("batch_stride", ctypes.c_longlong), ("head_stride", c_int), ("row_stride", c_int)]
+
+
+def head_layout(t: "torch.Tensor") -> HeadLayout | None:
+    """Layout of a 4-D [B, H, L, d] tensor or view for the strided entry points; None when they cannot take it
+    (last dimension not unit-stride, strides not multiples of 4 floats, storage offset not 16-byte aligned)."""
+    sb, sh, sl, sf = t.stride()
+    if t.dim() != 4 or sf != 1 or t.data_ptr() % 16:
+        return None
+    if sb % 4 or sh % 4 or sl % 4 or sl < t.shape[3] or min(sb, sh) < 0:
+        return None
+    if t.shape[2] * sl >= 1 << 29:
+        return None
+    return HeadLayout(sb, sh, sl)
 
 
 def use_current_stream(module, device) -> None:

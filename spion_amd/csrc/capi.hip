@@ -28,6 +28,16 @@ void sparse_forward(void*, const float*, const float*, const float*, const float
                     const int*, int, bool, bool);
 void sparse_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
                      float*, float*, float*, const int*, const int*, int, const float*, bool);
+struct HeadLayout {  // as in tile_kernels.h
+    long long bstride;
+    int hstride;
+    int ld;
+};
+void sparse_forward_strided(void*, const float*, const float*, const float*, const float*, float*, float*, const int*,
+                            const int*, int, int, const HeadLayout&, const HeadLayout&);
+void sparse_backward_strided(void*, const float*, const float*, const float*, const float*, const float*, const float*,
+                             float*, float*, float*, const int*, const int*, int, int, const HeadLayout&,
+                             const HeadLayout&, const HeadLayout&);
 void sparse_invalidate(void*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
@@ -192,6 +202,32 @@ void spion_attn_backward_rowmajor(void* h, const float* Q, const float* K, const
                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
     (void)SumMat;
     sparse_backward(h, Q, K, V, P, dO, nullptr, dS, dQ, dK, dV, Offsets, Columns, nnz, Out, true);
+}
+static spion::HeadLayout to_layout(const spion_head_layout* y) {
+    return spion::HeadLayout{y->batch_stride, y->head_stride, y->row_stride};
+}
+void spion_attn_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                                float* Out, const int* Offsets, const int* Columns, const int* SumMat, int nnz,
+                                int heads, const spion_head_layout* in, const spion_head_layout* out) {
+    (void)SumMat;
+    if (!in || !out) {
+        set_error("attn_forward_strided: null layout argument");
+        return;
+    }
+    sparse_forward_strided(h, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, heads, to_layout(in), to_layout(out));
+}
+void spion_attn_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P,
+                                 const float* Out, const float* dO, float* dQ, float* dK, float* dV,
+                                 const int* Offsets, const int* Columns, const int* SumMat, int nnz, int heads,
+                                 const spion_head_layout* in, const spion_head_layout* out,
+                                 const spion_head_layout* grad) {
+    (void)SumMat;
+    if (!in || !out || !grad) {
+        set_error("attn_backward_strided: null layout argument");
+        return;
+    }
+    sparse_backward_strided(h, Q, K, V, P, Out, dO, dQ, dK, dV, Offsets, Columns, nnz, heads, to_layout(in),
+                            to_layout(out), to_layout(grad));
 }
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
     return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));

@@ -715,12 +715,12 @@ static int heads_per_group(const SparseAttn* a) {
     return a->NB % 16 == 0 ? 2 : 1;
 }
 
-template <int D, bool MASK, bool KROW>
+template <int D, bool MASK, bool KROW, bool ST = false>
 static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, const float* V, const float* pen, float* P,
-                            float* O, const int* offs, int nnz) {
+                            float* O, const int* offs, int nnz, const Layouts& ly = Layouts{}) {
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
-    float* ocache = ocache_for_forward(a, P);
+    float* ocache = ST ? nullptr : ocache_for_forward(a, P);
     // Logit tiles stay in registers when every wavefront's share of the longest block row fits (MAXT tiles);
     // otherwise two sweeps.  (Launching the block rows by length class with 1, 2 and 4 wavefronts per row was
     // measured and brings nothing over four wavefronts for all.)
@@ -730,13 +730,13 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 #define SPION_LAUNCH(W)                                                                                              \
     do {                                                                                                             \
         if (pi.max_row_tiles <= W * MAXT)                                                                            \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
-                               a->NB, nnz, a->scale, 0, nbr, hc);                                                        \
+                               a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
         else                                                                                                         \
-            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
+            hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
-                               a->NB, nnz, a->scale, 0, nbr, hc);                                                        \
+                               a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
@@ -744,10 +744,10 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 #undef SPION_LAUNCH
 }
 
-template <int D, bool VROW>
+template <int D, bool VROW, bool ST = false>
 static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
                             const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz,
-                            const float* Out) {
+                            const float* Out, const Layouts& ly = Layouts{}) {
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
@@ -757,17 +757,19 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,   \
-                               dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
-                               a->scale, hc);                                                                       \
-        else if (a->bwd_passes & 1)                                                                                 \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, K, Vt, P,  \
-                               dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB, nnz,      \
-                               a->scale, hc);                                                                       \
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, K,   \
+                               Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB,    \
+                               nnz, a->scale, hc, ly);                                                              \
+        else if (a->bwd_passes & 1) {                                                                               \
+            if constexpr (!ST)                                                                                      \
+                hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream,  \
+                                   K, Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr,    \
+                                   a->NB, nnz, a->scale, hc, ly);                                                   \
+        }                                                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
-            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, dO,     \
-                               a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr,                          \
-                               a->NB, nnz, a->scale, hc);                                                           \
+            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, \
+                               dO, a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
+                               hc, ly);                                                                             \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
@@ -912,6 +914,107 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         default: launch_elem_bwd<128>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
     }
     check_launch("elem_bwd kernels");
+}
+
+// Heads that are views of other memory (the [B][L][H*d] output of a projection seen as [B][H][L][d]): the tile
+// kernels for d = 32 take the three strides of each tensor group and read / write the views in place.
+static bool check_layout(const char* who, const char* what, const SparseAttn* a, int heads, const HeadLayout& y) {
+    if (y.ld < a->d || y.ld % 4 || y.hstride % 4 || y.bstride % 4 || y.hstride < 0 || y.bstride < 0) {
+        set_error("%s: %s layout: strides must be non-negative multiples of 4 floats and the row stride >= emb_dim", who,
+                  what);
+        return false;
+    }
+    // every byte offset inside one head's slice is a 32-bit quantity in the kernels
+    if ((long long)a->L * y.ld >= (1ll << 29)) {
+        set_error("%s: %s layout: seq_len * row stride = %lld floats exceeds 2^29", who, what, (long long)a->L * y.ld);
+        return false;
+    }
+    (void)heads;
+    return true;
+}
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static SparseAttn* strided_handle(void* h, const char* who, const int* Offsets, const int* Columns, int nnz, int heads) {
+    SparseAttn* a = as_sparse(h, who);
+    if (!a) return nullptr;
+    if (a->is_bf16) {
+        set_error("%s: handle was created by the bf16 init", who);
+        return nullptr;
+    }
+    if (heads <= 0 || a->NB % heads) {
+        set_error("%s: heads = %d does not divide num_batches = %d", who, heads, a->NB);
+        return nullptr;
+    }
+    if (!Offsets || (nnz > 0 && !Columns)) {
+        set_error("%s: null pointer argument", who);
+        return nullptr;
+    }
+    if (!ensure_pattern(a, Offsets, Columns, nnz)) return nullptr;
+    if (!a->pat.tiled || a->d != 32) {
+        set_error("%s: strided heads are read in place only by the tile kernels for emb_dim 32 (pattern of aligned "
+                  "32x32 tiles); make the operands contiguous and use the row-major entry points", who);
+        return nullptr;
+    }
+    return a;
+}
+
+void sparse_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                            float* Out, const int* Offsets, const int* Columns, int nnz, int heads,
+                            const HeadLayout& in, const HeadLayout& out) {
+    const char* who = "attn_forward_strided";
+    SparseAttn* a = strided_handle(h, who, Offsets, Columns, nnz, heads);
+    if (!a) return;
+    if (a->has_mask != (Mask != nullptr)) {
+        set_error("%s: handle was created by the %s init", who, a->has_mask ? "mask" : "no-mask");
+        return;
+    }
+    if (!Q || !K || !V || !Attn || !Out) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Out)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!check_layout(who, "input", a, heads, in) || !check_layout(who, "output", a, heads, out)) return;
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = out;
+    ly.H = heads;
+    a->last_path = 1;
+    if (a->has_mask) launch_tile_fwd<32, true, true, true>(a, Q, K, V, Mask, Attn, Out, Offsets, nnz, ly);
+    else launch_tile_fwd<32, false, true, true>(a, Q, K, V, nullptr, Attn, Out, Offsets, nnz, ly);
+    check_launch("tile_fwd_kernel");
+}
+
+void sparse_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P, const float* Out,
+                             const float* dO, float* dQ, float* dK, float* dV, const int* Offsets, const int* Columns,
+                             int nnz, int heads, const HeadLayout& in, const HeadLayout& out, const HeadLayout& grad) {
+    const char* who = "attn_backward_strided";
+    SparseAttn* a = strided_handle(h, who, Offsets, Columns, nnz, heads);
+    if (!a) return;
+    if (!Q || !K || !V || !P || !Out || !dO || !dQ || !dK || !dV) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Out) || !aligned16(dO) || !aligned16(dQ) ||
+        !aligned16(dK) || !aligned16(dV)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!check_layout(who, "input", a, heads, in) || !check_layout(who, "output", a, heads, out) ||
+        !check_layout(who, "gradient", a, heads, grad))
+        return;
+    if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = grad;
+    ly.H = heads;
+    a->last_path = 1;
+    launch_tile_bwd<32, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);
+    check_launch("tile_bwd kernels");
 }
 
 // =================================================================================================

@@ -82,11 +82,11 @@ __device__ __forceinline__ void ldr_cols(rsrc_t r, int L, int voff, int soff, fl
 // B operand of a product over a tile's 32 rows from a row-major [.][D] head slice: slot (s, h) = tile row
 // acc_row(s, h).  voff = (4*(lane/32)*D + lane%32)*4, soff = byte offset of the tile's first row.
 template <int D>
-__device__ __forceinline__ void ldr_tile_b(rsrc_t r, int voff, int soff, float (&x)[D / 32][16]) {
+__device__ __forceinline__ void ldr_tile_b(rsrc_t r, int voff, int soff, float (&x)[D / 32][16], int ld = D) {
 #pragma unroll
     for (int c = 0; c < D / 32; ++c)
 #pragma unroll
-        for (int s = 0; s < 16; ++s) x[c][s] = ld1(r, voff, soff + ((8 * (s >> 2) + (s & 3)) * D + c * 32) * 4);
+        for (int s = 0; s < 16; ++s) x[c][s] = ld1(r, voff, soff + ((8 * (s >> 2) + (s & 3)) * ld + c * 32) * 4);
 }
 // 16 floats per lane laid out as 4 groups of 4 consecutive floats 8 apart (accumulator rows of one lane).
 __device__ __forceinline__ void ldr_4x4(rsrc_t r, int voff, int soff, float (&x)[16]) {
@@ -243,6 +243,35 @@ __device__ __forceinline__ void merge_max_sum(float& m, float& z, int w, int h, 
     }
 }
 
+// Where the [L][D] slice of head bh = b*H + hh of a [B][H][L][D] tensor lies when the tensor is a view of other
+// memory (the [B][L][H*D] output of a projection, say): element (b, hh, i, f) at b*bstride + hh*hstride + i*ld + f
+// floats.  One layout each for the inputs (Q, K, V), the outputs of the forward (Out, and dO with it) and the
+// gradients (dQ, dK, dV).
+struct HeadLayout {
+    long long bstride;
+    int hstride;
+    int ld;
+};
+struct Layouts {
+    HeadLayout in, out, grad;
+    int H;
+};
+// ST = false: the heads are contiguous [NB][L][D] slices and every figure below is a compile-time constant.
+template <bool ST, int D>
+__device__ __forceinline__ void head_slice(const HeadLayout& y, int H, int bh, int L, size_t& base, int& ld,
+                                           size_t& bytes) {
+    if constexpr (ST) {
+        const int b = bh / H, hh = bh - b * H;
+        base = (size_t)b * y.bstride + (size_t)hh * y.hstride;
+        ld = y.ld;
+        bytes = ((size_t)(L - 1) * y.ld + D) * 4;
+    } else {
+        base = (size_t)bh * L * D;
+        ld = D;
+        bytes = (size_t)L * D * 4;
+    }
+}
+
 // Work item -> (head, position in the strip order).  The heads are taken hc at a time; within such a group the
 // items walk the strip order (long strips first) with the group's heads innermost, so that all long strips of the
 // group start before any short one and the launch ends on short strips.  (Time stamps per work group on the north
@@ -285,12 +314,13 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // -------------------------------------------------------------------------------------------------
 // KROW: the K operand is row-major [NB][L][D] (what a caller has before it makes the transposed copy the
 // reference's ABI asks for) instead of feature-major [NB][D][L]; d = 32 only.
-template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false>
+template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
     const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
-    int NB, int nnz, float scale, int s0, int ns, int hc) {
+    int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
+    static_assert(!ST || (KROW && D == 32), "strided heads: row-major operands, d = 32");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
@@ -303,14 +333,18 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(Kt + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, hbytes, obytes;
+    int ild, old_;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, hbytes), rK = make_rsrc(Kt + ib, hbytes), rV = make_rsrc(V + ib, hbytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int p_base = offs[I * 32] * 4;
     const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
-    const int b_voff = (4 * h * D + li) * 4;
+    const int b_voff = (4 * h * ild + li) * 4;
     const int m_voff = 16 * h;
     float* T = lds_t[w];
     // P tile t of this block row: transpose to the col-owner layout and store full rows
@@ -323,12 +357,12 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float c2 = scale * LOG2E;
 
     float q[KH];
-    ldr_rows<D>(rQ, (li * D + h * KH) * 4, I * 32 * D * 4, q);
+    ldr_rows<D>(rQ, (li * ild + h * KH) * 4, I * 32 * ild * 4, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
     // operand over the head dimension of key tile J (lane = key, features h*D/2 ..)
     auto load_kf = [&](int J, float (&x)[KH]) {
-        if constexpr (KROW) ldr_rows<D>(rK, (li * D + h * KH) * 4, J * 32 * D * 4, x);
+        if constexpr (KROW) ldr_rows<D>(rK, (li * ild + h * KH) * 4, J * 32 * ild * 4, x);
         else ldr_cols<D>(rK, L, col_voff, J * 128, x);
     };
 
@@ -360,9 +394,9 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
         constexpr bool LIN = D == 32;
         float* Tx = T + 32 * TS;  // K^T tile, later V tile (LIN only)
         // a K tile is 32 features x 32 keys with rows L floats apart, or (KROW) 32 keys x 32 features, contiguous
-        constexpr int KSTEP = KROW ? 32 * D * 4 : 128;
-        const int kld = KROW ? D : L;
-        const int klin = lin_voff(l, kld), vlin = lin_voff(l, D), plin = lin_voff(l, rn);
+        const int KSTEP = KROW ? 32 * ild * 4 : 128;
+        const int kld = KROW ? ild : L;
+        const int klin = lin_voff(l, kld), vlin = lin_voff(l, ild), plin = lin_voff(l, rn);
         if constexpr (LIN) {
             f32x4 kraw[2][4];
             if (nu > 0) ldr_tile_lin(rK, klin, Js[0] * KSTEP, kld, kraw[0]);
@@ -429,12 +463,12 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
 
         if constexpr (LIN) {
             f32x4 vraw[2][4];
-            if (nu > 0) ldr_tile_lin(rV, vlin, Js[0] * 32 * D * 4, D, vraw[0]);
+            if (nu > 0) ldr_tile_lin(rV, vlin, Js[0] * 32 * ild * 4, ild, vraw[0]);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
                     const int t = w + u * WAVES;
-                    if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, D, vraw[(u + 1) & 1]);
+                    if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, Js[u + 1 < MAXT ? u + 1 : u] * 32 * ild * 4, ild, vraw[(u + 1) & 1]);
                     lds_put_lin(Tx, l, vraw[u & 1]);
                     float p[16], vb[1][16];
 #pragma unroll
@@ -450,12 +484,12 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
             }
         } else {
             float vbuf[2][D / 32][16];
-            if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * D * 4, vbuf[0]);
+            if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * ild * 4, vbuf[0], ild);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
                     const int t = w + u * WAVES;
-                    if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * D * 4, vbuf[(u + 1) & 1]);
+                    if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * ild * 4, vbuf[(u + 1) & 1], ild);
                     float p[16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
@@ -511,7 +545,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                 nu, xa, xb,
                 [&](PreKV& x, int i) {
                     fetch_k(x.k, i);
-                    ldr_tile_b<D>(rV, b_voff, tcol[t0 + w + min(i, nu - 1) * WAVES] * 32 * D * 4, x.vb);
+                    ldr_tile_b<D>(rV, b_voff, tcol[t0 + w + min(i, nu - 1) * WAVES] * 32 * ild * 4, x.vb, ild);
                 },
                 [&](PreKV& c, int i) {
                     f32x16 s = mma_feat_init<D>(c.k.k, q, init_of(c.k, m));
@@ -523,8 +557,8 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                 });
         }
     }
-    if (Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);
-    else reduce_store<D, WAVES>(o, O + hb, I * 32, w, li, h, lds);
+    if (!ST && Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);
+    else reduce_store<D, WAVES>(o, O + ob, I * 32, w, li, h, lds, old_);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -534,12 +568,13 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
 // the 32 x d result.  G receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------
 // VROW: the V operand is row-major [NB][L][D] instead of feature-major [NB][D][L]; d = 32 only.
-template <int D, int WAVES, bool HAVE_O, bool VROW = false>
+template <int D, int WAVES, bool HAVE_O, bool VROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
     float* __restrict__ dQ, const int* __restrict__ trp, const int* __restrict__ tcol,
-    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale, int hc) {
+    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
+    static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, d = 32, Out given");
     static_assert(!VROW || D == 32, "row-major V operand: d = 32 only");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
@@ -555,14 +590,18 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
     const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes), rdO = make_rsrc(dO + ob, obytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const int p_base = offs[I * 32] * 4;
     const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
-    const int b_voff = (4 * h * D + li) * 4;
-    const int r_voff = (li * D + h * KH) * 4;
+    const int b_voff = (4 * h * ild + li) * 4;
+    const int r_voff = (li * ild + h * KH) * 4, ro_voff = (li * old_ + h * KH) * 4;
     float* T = lds_t[w];
     // P tile as loaded (col owner) -> row-owner layout, the one dP^T comes in
     auto p_rows = [&](const float (&pc)[16], float (&pr)[16]) {
@@ -571,12 +610,12 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     };
 
     float go[KH];
-    ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, go);
+    ldr_rows<D>(rdO, ro_voff, I * 32 * old_ * 4, go);
 
     float g = 0.f;
     if (HAVE_O) {
         float oo[KH];
-        ldr_rows<D>(make_rsrc(Ocache + hb, hbytes), r_voff, I * 32 * D * 4, oo);
+        ldr_rows<D>(make_rsrc(Ocache + ob, obytes), ro_voff, I * 32 * old_ * 4, oo);
 #pragma unroll
         for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
         g += __shfl_xor(g, 32, 64);
@@ -590,7 +629,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             nu, xa, xb,
             [&](PreG& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
-                if constexpr (VROW) ldr_rows<D>(rV, r_voff, tcol[t0 + t] * 32 * D * 4, x.vt);
+                if constexpr (VROW) ldr_rows<D>(rV, r_voff, tcol[t0 + t] * 32 * ild * 4, x.vt);
                 else ldr_cols<D>(rV, L, col_voff, tcol[t0 + t] * 128, x.vt);
                 ldr_tile_cols(rP, pc_voff, p_base + t * 128, rn, x.pv);
             },
@@ -625,9 +664,9 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
         float* Tv = T;
         float* Tp = T + 32 * TS;
         float* Tk = T + 64 * TS;
-        constexpr int VSTEP = VROW ? 32 * D * 4 : 128;
-        const int vld = VROW ? D : L;
-        const int vl = lin_voff(l, vld), pl = lin_voff(l, rn), kl = lin_voff(l, D);
+        const int VSTEP = VROW ? 32 * ild * 4 : 128;
+        const int vld = VROW ? ild : L;
+        const int vl = lin_voff(l, vld), pl = lin_voff(l, rn), kl = lin_voff(l, ild);
         Pre xa, xb;
         tile_pipeline(
             nu, xa, xb,
@@ -637,7 +676,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
                 ldr_tile_lin(rV, vl, J * VSTEP, vld, x.vt);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) x.pv[i] = ld4_nt(rP, pl, p_base + t * 128 + 32 * i * rn);
-                ldr_tile_lin(rK, kl, J * 32 * D * 4, D, x.kb);
+                ldr_tile_lin(rK, kl, J * 32 * ild * 4, ild, x.kb);
             },
             [&](Pre& c, int) {
                 lds_put_lin(Tv, l, c.vt);
@@ -694,7 +733,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     }
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
-    reduce_store<D, WAVES>(acc, dQ + hb, I * 32, w, li, h, lds);
+    reduce_store<D, WAVES>(acc, dQ + gb, I * 32, w, li, h, lds, gld);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -703,12 +742,13 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
 // started from the stored -g, the 1/sqrt(d) of dK is applied to the 32 x d result.
 // -------------------------------------------------------------------------------------------------
 // VROW: as in the row pass.
-template <int D, int WAVES, bool VROW = false>
+template <int D, int WAVES, bool VROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
     const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
-    int hc) {
+    int hc, Layouts ly) {
+    static_assert(!ST || VROW, "strided heads: row-major operands, d = 32");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
@@ -718,15 +758,19 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const int J = tcp[nbr + 1 + pos];  // strips longest first
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes), rdO = make_rsrc(dO + hb, hbytes);
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes), rdO = make_rsrc(dO + ob, obytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
-    const int b_voff = (4 * h * D + li) * 4;
-    const int r_voff = (li * D + h * KH) * 4;
+    const int b_voff = (4 * h * ild + li) * 4, bo_voff = (4 * h * old_ + li) * 4;
+    const int r_voff = (li * ild + h * KH) * 4, ro_voff = (li * old_ + h * KH) * 4;
 
     float vt[KH];
-    if constexpr (VROW) ldr_rows<D>(rV, r_voff, J * 32 * D * 4, vt);
+    if constexpr (VROW) ldr_rows<D>(rV, r_voff, J * 32 * ild * 4, vt);
     else ldr_cols<D>(rV, L, (h * KH * L + li) * 4, J * 128, vt);
 
     f32x16 ak[D / 32], av[D / 32];
@@ -759,21 +803,21 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
             const int4 d = desc[w + min(i, nu - 1) * WAVES];
             const int I = d.x, rn = d.z;
             x.I = I;
-            if constexpr (!DEEP) ldr_rows<D>(rdO, r_voff, I * 32 * D * 4, x.go);
+            if constexpr (!DEEP) ldr_rows<D>(rdO, ro_voff, I * 32 * old_ * 4, x.go);
             const int pv = (4 * h * rn + li) * 4;
 #pragma unroll
             for (int r = 0; r < 16; ++r) x.p[r] = ld1_nt(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
             ldr_4x4(rG, 16 * h, I * 128, x.gneg);
             if constexpr (DEEP) {
-                ldr_tile_b<D>(rQ, b_voff, I * 32 * D * 4, x.qb);
-                ldr_tile_b<D>(rdO, b_voff, I * 32 * D * 4, x.ob);
+                ldr_tile_b<D>(rQ, b_voff, I * 32 * ild * 4, x.qb, ild);
+                ldr_tile_b<D>(rdO, bo_voff, I * 32 * old_ * 4, x.ob, old_);
             }
         },
         [&](Pre& c, int) {
             float qb2[D / 32][16], ob2[D / 32][16];
             if constexpr (!DEEP) {
-                ldr_tile_b<D>(rQ, b_voff, c.I * 32 * D * 4, qb2);
-                ldr_tile_b<D>(rdO, b_voff, c.I * 32 * D * 4, ob2);
+                ldr_tile_b<D>(rQ, b_voff, c.I * 32 * ild * 4, qb2, ild);
+                ldr_tile_b<D>(rdO, bo_voff, c.I * 32 * old_ * 4, ob2, old_);
             }
             f32x16 init;
 #pragma unroll
@@ -800,9 +844,9 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
         });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
-    reduce_store<D, WAVES>(ak, dK + hb, J * 32, w, li, h, lds);
+    reduce_store<D, WAVES>(ak, dK + gb, J * 32, w, li, h, lds, gld);
     if (WAVES > 1) __syncthreads();
-    reduce_store<D, WAVES>(av, dV + hb, J * 32, w, li, h, lds);
+    reduce_store<D, WAVES>(av, dV + gb, J * 32, w, li, h, lds, gld);
 }
 
 }  // namespace spion

@@ -121,7 +121,7 @@ __device__ __forceinline__ void reduce_store(f32x16 (&acc)[D / 32], float* __res
     constexpr int NC = D / 32;
     auto addr = [&](int c, int r) -> size_t {
         return TRANS ? (size_t)(c * 32 + acc_row(r, h)) * ld + row0 + li
-                     : (size_t)(row0 + acc_row(r, h)) * D + c * 32 + li;
+                     : (size_t)(row0 + acc_row(r, h)) * ld + c * 32 + li;
     };
     if (WAVES == 1) {
 #pragma unroll

@@ -114,6 +114,32 @@ class SparseABI:
         _lib.check_error("spion_attn_backward_rowmajor")
         return dQ, dK, dV
 
+    def forward_strided(self, q, k, v, out, penalty=None):
+        """q, k, v, out: [B, H, L, d] views (any strides the library takes), read and written in place.  Returns P."""
+        import ctypes
+        P = torch.full((self.NB * max(self.nnz, 1),), float("nan"), device=self.dev)
+        lin, lout = _lib.head_layout(q), _lib.head_layout(out)
+        assert lin is not None and lout is not None
+        assert k.stride() == q.stride() and v.stride() == q.stride()
+        _lib.core().spion_attn_forward_strided(
+            self.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), penalty.data_ptr() if penalty is not None else None,
+            P.data_ptr(), out.data_ptr(), self.offsets.data_ptr(), self.columns.data_ptr(), self.sum_mat.data_ptr(),
+            self.nnz, q.shape[1], ctypes.addressof(lin), ctypes.addressof(lout))
+        _lib.check_error("spion_attn_forward_strided")
+        return P[: self.NB * self.nnz].view(self.NB, self.nnz)
+
+    def backward_strided(self, q, k, v, P, out, dout, dq, dk, dv):
+        import ctypes
+        lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+        assert lin is not None and lout is not None and lgrad is not None
+        assert dout.stride() == out.stride() and dk.stride() == dq.stride() and dv.stride() == dq.stride()
+        _lib.core().spion_attn_backward_strided(
+            self.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), P.contiguous().data_ptr(), out.data_ptr(),
+            dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), self.offsets.data_ptr(),
+            self.columns.data_ptr(), self.sum_mat.data_ptr(), self.nnz, q.shape[1], ctypes.addressof(lin),
+            ctypes.addressof(lout), ctypes.addressof(lgrad))
+        _lib.check_error("spion_attn_backward_strided")
+
     def last_path(self):
         return _lib.core().spion_last_path(self.handle)
 

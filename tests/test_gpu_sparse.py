@@ -412,6 +412,108 @@ def test_rowmajor_entry_points_match_oracle(kind, d, with_mask):
     abi.close()
 
 
+def _head_views(B, H, L, d, layout, n, seed, fill=None):
+    """n tensors seen as [B, H, L, d], in memory as the layer has them: "proj": each a [B, L, H*d] projection;
+    "fused": slices of one [B, L, n, H, d+4] buffer (one GEMM for all, padded rows); "plain": contiguous."""
+    g = torch.Generator().manual_seed(seed)
+    if layout == "plain":
+        bufs = [torch.randn(B, H, L, d, generator=g).cuda() for _ in range(n)]
+        views = bufs
+    elif layout == "proj":
+        bufs = [torch.randn(B, L, H * d, generator=g).cuda() for _ in range(n)]
+        views = [b.view(B, L, H, d).transpose(1, 2) for b in bufs]
+    else:
+        buf = torch.randn(B, L, n, H, d + 4, generator=g).cuda()
+        bufs = [buf]
+        views = [buf[:, :, i, :, :d].transpose(1, 2) for i in range(n)]
+    if fill is not None:
+        for b in bufs:
+            b.fill_(fill)
+    return bufs, views
+
+
+@pytest.mark.parametrize("layout,kind,with_mask", [("proj", "tile", False), ("fused", "tile", True), ("plain", "tile", False),
+                                                   ("proj", "tile_rows", False), ("fused", "many_rows", False)])
+def test_strided_entry_points(layout, kind, with_mask):
+    """spion_attn_forward_strided / spion_attn_backward_strided: heads read and written in place in the memory of
+    [B, L, H*d] projections.  Same kernels, same arithmetic as the row-major entry points on contiguous copies:
+    bit-identical results; padding between the heads' rows is left alone."""
+    d, H, bs = 32, 2, 32
+    B, L = {"tile": (2, 256), "tile_rows": (1, 2048), "many_rows": (8, 4096)}[kind]
+    NB = B * H
+    mat = _random_block_mask(L // bs, 0.3 if kind != "many_rows" else 0.05, seed=7)
+    if kind == "tile_rows":
+        mat[3, :] = 1
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    _, (q, k, v) = _head_views(B, H, L, d, layout, 3, seed=41)
+    _, (dout,) = _head_views(B, H, L, d, "proj" if layout != "plain" else "plain", 1, seed=42)
+    obufs, (out,) = _head_views(B, H, L, d, "proj" if layout != "plain" else "plain", 1, seed=0, fill=float("nan"))
+    gbufs, (dq, dk, dv) = _head_views(B, H, L, d, layout, 3, seed=0, fill=-7.0)
+    pen = None
+    if with_mask:
+        valid = torch.tensor([L, L - 40, L // 2, L - 1][:NB])
+        pen = (1e6 * (torch.arange(L)[None, :] >= valid[:, None]).float()).contiguous().cuda()
+    P = abi.forward_strided(q, k, v, out, pen)
+    abi.backward_strided(q, k, v, P, out, dout, dq, dk, dv)
+    torch.cuda.synchronize()
+    assert abi.last_path() == 1
+    flat = lambda t: t.reshape(NB, L, d).contiguous()
+    Qc, Kc, Vc, dOc = flat(q), flat(k), flat(v), flat(dout)
+    O2, P2 = abi.forward_rowmajor(Qc, Kc, Vc, pen)
+    g2 = abi.backward_rowmajor(Qc, Kc, Vc, P2, O2, dOc)
+    torch.cuda.synchronize()
+    assert torch.equal(P, P2) and torch.equal(flat(out), O2)
+    for name, a, b in zip(("dQ", "dK", "dV"), (dq, dk, dv), g2):
+        assert torch.equal(flat(a), b), name
+    if layout == "fused":
+        assert (gbufs[0][..., d:] == -7.0).all(), "padding between the heads' rows was written"
+    if kind != "many_rows":
+        ref = oracle_fwd_bwd(Qc, Kc, Vc, dOc, sm, off, col, pen)
+        assert_close(P.cpu().numpy(), ref["P"], what=f"strided {layout} P")
+        assert_close(flat(out).cpu().numpy(), ref["O"], what=f"strided {layout} O")
+        for name, a in zip(("dQ", "dK", "dV"), (dq, dk, dv)):
+            assert_close(flat(a).cpu().numpy(), ref[name], what=f"strided {layout} {name}")
+    abi.close()
+
+
+def test_strided_entry_points_refuse_what_they_cannot_serve():
+    import ctypes
+    from spion_amd import _lib
+    L, bs, B, H = 128, 32, 1, 2
+    mat = _random_block_mask(L // bs, 0.5, seed=3)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+
+    def call(abi, q, out, heads=H, lin=None):
+        P = torch.zeros(abi.NB * abi.nnz, device="cuda")
+        lin = lin or _lib.head_layout(q)
+        lout = _lib.head_layout(out)
+        _lib.core().spion_attn_forward_strided(
+            abi.handle, q.data_ptr(), q.data_ptr(), q.data_ptr(), None, P.data_ptr(), out.data_ptr(),
+            abi.offsets.data_ptr(), abi.columns.data_ptr(), abi.sum_mat.data_ptr(), abi.nnz, heads,
+            ctypes.addressof(lin), ctypes.addressof(lout))
+
+    abi64 = SparseABI(64, L, B * H, bs, with_mask=False)
+    abi64.set_pattern(sm, off, col)
+    q64 = torch.zeros(B, H, L, 64, device="cuda")
+    call(abi64, q64, torch.zeros_like(q64))
+    with pytest.raises(RuntimeError, match="emb_dim 32"):
+        _lib.check_error("d=64")
+    abi64.close()
+    abi = SparseABI(32, L, B * H, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    q = torch.zeros(B, H, L, 32, device="cuda")
+    call(abi, q, torch.zeros_like(q), heads=3)
+    with pytest.raises(RuntimeError, match="does not divide"):
+        _lib.check_error("heads")
+    call(abi, q, torch.zeros_like(q), lin=_lib.HeadLayout(H * L * 32, L * 32, 30))
+    with pytest.raises(RuntimeError, match="multiples of 4"):
+        _lib.check_error("row stride")
+    assert _lib.head_layout(torch.zeros(B, H, L, 33, device="cuda")[..., 1:]) is None   # 4-byte offset
+    abi.close()
+
+
 @pytest.mark.parametrize("shape", [(3, 512, 32), (2, 256, 64), (2, 100, 32), (1, 70, 45), (4, 2, 1024, 32)])
 def test_library_transpose_is_exact(shape):
     from spion_amd import _lib
