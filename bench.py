@@ -568,6 +568,33 @@ def main():
     for t in (q, k, v):
         t.grad = None
     _lib.use_current_stream(module, dev)  # the capture left the handle on its own stream
+    # ---- the same step with the heads as the layer hands them over: views of [B, L, H*d] projections ------
+    views = None
+    if getattr(module, "reads_views", False):
+        qv, kv, vv = (t.detach().transpose(1, 2).contiguous().transpose(1, 2).requires_grad_() for t in (q, k, v))
+        dov = do.transpose(1, 2).contiguous().transpose(1, 2)
+
+        def step_views():
+            for t in (qv, kv, vv):
+                t.grad = None
+            o, _ = module(qv, kv, vv, key_mask, mat)
+            o.backward(dov)
+
+        views = {}
+        for name, flag in (("in_place_ms", True), ("with_copies_ms", False)):
+            module.reads_views = flag
+            for _ in range(args.warmup):
+                step_views()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                step_views()
+            torch.cuda.synchronize()
+            views[name] = round(1e3 * (time.perf_counter() - t0) / args.steps, 4)
+        module.reads_views = True
+        views["what"] = ("module step on heads that are views of [B,L,H*d] projections: read and written in place "
+                         "by the strided entry points, against the reference's contiguous copies first")
+        del qv, kv, vv, dov
     # the module hands the forward's output to the backward itself; a caller of the reference's ABI cannot, so
     # the timings below run with the library's kept copies of Out, as such a caller would
     _lib.core().spion_use_output_cache(handle, 1)
@@ -685,6 +712,8 @@ def main():
                                "what": "the module's forward + backward recorded once as a HIP graph and replayed"}
     else:
         result["hip_graph"] = {"error": graph_ms}
+    if views:
+        result["projection_views"] = views
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(result))

@@ -9,6 +9,8 @@ only; the gradient of the returned probabilities is ignored, models/attention_bl
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 import torch.nn as nn
 
@@ -21,7 +23,13 @@ class _BlockAttnFunction(torch.autograd.Function):
     and of V for the backward because its ABI takes them that way, and its backward is not handed the forward's
     output.  Here every tensor stays row-major and autograd's saved ``out`` goes to the backward: the library's
     row-major entry points (spion_attn_forward_rowmajor / spion_attn_backward_rowmajor) take them as they are.
-    ``attn_cpp`` (the drop-in with the reference's four symbols) is still what created the handle."""
+    ``attn_cpp`` (the drop-in with the reference's four symbols) is still what created the handle.
+
+    The reference also starts with ``.contiguous()`` copies of query, key and value (models/attention_blockcuda.py:
+    36-48), which arrive as [B,H,L,d] views of [B,L,H*d] projections (models/attention.py:136-139).  For head
+    dimension 32 and block sizes that are multiples of 32 (the tile kernels) the strided entry points read the
+    views in place, write ``out`` in the same interleaved layout (so that combine_heads, models/attention.py:131-134,
+    is a view as well) and the gradients likewise: no copy on either side of the kernels."""
 
     @staticmethod
     def forward(ctx, query, key, value, mask, mat, module):
@@ -35,21 +43,38 @@ class _BlockAttnFunction(torch.autograd.Function):
                 f"({m.batch_size}, {m.num_heads}, {L}, {d})"
             )
         dev = query.device
-        q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+        shape = (m.batch_size, m.num_heads, L, d)
         p_flat = torch.empty(nb_ * idx.nnz, dtype=torch.float32, device=dev)
-        out = torch.empty((m.batch_size, m.num_heads, L, d), dtype=torch.float32, device=dev)
         pen_ptr = None
         if m.with_mask:
             pen = (1e6 * (1.0 - mask.repeat(1, m.num_heads))).to(torch.float32).contiguous()  # [B, H*L]
             pen_ptr = pen.data_ptr()
-        _lib.core().spion_attn_forward_rowmajor(m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
-                                                p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
-                                                idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
+        lay = None
+        if m.reads_views and not (query.is_contiguous() and key.is_contiguous() and value.is_contiguous()):
+            lay = _lib.head_layout(query)
+            if lay is None or key.stride() != query.stride() or value.stride() != query.stride() \
+                    or _lib.head_layout(key) is None or _lib.head_layout(value) is None:
+                lay = None
+        if lay is not None:
+            q, k, v = query, key, value
+            out = _empty_heads(shape, interleaved=query.stride(1) < query.stride(2), device=dev)
+            lout = _lib.head_layout(out)
+            _lib.core().spion_attn_forward_strided(
+                m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr, p_flat.data_ptr(), out.data_ptr(),
+                idx.offsets.data_ptr(), idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz, m.num_heads,
+                ctypes.addressof(lay), ctypes.addressof(lout))
+        else:
+            q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
+            out = torch.empty(shape, dtype=torch.float32, device=dev)
+            _lib.core().spion_attn_forward_rowmajor(m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
+                                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
+                                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
         _lib.check_error("attn_forward")
         ctx.save_for_backward(q, k, v, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
         ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
         ctx.nnz = idx.nnz
+        ctx.strided = lay is not None
         if m.with_mask:
             ctx.mark_non_differentiable(p_flat)
         return out, p_flat
@@ -63,10 +88,25 @@ class _BlockAttnFunction(torch.autograd.Function):
         n_total = m.num_batches * ctx.nnz
         if grad_output is None:  # only the probabilities were used downstream: their gradient is ignored
             grad_output = torch.zeros(m.batch_size, m.num_heads, m.seq_len, m.emb_dim, dtype=torch.float32, device=dev)
+        core = _lib.core()
+        if ctx.strided:
+            go = grad_output
+            if go.stride() != out.stride() or _lib.head_layout(go) is None:
+                go = torch.empty_like(out).copy_(grad_output)  # preserves out's strides
+            interleaved = q.stride(1) < q.stride(2)
+            shape = tuple(q.shape)
+            dq, dk, dv = (_empty_heads(shape, interleaved, dev) for _ in range(3))
+            lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+            core.spion_attn_backward_strided(
+                m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), p_flat.data_ptr(), out.data_ptr(),
+                go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), offsets.data_ptr(), columns.data_ptr(),
+                sum_mat.data_ptr(), ctx.nnz, m.num_heads, ctypes.addressof(lin), ctypes.addressof(lout),
+                ctypes.addressof(lgrad))
+            _lib.check_error("attn_backward")
+            return dq, dk, dv, None, None, None
         go = grad_output.contiguous()
         # Of the ABI's two [NB*nnz] scratch arguments (models/attention_blockcuda.py:83-84) the tile kernels use
         # neither and the element kernels only dS: nothing that size is allocated unless it is needed.
-        core = _lib.core()
         scratch_ds = None
         if core.spion_last_path(m.attn_handle) != 1:
             scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
@@ -80,6 +120,14 @@ class _BlockAttnFunction(torch.autograd.Function):
             offsets.data_ptr(), columns.data_ptr(), sum_mat.data_ptr(), ctx.nnz)
         _lib.check_error("attn_backward")
         return dq, dk, dv, None, None, None
+
+
+def _empty_heads(shape, interleaved, device):
+    """Uninitialised [B,H,L,d] tensor; ``interleaved``: in memory [B,L,H,d], i.e. [B,L,H*d] once the heads are merged."""
+    B, H, L, d = shape
+    if interleaved:
+        return torch.empty((B, L, H, d), dtype=torch.float32, device=device).transpose(1, 2)
+    return torch.empty(shape, dtype=torch.float32, device=device)
 
 
 class _BlockAttentionBase(nn.Module):
@@ -104,6 +152,8 @@ class _BlockAttentionBase(nn.Module):
         self.csr_cache = CsrCache()
         self.attn_func = _BlockAttnFunction
         _lib.core().spion_use_output_cache(attn_handle, 0)  # the backward is handed the output instead
+        # block masks whose blocks are unions of 32x32 tiles run on the tile kernels; those for d = 32 take views
+        self.reads_views = self.emb_dim == 32 and self.block_size % 32 == 0 and self.seq_len % 32 == 0
 
 
 class CUDABlockAttention(_BlockAttentionBase):

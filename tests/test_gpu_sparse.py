@@ -319,6 +319,58 @@ def test_block_modules_autograd_match_dense_statement(with_mask):
         assert_close(a.grad.cpu().numpy() / 2.0, b.grad.numpy(), what=f"module {name}")  # two backward passes accumulated
 
 
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_block_modules_read_projection_views_in_place(with_mask):
+    """Heads handed over as views of [B, L, H*d] projections (what models/attention.py:136-139 makes): the module
+    takes them without copies, returns ``out`` in the same interleaved memory, and every result equals, bit for bit,
+    what it returns for contiguous copies of the same tensors."""
+    import spion_amd
+
+    B, H, L, d, bs = 2, 2, 256, 32, 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    mat_np = _random_block_mask(L // bs, 0.3, seed=5)
+    mat = torch.from_numpy(mat_np).cuda()
+    if with_mask:
+        cpp = spion_amd.Attention._blockcuda_mask_compile_module()
+        mod = spion_amd.CUDABlockMaskAttention(cfg, cpp, cpp.init(d, L, B * H, bs))
+    else:
+        cpp = spion_amd.Attention._blockcuda_compile_module()
+        mod = spion_amd.CUDABlockAttention(cfg, cpp, cpp.init(d, L, B * H, bs))
+    assert mod.reads_views
+    g = torch.Generator().manual_seed(11)
+    proj = [torch.randn(B, L, H * d, generator=g).cuda().requires_grad_() for _ in range(3)]
+    dmerged = torch.randn(B, L, H * d, generator=g).cuda()
+    key_mask = torch.ones(B, L)
+    if with_mask:
+        key_mask[1, 77:] = 0
+    key_mask = key_mask.cuda()
+    split = lambda x: x.view(B, L, H, d).transpose(1, 2)
+    # (a) views in, merged output out
+    out_v, _ = mod(*(split(x) for x in proj), key_mask, mat)
+    assert out_v.transpose(1, 2).is_contiguous()           # [B, L, H, d] memory: merging the heads is a view
+    merged = out_v.transpose(1, 2).reshape(B, L, H * d)
+    assert merged.data_ptr() == out_v.data_ptr()
+    merged.backward(dmerged)
+    grads_v = [x.grad.clone() for x in proj]
+    for x in proj:
+        x.grad = None
+    # (b) contiguous copies in
+    out_c, _ = mod(*(split(x).contiguous() for x in proj), key_mask, mat)
+    assert out_c.is_contiguous()
+    out_c.transpose(1, 2).reshape(B, L, H * d).backward(dmerged)
+    assert torch.equal(out_v, out_c)
+    for a, x in zip(grads_v, proj):
+        assert torch.equal(a, x.grad)
+    # and against the float64 model of the layer
+    qc, kc, vc = (split(x.detach().double().cpu()).requires_grad_() for x in proj)
+    pat = torch.from_numpy(np.repeat(np.repeat(mat_np, bs, 0), bs, 1)).double()
+    O, _ = osa.dense_masked_attention(qc, kc, vc, pat, key_mask.double().cpu() if with_mask else None)
+    O.backward(split(dmerged.double().cpu()))
+    assert_close(out_v.detach().cpu().numpy(), O.detach().numpy(), what="views: out")
+    for name, a, b in zip(("dq", "dk", "dv"), grads_v, (qc, kc, vc)):
+        assert_close(split(a).cpu().numpy(), b.grad.numpy(), what=f"views: {name}")
+
+
 # ---------------------------------------------------------------------------------- error handling (host side)
 def test_inconsistent_csr_is_reported_not_launched():
     from spion_amd import _lib
