@@ -259,6 +259,22 @@ void spion_attn_backward_strided(void* handle, const float* Q, const float* K, c
                                  int heads, const spion_head_layout* in, const spion_head_layout* out,
                                  const spion_head_layout* grad);
 
+/* The dense phase on the same views: the reference's dense modules transpose Q and V before the forward and K
+ * and grad_output before the backward (models/attention_cuda.py:22-31,52-62) because its GEMM calls
+ * (models/attn.cu:179-262) take feature-major operands, and hand Out and the gradients back feature-major.
+ * Here Q, K, V, Out, dO, dQ, dK, dV are all [B][H][L][d] views described as above (a contiguous [NB][L][d]
+ * tensor is the layout {H*L*d, L*d, d}); Attn / P is the same [NB][key][query] map as in attn_forward.  Mask:
+ * NULL for a handle of spion_dense_init, the [NB][L] penalty for one of spion_densemask_init.  emb_dim 32 and
+ * seq_len <= 16384 only.  No copy of Out is kept: the backward takes Out (required). */
+void spion_dense_forward_strided(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
+                                 float* Attn, float* Out,
+                                 int heads, const spion_head_layout* in, const spion_head_layout* out);
+void spion_dense_backward_strided(void* handle, const float* Q, const float* K, const float* V, const float* P,
+                                  const float* Out, const float* dO,
+                                  float* dQ, float* dK, float* dV,
+                                  int heads, const spion_head_layout* in, const spion_head_layout* out,
+                                  const spion_head_layout* grad);
+
 /* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
  * attention entry points take.  Returns 0 on success. */
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream);

@@ -38,6 +38,10 @@ void sparse_forward_strided(void*, const float*, const float*, const float*, con
 void sparse_backward_strided(void*, const float*, const float*, const float*, const float*, const float*, const float*,
                              float*, float*, float*, const int*, const int*, int, int, const HeadLayout&,
                              const HeadLayout&, const HeadLayout&);
+void dense_forward_strided(void*, const float*, const float*, const float*, const float*, float*, float*, int,
+                           const HeadLayout&, const HeadLayout&);
+void dense_backward_strided(void*, const float*, const float*, const float*, const float*, const float*, const float*,
+                            float*, float*, float*, int, const HeadLayout&, const HeadLayout&, const HeadLayout&);
 void sparse_invalidate(void*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
@@ -228,6 +232,24 @@ void spion_attn_backward_strided(void* h, const float* Q, const float* K, const 
     }
     sparse_backward_strided(h, Q, K, V, P, Out, dO, dQ, dK, dV, Offsets, Columns, nnz, heads, to_layout(in),
                             to_layout(out), to_layout(grad));
+}
+void spion_dense_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                                 float* Out, int heads, const spion_head_layout* in, const spion_head_layout* out) {
+    if (!in || !out) {
+        set_error("dense attn_forward_strided: null layout argument");
+        return;
+    }
+    dense_forward_strided(h, Q, K, V, Mask, Attn, Out, heads, to_layout(in), to_layout(out));
+}
+void spion_dense_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P,
+                                  const float* Out, const float* dO, float* dQ, float* dK, float* dV, int heads,
+                                  const spion_head_layout* in, const spion_head_layout* out,
+                                  const spion_head_layout* grad) {
+    if (!in || !out || !grad) {
+        set_error("dense attn_backward_strided: null layout argument");
+        return;
+    }
+    dense_backward_strided(h, Q, K, V, P, Out, dO, dQ, dK, dV, heads, to_layout(in), to_layout(out), to_layout(grad));
 }
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
     return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));

@@ -103,11 +103,13 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
 // share of the strip (at most 8) in registers, so a tile costs one QK^T chain and one PV chain instead of the
 // two-sweep kernel's three; K, V^T and map tiles move as four 16-byte instructions each and change layout in
 // wave-private LDS tiles; the map is written non-temporally.
-template <bool MASK>
+// RM: Q, V and Out are row-major head slices located by `ly` (heads possibly interleaved in [B][L][H*32] memory,
+// tile_kernels.h) instead of the feature-major [NB][32][L] operands of the reference's ABI; K likewise.
+template <bool MASK, bool RM = false>
 SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
-    int L, int nbr, int NB, float scale) {
+    int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16, WAVES = 4, MAXT = 8;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
@@ -116,17 +118,23 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w+4, ... of this wavefront
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes);
+    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, hbytes, obytes;
+    int ild, old_;
+    head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes);
     const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     float* T = lds_t[w];         // map tile on its way to memory
     float* Tx = T + 32 * TS;     // K tile, later V^T tile
-    const int klin = lin_voff(l, D), vlin = lin_voff(l, L);
+    const int klin = lin_voff(l, ild), alin = lin_voff(l, L);
+    const int vld = RM ? ild : L, vlin = lin_voff(l, vld), VSTEP = RM ? 32 * ild * 4 : 128;
     const float c2 = scale * LOG2E;
 
     float q[KH];
-    ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
+    if constexpr (RM) ldr_rows<D>(rQ, (li * ild + h * KH) * 4, I * 32 * ild * 4, q);
+    else ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
     auto chain_init = [&](int J) -> f32x16 {  // minus the key penalties of the tile, log2 domain
@@ -143,12 +151,12 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     f32x16 S[MAXT];
     {
         f32x4 kraw[2][4];
-        if (nu > 0) ldr_tile_lin(rK, klin, w * 32 * D * 4, D, kraw[0]);
+        if (nu > 0) ldr_tile_lin(rK, klin, w * 32 * ild * 4, ild, kraw[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int J = w + u * WAVES;
-                if (u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * D * 4, D, kraw[(u + 1) & 1]);
+                if (u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * ild * 4, ild, kraw[(u + 1) & 1]);
                 lds_put_lin(Tx, l, kraw[u & 1]);
                 float kf[KH];
                 lds_get_feat32(Tx, li, h, kf);
@@ -192,26 +200,31 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     f32x16 o[1] = {splat16(0.f)};  // O^T: register = feature, lane = query
     {
         f32x4 vraw[2][4];
-        if (nu > 0) ldr_tile_lin(rV, vlin, w * 128, L, vraw[0]);
+        if (nu > 0) ldr_tile_lin(rV, vlin, w * VSTEP, vld, vraw[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int J = w + u * WAVES;
-                if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * 128, L, vraw[(u + 1) & 1]);
+                if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * VSTEP, vld, vraw[(u + 1) & 1]);
                 lds_put_lin(Tx, l, vraw[u & 1]);
                 float p[16], vb[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
                 lds_put_cols(T, li, h, p);        // T[key][query]: the map is stored key-major
-                lds_get_rows(Tx, li, h, vb);      // vb[s] = V[key acc_row(s, h)][feature li]
+                if constexpr (RM) lds_get_cols(Tx, li, h, vb);  // vb[s] = V[key acc_row(s, h)][feature li]
+                else lds_get_rows(Tx, li, h, vb);
                 f32x4 pl[4];
                 lds_get_lin(T, l, pl);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
-                str_tile_lin(rA, vlin, (J * 32 * L + I * 32) * 4, L, pl);
+                str_tile_lin(rA, alin, (J * 32 * L + I * 32) * 4, L, pl);
             }
         }
+    }
+    if constexpr (RM) {
+        reduce_store_rows<WAVES>(o[0], Out + ob, I * 32, w, li, h, lds, old_);
+        return;
     }
     reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
     if (OutCopy) {
@@ -226,11 +239,11 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
 // accumulates O^T.  Tiles are fetched linearly one tile ahead and re-laid out in wave-private LDS tiles, as in
 // the kernels above.  48 MFMA per tile against the 32 of the register-resident kernel, which is why that one is
 // used whenever a strip's logits fit in the registers of four wavefronts.
-template <bool MASK>
+template <bool MASK, bool RM = false>
 SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
-    int L, int nbr, int NB, float scale) {
+    int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16, WAVES = 4;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
@@ -239,18 +252,24 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(Vt + hb, hbytes);
+    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, hbytes, obytes;
+    int ild, old_;
+    head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes);
     const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     float* T = lds_t[w];          // map tile on its way to memory
     float* Tk = T + 32 * TS;
     float* Tv = T + 64 * TS;
-    const int klin = lin_voff(l, D), vlin = lin_voff(l, L);
+    const int klin = lin_voff(l, ild), alin = lin_voff(l, L);
+    const int vld = RM ? ild : L, vlin = lin_voff(l, vld), VSTEP = RM ? 32 * ild * 4 : 128;
     const float c2 = scale * LOG2E;
 
     float q[KH];
-    ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
+    if constexpr (RM) ldr_rows<D>(rQ, (li * ild + h * KH) * 4, I * 32 * ild * 4, q);
+    else ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
 
@@ -279,7 +298,7 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
             nu, xa, xb,
             [&](Pre1& x, int i) {
                 const int J = w + min(i, nu - 1) * WAVES;
-                ldr_tile_lin(rK, klin, J * 32 * D * 4, D, x.k);
+                ldr_tile_lin(rK, klin, J * 32 * ild * 4, ild, x.k);
                 penalties(x.pj, J);
             },
             [&](Pre1& c, int) {
@@ -330,8 +349,8 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
             nu, xa, xb,
             [&](Pre2& x, int i) {
                 const int J = w + min(i, nu - 1) * WAVES;
-                ldr_tile_lin(rK, klin, J * 32 * D * 4, D, x.k);
-                ldr_tile_lin(rV, vlin, J * 128, L, x.v);
+                ldr_tile_lin(rK, klin, J * 32 * ild * 4, ild, x.k);
+                ldr_tile_lin(rV, vlin, J * VSTEP, vld, x.v);
                 penalties(x.pj, J);
             },
             [&](Pre2& c, int i) {
@@ -340,7 +359,8 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
                 lds_put_lin(Tv, l, c.v);
                 float kf[KH], vb[16];
                 lds_get_feat32(Tk, li, h, kf);
-                lds_get_rows(Tv, li, h, vb);  // V[key acc_row(s, h)][feature li]
+                if constexpr (RM) lds_get_cols(Tv, li, h, vb);  // V[key acc_row(s, h)][feature li]
+                else lds_get_rows(Tv, li, h, vb);
                 __builtin_amdgcn_sched_barrier(0);
                 f32x16 init = minus_m;
                 if constexpr (MASK) {
@@ -356,8 +376,12 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
                 lds_get_lin(T, l, pl);
 #pragma unroll
                 for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
-                str_tile_lin(rA, vlin, (J * 32 * L + I * 32) * 4, L, pl);
+                str_tile_lin(rA, alin, (J * 32 * L + I * 32) * 4, L, pl);
             });
+    }
+    if constexpr (RM) {
+        reduce_store_rows<WAVES>(o[0], Out + ob, I * 32, w, li, h, lds, old_);
+        return;
     }
     reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
     if (OutCopy) {
@@ -482,11 +506,12 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_col_kernel(
 // on the dense layouts.  Every operand tile -- V, K^T, Q^T, dO^T and the key-major map tile -- is fetched as four
 // 16-byte instructions one tile ahead and turned into MFMA operands through wave-private LDS copies; -g enters as
 // the initial accumulator of the dP chain; the 1/sqrt(d) is applied to the 32 x d results.
-template <int WAVES>
+// RM: K, dO, Out (OutCopy) and dQ are row-major head slices located by `ly`, V as well.
+template <int WAVES, bool RM = false>
 SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     const float* __restrict__ Kt, const float* __restrict__ V, const float* __restrict__ Attn,
     const float* __restrict__ dOt, const float* __restrict__ OutCopy, float* __restrict__ G,
-    float* __restrict__ dQ, int L, int nbr, int NB, float scale) {
+    float* __restrict__ dQ, int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS];
@@ -495,16 +520,26 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     const int bh = NB - 1 - item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rK = make_rsrc(Kt + hb, hbytes), rV = make_rsrc(V + hb, hbytes), rdO = make_rsrc(dOt + hb, hbytes);
+    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<RM, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rK = make_rsrc(Kt + ib, hbytes), rV = make_rsrc(V + ib, hbytes), rdO = make_rsrc(dOt + ob, obytes);
     const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
     float* Tv = lds_t[w];
     float* Tp = Tv + 32 * TS;
     float* Tk = Tv + 64 * TS;
 
     float go[KH], oo[KH];
-    ldr_cols<D>(rdO, L, (h * KH * L + li) * 4, I * 128, go);
-    ldr_cols<D>(make_rsrc(OutCopy + hb, hbytes), L, (h * KH * L + li) * 4, I * 128, oo);
+    if constexpr (RM) {
+        ldr_rows<D>(rdO, (li * old_ + h * KH) * 4, I * 32 * old_ * 4, go);
+        ldr_rows<D>(make_rsrc(OutCopy + ob, obytes), (li * old_ + h * KH) * 4, I * 32 * old_ * 4, oo);
+    } else {
+        ldr_cols<D>(rdO, L, (h * KH * L + li) * 4, I * 128, go);
+        ldr_cols<D>(make_rsrc(OutCopy + hb, hbytes), L, (h * KH * L + li) * 4, I * 128, oo);
+    }
     float g = 0.f;
 #pragma unroll
     for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
@@ -516,16 +551,17 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     struct Pre {
         f32x4 v[4], p[4], k[4];
     };
-    const int vl = lin_voff(l, D), ll = lin_voff(l, L);
+    const int vl = lin_voff(l, ild), ll = lin_voff(l, L);
+    const int kld = RM ? ild : L, kl = lin_voff(l, kld), KSTEP = RM ? 32 * ild * 4 : 128;
     Pre xa, xb;
     tile_pipeline(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int J = w + min(i, nu - 1) * WAVES;
-            ldr_tile_lin(rV, vl, J * 32 * D * 4, D, x.v);
+            ldr_tile_lin(rV, vl, J * 32 * ild * 4, ild, x.v);
 #pragma unroll
             for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
-            ldr_tile_lin(rK, ll, J * 128, L, x.k);
+            ldr_tile_lin(rK, kl, J * KSTEP, kld, x.k);
         },
         [&](Pre& c, int) {
             lds_put_lin(Tv, l, c.v);
@@ -534,7 +570,8 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
             float vt[16], pr[16], kb[16];
             lds_get_feat32(Tv, li, h, vt);  // V[key li][feature 16h + s]
             lds_get_cols(Tp, li, h, pr);    // P[query li][key acc_row(r, h)]
-            lds_get_rows(Tk, li, h, kb);    // K^T[feature li][key acc_row(s, h)]
+            if constexpr (RM) lds_get_cols(Tk, li, h, kb);  // K^T[feature li][key acc_row(s, h)]
+            else lds_get_rows(Tk, li, h, kb);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // register = key, lane = query: dO_i . v_j - g_i
             float ds[16];
@@ -544,14 +581,15 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
             for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(kb[s], ds[s], acc, 0, 0, 0);
         });
     f32x16 out[1] = {acc * scale};
-    reduce_store<D, WAVES, true>(out, dQ + hb, I * 32, w, li, h, lds, L);
+    if constexpr (RM) reduce_store_rows<WAVES>(out[0], dQ + gb, I * 32, w, li, h, lds, gld);
+    else reduce_store<D, WAVES, true>(out, dQ + hb, I * 32, w, li, h, lds, L);
 }
 
-template <int WAVES>
+template <int WAVES, bool RM = false>
 SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     const float* __restrict__ Qt, const float* __restrict__ V, const float* __restrict__ Attn,
     const float* __restrict__ dOt, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
-    int L, int nbr, int NB, float scale) {
+    int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS + 32];
@@ -559,8 +597,13 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     const int bh = item / nbr, J = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 4;
-    const rsrc_t rQ = make_rsrc(Qt + hb, hbytes), rV = make_rsrc(V + hb, hbytes), rdO = make_rsrc(dOt + hb, hbytes);
+    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<RM, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rV = make_rsrc(V + ib, hbytes), rdO = make_rsrc(dOt + ob, obytes);
     const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
     const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
     float* To = lds_t[w];
@@ -569,7 +612,7 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     float* Tg = To + 96 * TS;
 
     float v[KH];
-    ldr_rows<D>(rV, (li * D + h * KH) * 4, J * 32 * D * 4, v);
+    ldr_rows<D>(rV, (li * ild + h * KH) * 4, J * 32 * ild * 4, v);
 
     f32x16 ak = splat16(0.f), av = splat16(0.f);  // dK^T, dV^T: register = feature, lane = key
     struct Pre {
@@ -577,15 +620,17 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
         float gneg;  // of query li; spread over the registers of dP through LDS
     };
     const int ll = lin_voff(l, L);
+    const int qld = RM ? ild : L, ql = lin_voff(l, qld), QSTEP = RM ? 32 * ild * 4 : 128;
+    const int dld = RM ? old_ : L, dl = lin_voff(l, dld), DSTEP = RM ? 32 * old_ * 4 : 128;
     Pre xa, xb;
     tile_pipeline(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int I = w + min(i, nu - 1) * WAVES;
-            ldr_tile_lin(rdO, ll, I * 128, L, x.o);
+            ldr_tile_lin(rdO, dl, I * DSTEP, dld, x.o);
 #pragma unroll
             for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
-            ldr_tile_lin(rQ, ll, I * 128, L, x.q);
+            ldr_tile_lin(rQ, ql, I * QSTEP, qld, x.q);
             x.gneg = ld1(rG, li * 4, I * 128);
         },
         [&](Pre& c, int) {
@@ -595,10 +640,16 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
             Tg[li] = c.gneg;
             float go[16], ob[16], p[16], qb[16], gn[16];
             lds_get_rows(Tg, 0, h, gn);         // -g[query acc_row(r, h)]
-            lds_get_featcols32(To, li, h, go);  // dO[query li][feature 16h + s]
             lds_get_rows(Tp, li, h, p);         // P[query acc_row(r, h)][key li]
-            lds_get_rows(Tq, li, h, qb);        // Q^T[feature li][query acc_row(s, h)]
-            lds_get_rows(To, li, h, ob);        // dO^T[feature li][query acc_row(s, h)]
+            if constexpr (RM) {
+                lds_get_feat32(To, li, h, go);  // dO[query li][feature 16h + s]
+                lds_get_cols(Tq, li, h, qb);    // Q^T[feature li][query acc_row(s, h)]
+                lds_get_cols(To, li, h, ob);    // dO^T[feature li][query acc_row(s, h)]
+            } else {
+                lds_get_featcols32(To, li, h, go);
+                lds_get_rows(Tq, li, h, qb);
+                lds_get_rows(To, li, h, ob);
+            }
             __builtin_amdgcn_sched_barrier(0);
             f32x16 init;
 #pragma unroll
@@ -613,6 +664,12 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
             for (int s = 0; s < 16; ++s) av = __builtin_amdgcn_mfma_f32_32x32x2f32(ob[s], p[s], av, 0, 0, 0);
         });
     f32x16 out[1] = {ak * scale};
+    if constexpr (RM) {
+        reduce_store_rows<WAVES>(out[0], dK + gb, J * 32, w, li, h, lds, gld);
+        __syncthreads();
+        reduce_store_rows<WAVES>(av, dV + gb, J * 32, w, li, h, lds, gld);
+        return;
+    }
     reduce_store<D, WAVES, true>(out, dK + hb, J * 32, w, li, h, lds, L);
     __syncthreads();
     out[0] = av;
@@ -685,20 +742,20 @@ static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, cons
         const dim3 block4(64 * 4);
         if (a->has_mask)
             hipLaunchKernelGGL(dense_fwd_reg_kernel<true>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
-                               a->ws_out, a->L, nbr, a->NB, a->scale);
+                               a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
         else
             hipLaunchKernelGGL(dense_fwd_reg_kernel<false>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn, Out,
-                               a->ws_out, a->L, nbr, a->NB, a->scale);
+                               a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
         return;
     }
     if (D == 32 && a->L <= 16384) {  // 32-bit byte offsets into one head's map: L*L*4 < 2^31
         const dim3 block4(64 * 4);
         if (a->has_mask)
             hipLaunchKernelGGL(dense_fwd_sweep32_kernel<true>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn,
-                               Out, a->ws_out, a->L, nbr, a->NB, a->scale);
+                               Out, a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
         else
             hipLaunchKernelGGL(dense_fwd_sweep32_kernel<false>, grid, block4, 0, a->hdr.stream, Qt, K, Vt, Mask, Attn,
-                               Out, a->ws_out, a->L, nbr, a->NB, a->scale);
+                               Out, a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
         return;
     }
     if (a->has_mask)
@@ -718,9 +775,9 @@ static void dense_bwd_launch(DenseAttn* a, const float* Qt, const float* Kt, con
     if (D == 32 && a->L <= 16384 && a->out_key == P && a->ws_out) {
         const dim3 block4(64 * 4);
         hipLaunchKernelGGL(dense_bwd_row32_kernel<4>, grid, block4, 0, a->hdr.stream, Kt, V, P, dOt, a->ws_out,
-                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale);
+                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale, Layouts{});
         hipLaunchKernelGGL(dense_bwd_col32_kernel<4>, grid, block4, 0, a->hdr.stream, Qt, V, P, dOt, a->ws_rowsum, dK,
-                           dV, a->L, nbr, a->NB, a->scale);
+                           dV, a->L, nbr, a->NB, a->scale, Layouts{});
         return;
     }
     if (a->out_key == P && a->ws_out)
@@ -761,6 +818,107 @@ void dense_backward(void* h, const float* Qt, const float* Kt, const float* V, c
     if (!a->ws_rowsum && !SPION_HIP_OK(hipMalloc((void**)&a->ws_rowsum, sizeof(float) * (size_t)a->NB * a->L))) return;
     if (a->d == 32) dense_bwd_launch<32>(a, Qt, Kt, V, P, dOt, dQ, dK, dV);
     else dense_bwd_launch<64>(a, Qt, Kt, V, P, dOt, dQ, dK, dV);
+    check_launch("dense_bwd kernels");
+}
+
+// Row-major / strided heads (d = 32, L <= 16384): Q, K, V, Out, dO and the gradients are [B][H][L][32] views with
+// one layout per tensor group (tile_kernels.h), read and written in place; the map stays [NB][key][query].
+static DenseAttn* dense_strided_handle(void* h, const char* who, int heads, const HeadLayout* const* lays, int n) {
+    DenseAttn* a = as_dense(h, who);
+    if (!a) return nullptr;
+    if (a->d != 32 || a->L > 16384) {
+        set_error("%s: strided heads are served for emb_dim 32 and seq_len <= 16384 only", who);
+        return nullptr;
+    }
+    if (heads <= 0 || a->NB % heads) {
+        set_error("%s: heads = %d does not divide num_batches = %d", who, heads, a->NB);
+        return nullptr;
+    }
+    for (int i = 0; i < n; ++i) {
+        const HeadLayout& y = *lays[i];
+        if (y.ld < a->d || y.ld % 4 || y.hstride % 4 || y.bstride % 4 || y.hstride < 0 || y.bstride < 0 ||
+            (long long)a->L * y.ld >= (1ll << 29)) {
+            set_error("%s: layout %d: strides must be non-negative multiples of 4 floats, row stride >= emb_dim, "
+                      "seq_len * row stride < 2^29", who, i);
+            return nullptr;
+        }
+    }
+    return a;
+}
+static bool dense_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+void dense_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                           float* Out, int heads, const HeadLayout& in, const HeadLayout& out) {
+    const char* who = "dense attn_forward_strided";
+    const HeadLayout* lays[2] = {&in, &out};
+    DenseAttn* a = dense_strided_handle(h, who, heads, lays, 2);
+    if (!a) return;
+    if (a->has_mask != (Mask != nullptr)) {
+        set_error("%s: handle was created by the %s init", who, a->has_mask ? "mask" : "no-mask");
+        return;
+    }
+    if (!Q || !K || !V || !Attn || !Out) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    if (!dense_aligned16(Q) || !dense_aligned16(K) || !dense_aligned16(V) || !dense_aligned16(Out)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = out;
+    ly.H = heads;
+    const int nbr = a->L / 32;
+    const dim3 grid(nbr * a->NB), block4(64 * 4);
+    a->out_key = nullptr;  // no kept copy: the strided backward is handed Out
+    if (nbr <= 32) {
+        if (a->has_mask)
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<true, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn,
+                               Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+        else
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<false, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn,
+                               Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+    } else {
+        if (a->has_mask)
+            hipLaunchKernelGGL((dense_fwd_sweep32_kernel<true, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask,
+                               Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+        else
+            hipLaunchKernelGGL((dense_fwd_sweep32_kernel<false, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask,
+                               Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+    }
+    check_launch("dense_fwd kernels");
+}
+
+void dense_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P, const float* Out,
+                            const float* dO, float* dQ, float* dK, float* dV, int heads, const HeadLayout& in,
+                            const HeadLayout& out, const HeadLayout& grad) {
+    const char* who = "dense attn_backward_strided";
+    const HeadLayout* lays[3] = {&in, &out, &grad};
+    DenseAttn* a = dense_strided_handle(h, who, heads, lays, 3);
+    if (!a) return;
+    if (!Q || !K || !V || !P || !Out || !dO || !dQ || !dK || !dV) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    if (!dense_aligned16(Q) || !dense_aligned16(K) || !dense_aligned16(V) || !dense_aligned16(Out) ||
+        !dense_aligned16(dO) || !dense_aligned16(dQ) || !dense_aligned16(dK) || !dense_aligned16(dV)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!a->ws_rowsum && !SPION_HIP_OK(hipMalloc((void**)&a->ws_rowsum, sizeof(float) * (size_t)a->NB * a->L))) return;
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = grad;
+    ly.H = heads;
+    const int nbr = a->L / 32;
+    const dim3 grid(nbr * a->NB), block4(64 * 4);
+    hipLaunchKernelGGL((dense_bwd_row32_kernel<4, true>), grid, block4, 0, a->hdr.stream, K, V, P, dO, Out,
+                       a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale, ly);
+    hipLaunchKernelGGL((dense_bwd_col32_kernel<4, true>), grid, block4, 0, a->hdr.stream, Q, V, P, dO, a->ws_rowsum, dK,
+                       dV, a->L, nbr, a->NB, a->scale, ly);
     check_launch("dense_bwd kernels");
 }
 

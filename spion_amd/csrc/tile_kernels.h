@@ -28,7 +28,6 @@ namespace spion {
 #define SPION_TILE_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2, 2)))
 #define SPION_TILE_KERNEL3(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 constexpr float LOG2E = 1.4426950408889634f;

@@ -9,6 +9,7 @@ namespace spion {
 // wavefront helpers
 // =================================================================================================
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -146,6 +147,36 @@ __device__ __forceinline__ void reduce_store(f32x16 (&acc)[D / 32], float* __res
             for (int ww = 0; ww < WAVES; ++ww) s += lds[((ww * NC + c) * 16 + r) * 64 + l];
             out[addr(c, r)] = s;
         }
+}
+
+// A transposed 32-feature accumulator (register = feature acc_row(r, h), lane = row li of the strip) summed over
+// the waves and written row-major, rows `ld` floats apart: register group g = r/4 is four consecutive features,
+// one 16-byte store per lane; wave g % WAVES writes group g.
+template <int WAVES>
+__device__ __forceinline__ void reduce_store_rows(const f32x16& acc, float* __restrict__ out, int row0, int w, int li,
+                                                  int h, float* __restrict__ lds, size_t ld) {
+    const int l = h * 32 + li;
+    if (WAVES > 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lds[(w * 16 + r) * 64 + l] = acc[r];
+        __syncthreads();
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        if (WAVES > 1 && (g % WAVES) != w) continue;
+        float s[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int r = 4 * g + j;
+            s[j] = acc[r];
+            if (WAVES > 1) {
+                s[j] = 0.f;
+#pragma unroll
+                for (int ww = 0; ww < WAVES; ++ww) s[j] += lds[(ww * 16 + r) * 64 + l];
+            }
+        }
+        *reinterpret_cast<f32x4*>(out + (size_t)(row0 + li) * ld + 8 * g + 4 * h) = (f32x4){s[0], s[1], s[2], s[3]};
+    }
 }
 
 // Like reduce_store (row-major form), but the reduced tile goes to two arrays.

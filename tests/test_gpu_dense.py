@@ -65,6 +65,79 @@ def test_dense_matches_oracle(L, d, NB, with_mask):
         assert (got["P"][0][:, 130:] == 0).all() and (got["P"][2][:, 33:] == 0).all()
 
 
+def _views(B, H, L, d, layout, n, seed, fill=None):
+    """n tensors seen as [B, H, L, d]: "plain" contiguous, "proj" each a [B, L, H*d] projection, "fused" slices of
+    one [B, L, n, H, d+4] buffer."""
+    g = torch.Generator().manual_seed(seed)
+    if layout == "plain":
+        bufs = [torch.randn(B, H, L, d, generator=g).cuda() for _ in range(n)]
+        views = bufs
+    elif layout == "proj":
+        bufs = [torch.randn(B, L, H * d, generator=g).cuda() for _ in range(n)]
+        views = [b.view(B, L, H, d).transpose(1, 2) for b in bufs]
+    else:
+        buf = torch.randn(B, L, n, H, d + 4, generator=g).cuda()
+        bufs = [buf]
+        views = [buf[:, :, i, :, :d].transpose(1, 2) for i in range(n)]
+    if fill is not None:
+        for b in bufs:
+            b.fill_(fill)
+    return bufs, views
+
+
+@pytest.mark.parametrize("layout,L,with_mask", [("plain", 256, False), ("proj", 256, True), ("fused", 160, False),
+                                                ("proj", 1024, False), ("proj", 1088, True), ("fused", 2048, False)])
+def test_dense_strided_entry_points(layout, L, with_mask):
+    """spion_dense_forward_strided / spion_dense_backward_strided: row-major heads, possibly interleaved in the
+    memory of [B, L, H*d] projections, against the oracle and, bit for bit, against the reference's ABI on
+    transposed copies of the same tensors."""
+    import ctypes
+    d, B, H = 32, 2, 2
+    NB = B * H
+    lib = Attention._cuda_mask_compile_module() if with_mask else Attention._cuda_compile_module()
+    h = lib.init(d, L, NB)
+    _lib.check_error("init")
+    _, (q, k, v) = _views(B, H, L, d, layout, 3, seed=L)
+    _, (dout,) = _views(B, H, L, d, "plain" if layout == "plain" else "proj", 1, seed=L + 1)
+    _, (out,) = _views(B, H, L, d, "plain" if layout == "plain" else "proj", 1, seed=0, fill=float("nan"))
+    gbufs, (dq, dk, dv) = _views(B, H, L, d, layout, 3, seed=0, fill=-7.0)
+    pen = pen_np = None
+    if with_mask:
+        km = np.ones((B, L), np.float32)
+        km[0, 130:] = 0
+        km[1, 33:] = 0
+        pen_np = osa.key_penalty_from_mask(km, H)
+        pen = torch.from_numpy(pen_np).cuda()
+    attn = torch.full((NB, L, L), float("nan"), device="cuda")
+    lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+    A = ctypes.addressof
+    core = _lib.core()
+    core.spion_dense_forward_strided(h, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen.data_ptr() if with_mask else None,
+                                     attn.data_ptr(), out.data_ptr(), H, A(lin), A(lout))
+    _lib.check_error("dense forward strided")
+    core.spion_dense_backward_strided(h, q.data_ptr(), k.data_ptr(), v.data_ptr(), attn.data_ptr(), out.data_ptr(),
+                                      dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), H, A(lin), A(lout),
+                                      A(lgrad))
+    _lib.check_error("dense backward strided")
+    torch.cuda.synchronize()
+    lib.destroy(h)
+    flat = lambda t: t.reshape(NB, L, d).contiguous()
+    Q, K, V, dO = flat(q), flat(k), flat(v), flat(dout)
+    abi = _run_dense(d, L, NB, Q, K, V, dO, pen)
+    got = dict(O=flat(out).cpu().numpy(), P=attn.transpose(1, 2).cpu().numpy(), dQ=flat(dq).cpu().numpy(),
+               dK=flat(dk).cpu().numpy(), dV=flat(dv).cpu().numpy())
+    for name in ("P", "O", "dQ", "dK", "dV"):
+        assert np.array_equal(got[name], abi[name]), f"{name}: differs from the reference ABI's result"
+    if layout == "fused":
+        assert (gbufs[0][..., d:] == -7.0).all(), "padding between the heads' rows was written"
+    if L <= 1088:
+        f = lambda t: t.cpu().numpy().astype(np.float64)
+        O, P = oda.dense_attention_forward(f(Q), f(K), f(V), None if pen_np is None else pen_np.astype(np.float64))
+        gQ, gK, gV = oda.dense_attention_backward(f(Q), f(K), f(V), P, f(dO))
+        for name, ref in (("P", P), ("O", O), ("dQ", gQ), ("dK", gK), ("dV", gV)):
+            assert_close(got[name], ref, what=f"dense strided {layout} L={L} {name}")
+
+
 def test_dense_backward_without_the_kept_output():
     L, d, NB = 256, 32, 2
     g = torch.Generator().manual_seed(5)
