@@ -395,12 +395,41 @@ def bench_dense_phase(args, dev):
         step()
     torch.cuda.synchronize()
     ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    # the same step through the reference's ABI (feature-major operands: four transposes a step)
+    module.reads_views = False
+    for _ in range(max(3, args.warmup // 4)):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(5, args.steps // 4)):
+        step()
+    torch.cuda.synchronize()
+    ms_step_abi = 1e3 * (time.perf_counter() - t0) / max(5, args.steps // 4)
+    module.reads_views = True
+
+    # the kernels the module runs: row-major operands at the strided entry points
+    import ctypes
+    core = _lib.core()
+    Qr, Kr, Vr, dOr = (t.detach().contiguous() for t in (q, k, v, do))
+    out_r = torch.empty_like(Qr)
+    attn = torch.empty(NB, L, L, device=dev)
+    gq, gk, gv = (torch.empty_like(Qr) for _ in range(3))
+    lay = _lib.head_layout(Qr)
+    A = ctypes.addressof(lay)
+    t_fwd_rm = _event_ms(lambda: core.spion_dense_forward_strided(
+        handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), None, attn.data_ptr(), out_r.data_ptr(), H, A, A),
+        max(10, args.steps // 4))
+    _lib.check_error("dense forward (row-major)")
+    t_bwd_rm = _event_ms(lambda: core.spion_dense_backward_strided(
+        handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), attn.data_ptr(), out_r.data_ptr(), dOr.data_ptr(),
+        gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), H, A, A, A), max(10, args.steps // 4))
+    _lib.check_error("dense backward (row-major)")
+    del Qr, Kr, Vr, dOr, out_r, gq, gk, gv
 
     # forward kernel alone at the C ABI (operands in the layouts it takes: Qt, Vt feature-major)
     Qt = _lib.transpose_last2(q.detach().reshape(NB, L, d))
     Vt = _lib.transpose_last2(v.detach().reshape(NB, L, d))
     K = k.detach().reshape(NB, L, d).contiguous()
-    attn = torch.empty(NB, L, L, device=dev)
     out_t = torch.empty(NB, d, L, device=dev)
     t_fwd = _event_ms(lambda: cpp.attn_forward(handle, Qt.data_ptr(), K.data_ptr(), Vt.data_ptr(), attn.data_ptr(),
                                                out_t.data_ptr()), max(10, args.steps // 4))
@@ -415,12 +444,14 @@ def bench_dense_phase(args, dev):
                                                 dv.data_ptr()), max(10, args.steps // 4))
     _lib.check_error("dense backward")
     alg_flops = 12.0 * L * L * d * NB
-    roof = dict(bound="mfma", kernel="dense_fwd_reg_kernel", achieved=alg_flops / 3.0 / t_fwd / 1e9,
+    roof = dict(bound="mfma", kernel="dense_fwd_reg_kernel", achieved=alg_flops / 3.0 / t_fwd_rm / 1e9,
                 peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s", traffic=None)
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd, 4),
-                         "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd, 4)}
-    roof["backward_frac"] = alg_flops * 2.0 / 3.0 / t_bwd / 1e9 / PEAK_FP32_MFMA_TFLOPS
+    roof["kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd_rm, 4),
+                         "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd_rm, 4)}
+    roof["backward_frac"] = alg_flops * 2.0 / 3.0 / t_bwd_rm / 1e9 / PEAK_FP32_MFMA_TFLOPS
+    roof["reference_abi_kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd, 4),
+                                       "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd, 4)}
     result = {
         "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -428,6 +459,7 @@ def bench_dense_phase(args, dev):
         "data": "synthetic (seeded N(0,1) tensors)",
         "config": {"workload": f"dense_phase: softmax attention fwd+bwd with the full probability map, B={B} H={H} L={L} d={d}"},
         "algorithmic": {"gflop": alg_flops / 1e9, "map_gbytes": 4.0 * NB * L * L / 1e9},
+        "reference_abi_step_ms": round(ms_step_abi, 4),
         "roofline": roof,
     }
     if not args.no_cpu_baseline:

@@ -7,13 +7,36 @@ library fills (models/attention_cuda.py:32-36).  ``mask`` is ignored by this var
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 import torch.nn as nn
 
 from . import _lib
 
 
+def _head_views(tensors):
+    """The tensors as the strided entry points can take them (one common layout), or None."""
+    lay = _lib.head_layout(tensors[0])
+    if lay is None or any(t.stride() != tensors[0].stride() or _lib.head_layout(t) is None for t in tensors[1:]):
+        return None
+    return lay
+
+
+def _empty_heads(shape, interleaved, device):
+    B, H, L, d = shape
+    if interleaved:  # memory [B, L, H, d]: merging the heads afterwards is a view
+        return torch.empty((B, L, H, d), dtype=torch.float32, device=device).transpose(1, 2)
+    return torch.empty(shape, dtype=torch.float32, device=device)
+
+
 class _DenseAttnFunction(torch.autograd.Function):
+    """The reference's function (models/attention_cuda.py:18-74) transposes Q and V for the forward and K and
+    grad_output for the backward, because its ABI takes feature-major operands, and returns feature-major results
+    as permuted views.  For head dimension 32 and sequences up to 16384 the library's strided entry points
+    (spion_dense_forward_strided / spion_dense_backward_strided) take every tensor row-major -- also as views of
+    [B, L, H*d] projections -- and nothing is transposed or copied; other shapes go through the reference's ABI."""
+
     @staticmethod
     def forward(ctx, query, key, value, mask, module):
         m = module
@@ -22,6 +45,28 @@ class _DenseAttnFunction(torch.autograd.Function):
         if tuple(query.shape) != (B, H, L, d):
             raise ValueError(f"query shape {tuple(query.shape)} does not match the handle ({B}, {H}, {L}, {d})")
         dev = query.device
+        ctx.strided = False
+        if m.reads_views:
+            lay = _head_views((query, key, value))
+            if lay is None:
+                query, key, value = query.contiguous(), key.contiguous(), value.contiguous()
+                lay = _lib.head_layout(query)
+            attn = torch.empty((B, H, L, L), dtype=torch.float32, device=dev)  # memory [key][query]
+            out = _empty_heads((B, H, L, d), query.stride(1) < query.stride(2), dev)
+            lout = _lib.head_layout(out)
+            pen_ptr = None
+            if m.with_mask:
+                pen = (1e6 * (1.0 - mask.repeat(1, H))).to(torch.float32).contiguous()
+                pen_ptr = pen.data_ptr()
+            _lib.core().spion_dense_forward_strided(
+                m.attn_handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pen_ptr, attn.data_ptr(),
+                out.data_ptr(), H, ctypes.addressof(lay), ctypes.addressof(lout))
+            _lib.check_error("attn_forward")
+            ctx.save_for_backward(query, key, value, attn, out)
+            ctx.set_materialize_grads(False)
+            ctx.module = m
+            ctx.strided = True
+            return out, attn.permute(0, 1, 3, 2)
         qt = _lib.transpose_last2(query)  # [B,H,d,L]
         k = key.contiguous()
         vt = _lib.transpose_last2(value)
@@ -44,8 +89,24 @@ class _DenseAttnFunction(torch.autograd.Function):
     def backward(ctx, grad_output, grad_weights):
         m = ctx.module
         _lib.use_current_stream(m, ctx.saved_tensors[0].device)
-        qt, key, value, attn = ctx.saved_tensors
         B, H, L, d = m.batch_size, m.num_heads, m.seq_len, m.emb_dim
+        if ctx.strided:
+            q, k, v, attn, out = ctx.saved_tensors
+            dev = q.device
+            if grad_output is None:  # only the returned map was used downstream: its gradient is ignored
+                grad_output = torch.zeros(B, H, L, d, dtype=torch.float32, device=dev)
+            go = grad_output
+            if go.stride() != out.stride() or _lib.head_layout(go) is None:
+                go = torch.empty_like(out).copy_(grad_output)  # keeps out's strides
+            dq, dk, dv = (_empty_heads((B, H, L, d), q.stride(1) < q.stride(2), dev) for _ in range(3))
+            lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+            _lib.core().spion_dense_backward_strided(
+                m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), attn.data_ptr(), out.data_ptr(),
+                go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), H, ctypes.addressof(lin),
+                ctypes.addressof(lout), ctypes.addressof(lgrad))
+            _lib.check_error("attn_backward")
+            return dq, dk, dv, None, None
+        qt, key, value, attn = ctx.saved_tensors
         dev = qt.device
         kt = _lib.transpose_last2(key)
         v = value.contiguous()
@@ -83,6 +144,8 @@ class _DenseAttentionBase(nn.Module):
         self.attn_cpp = attn_cpp
         self.attn_handle = attn_handle
         self.attn_func = _DenseAttnFunction
+        # shapes the strided entry points serve; everything else goes through the reference's ABI
+        self.reads_views = self.emb_dim == 32 and self.seq_len <= 16384
 
     def forward(self, query, key, value, mask):
         return self.attn_func.apply(query, key, value, mask, self)
