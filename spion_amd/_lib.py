@@ -149,6 +149,21 @@ def head_layout(t: "torch.Tensor") -> HeadLayout | None:
     return HeadLayout(sb, sh, sl)
 
 
+def adjacent_head_views(q, k, v):
+    """True when q, k, v ([B,H,L,d] views) are the three slices of one [B, L, 3, H, d] buffer, in this order."""
+    B, H, L, d = q.shape
+    strides = (L * 3 * H * d, d, 3 * H * d, 1)
+    step = H * d * q.element_size()
+    return (q.stride() == strides and k.stride() == strides and v.stride() == strides
+            and k.data_ptr() - q.data_ptr() == step and v.data_ptr() - k.data_ptr() == step)
+
+
+def empty_adjacent_heads(B, H, L, d, device):
+    """Three uninitialised [B,H,L,d] views that are the slices of one [B, L, 3, H, d] buffer."""
+    buf = torch.empty((B, L, 3, H, d), dtype=torch.float32, device=device)
+    return tuple(buf[:, :, i].transpose(1, 2) for i in range(3))
+
+
 def use_current_stream(module, device) -> None:
     """Point the module's handle at torch's current stream on ``device`` (the reference runs on the legacy
     default stream only): what makes the modules usable on side streams and under HIP graph capture.  One

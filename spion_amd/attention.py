@@ -39,6 +39,41 @@ class SoftmaxAttention(nn.Module):
         return torch.matmul(attn, V), attn
 
 
+class _FusedQKV(torch.autograd.Function):
+    """The three projections of models/attention.py:84-86 as one GEMM: X [B,L,dim] times the stacked weights gives one
+    [B, L, 3, H, d] buffer whose slices are returned as the [B,H,L,d] heads (what split_heads, :136-139, makes of
+    each projection).  The attention modules read such views in place and hand back gradients that are slices of one
+    buffer again, so the backward is one GEMM for dX and one for the stacked weight gradient, without a copy."""
+
+    @staticmethod
+    def forward(ctx, X, wq, wk, wv, bq, bk, bv, H, d):
+        B, L, dim = X.shape
+        w = torch.cat((wq, wk, wv), 0)
+        b = torch.cat((bq, bk, bv), 0)
+        X2 = X.reshape(B * L, dim)
+        qkv = torch.addmm(b, X2, w.t()).view(B, L, 3, H, d)
+        ctx.save_for_backward(X2, w)
+        ctx.dims = (B, H, L, d, dim)
+        return tuple(qkv[:, :, i].transpose(1, 2) for i in range(3))
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv):
+        X2, w = ctx.saved_tensors
+        B, H, L, d, dim = ctx.dims
+        n = H * d
+        if any(g is None for g in (dq, dk, dv)):
+            z = next(g for g in (dq, dk, dv) if g is not None)
+            dq, dk, dv = (torch.zeros_like(z) if g is None else g for g in (dq, dk, dv))
+        if _lib.adjacent_head_views(dq, dk, dv):
+            g2 = torch.as_strided(dq, (B * L, 3 * n), (3 * n, 1))
+        else:
+            g2 = torch.stack([g.transpose(1, 2) for g in (dq, dk, dv)], 2).reshape(B * L, 3 * n)
+        dX = (g2 @ w).view(B, L, dim) if ctx.needs_input_grad[0] else None
+        dW = g2.t() @ X2
+        db = g2.sum(0)
+        return (dX, dW[:n], dW[n:2 * n], dW[2 * n:], db[:n], db[n:2 * n], db[2 * n:], None, None)
+
+
 class Attention(nn.Module):
     def __init__(self, config, inference=False):
         super().__init__()
@@ -50,6 +85,8 @@ class Attention(nn.Module):
         self.block_size = config["block_size"]
         self.num_blocks = int(self.seq_len / self.block_size)
 
+        # one GEMM for the three projections (same parameters, same state dict as the reference's three layers)
+        self.fused_qkv = bool(config.get("fused_qkv", True))
         self.W_q = nn.Linear(self.dim, self.num_head * self.head_dim)
         self.W_k = nn.Linear(self.dim, self.num_head * self.head_dim)
         self.W_v = nn.Linear(self.dim, self.num_head * self.head_dim)
@@ -75,9 +112,13 @@ class Attention(nn.Module):
         self.ff = nn.Linear(self.num_head * self.head_dim, self.dim)
 
     def forward(self, X, mask, mat=None):
-        Q = self.split_heads(self.W_q(X))
-        K = self.split_heads(self.W_k(X))
-        V = self.split_heads(self.W_v(X))
+        if self.fused_qkv and X.dtype == torch.float32 and not torch.is_autocast_enabled():
+            Q, K, V = _FusedQKV.apply(X, self.W_q.weight, self.W_k.weight, self.W_v.weight, self.W_q.bias,
+                                      self.W_k.bias, self.W_v.bias, self.num_head, self.head_dim)
+        else:
+            Q = self.split_heads(self.W_q(X))
+            K = self.split_heads(self.W_k(X))
+            V = self.split_heads(self.W_v(X))
         # the kernels are fp32: leave autocast for the attention core (models/attention.py:88-92)
         with torch.autocast(device_type=X.device.type, enabled=False):
             if mat is None:

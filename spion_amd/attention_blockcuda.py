@@ -95,7 +95,10 @@ class _BlockAttnFunction(torch.autograd.Function):
                 go = torch.empty_like(out).copy_(grad_output)  # preserves out's strides
             interleaved = q.stride(1) < q.stride(2)
             shape = tuple(q.shape)
-            dq, dk, dv = (_empty_heads(shape, interleaved, dev) for _ in range(3))
+            if _lib.adjacent_head_views(q, k, v):  # slices of one fused projection: the gradients likewise
+                dq, dk, dv = _lib.empty_adjacent_heads(*shape, dev)
+            else:
+                dq, dk, dv = (_empty_heads(shape, interleaved, dev) for _ in range(3))
             lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
             core.spion_attn_backward_strided(
                 m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), p_flat.data_ptr(), out.data_ptr(),

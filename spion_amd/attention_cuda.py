@@ -98,7 +98,10 @@ class _DenseAttnFunction(torch.autograd.Function):
             go = grad_output
             if go.stride() != out.stride() or _lib.head_layout(go) is None:
                 go = torch.empty_like(out).copy_(grad_output)  # keeps out's strides
-            dq, dk, dv = (_empty_heads((B, H, L, d), q.stride(1) < q.stride(2), dev) for _ in range(3))
+            if _lib.adjacent_head_views(q, k, v):  # slices of one fused projection: the gradients likewise
+                dq, dk, dv = _lib.empty_adjacent_heads(B, H, L, d, dev)
+            else:
+                dq, dk, dv = (_empty_heads((B, H, L, d), q.stride(1) < q.stride(2), dev) for _ in range(3))
             lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
             _lib.core().spion_dense_backward_strided(
                 m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), attn.data_ptr(), out.data_ptr(),
