@@ -41,8 +41,10 @@ def _eager_step(module, args, q, k, v, do):
     return out.detach().clone(), [t.grad.clone() for t in (q, k, v)]
 
 
-@pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16"])
+@pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16", "block_views", "blockmask_views", "dense_views"])
 def test_whole_step_graph_replays_match_eager(kind):
+    views = kind.endswith("_views")  # heads as views of [B, L, H*d] projections: the strided entry points
+    kind = kind.split("_")[0]
     B, H, L, d, bs = 2, 2, 256, 32, 32
     cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
     mat = torch.from_numpy(workloads.band_random_block_mask(L // bs, 1, extra_frac=0.1, seed=3)).cuda()
@@ -62,6 +64,9 @@ def test_whole_step_graph_replays_match_eager(kind):
         module, args = spion_amd.BlockAttentionBF16(cfg), (key_mask, mat)
     dtype = torch.bfloat16 if kind == "bf16" else torch.float32
     q, k, v, do = (t.to(dtype) for t in workloads.qkv(B, H, L, d, seed=11, device="cuda"))
+    if views:
+        q, k, v, do = (t.transpose(1, 2).contiguous().transpose(1, 2) for t in (q, k, v, do))
+        assert module.reads_views and not q.is_contiguous()
     for t in (q, k, v):
         t.requires_grad_()
     ref_out, ref_grads = _eager_step(module, args, q, k, v, do)
