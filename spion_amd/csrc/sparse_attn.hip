@@ -325,6 +325,7 @@ struct PatternIndex {
     int* d_blob = nullptr;  // one allocation holding every array below
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
+    int *d_rdesc = nullptr, *d_cdesc = nullptr;  // per strip in launch order: {strip, first tile, tiles, P offset}
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
     // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
@@ -529,7 +530,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         return o;
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
-    size_t o_lgr = 0, o_lgc = 0;
+    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_cdesc = 0;
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -566,6 +567,23 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         };
         append_order(trp, true);
         append_order(tcp, false);
+        // One 16-byte descriptor per strip in that order, {strip, first tile, tiles, offset of the strip's first
+        // element in a head's P}: a work-group learns everything about its strip from one scalar load instead of
+        // three dependent ones.
+        std::vector<int> rdesc(4 * (size_t)nbr), cdesc(4 * (size_t)nbr);
+        for (int p = 0; p < nbr; ++p) {
+            const int I = trp[nbr + 1 + p], J = tcp[nbr + 1 + p];
+            rdesc[4 * p + 0] = I;
+            rdesc[4 * p + 1] = trp[I];
+            rdesc[4 * p + 2] = trp[I + 1] - trp[I];
+            rdesc[4 * p + 3] = off[I * 32];
+            cdesc[4 * p + 0] = J;
+            cdesc[4 * p + 1] = tcp[J];
+            cdesc[4 * p + 2] = tcp[J + 1] - tcp[J];
+            cdesc[4 * p + 3] = 0;
+        }
+        o_rdesc = append(rdesc);
+        o_cdesc = append(cdesc);
         pi.n_wg_row = (int)wgr.wg.size() / 4;
         pi.n_wg_col = (int)wgc.wg.size() / 4;
         pi.chunk_row = wgr.chunk;
@@ -611,6 +629,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcol = pi.d_blob + o_tcol;
         pi.d_tcp = pi.d_blob + o_tcp;
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
+        pi.d_rdesc = pi.d_blob + o_rdesc;
+        pi.d_cdesc = pi.d_blob + o_cdesc;
         pi.d_wg_row = pi.d_blob + o_wgr;
         pi.d_wg_col = pi.d_blob + o_wgc;
         pi.d_long_row = pi.d_blob + o_lgr;
@@ -731,11 +751,11 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     do {                                                                                                             \
         if (pi.max_row_tiles <= W * MAXT)                                                                            \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
-                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_rdesc, pi.d_tcol, a->L, nbr,     \
                                a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
         else                                                                                                         \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
-                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_trp, pi.d_tcol, offs, a->L, nbr,     \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_rdesc, pi.d_tcol, a->L, nbr,     \
                                a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
@@ -758,17 +778,17 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
             hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, K,   \
-                               Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr, a->NB,    \
+                               Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB,    \
                                nnz, a->scale, hc, ly);                                                              \
         else if (a->bwd_passes & 1) {                                                                               \
             if constexpr (!ST)                                                                                      \
                 hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream,  \
-                                   K, Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_trp, pi.d_tcol, offs, a->L, nbr,    \
+                                   K, Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr,    \
                                    a->NB, nnz, a->scale, hc, ly);                                                   \
         }                                                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, \
-                               dO, a->ws_rowsum, dK, dV, pi.d_tcp, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
+                               dO, a->ws_rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
                                hc, ly);                                                                             \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);

@@ -317,7 +317,7 @@ template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = fa
 SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
-    const int* __restrict__ trp, const int* __restrict__ tcol, const int* __restrict__ offs, int L, int nbr,
+    const int* __restrict__ rdesc, const int* __restrict__ tcol, int L, int nbr,
     int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
     static_assert(!ST || (KROW && D == 32), "strided heads: row-major operands, d = 32");
     constexpr int KH = D / 2;
@@ -328,9 +328,9 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const int item = xcd_remap(blockIdx.x, ns * NB);
     int bh, pos;
     item_to_head_strip(item, ns, hc, bh, pos);
-    const int I = trp[nbr + 1 + s0 + pos];
+    const int4 sd = reinterpret_cast<const int4*>(rdesc)[s0 + pos];  // {strip, first tile, tiles, P offset}
+    const int I = sd.x, t0 = sd.y, cnt = sd.z;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
     const size_t hb = (size_t)bh * L * D;
     size_t ib, ob, hbytes, obytes;
@@ -340,7 +340,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const rsrc_t rQ = make_rsrc(Q + ib, hbytes), rK = make_rsrc(Kt + ib, hbytes), rV = make_rsrc(V + ib, hbytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int p_base = offs[I * 32] * 4;
+    const int p_base = sd.w * 4;
     const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
     const int b_voff = (4 * h * ild + li) * 4;
@@ -571,8 +571,8 @@ template <int D, int WAVES, bool HAVE_O, bool VROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
-    float* __restrict__ dQ, const int* __restrict__ trp, const int* __restrict__ tcol,
-    const int* __restrict__ offs, int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
+    float* __restrict__ dQ, const int* __restrict__ rdesc, const int* __restrict__ tcol,
+    int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
     static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, d = 32, Out given");
     static_assert(!VROW || D == 32, "row-major V operand: d = 32 only");
     constexpr int KH = D / 2;
@@ -584,9 +584,9 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     int bh, pos;
     item_to_head_strip(item, nbr, hc, bh, pos);
     bh = NB - 1 - bh;
-    const int I = trp[nbr + 1 + pos];  // strips longest first
+    const int4 sd = reinterpret_cast<const int4*>(rdesc)[pos];  // strips longest first: {strip, first tile, tiles, P offset}
+    const int I = sd.x, t0 = sd.y, cnt = sd.z;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const int rn = cnt * 32;
     const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
     size_t ib, ob, gb, hbytes, obytes, gbytes;
@@ -596,7 +596,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
     const rsrc_t rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes), rdO = make_rsrc(dO + ob, obytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
-    const int p_base = offs[I * 32] * 4;
+    const int p_base = sd.w * 4;
     const int pc_voff = (4 * h * rn + li) * 4;  // col-owner access to a P tile
     const int col_voff = (h * KH * L + li) * 4;
     const int b_voff = (4 * h * ild + li) * 4;
@@ -745,7 +745,7 @@ template <int D, int WAVES, bool VROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
-    const int* __restrict__ tcp, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
+    const int* __restrict__ cdesc, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
     int hc, Layouts ly) {
     static_assert(!ST || VROW, "strided heads: row-major operands, d = 32");
     constexpr int KH = D / 2;
@@ -754,9 +754,9 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     int bh, pos;
     item_to_head_strip(item, nbr, hc, bh, pos);
-    const int J = tcp[nbr + 1 + pos];  // strips longest first
+    const int4 sd = reinterpret_cast<const int4*>(cdesc)[pos];  // strips longest first: {strip, first tile, tiles, 0}
+    const int J = sd.x, e0 = sd.y, cnt = sd.z;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int e0 = tcp[J], cnt = tcp[J + 1] - e0;
     size_t ib, ob, gb, hbytes, obytes, gbytes;
     int ild, old_, gld;
     head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
