@@ -726,8 +726,7 @@ static int pick_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, bool
     return 4;
 }
 
-// Heads whose strips are interleaved in launch order (see item_to_head_strip): as many as share an XCD's slice of
-// the launch, at most 8 -- their K and V (2 * L * d floats a head) stay within reach of that XCD's L2.
+// Heads whose strips are interleaved in launch order (see item_to_head_strip).
 static int heads_per_group(const SparseAttn* a) {
     // Two heads share a stretch of the launch order when every die's share of the heads is even: the long strips of
     // both come first, so the last work groups of a die are short ones (north star shape: step 2 % shorter than
