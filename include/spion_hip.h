@@ -239,7 +239,9 @@ void spion_attn_backward_rowmajor(void* handle, const float* Q, const float* K, 
  * write such views in place.  Element (b, h, i, f) of a tensor lies batch_stride*b + head_stride*h +
  * row_stride*i + f floats after its pointer; one layout for the inputs Q, K, V, one for Out and dO, one for
  * the gradients dQ, dK, dV.  heads = H (num_batches of the handle = B*H, head index fastest).  Strides are
- * multiples of 4 floats, pointers 16-byte aligned, seq_len * row_stride < 2^29.  Served by the tile kernels
+ * multiples of 4 floats, pointers 16-byte aligned, seq_len * row_stride < 2^29; the layouts of tensors that are
+ * written (out, grad) must not map two elements to one address, those of inputs may (head_stride 0: one K / V
+ * head shared by all query heads).  Served by the tile kernels
  * for emb_dim 32 (patterns of aligned 32x32 tiles); otherwise an error is recorded and the caller makes
  * contiguous copies for the row-major entry points above.  Attn / P stay [NB][nnz] as everywhere.  The kept
  * copies of Out are not used: the backward takes Out (required). */

@@ -865,6 +865,10 @@ void dense_forward_strided(void* h, const float* Q, const float* K, const float*
         set_error("%s: operand pointers must be 16-byte aligned", who);
         return;
     }
+    if (!layout_is_injective(out, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the output layout maps two elements to one address", who);
+        return;
+    }
     Layouts ly{};
     ly.in = in;
     ly.out = out;
@@ -905,6 +909,10 @@ void dense_backward_strided(void* h, const float* Q, const float* K, const float
     if (!dense_aligned16(Q) || !dense_aligned16(K) || !dense_aligned16(V) || !dense_aligned16(Out) ||
         !dense_aligned16(dO) || !dense_aligned16(dQ) || !dense_aligned16(dK) || !dense_aligned16(dV)) {
         set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!layout_is_injective(grad, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the gradient layout maps two elements to one address", who);
         return;
     }
     if (!a->ws_rowsum && !SPION_HIP_OK(hipMalloc((void**)&a->ws_rowsum, sizeof(float) * (size_t)a->NB * a->L))) return;

@@ -996,6 +996,10 @@ void sparse_forward_strided(void* h, const float* Q, const float* K, const float
         return;
     }
     if (!check_layout(who, "input", a, heads, in) || !check_layout(who, "output", a, heads, out)) return;
+    if (!layout_is_injective(out, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the output layout maps two elements to one address", who);
+        return;
+    }
     Layouts ly{};
     ly.in = in;
     ly.out = out;
@@ -1025,6 +1029,10 @@ void sparse_backward_strided(void* h, const float* Q, const float* K, const floa
     if (!check_layout(who, "input", a, heads, in) || !check_layout(who, "output", a, heads, out) ||
         !check_layout(who, "gradient", a, heads, grad))
         return;
+    if (!layout_is_injective(grad, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the gradient layout maps two elements to one address", who);
+        return;
+    }
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
     Layouts ly{};
     ly.in = in;

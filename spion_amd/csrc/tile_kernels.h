@@ -255,6 +255,16 @@ struct Layouts {
     HeadLayout in, out, grad;
     int H;
 };
+// Host side: true when no two elements of a [B][H][L][d] view with this layout share an address (required of every
+// tensor the kernels write).  Heads either follow one another as whole blocks or are interleaved inside the rows.
+inline bool layout_is_injective(const HeadLayout& y, int B, int H, int L, int d) {
+    const long long row_span = (long long)(L - 1) * y.ld + d;
+    const bool blocks = H == 1 || y.hstride >= row_span;
+    const bool interleaved = y.hstride >= d && y.ld >= (long long)(H - 1) * y.hstride + d;
+    if (!blocks && !interleaved) return false;
+    const long long batch_span = (long long)(H - 1) * y.hstride + row_span;
+    return B == 1 || y.bstride >= batch_span;
+}
 // ST = false: the heads are contiguous [NB][L][D] slices and every figure below is a compile-time constant.
 template <bool ST, int D>
 __device__ __forceinline__ void head_slice(const HeadLayout& y, int H, int bh, int L, size_t& base, int& ld,

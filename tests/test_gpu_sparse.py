@@ -563,6 +563,13 @@ def test_strided_entry_points_refuse_what_they_cannot_serve():
     with pytest.raises(RuntimeError, match="multiples of 4"):
         _lib.check_error("row stride")
     assert _lib.head_layout(torch.zeros(B, H, L, 33, device="cuda")[..., 1:]) is None   # 4-byte offset
+    # inputs may share memory between heads (one K/V head for all query heads), outputs may not
+    shared = q[:, :1].expand(B, H, L, 32)
+    call(abi, shared, torch.zeros_like(q))
+    _lib.check_error("shared input heads")
+    call(abi, q, shared)
+    with pytest.raises(RuntimeError, match="two elements to one address"):
+        _lib.check_error("aliased output")
     abi.close()
 
 
