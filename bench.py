@@ -706,6 +706,13 @@ def main():
     if wl["name"] == "north_star":  # the workload the committed byte counters were taken on
         roof["traffic"] = _profiled_traffic_bytes(dom)
     roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
+    if path == 1:
+        # MFMA instructions a 32x32 tile costs each kernel against the 32 of its algorithmic share (d = 32): the
+        # column pass recomputes dP (48), the forward's two-sweep form recomputes the logits (48)
+        executed = {"tile_fwd_kernel": 1.0, "tile_bwd_row_kernel": 1.0, "tile_bwd_col_kernel": 1.5}
+        roof["frac_per_kernel"] = {k_: round(third / v_ / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4) for k_, v_ in kernels.items()}
+        roof["frac_on_executed_mfma"] = {k_: round(executed[k_] * third / v_ / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
+                                         for k_, v_ in kernels.items()}
 
     result = {
         "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
