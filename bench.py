@@ -707,8 +707,8 @@ def main():
         roof["traffic"] = _profiled_traffic_bytes(dom)
     roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
     if path == 1:
-        # MFMA instructions a 32x32 tile costs each kernel against the 32 of its algorithmic share (d = 32): the
-        # column pass recomputes dP (48), the forward's two-sweep form recomputes the logits (48)
+        # MFMA work a tile costs each kernel against its algorithmic share: the column pass recomputes dP (1.5x);
+        # the forward is taken in its register-resident form (1x; its two-sweep form for very long rows is 1.5x)
         executed = {"tile_fwd_kernel": 1.0, "tile_bwd_row_kernel": 1.0, "tile_bwd_col_kernel": 1.5}
         roof["frac_per_kernel"] = {k_: round(third / v_ / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4) for k_, v_ in kernels.items()}
         roof["frac_on_executed_mfma"] = {k_: round(executed[k_] * third / v_ / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
