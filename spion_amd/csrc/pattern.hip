@@ -13,7 +13,7 @@ namespace spion {
 
 constexpr int POOL_THREADS = 256;
 constexpr int WALK_THREADS = 1024;
-constexpr int POOLED_LDS = 8192;  // block grids up to 90 x 90 are walked from LDS
+constexpr int POOLED_LDS = 36864;  // block grids up to 192 x 192 are walked from LDS (144 KB of the CU's 160)
 
 // pooled[I][J] = (1/bs^2) sum_{i in I, j in J} sum_{t=-hk..hk} A[i+t][j+t]  (zero outside the map).
 // Regrouped per source element A[p][q]: its weight is the number of shifts t that land in the block.
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(WALK_THREADS) void threshold_walk_kernel(const floa
     __shared__ int sh[2];
     __shared__ int s_cnt;
     __shared__ uint32_t s_min;
-    __shared__ float s_pooled[POOLED_LDS];
+    extern __shared__ float s_pooled[];  // N floats when N <= POOLED_LDS (sized by the launch)
     const int map = blockIdx.x, N = nb * nb;
     const float* pooled = pooled_all + (size_t)map * N;
     float* mat = mat_all + (size_t)map * N;
@@ -318,8 +318,18 @@ int pattern_generate(const float* Score, int n_maps, int L, int bs, int ksize, i
     if (!check_launch("conv_pool_kernel")) return 1;
     int topk = 0;
     if (mode == SPION_PATTERN_TOPK) topk = (int)((double)(nb * nb) * param - (double)nb);  // main_conv.py:247
-    hipLaunchKernelGGL(threshold_walk_kernel, dim3(n_maps), dim3(WALK_THREADS), 0, stream, pooled, Mat, Thresh, nb, mode,
-                       (float)param, topk);
+    const size_t walk_lds = (size_t)nb * nb <= (size_t)POOLED_LDS ? sizeof(float) * nb * nb : 0;
+    if (walk_lds > 32 * 1024) {  // beyond what a launch may ask for without saying so first
+        static std::once_flag once;
+        static hipError_t attr_err = hipSuccess;
+        std::call_once(once, [] {
+            attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(threshold_walk_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, sizeof(float) * POOLED_LDS);
+        });
+        if (!SPION_HIP_OK(attr_err)) return 1;
+    }
+    hipLaunchKernelGGL(threshold_walk_kernel, dim3(n_maps), dim3(WALK_THREADS), walk_lds, stream, pooled, Mat, Thresh, nb,
+                       mode, (float)param, topk);
     if (!check_launch("threshold_walk_kernel")) return 1;
     return 0;
 }

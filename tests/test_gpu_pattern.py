@@ -42,6 +42,16 @@ def test_pattern_small_maps(L, bs, q, ksize):
     _check_maps(maps, bs, q, ksize)
 
 
+@pytest.mark.parametrize("L,bs", [(4096, 32), (6400, 32)])
+def test_pattern_large_block_grids(L, bs):
+    """Block grids of 128 x 128 (pooled map walked from LDS) and 200 x 200 (walked from global memory)."""
+    g = torch.Generator().manual_seed(L)
+    maps = torch.rand(1, L, L, generator=g)
+    maps = maps / maps.sum(-1, keepdim=True)
+    maps[0] += (2.0 / L) * torch.eye(L)
+    _check_maps(maps, bs, 0.95, 31)
+
+
 def test_pattern_config2_bit_exact_against_both_routes():
     """Config 2: two 1024x1024 maps, 31x31 diagonal filter, 32x32 pooling, q = 0.90.
     The seed is one whose decision margin exceeds the float32-route error (tests/golden/config2.json),
