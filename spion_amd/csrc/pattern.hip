@@ -6,6 +6,7 @@
 #include "common.h"
 #include "../../include/spion_hip.h"
 
+#include <algorithm>
 #include <cmath>
 #include <mutex>
 
@@ -41,6 +42,66 @@ __global__ __launch_bounds__(POOL_THREADS) void conv_pool_kernel(const float* __
         __syncthreads();
     }
     if (threadIdx.x == 0) pooled[((size_t)map * nb + I) * nb + J] = (float)(red[0] / ((double)bs * (double)bs));
+}
+
+// The same sums for block sizes of at least twice the filter's reach (bs >= 2 hk, so a column feeds its own block
+// and at most one neighbour): one work-group per (block row, group of adjacent blocks, map); thread (column, row
+// group) walks its share of the bs + 2 hk rows of one column -- consecutive threads read consecutive floats -- and
+// keeps two fp64 sums, for the column's own block and for the neighbour it reaches into; one wavefront per block
+// then adds the block's partial sums in a fixed order.  Every element is read once per block row it touches
+// ((bs + 2 hk) / bs times, the repeats from L2) instead of once per block, and in full rows.
+constexpr int CP_COLS = 256, CP_RG = 4;
+__global__ __launch_bounds__(CP_COLS* CP_RG) void conv_pool_cols_kernel(const float* __restrict__ A,
+                                                                         float* __restrict__ pooled, int L, int bs,
+                                                                         int nb, int hk, int gb) {
+    __shared__ double part[CP_RG][2][CP_COLS];
+    const int I = blockIdx.y, map = blockIdx.z;
+    const int Jg = blockIdx.x * gb;  // first block of this group
+    const float* Am = A + (size_t)map * L * L;
+    const int cc = threadIdx.x % CP_COLS, rg = threadIdx.x / CP_COLS;
+    const int ncols = gb * bs + 2 * hk;
+    const int q = Jg * bs - hk + cc;
+    const int p0 = max(0, I * bs - hk), p1 = min(L, I * bs + bs + hk);
+    double a0 = 0.0, a1 = 0.0;
+    if (cc < ncols && q >= 0 && q < L) {
+        const int J0 = q / bs, c = q - J0 * bs;
+        int dq1 = 0;
+        bool has1 = false;
+        if (c < hk) {  // reaches into the block on the left
+            dq1 = c + bs;
+            has1 = J0 > 0;
+        } else if (c >= bs - hk) {  // ... on the right
+            dq1 = c - bs;
+            has1 = J0 + 1 < nb;
+        }
+        auto weight = [&](int dp, int dq) {  // shifts t with dp - t and dq - t inside the block
+            const int lo = max(-hk, max(dp, dq) - bs + 1), hi = min(hk, min(dp, dq));
+            return max(0, hi - lo + 1);
+        };
+        const float* col = Am + q;
+#pragma unroll 8
+        for (int p = p0 + rg; p < p1; p += CP_RG) {
+            const int dp = p - I * bs;
+            const double v = (double)col[(size_t)p * L];
+            a0 += v * (double)weight(dp, c);
+            if (has1) a1 += v * (double)weight(dp, dq1);
+        }
+    }
+    part[rg][0][cc] = a0;
+    part[rg][1][cc] = a1;
+    __syncthreads();
+    // wavefront b adds up block b: entries e = 0 .. CP_RG (bs + 2 hk) - 1, lane-strided, then a butterfly
+    const int b = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (b < gb && Jg + b < nb) {
+        const int base = hk + b * bs, span = bs + 2 * hk;
+        double s = 0.0;
+        for (int e = lane; e < CP_RG * span; e += 64) {
+            const int r = e / span, k = e - r * span - hk;  // column base + k, k = -hk .. bs + hk - 1
+            s += part[r][(k < 0 || k >= bs) ? 1 : 0][base + k];
+        }
+        for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+        if (lane == 0) pooled[((size_t)map * nb + I) * nb + Jg + b] = (float)(s / ((double)bs * (double)bs));
+    }
 }
 
 __device__ __forceinline__ uint32_t float_key(float f) {  // order-preserving map to unsigned
@@ -313,8 +374,15 @@ int pattern_generate(const float* Score, int n_maps, int L, int bs, int ksize, i
         }
         pooled = g_pool_ws;
     }
-    hipLaunchKernelGGL(conv_pool_kernel, dim3(nb, nb, n_maps), dim3(POOL_THREADS), 0, stream, Score, pooled, L, bs, nb,
-                       ksize / 2);
+    const int hk = ksize / 2;
+    // blocks per work-group of the streaming kernel (0: block size too small for it, or too wide)
+    const int gb = bs >= 2 * hk && bs + 2 * hk <= CP_COLS ? std::min((CP_COLS - 2 * hk) / bs, CP_COLS * CP_RG / 64) : 0;
+    if (gb > 0)
+        hipLaunchKernelGGL(conv_pool_cols_kernel, dim3((nb + gb - 1) / gb, nb, n_maps), dim3(CP_COLS * CP_RG), 0, stream,
+                           Score, pooled, L, bs, nb, hk, gb);
+    else
+        hipLaunchKernelGGL(conv_pool_kernel, dim3(nb, nb, n_maps), dim3(POOL_THREADS), 0, stream, Score, pooled, L, bs,
+                           nb, hk);
     if (!check_launch("conv_pool_kernel")) return 1;
     int topk = 0;
     if (mode == SPION_PATTERN_TOPK) topk = (int)((double)(nb * nb) * param - (double)nb);  // main_conv.py:247
