@@ -186,7 +186,7 @@ def bench_pattern_discovery(args, dev):
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
         "data": "synthetic (seeded softmax(QK^T) maps with a diagonal band boost)",
         "config": {"workload": f"config2: {n_maps} score maps {L}x{L}, 31x31 diagonal filter, {bs}x{bs} pooling, q={q}"},
-        "roofline": {"bound": "hbm", "kernel": "conv_pool_kernel + threshold_walk_kernel", "achieved": bytes_read / t_evt / 1e6,
+        "roofline": {"bound": "hbm", "kernel": "conv_pool_cols_kernel + threshold_walk_kernel", "achieved": bytes_read / t_evt / 1e6,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": bytes_read / t_evt / 1e6 / PEAK_HBM_GBS, "traffic": None,
                      "event_ms": t_evt},
         "cpu_baseline": {"value": n_maps / (cpu_ms / 1e3), "unit": "maps/s", "cores": min(os.cpu_count() or 1, torch.get_num_threads()),
