@@ -325,7 +325,8 @@ struct PatternIndex {
     int* d_blob = nullptr;  // one allocation holding every array below
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
-    int *d_rdesc = nullptr, *d_cdesc = nullptr;  // per strip in launch order: {strip, first tile, tiles, P offset}
+    // per strip in launch order, {strip, first tile, tiles, P offset}: row pass, forward, column pass
+    int *d_rdesc = nullptr, *d_fdesc = nullptr, *d_cdesc = nullptr;
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
     // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
@@ -530,7 +531,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         return o;
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
-    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_cdesc = 0;
+    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0;
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -567,22 +568,39 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         };
         append_order(trp, true);
         append_order(tcp, false);
-        // One 16-byte descriptor per strip in that order, {strip, first tile, tiles, offset of the strip's first
+        // One 16-byte descriptor per strip in launch order, {strip, first tile, tiles, offset of the strip's first
         // element in a head's P}: a work-group learns everything about its strip from one scalar load instead of
-        // three dependent ones.
-        std::vector<int> rdesc(4 * (size_t)nbr), cdesc(4 * (size_t)nbr);
+        // three dependent ones.  The row pass walks the bucketed order above.  The forward and the column pass
+        // walk the strips by descending length (equal lengths in index order): the launch then ends on the
+        // shortest strips.  Measured: on one machine the north star's column pass went 0.203 -> 0.193 ms and the
+        // forward -1 %, on another neither moved; one round of 512 work-groups at L = 1024: forward 0.0094 ->
+        // 0.0088 ms; the row pass is 0-3 % slower in that order on the large shapes, hence its own.
+        auto by_length = [&](const std::vector<int>& ptr) {
+            std::vector<int> order(nbr);
+            for (int i = 0; i < nbr; ++i) order[i] = i;
+            std::stable_sort(order.begin(), order.end(),
+                             [&](int x, int y) { return ptr[x + 1] - ptr[x] > ptr[y + 1] - ptr[y]; });
+            return order;
+        };
+        const std::vector<int> rows_sorted = by_length(trp), cols_sorted = by_length(tcp);
+        std::vector<int> rdesc(4 * (size_t)nbr), fdesc(4 * (size_t)nbr), cdesc(4 * (size_t)nbr);
         for (int p = 0; p < nbr; ++p) {
-            const int I = trp[nbr + 1 + p], J = tcp[nbr + 1 + p];
+            const int I = trp[nbr + 1 + p], F = rows_sorted[p], J = cols_sorted[p];
             rdesc[4 * p + 0] = I;
             rdesc[4 * p + 1] = trp[I];
             rdesc[4 * p + 2] = trp[I + 1] - trp[I];
             rdesc[4 * p + 3] = off[I * 32];
+            fdesc[4 * p + 0] = F;
+            fdesc[4 * p + 1] = trp[F];
+            fdesc[4 * p + 2] = trp[F + 1] - trp[F];
+            fdesc[4 * p + 3] = off[F * 32];
             cdesc[4 * p + 0] = J;
             cdesc[4 * p + 1] = tcp[J];
             cdesc[4 * p + 2] = tcp[J + 1] - tcp[J];
             cdesc[4 * p + 3] = 0;
         }
         o_rdesc = append(rdesc);
+        o_fdesc = append(fdesc);
         o_cdesc = append(cdesc);
         pi.n_wg_row = (int)wgr.wg.size() / 4;
         pi.n_wg_col = (int)wgc.wg.size() / 4;
@@ -630,6 +648,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcp = pi.d_blob + o_tcp;
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
         pi.d_rdesc = pi.d_blob + o_rdesc;
+        pi.d_fdesc = pi.d_blob + o_fdesc;
         pi.d_cdesc = pi.d_blob + o_cdesc;
         pi.d_wg_row = pi.d_blob + o_wgr;
         pi.d_wg_col = pi.d_blob + o_wgc;
@@ -750,11 +769,11 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     do {                                                                                                             \
         if (pi.max_row_tiles <= W * MAXT)                                                                            \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, MAXT, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,        \
-                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_rdesc, pi.d_tcol, a->L, nbr,     \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr,     \
                                a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
         else                                                                                                         \
             hipLaunchKernelGGL((tile_fwd_kernel<D, W, MASK, 0, KROW, ST>), dim3(nbr * a->NB), dim3(64 * W), 0,           \
-                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_rdesc, pi.d_tcol, a->L, nbr,     \
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr,     \
                                a->NB, nnz, a->scale, 0, nbr, hc, ly);                                                    \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
