@@ -120,3 +120,81 @@ def test_random_dense_shapes(seed):
     dQ, dK, dV = oda.dense_attention_backward(f(Q), f(K), f(V), P, f(dO))
     for name, ref in (("P", P), ("O", O), ("dQ", dQ), ("dK", dK), ("dV", dV)):
         assert_close(got[name], ref, what=f"seed {seed}: dense L={L} d={d} NB={NB} mask={with_mask} {name}")
+
+
+def _random_views(rng, B, H, L, d, n, gen, fill=None):
+    """n [B, H, L, d] views in one of the memory layouts a layer produces, drawn at random: contiguous, each a
+    [B, L, H*d] projection, slices of one fused buffer, the latter two with padded rows."""
+    kind = str(rng.choice(["plain", "proj", "fused"]))
+    pad = int(rng.choice([0, 4, 12]))
+    if kind == "plain":
+        views = [torch.randn(B, H, L, d, generator=gen).cuda() for _ in range(n)]
+    elif kind == "proj":
+        views = [torch.randn(B, L, H, d + pad, generator=gen).cuda()[..., :d].transpose(1, 2) for _ in range(n)]
+    else:
+        buf = torch.randn(B, L, n, H, d + pad, generator=gen).cuda()
+        views = [buf[:, :, i, :, :d].transpose(1, 2) for i in range(n)]
+    if fill is not None:
+        for v in views:
+            v.fill_(fill)
+    return kind, views
+
+
+@pytest.mark.parametrize("seed", range(500, 510))
+def test_random_strided_heads(seed):
+    """The strided entry points of the sparse and the dense phase on random shapes, patterns and memory layouts:
+    bit for bit what the row-major entry points / the reference's ABI give for contiguous copies, which the other
+    sweeps hold against the oracle."""
+    from spion_amd import _lib
+    from spion_amd.attention import Attention
+    from tests.test_gpu_dense import _run_dense
+    import ctypes
+
+    c = _draw(seed, [32])
+    rng = np.random.default_rng(seed + 7)
+    H = int(rng.choice([1, 2, 3]))
+    B = max(1, c["NB"] // H)
+    NB, L, d = B * H, c["L"], 32
+    pen = c["pen"]
+    if pen is not None:
+        pen = pen[:1].repeat(NB, 1).contiguous()
+    gen = torch.Generator().manual_seed(seed)
+    kq, (q, k, v) = _random_views(rng, B, H, L, d, 3, gen)
+    ko, (out, dout) = _random_views(rng, B, H, L, d, 2, gen)
+    kg, (dq, dk, dv) = _random_views(rng, B, H, L, d, 3, gen, fill=float("nan"))
+    tag = f"{c['tag']} B={B} H={H} layouts {kq}/{ko}/{kg}"
+    flat = lambda t: t.reshape(NB, L, d).contiguous()
+    # sparse
+    sm, off, col = osa.build_csr_from_block_mask(c["mat"], c["bs"])
+    abi = SparseABI(d, L, NB, c["bs"], with_mask=pen is not None)
+    abi.set_pattern(sm, off, col)
+    P = abi.forward_strided(q, k, v, out, pen)
+    abi.backward_strided(q, k, v, P, out, dout, dq, dk, dv)
+    O2, P2 = abi.forward_rowmajor(flat(q), flat(k), flat(v), pen)
+    g2 = abi.backward_rowmajor(flat(q), flat(k), flat(v), P2, O2, flat(dout))
+    torch.cuda.synchronize()
+    assert torch.equal(P, P2) and torch.equal(flat(out), O2), tag
+    for name, a, b in zip(("dQ", "dK", "dV"), (dq, dk, dv), g2):
+        assert torch.equal(flat(a), b), f"{tag}: sparse {name}"
+    abi.close()
+    # dense phase
+    lib = Attention._cuda_mask_compile_module() if pen is not None else Attention._cuda_compile_module()
+    h = lib.init(d, L, NB)
+    _lib.check_error("init")
+    attn = torch.full((NB, L, L), float("nan"), device="cuda")
+    lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+    A = ctypes.addressof
+    core = _lib.core()
+    core.spion_dense_forward_strided(h, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen.data_ptr() if pen is not None else None,
+                                     attn.data_ptr(), out.data_ptr(), H, A(lin), A(lout))
+    _lib.check_error("dense forward strided")
+    core.spion_dense_backward_strided(h, q.data_ptr(), k.data_ptr(), v.data_ptr(), attn.data_ptr(), out.data_ptr(),
+                                      dout.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), H, A(lin), A(lout),
+                                      A(lgrad))
+    _lib.check_error("dense backward strided")
+    torch.cuda.synchronize()
+    lib.destroy(h)
+    ref = _run_dense(d, L, NB, flat(q), flat(k), flat(v), flat(dout), pen)
+    got = dict(O=flat(out), P=attn.transpose(1, 2), dQ=flat(dq), dK=flat(dk), dV=flat(dv))
+    for name in ("P", "O", "dQ", "dK", "dV"):
+        assert np.array_equal(got[name].cpu().numpy(), ref[name]), f"{tag}: dense {name}"
