@@ -706,6 +706,15 @@ def main():
     if wl["name"] == "north_star":  # the workload the committed byte counters were taken on
         roof["traffic"] = _profiled_traffic_bytes(dom)
     roof["kernel_ms"] = {k_: round(v_, 4) for k_, v_ in kernels.items()}
+    if path == 2:
+        # what the element kernels actually move: per pattern entry two gathered rows of d floats (K and V in the
+        # forward and the row pass, Q and dO in the column pass), served by the caches, not by HBM
+        gbytes = 2.0 * 4.0 * d * nnz * NB
+        roof["gathered_rows"] = {
+            "gbytes_per_kernel": round(gbytes / 1e9, 2),
+            "tbytes_per_s": {k_: round(gbytes / v_ / 1e9, 2) for k_, v_ in kernels.items()},
+            "what": "bytes of gathered operand rows per kernel over its time; for scale, 256 CUs x 64 B per clock "
+                    "at 2.4 GHz of vector L1 bandwidth would be 39 TB/s"}
     if path == 1:
         # MFMA work a tile costs each kernel against its algorithmic share: the column pass recomputes dP (1.5x);
         # the forward is taken in its register-resident form (1x; its two-sweep form for very long rows is 1.5x)
