@@ -48,6 +48,34 @@ def _event_ms(fn, iters, warm=3):
     return start.elapsed_time(end) / iters
 
 
+def _spin_up(step, min_ms=300.0):
+    """Untimed repetitions of ``step`` for at least ``min_ms`` of wall time, in batches separated by a
+    synchronisation.  The shader clock of an idle MI355X needs some tens of milliseconds of continuous load to
+    reach its steady value; without this a short run (few warm-up steps) is timed on the ramp.  Returns the
+    wall time spent, in ms."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while True:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+        el = 1e3 * (time.perf_counter() - t0)
+        if el >= min_ms:
+            return el
+
+
+def _timed_steps(step, steps, warmup):
+    """``warmup`` untimed steps, then exactly ``steps`` timed ones between two synchronisations: ms per step."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return 1e3 * (time.perf_counter() - t0) / steps
+
+
 def _profiled_traffic_bytes(kernel):
     """HBM bytes per launch of ``kernel`` on the north-star workload as measured with rocprofv3 --pmc
     (FETCH_SIZE / WRITE_SIZE scaled by a copy kernel of known size): the 'HBM MiB/launch' column of the
@@ -163,14 +191,8 @@ def bench_pattern_discovery(args, dev):
     def step():
         return spion_amd.discover_block_masks(maps, bs, mode="conv_ff", threshold=q)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    spinup_ms = _spin_up(step, args.spinup_ms)
+    ms_step = _timed_steps(step, args.steps, args.warmup)
     t_evt = _event_ms(step, max(10, args.steps))
     bytes_read = 4.0 * L * L * n_maps
     t1 = time.perf_counter()
@@ -183,7 +205,7 @@ def bench_pattern_discovery(args, dev):
     return {
         "metric": "pattern discovery (conv filter + block pool + quantile + path walk), maps per second, 1 GPU",
         "value": n_maps / (ms_step / 1e3), "unit": "maps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
         "data": "synthetic (seeded softmax(QK^T) maps with a diagonal band boost)",
         "config": {"workload": f"config2: {n_maps} score maps {L}x{L}, 31x31 diagonal filter, {bs}x{bs} pooling, q={q}"},
         "roofline": {"bound": "hbm", "kernel": "conv_pool_cols_kernel + threshold_walk_kernel", "achieved": bytes_read / t_evt / 1e6,
@@ -222,14 +244,8 @@ def bench_encoder_step(args, dev):
         loss.mean().backward()
         opt.step()
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    spinup_ms = _spin_up(step, args.spinup_ms)
+    ms_step = _timed_steps(step, args.steps, args.warmup)
 
     # attention share: the two layers' C-ABI kernels, from HIP events around a forward+backward of one layer's
     # attention core at the same shape
@@ -247,7 +263,7 @@ def bench_encoder_step(args, dev):
     return {
         "metric": "2-layer sparse encoder training step (fwd+bwd+AdamW), samples per second, 1 GPU",
         "value": B / (ms_step / 1e3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (uniform token ids, uniform labels, random-init weights)",
         "config": {"workload": f"config3: 2-layer encoder step, batch {B}, L={L}, d_model 64, FFN 128, H={H}, d_head {d}, "
                                f"block {cfg['block_size']}, discovered block densities {[round(x, 3) for x in density]}"},
@@ -289,14 +305,8 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
         out, _ = module(q, k, v, ones, mat)
         out.backward(do)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    spinup_ms = _spin_up(step, args.spinup_ms)
+    ms_step = _timed_steps(step, args.steps, args.warmup)
 
     core = _lib.core()
     idx = module.csr_cache.get(mat, bs)
@@ -342,7 +352,7 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
     result = {
         "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": f"synthetic (seeded N(0,1)*{in_scale:g} tensors rounded to bf16, seeded block mask)",
         "config": {"workload": f"{shape}{'_bf16' if shape != 'config5' else ''}: bf16 sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, block {bs}, "
                                f"nnz/head={nnz}, block density={round(float(mat_np.mean()), 4)}",
@@ -387,14 +397,8 @@ def bench_dense_phase(args, dev):
         out, _ = module(q, k, v, ones)
         out.backward(do)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    spinup_ms = _spin_up(step, args.spinup_ms)
+    ms_step = _timed_steps(step, args.steps, args.warmup)
     # the same step through the reference's ABI (feature-major operands: four transposes a step)
     module.reads_views = False
     for _ in range(max(3, args.warmup // 4)):
@@ -455,7 +459,7 @@ def bench_dense_phase(args, dev):
     result = {
         "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded N(0,1) tensors)",
         "config": {"workload": f"dense_phase: softmax attention fwd+bwd with the full probability map, B={B} H={H} L={L} d={d}"},
         "algorithmic": {"gflop": alg_flops / 1e9, "map_gbytes": 4.0 * NB * L * L / 1e9},
@@ -492,6 +496,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="north_star")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-config1", action="store_true", help="north_star only: leave out the L = 1024 sub-object")
+    ap.add_argument("--spinup-ms", type=float, default=300.0,
+                    help="untimed repetitions of the step for this long before the warm-up (clock ramp)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB device copy a few times (calibrates rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -530,7 +537,24 @@ def main():
         print(json.dumps(bench_bf16_scale_up(args, dev, "north_star")))
         return
 
-    wl = build_workload(args.workload)
+    result = bench_sparse_layer(args, dev, args.workload, full=True)
+    if args.workload == "north_star" and not args.no_config1:
+        # the metric is quoted at L = 1024 and L = 4096: the L = 1024 point (configuration 1) rides in the same line
+        c1 = bench_sparse_layer(args, dev, "config1", full=False)
+        result["config1"] = {k_: c1[k_] for k_ in ("value", "unit", "ms_per_step", "spinup_ms", "config", "hip_graph",
+                                                    "rowmajor_abi_ms", "kernels_effective_tflops", "roofline",
+                                                    "algorithmic") if k_ in c1}
+    print(json.dumps(result))
+
+
+def bench_sparse_layer(args, dev, workload, full=True):
+    """Forward + backward of the drop-in sparse attention module on one of the fp32 workloads.  ``full`` adds the
+    legs that only describe the default workload further (reference-ABI timings, projection views, CPU baseline)."""
+    import spion_amd
+    from spion_amd import _lib, workloads
+    from spion_amd.attention import Attention
+
+    wl = build_workload(workload)
     B, H, L, d, bs, nnz = wl["B"], wl["H"], wl["L"], wl["d"], wl["bs"], wl["nnz"]
     NB = B * H
     q, k, v, do = workloads.qkv(B, H, L, d, scale=wl["scale"], seed=0, device=dev)
@@ -561,14 +585,8 @@ def main():
         out, _ = module(q, k, v, key_mask, mat)
         out.backward(do)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+    spinup_ms = _spin_up(step, args.spinup_ms)
+    ms_step = _timed_steps(step, args.steps, args.warmup)
     path = _lib.core().spion_last_path(handle)
 
     # ---- the same step recorded once as a HIP graph and replayed (what a launch-bound caller would do) ----------
@@ -586,14 +604,8 @@ def main():
         with torch.cuda.graph(graph):
             out_g, _ = module(q, k, v, key_mask, mat)
             out_g.backward(do)
-        for _ in range(args.warmup):
-            graph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            graph.replay()
-        torch.cuda.synchronize()
-        graph_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+        _spin_up(graph.replay, min(args.spinup_ms, 100.0))
+        graph_ms = _timed_steps(graph.replay, args.steps, args.warmup)
         del graph, out_g
     except Exception as e:  # the eager figures above stand on their own
         graph_ms = f"capture failed: {type(e).__name__}: {e}"
@@ -602,7 +614,7 @@ def main():
     _lib.use_current_stream(module, dev)  # the capture left the handle on its own stream
     # ---- the same step with the heads as the layer hands them over: views of [B, L, H*d] projections ------
     views = None
-    if getattr(module, "reads_views", False):
+    if full and getattr(module, "reads_views", False):
         qv, kv, vv = (t.detach().transpose(1, 2).contiguous().transpose(1, 2).requires_grad_() for t in (q, k, v))
         dov = do.transpose(1, 2).contiguous().transpose(1, 2)
 
@@ -615,14 +627,7 @@ def main():
         views = {}
         for name, flag in (("in_place_ms", True), ("with_copies_ms", False)):
             module.reads_views = flag
-            for _ in range(args.warmup):
-                step_views()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                step_views()
-            torch.cuda.synchronize()
-            views[name] = round(1e3 * (time.perf_counter() - t0) / args.steps, 4)
+            views[name] = round(_timed_steps(step_views, args.steps, args.warmup), 4)
         module.reads_views = True
         views["what"] = ("module step on heads that are views of [B,L,H*d] projections: read and written in place "
                          "by the strided entry points, against the reference's contiguous copies first")
@@ -731,6 +736,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_step,
+        "spinup_ms": round(spinup_ms, 1),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -762,9 +768,10 @@ def main():
         result["hip_graph"] = {"error": graph_ms}
     if views:
         result["projection_views"] = views
-    if not args.no_cpu_baseline:
+    if full and not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(wl)
-    print(json.dumps(result))
+    cpp.destroy(handle)
+    return result
 
 
 if __name__ == "__main__":

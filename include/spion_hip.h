@@ -185,20 +185,36 @@ void spion_clear_error(void);
 /* Launch this handle's work on `stream` (a hipStream_t; NULL = null stream).  Any family. */
 void spion_set_stream(void* handle, void* stream);
 
-/* Forget the analysed pattern of a sparse handle.  The analysis is cached under the key
- * (Offsets pointer, Columns pointer, nnz); call this if index arrays were rewritten in place. */
+/* The analysis of a pattern (tile detection, transposed index) is cached per handle under the key
+ * (Offsets pointer, Columns pointer, nnz), up to 8 patterns per handle, least recently used evicted.  The key
+ * says nothing about the arrays' contents.  A caller that frees index arrays, or rewrites them in place, MUST
+ * drop the key before the addresses can carry another pattern -- with spion_forget_pattern for that one pair of
+ * arrays, or spion_invalidate_pattern for everything the handle holds; otherwise a later pattern at the same
+ * addresses with the same nnz silently runs on the old index.  (The Python modules do this when their mask
+ * cache evicts an entry.) */
 void spion_invalidate_pattern(void* handle);
+void spion_forget_pattern(void* handle, const int* Offsets, const int* Columns);
+
+/* Analyse a pattern ahead of its first use from HOST copies of the index arrays (host_Offsets [L+1],
+ * host_Columns [nnz]: host pointers) and file it under the device arrays Offsets / Columns: the first
+ * attn_forward with that pair then copies nothing back to the host and does not wait for the stream -- what a
+ * loader of saved masks does once per mask (the reference rebuilds the index on every forward,
+ * models/attention_blockcuda.py:26-43, and loads masks in main_inference.py:164-172).  Also the way to make a
+ * pattern known before a HIP graph capture.  Returns 0 on success; on a
+ * malformed index nothing is filed and the error is recorded. */
+int spion_register_pattern(void* handle, const int* Offsets, const int* Columns, int nnz,
+                           const int* host_Offsets, const int* host_Columns);
 
 /* Which kernel family the last forward/backward of a sparse handle used:
  * 0 = none yet, 1 = MFMA 32x32 tile path, 2 = element (gather) path. */
 int spion_last_path(void* handle);
 
-/* Force the element path even for tile-structured patterns (testing / comparison). */
-void spion_force_element_path(void* handle, int on);
-
-/* Profiling aid: run only part of a sparse handle's backward.  bit 0 = row pass (row sums and dQ),
- * bit 1 = column pass (dK, dV; needs the row sums of an earlier row pass).  Default 3 = both. */
-void spion_set_backward_passes(void* handle, int mask);
+/* Most recent failure recorded by a call on THIS handle ("" if none), besides the process-wide slot of
+ * spion_last_error, which any thread or handle can overwrite.  Every failure is also written to stderr unless
+ * the environment has SPION_QUIET=1; SPION_ABORT_ON_ERROR=1 makes a failure abort the process (for callers of the
+ * void-returning drop-in symbols, who have no other signal). */
+const char* spion_handle_error(void* handle);
+void spion_clear_handle_error(void* handle);
 
 /* The forward of the MFMA tile path keeps a private copy of Out, filed under the Attn pointer it filled
  * (up to 4 per handle, NB*L*d floats each); a backward given the same P pointer then gets its softmax

@@ -1,0 +1,24 @@
+/*
+ * spion_hip_debug.h -- testing and profiling aids of libspion_hip.so.  Not product surface: nothing in a
+ * deployment needs them; the test-suite and the benchmark use them to compare kernel families and to time the
+ * two backward kernels separately.  No counterpart in the reference.
+ */
+#ifndef SPION_HIP_DEBUG_H
+#define SPION_HIP_DEBUG_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Force the element path even for tile-structured patterns (testing / comparison).  Drops every analysed
+ * pattern of the handle. */
+void spion_force_element_path(void* handle, int on);
+
+/* Run only part of a sparse handle's backward.  bit 0 = row pass (row sums and dQ), bit 1 = column pass (dK, dV;
+ * needs the row sums of an earlier row pass).  Default 3 = both. */
+void spion_set_backward_passes(void* handle, int mask);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPION_HIP_DEBUG_H */

@@ -36,7 +36,9 @@ def _cdll(name: str) -> ctypes.CDLL:
             f"{path} is missing: build the HIP libraries first (python -m spion_amd.build). "
             "spion_amd has no CPU fallback."
         )
-    lib = ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+    # default (local) symbol scope, as the reference loads its libraries: the drop-ins' generic names (init,
+    # destroy, ...) stay out of the process-wide scope; they find libspion_hip.so through DT_NEEDED + $ORIGIN
+    lib = ctypes.CDLL(path)
     _cache[name] = lib
     return lib
 
@@ -54,6 +56,14 @@ def core() -> ctypes.CDLL:
     lib.spion_set_stream.restype = None
     lib.spion_invalidate_pattern.argtypes = [_P]
     lib.spion_invalidate_pattern.restype = None
+    lib.spion_forget_pattern.argtypes = [_P, _P, _P]
+    lib.spion_forget_pattern.restype = None
+    lib.spion_register_pattern.argtypes = [_P, _P, _P, c_int, _P, _P]
+    lib.spion_register_pattern.restype = c_int
+    lib.spion_handle_error.argtypes = [_P]
+    lib.spion_handle_error.restype = c_char_p
+    lib.spion_clear_handle_error.argtypes = [_P]
+    lib.spion_clear_handle_error.restype = None
     lib.spion_last_path.argtypes = [_P]
     lib.spion_last_path.restype = c_int
     lib.spion_force_element_path.argtypes = [_P, c_int]

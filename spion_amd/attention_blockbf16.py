@@ -76,7 +76,7 @@ class BlockAttentionBF16(nn.Module):
             attn_handle = self.lib.spion_block_bf16_init(self.emb_dim, self.seq_len, self.num_batches, self.block_size)
             _lib.check_error("spion_block_bf16_init")
         self.attn_handle = attn_handle
-        self.csr_cache = CsrCache()
+        self.csr_cache = CsrCache(handle=attn_handle)
 
     def forward(self, query, key, value, mask, mat):
         return _BlockBF16Function.apply(query, key, value, mask, mat, self), 0

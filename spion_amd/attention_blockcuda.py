@@ -152,7 +152,7 @@ class _BlockAttentionBase(nn.Module):
         self.num_blocks = int(self.seq_len / self.block_size)
         self.attn_cpp = attn_cpp
         self.attn_handle = attn_handle
-        self.csr_cache = CsrCache()
+        self.csr_cache = CsrCache(handle=attn_handle)
         self.attn_func = _BlockAttnFunction
         _lib.core().spion_use_output_cache(attn_handle, 0)  # the backward is handed the output instead
         # block masks whose blocks are unions of 32x32 tiles run on the tile kernels; those for d = 32 take views

@@ -5,6 +5,11 @@ The reference rebuilds the index on every forward call with an O(L^2) nearest-ne
 is built once per distinct mask (one host round trip) and reused; a cache entry keeps a reference to the
 mask tensor, so neither its address nor its version counter can be recycled while the entry lives.
 
+The library analyses an index once per (Offsets address, Columns address, nnz) and trusts that key.  A cache
+that belongs to a handle therefore registers every new index with the library straight from its host arrays
+(no copy back, no wait for the stream in the first forward) and tells the library to forget an index when its
+entry is evicted -- before torch can hand the freed addresses to another index.
+
 Layout produced (all int32, on the mask's device), as the C ABI expects:
   sum_mat [L]   entries per row  = block_size * (non-zero blocks in the row's block row)
   offsets [L+1] exclusive prefix sum of sum_mat
@@ -49,12 +54,60 @@ def block_mask_to_csr_host(mat: np.ndarray, block_size: int):
     return sum_mat, offsets.astype(np.int32), columns.astype(np.int32)
 
 
-class CsrCache:
-    """LRU cache: (mask storage address, version, shape, block size) -> CsrIndex."""
+def index_from_host(sum_mat: np.ndarray, offsets: np.ndarray, columns: np.ndarray, device, handle=None,
+                    keepalive=None) -> CsrIndex:
+    """Device copies of a host-built CSR index; with ``handle`` the pattern is registered with the library from
+    the host arrays (spion_register_pattern), so that its first use neither copies the index back nor waits."""
+    offsets = np.ascontiguousarray(offsets, dtype=np.int32)
+    columns = np.ascontiguousarray(columns, dtype=np.int32)
+    sum_mat = np.ascontiguousarray(sum_mat, dtype=np.int32)
+    nnz = int(offsets[-1])
+    entry = CsrIndex(
+        sum_mat=torch.from_numpy(sum_mat).to(device),
+        offsets=torch.from_numpy(offsets).to(device),
+        columns=torch.from_numpy(columns).to(device) if columns.size else torch.zeros(1, dtype=torch.int32, device=device),
+        nnz=nnz,
+        keepalive=keepalive,
+    )
+    if handle:
+        from . import _lib
 
-    def __init__(self, capacity: int = 8):
+        rc = _lib.core().spion_register_pattern(handle, entry.offsets.data_ptr(), entry.columns.data_ptr(), nnz,
+                                                offsets.ctypes.data, columns.ctypes.data if columns.size else None)
+        if rc != 0:
+            _lib.check_error("spion_register_pattern")
+    return entry
+
+
+class CsrCache:
+    """LRU cache: (mask storage address, version, shape, block size) -> CsrIndex.  ``handle``: the sparse handle
+    the indices are used with (None: indices are not registered and evictions are not reported)."""
+
+    def __init__(self, capacity: int = 8, handle=None):
         self.capacity = capacity
+        self.handle = handle
         self._entries: "OrderedDict[tuple, CsrIndex]" = OrderedDict()
+
+    def _forget(self, entry: CsrIndex) -> None:
+        if self.handle:
+            from . import _lib
+
+            _lib.core().spion_forget_pattern(self.handle, entry.offsets.data_ptr(), entry.columns.data_ptr())
+
+    def put(self, mat: torch.Tensor, block_size: int, entry: CsrIndex) -> None:
+        """File a prebuilt index (a sidecar built when the masks were loaded) under ``mat``."""
+        key = (mat.data_ptr(), mat._version, tuple(mat.shape), tuple(mat.stride()), int(block_size), str(mat.device))
+        old = self._entries.pop(key, None)
+        if old is not None and old is not entry:
+            self._forget(old)
+        entry.keepalive = mat
+        self._entries[key] = entry
+        self._trim()
+
+    def _trim(self) -> None:
+        while len(self._entries) > self.capacity:
+            _, old = self._entries.popitem(last=False)
+            self._forget(old)
 
     def get(self, mat: torch.Tensor, block_size: int) -> CsrIndex:
         key = (mat.data_ptr(), mat._version, tuple(mat.shape), tuple(mat.stride()), int(block_size), str(mat.device))
@@ -65,15 +118,7 @@ class CsrCache:
         if mat.dim() != 2 or mat.shape[0] != mat.shape[1]:
             raise ValueError(f"block mask must be square [nb, nb], got {tuple(mat.shape)}")
         sum_mat, offsets, columns = block_mask_to_csr_host(mat.detach().cpu().numpy(), block_size)
-        dev = mat.device
-        entry = CsrIndex(
-            sum_mat=torch.from_numpy(sum_mat).to(dev),
-            offsets=torch.from_numpy(offsets).to(dev),
-            columns=torch.from_numpy(columns).to(dev) if columns.size else torch.zeros(1, dtype=torch.int32, device=dev),
-            nnz=int(offsets[-1]),
-            keepalive=mat,
-        )
+        entry = index_from_host(sum_mat, offsets, columns, mat.device, self.handle, keepalive=mat)
         self._entries[key] = entry
-        while len(self._entries) > self.capacity:
-            self._entries.popitem(last=False)
+        self._trim()
         return entry

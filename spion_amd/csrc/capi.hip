@@ -1,20 +1,38 @@
 // extern "C" surface of libspion_hip.so (declared in include/spion_hip.h) and the error slot.
 #include "common.h"
+
+#include <cstdlib>
 #include "../../include/spion_hip.h"
 
 namespace spion {
 
 static std::mutex g_err_mutex;
 static std::string g_err;
+static thread_local HandleHeader* t_handle = nullptr;
 
+void note_current_handle(HandleHeader* h) { t_handle = h; }
+
+// The entry points return void like the reference's, and the reference's Python never asks for an error: so a
+// failure is also written to stderr (SPION_QUIET=1 silences it) and SPION_ABORT_ON_ERROR=1 turns it into an abort,
+// for callers that would otherwise go on with unwritten output buffers.
 void set_error(const char* fmt, ...) {
     char buf[1024];
     va_list ap;
     va_start(ap, fmt);
     vsnprintf(buf, sizeof(buf), fmt, ap);
     va_end(ap);
-    std::lock_guard<std::mutex> lock(g_err_mutex);
-    g_err = buf;
+    {
+        std::lock_guard<std::mutex> lock(g_err_mutex);
+        g_err = buf;
+        if (t_handle) {
+            strncpy(t_handle->err, buf, sizeof(t_handle->err) - 1);
+            t_handle->err[sizeof(t_handle->err) - 1] = 0;
+        }
+    }
+    const char* quiet = getenv("SPION_QUIET");
+    if (!quiet || quiet[0] != '1') fprintf(stderr, "spion_hip: error: %s\n", buf);
+    const char* fatal = getenv("SPION_ABORT_ON_ERROR");
+    if (fatal && fatal[0] == '1') abort();
 }
 bool error_pending() {
     std::lock_guard<std::mutex> lock(g_err_mutex);
@@ -43,6 +61,8 @@ void dense_forward_strided(void*, const float*, const float*, const float*, cons
 void dense_backward_strided(void*, const float*, const float*, const float*, const float*, const float*, const float*,
                             float*, float*, float*, int, const HeadLayout&, const HeadLayout&, const HeadLayout&);
 void sparse_invalidate(void*);
+int sparse_register_pattern(void*, const int*, const int*, int, const int*, const int*);
+void sparse_forget_pattern(void*, const int*, const int*);
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
@@ -69,6 +89,7 @@ extern "C" {
 
 // ---- sparse, bf16 tensors (no reference counterpart) ---------------------------------------------
 void* spion_block_bf16_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    note_current_handle(nullptr);
     return sparse_bf16_init(emb_dim, seq_len, num_batches, block_size);
 }
 void spion_block_bf16_attn_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
@@ -86,6 +107,7 @@ void spion_block_bf16_destroy(void* h) { sparse_destroy(h); }
 
 // ---- sparse, no key mask -----------------------------------------------------------------------
 void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    note_current_handle(nullptr);
     return sparse_init(emb_dim, seq_len, num_batches, block_size, false);
 }
 void spion_block_attn_forward(void* h, const float* Q, const float* Kt, const float* V, float* Attn, float* Out,
@@ -103,6 +125,7 @@ void spion_block_destroy(void* h) { sparse_destroy(h); }
 
 // ---- sparse, key mask --------------------------------------------------------------------------
 void* spion_blockmask_init(int emb_dim, int seq_len, int num_batches, int block_size) {
+    note_current_handle(nullptr);
     return sparse_init(emb_dim, seq_len, num_batches, block_size, true);
 }
 void spion_blockmask_attn_forward(void* h, const float* Q, const float* Kt, const float* V, const float* Mask,
@@ -121,6 +144,7 @@ void spion_blockmask_destroy(void* h) { sparse_destroy(h); }
 
 // ---- dense phase ---------------------------------------------------------------------------------
 void* spion_dense_init(int emb_dim, int seq_len, int num_batches) {
+    note_current_handle(nullptr);
     return dense_init(emb_dim, seq_len, num_batches, false);
 }
 void spion_dense_attn_forward(void* h, const float* Qt, const float* K, const float* Vt, float* Attn, float* Out) {
@@ -137,6 +161,7 @@ void spion_dense_attn_backward(void* h, const float* Qt, const float* Kt, const 
 void spion_dense_destroy(void* h) { dense_destroy(h); }
 
 void* spion_densemask_init(int emb_dim, int seq_len, int num_batches) {
+    note_current_handle(nullptr);
     return dense_init(emb_dim, seq_len, num_batches, true);
 }
 void spion_densemask_attn_forward(void* h, const float* Qt, const float* K, const float* Vt, const float* Mask,
@@ -156,12 +181,14 @@ void spion_densemask_destroy(void* h) { dense_destroy(h); }
 // ---- pattern discovery ---------------------------------------------------------------------------
 int spion_pattern_generate(const float* Score, int n_maps, int seq_len, int block_size, int conv_ksize, int mode,
                            double param, float* Mat, float* Pooled, float* Thresh, void* stream) {
+    note_current_handle(nullptr);
     return pattern_generate(Score, n_maps, seq_len, block_size, conv_ksize, mode, param, Mat, Pooled, Thresh,
                             static_cast<hipStream_t>(stream));
 }
 
 int spion_score_map_mean(const float* Attn, int batch, int heads, int seq_len, int key_major, float* Mean,
                          void* stream) {
+    note_current_handle(nullptr);
     return score_map_mean(Attn, batch, heads, seq_len, key_major, Mean, static_cast<hipStream_t>(stream));
 }
 
@@ -176,6 +203,15 @@ void spion_clear_error(void) {
     std::lock_guard<std::mutex> lock(g_err_mutex);
     g_err.clear();
 }
+const char* spion_handle_error(void* h) {
+    HandleHeader* hd = static_cast<HandleHeader*>(h);
+    if (!hd || (hd->magic != KIND_SPARSE && hd->magic != KIND_DENSE)) return "not a spion handle";
+    return hd->err;
+}
+void spion_clear_handle_error(void* h) {
+    HandleHeader* hd = static_cast<HandleHeader*>(h);
+    if (hd && (hd->magic == KIND_SPARSE || hd->magic == KIND_DENSE)) hd->err[0] = 0;
+}
 void spion_set_stream(void* h, void* stream) {
     HandleHeader* hd = static_cast<HandleHeader*>(h);
     if (!hd || (hd->magic != KIND_SPARSE && hd->magic != KIND_DENSE)) {
@@ -185,6 +221,11 @@ void spion_set_stream(void* h, void* stream) {
     hd->stream = static_cast<hipStream_t>(stream);
 }
 void spion_invalidate_pattern(void* h) { sparse_invalidate(h); }
+int spion_register_pattern(void* h, const int* Offsets, const int* Columns, int nnz, const int* host_Offsets,
+                           const int* host_Columns) {
+    return sparse_register_pattern(h, Offsets, Columns, nnz, host_Offsets, host_Columns);
+}
+void spion_forget_pattern(void* h, const int* Offsets, const int* Columns) { sparse_forget_pattern(h, Offsets, Columns); }
 int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
@@ -252,6 +293,7 @@ void spion_dense_backward_strided(void* h, const float* Q, const float* K, const
     dense_backward_strided(h, Q, K, V, P, Out, dO, dQ, dK, dV, heads, to_layout(in), to_layout(out), to_layout(grad));
 }
 int spion_transpose_last2(const float* in, float* out, int batch, int rows, int cols, void* stream) {
+    note_current_handle(nullptr);
     return transpose_last2(in, out, batch, rows, cols, static_cast<hipStream_t>(stream));
 }
 const char* spion_version(void) { return "spion_hip 0.1 (gfx950)"; }

@@ -35,7 +35,12 @@ enum HandleKind : uint32_t {
 struct HandleHeader {
     uint32_t magic;
     hipStream_t stream;
+    char err[256];  // most recent failure of a call on this handle ("" if none), besides the process-wide slot
 };
+
+// The handle the calling thread is working on (set by the handle checks of every entry point, cleared by
+// entry points without a handle): set_error files the message there as well.
+void note_current_handle(HandleHeader* h);
 
 inline bool check_launch(const char* what) {
     hipError_t e = hipGetLastError();

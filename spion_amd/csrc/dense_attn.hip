@@ -691,6 +691,7 @@ struct DenseAttn {
 
 static DenseAttn* as_dense(void* h, const char* who) {
     DenseAttn* a = static_cast<DenseAttn*>(h);
+    note_current_handle(a && a->hdr.magic == KIND_DENSE ? &a->hdr : nullptr);
     if (!a || a->hdr.magic != KIND_DENSE) {
         set_error("%s: not a dense-attention handle", who);
         return nullptr;
@@ -711,6 +712,7 @@ void* dense_init(int emb_dim, int seq_len, int num_batches, bool has_mask) {
     DenseAttn* a = new DenseAttn();
     a->hdr.magic = KIND_DENSE;
     a->hdr.stream = nullptr;
+    a->hdr.err[0] = 0;
     a->d = emb_dim;
     a->L = seq_len;
     a->NB = num_batches;
@@ -725,6 +727,7 @@ void dense_destroy(void* h) {
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_out) (void)hipFree(a->ws_out);
     a->hdr.magic = 0;
+    note_current_handle(nullptr);
     delete a;
 }
 

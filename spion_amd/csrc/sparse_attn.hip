@@ -345,7 +345,19 @@ struct SparseAttn {
     int d, L, NB, bs;
     bool has_mask;
     float scale;
+    // Analysed patterns, keyed by (Offsets pointer, Columns pointer, nnz): a handle that alternates between a few
+    // masks (one per layer, or train / eval masks) analyses each once.  `pat` is a non-owning view of the slot in
+    // use; the slots own the device memory.  A key says nothing about the arrays' contents: whoever frees or
+    // rewrites index arrays must drop the key (spion_forget_pattern / spion_invalidate_pattern).
+    static constexpr int PAT_SLOTS = 8;
+    PatternIndex pats[PAT_SLOTS];
+    uint64_t pat_stamp[PAT_SLOTS] = {};
+    uint64_t pat_clock = 0;
     PatternIndex pat;
+    void release_patterns() {
+        for (auto& p : pats) p.release();
+        pat = PatternIndex();
+    }
     float* ws_rowsum = nullptr;  // [NB][L]   g of the backward (tile path)
     // Copies of O kept by the forward of the tile path, keyed by the Attn (P) buffer that forward
     // filled: a backward that is handed the same P pointer gets its row sums g_i = dO_i . O_i from the
@@ -371,6 +383,7 @@ struct SparseAttn {
 
 static SparseAttn* as_sparse(void* h, const char* who) {
     SparseAttn* a = static_cast<SparseAttn*>(h);
+    note_current_handle(a && a->hdr.magic == KIND_SPARSE ? &a->hdr : nullptr);
     if (!a || a->hdr.magic != KIND_SPARSE) {
         set_error("%s: not a sparse-attention handle", who);
         return nullptr;
@@ -398,6 +411,7 @@ void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, boo
     SparseAttn* a = new SparseAttn();
     a->hdr.magic = KIND_SPARSE;
     a->hdr.stream = nullptr;
+    a->hdr.err[0] = 0;
     a->d = emb_dim;
     a->L = seq_len;
     a->NB = num_batches;
@@ -410,13 +424,14 @@ void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, boo
 void sparse_destroy(void* h) {
     SparseAttn* a = as_sparse(h, "destroy");
     if (!a) return;
-    a->pat.release();
+    a->release_patterns();
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
     if (a->ws_part) (void)hipFree(a->ws_part);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
     a->hdr.magic = 0;
+    note_current_handle(nullptr);
     delete a;
 }
 
@@ -456,11 +471,11 @@ static WgList build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles
     return out;
 }
 
-// Copy the index to the host once, validate it, detect the tile structure and build the transposed
-// index.  Returns false (error recorded) if the CSR is inconsistent.
-static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Columns, int nnz) {
-    PatternIndex& pi = a->pat;
-    pi.release();
+// Copy the index to the host once (unless the caller hands over host copies), validate it, detect the tile
+// structure and build the transposed index.  Returns false (error recorded) if the CSR is inconsistent.
+static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Columns, int nnz,
+                            const int* host_off = nullptr, const int* host_col = nullptr) {
+    PatternIndex pi;
     const int L = a->L;
     if (nnz < 0) {
         set_error("pattern: nnz %d is negative", nnz);
@@ -470,13 +485,22 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         set_error("pattern: nnz %d too large (one head's map must stay under 2 GiB)", nnz);
         return false;
     }
-    std::vector<int> off(L + 1), col((size_t)nnz);
-    if (!SPION_HIP_OK(hipMemcpyAsync(off.data(), Offsets, sizeof(int) * (L + 1), hipMemcpyDeviceToHost, a->hdr.stream)))
-        return false;
-    if (nnz && !SPION_HIP_OK(hipMemcpyAsync(col.data(), Columns, sizeof(int) * (size_t)nnz, hipMemcpyDeviceToHost,
-                                            a->hdr.stream)))
-        return false;
-    if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
+    std::vector<int> off_copy, col_copy;
+    if (!host_off || (nnz && !host_col)) {
+        off_copy.resize(L + 1);
+        col_copy.resize((size_t)nnz);
+        if (!SPION_HIP_OK(hipMemcpyAsync(off_copy.data(), Offsets, sizeof(int) * (L + 1), hipMemcpyDeviceToHost,
+                                         a->hdr.stream)))
+            return false;
+        if (nnz && !SPION_HIP_OK(hipMemcpyAsync(col_copy.data(), Columns, sizeof(int) * (size_t)nnz,
+                                                hipMemcpyDeviceToHost, a->hdr.stream)))
+            return false;
+        if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
+        host_off = off_copy.data();
+        host_col = col_copy.data();
+    }
+    const int* off = host_off;
+    const int* col = host_col;
 
     if (off[0] != 0 || off[L] != nnz) {
         set_error("pattern: Offsets[0]=%d, Offsets[L]=%d do not match nnz=%d", off[0], off[L], nnz);
@@ -664,13 +688,65 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
     pi.key_col = Columns;
     pi.key_nnz = nnz;
     pi.valid = true;
+    // install: the slot already filed under this key (re-registration), else a free one, else the least recently used
+    int slot = -1;
+    for (int i = 0; i < SparseAttn::PAT_SLOTS; ++i)
+        if (a->pats[i].valid && a->pats[i].key_off == Offsets && a->pats[i].key_col == Columns) slot = i;
+    for (int i = 0; i < SparseAttn::PAT_SLOTS && slot < 0; ++i)
+        if (!a->pats[i].valid) slot = i;
+    if (slot < 0) {
+        slot = 0;
+        for (int i = 1; i < SparseAttn::PAT_SLOTS; ++i)
+            if (a->pat_stamp[i] < a->pat_stamp[slot]) slot = i;
+    }
+    a->pats[slot].release();  // hipFree waits for the kernels that may still read the evicted index
+    a->pats[slot] = pi;
+    a->pat_stamp[slot] = ++a->pat_clock;
+    a->pat = pi;
     return true;
 }
 
 static bool ensure_pattern(SparseAttn* a, const int* Offsets, const int* Columns, int nnz) {
-    PatternIndex& pi = a->pat;
-    if (pi.valid && pi.key_off == Offsets && pi.key_col == Columns && pi.key_nnz == nnz) return true;
+    const PatternIndex& cur = a->pat;
+    if (cur.valid && cur.key_off == Offsets && cur.key_col == Columns && cur.key_nnz == nnz) return true;
+    for (int i = 0; i < SparseAttn::PAT_SLOTS; ++i) {
+        const PatternIndex& pi = a->pats[i];
+        if (pi.valid && pi.key_off == Offsets && pi.key_col == Columns && pi.key_nnz == nnz) {
+            a->pat_stamp[i] = ++a->pat_clock;
+            a->pat = pi;
+            return true;
+        }
+    }
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+    if (cap != hipStreamCaptureStatusNone) {
+        set_error("pattern: an index that was never analysed cannot be analysed while its stream is being captured "
+                  "(run the call once before the capture, or register the pattern)");
+        return false;
+    }
     return analyse_pattern(a, Offsets, Columns, nnz);
+}
+
+// Analyse a pattern from host copies of its index arrays and file it under the device arrays' key: the first
+// forward then copies nothing back and does not wait for the stream.
+int sparse_register_pattern(void* h, const int* Offsets, const int* Columns, int nnz, const int* host_off,
+                            const int* host_col) {
+    SparseAttn* a = as_sparse(h, "spion_register_pattern");
+    if (!a) return 1;
+    if (!Offsets || !host_off || (nnz > 0 && (!Columns || !host_col))) {
+        set_error("spion_register_pattern: null pointer argument");
+        return 1;
+    }
+    return analyse_pattern(a, Offsets, Columns, nnz, host_off, host_col) ? 0 : 1;
+}
+
+// Drop the analysis filed under (Offsets, Columns), if any.
+void sparse_forget_pattern(void* h, const int* Offsets, const int* Columns) {
+    SparseAttn* a = as_sparse(h, "spion_forget_pattern");
+    if (!a) return;
+    for (auto& pi : a->pats)
+        if (pi.valid && pi.key_off == Offsets && pi.key_col == Columns) pi.release();
+    if (a->pat.valid && a->pat.key_off == Offsets && a->pat.key_col == Columns) a->pat = PatternIndex();
 }
 
 static bool ensure_ws(float** p, size_t count) {
@@ -711,6 +787,13 @@ static float* ocache_for_forward(SparseAttn* a, const float* key) {
     pick->key = key;
     pick->stamp = ++a->ostamp;
     return pick->buf;
+}
+// A forward that fills P buffer `key` without refreshing a kept copy of O (strided heads, element kernels) must
+// not leave an older copy filed under that pointer: a later backward handed the same P would take its row sums
+// from it.
+static void ocache_drop(SparseAttn* a, const float* key) {
+    for (auto& sl : a->oslot)
+        if (sl.key == key) sl.key = nullptr;
 }
 static const float* ocache_for_backward(SparseAttn* a, const float* key) {
     if (!a->use_ocache) return nullptr;
@@ -759,6 +842,7 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     float* ocache = ST ? nullptr : ocache_for_forward(a, P);
+    if (!ocache) ocache_drop(a, P);
     // Logit tiles stay in registers when every wavefront's share of the longest block row fits (MAXT tiles);
     // otherwise two sweeps.  (Launching the block rows by length class with 1, 2 and 4 wavefronts per row was
     // measured and brings nothing over four wavefronts for all.)
@@ -785,8 +869,9 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 template <int D, bool VROW, bool ST = false>
 static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
                             const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz,
-                            const float* Out, const Layouts& ly = Layouts{}) {
+                            const float* Out, const Layouts& ly = Layouts{}, float* rowsum = nullptr) {
     const PatternIndex& pi = a->pat;
+    if (!rowsum) rowsum = a->ws_rowsum;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB);
     const int wv = pick_waves(a, pi, nbr, false);
@@ -796,17 +881,17 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     do {                                                                                                            \
         if ((a->bwd_passes & 1) && ocache)                                                                          \
             hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, K,   \
-                               Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB,    \
+                               Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB,    \
                                nnz, a->scale, hc, ly);                                                              \
         else if (a->bwd_passes & 1) {                                                                               \
             if constexpr (!ST)                                                                                      \
                 hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream,  \
-                                   K, Vt, P, dO, ocache, a->ws_rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr,    \
+                                   K, Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr,    \
                                    a->NB, nnz, a->scale, hc, ly);                                                   \
         }                                                                                                           \
         if (a->bwd_passes & 2)                                                                                      \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, \
-                               dO, a->ws_rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
+                               dO, rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
                                hc, ly);                                                                             \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
@@ -885,6 +970,7 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
         return;
     }
     a->last_path = 2;
+    ocache_drop(a, Attn);
     const float* Krm = Kt;  // the element kernels read K row-major
     if (!krow) {
         if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
@@ -1250,7 +1336,7 @@ int transpose_last2(const float* in, float* out, int batch, int rows, int cols, 
 
 void sparse_invalidate(void* h) {
     SparseAttn* a = as_sparse(h, "spion_invalidate_pattern");
-    if (a) a->pat.release();
+    if (a) a->release_patterns();
 }
 int sparse_last_path(void* h) {
     SparseAttn* a = as_sparse(h, "spion_last_path");
@@ -1270,7 +1356,7 @@ void sparse_force_element(void* h, int on) {
     SparseAttn* a = as_sparse(h, "spion_force_element_path");
     if (!a) return;
     a->force_element = on != 0;
-    a->pat.release();
+    a->release_patterns();
 }
 
 }  // namespace spion

@@ -1,16 +1,21 @@
 """Writes tests/golden/config2.json and config2_masks.npy (pattern-discovery configuration 2).
 
-Runs the oracle only (no reference code).  For seeds 0, 1, 2, ... it builds the two 1024x1024 score maps,
-computes the masks along the float32 PyTorch route and the float64 closed-form route, measures the
-relative difference of the two pooled maps and the decision margin of every comparison the walks make,
-and keeps the first seed for which the margin exceeds 8x the route difference and the masks agree.
-Rejected seeds are listed in the JSON.
+Runs the oracle only (no reference code).  For every seed of a range it builds the two 1024x1024 score maps and
+measures the decision margin: the smallest relative gap over every comparison the path walks make (down > right,
+. > diagonal, . > threshold) on the float64-route pooled map.  It keeps the seed with the largest margin, then
+checks on that seed that the float32 PyTorch route (the reference's: F.conv2d, avg_pool2d, torch.quantile) and
+the float64 closed-form route give the same masks and that the margin exceeds 100 times the relative difference
+between the two routes' pooled maps -- so any correct summation order yields the identical mask.
 
-    python tests/golden/make_config2.py
+A walk makes about ten thousand comparisons per map, so margins above 1e-3 are out of reach: over seeds 0..2999
+the best is 6.3e-4 (seed 2608), the median 2e-5.  The float32 route differs from the float64 one by about 2e-6.
+
+    python tests/golden/make_config2.py [first_seed last_seed]      (default 0 3000: about a quarter of an hour on 8 cores)
 """
 import json
 import os
 import sys
+from multiprocessing import Pool
 
 import numpy as np
 
@@ -21,32 +26,40 @@ from oracle import pattern as op  # noqa: E402
 from spion_amd import workloads  # noqa: E402
 
 Q, BS, L = 0.90, 32, 1024
+MIN_FACTOR = 100.0
+
+
+def margins_of(seed):
+    maps = workloads.score_maps_config2(2, L, 32, seed=seed).numpy()
+    return seed, [op.decision_margin(op.pooled_map(maps[i], BS, 31, "fp64"), Q) for i in range(2)]
 
 
 def main():
-    rejected = []
-    for seed in range(64):
-        maps = workloads.score_maps_config2(2, L, 32, seed=seed).numpy()
-        ok, masks, margins, errs = True, [], [], []
-        for i in range(2):
-            m64, p64, t64 = op.generate_mask_conv_ff(maps[i], BS, Q, route="fp64")
-            m32, p32, t32 = op.generate_mask_conv_ff(maps[i], BS, Q, route="torch")
-            err = float(np.max(np.abs(p64.astype(np.float64) - p32) / np.abs(p64)))
-            margin = op.decision_margin(p64, Q)
-            margins.append(margin)
-            errs.append(err)
-            masks.append(m64)
-            ok = ok and margin > 8 * err and np.array_equal(m64, m32)
-        print(f"seed {seed}: margins {margins} route errors {errs} -> {'ok' if ok else 'rejected'}", flush=True)
-        if ok:
-            np.save(os.path.join(HERE, "config2_masks.npy"), np.stack(masks).astype(np.int8))
-            meta = dict(seed=seed, quantile=Q, block_size=BS, seq_len=L, decision_margin=margins,
-                        fp32_route_rel_error=errs, rejected_seeds=rejected,
-                        blocks_set=[int(m.sum()) for m in masks])
-            json.dump(meta, open(os.path.join(HERE, "config2.json"), "w"), indent=1)
-            return
-        rejected.append(dict(seed=seed, decision_margin=margins, fp32_route_rel_error=errs))
-    raise SystemExit("no seed passed the margin screen")
+    lo, hi = (int(sys.argv[1]), int(sys.argv[2])) if len(sys.argv) == 3 else (0, 3000)
+    with Pool(min(8, os.cpu_count() or 1)) as pool:
+        scan = pool.map(margins_of, range(lo, hi), chunksize=8)
+    scan.sort(key=lambda r: -min(r[1]))
+    seed, margins = scan[0]
+    maps = workloads.score_maps_config2(2, L, 32, seed=seed).numpy()
+    masks, errs = [], []
+    for i in range(2):
+        m64, p64, _ = op.generate_mask_conv_ff(maps[i], BS, Q, route="fp64")
+        m32, p32, _ = op.generate_mask_conv_ff(maps[i], BS, Q, route="torch")
+        errs.append(float(np.max(np.abs(p64.astype(np.float64) - p32) / np.abs(p64))))
+        if not np.array_equal(m64, m32):
+            raise SystemExit(f"seed {seed}: the float32 and float64 routes disagree on map {i}")
+        masks.append(m64)
+    if min(margins) <= MIN_FACTOR * max(errs):
+        raise SystemExit(f"seed {seed}: margin {min(margins):.3e} is not {MIN_FACTOR:g}x the route error {max(errs):.3e}")
+    np.save(os.path.join(HERE, "config2_masks.npy"), np.stack(masks).astype(np.int8))
+    all_min = sorted(min(r[1]) for r in scan)
+    meta = dict(seed=seed, quantile=Q, block_size=BS, seq_len=L, decision_margin=margins,
+                fp32_route_rel_error=errs, margin_over_route_error=min(margins) / max(errs),
+                seeds_scanned=[lo, hi], median_margin_of_scan=all_min[len(all_min) // 2],
+                runners_up=[dict(seed=s, decision_margin=m) for s, m in scan[1:6]],
+                blocks_set=[int(m.sum()) for m in masks])
+    json.dump(meta, open(os.path.join(HERE, "config2.json"), "w"), indent=1)
+    print(json.dumps(meta, indent=1))
 
 
 if __name__ == "__main__":

@@ -12,12 +12,17 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def test_every_declared_symbol_is_exported():
-    hdr = open(os.path.join(ROOT, "include", "spion_hip.h")).read()
-    names = sorted(set(re.findall(r"\b(spion_\w+)\s*\(", hdr)))
-    assert len(names) >= 24
+    inc = os.path.join(ROOT, "include")
+    headers = sorted(f for f in os.listdir(inc) if f.endswith(".h"))
+    assert "spion_hip.h" in headers
     lib = ctypes.CDLL(_lib.lib_path("libspion_hip.so"))
-    for n in names:
-        assert hasattr(lib, n), f"{n} declared in include/spion_hip.h but not exported"
+    total = 0
+    for h in headers:
+        names = sorted(set(re.findall(r"\b(spion_\w+)\s*\(", open(os.path.join(inc, h)).read())))
+        total += len(names)
+        for n in names:
+            assert hasattr(lib, n), f"{n} declared in include/{h} but not exported"
+    assert total >= 30
 
 
 @pytest.mark.parametrize("loader", ["_cuda_compile_module", "_cuda_mask_compile_module",

@@ -16,10 +16,15 @@ GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 
 
 def _check_maps(maps, bs, q, ksize):
+    """GPU masks against (1) the oracle's walk on the GPU's own pooled map (always) and (2) the mask of the
+    independent float64 route, whenever every decision of that route's walk is further from flipping than eight
+    times the difference between the two pooled maps (or the maps are bit-identical).  At least one map of every
+    call must take the second comparison: a call whose maps all sit on a near-tie fails instead of passing unseen."""
     mode = "conv_ff" if ksize else "ff"
     mat, pooled, thresh = discover_block_masks(maps.cuda(), bs, mode=mode, threshold=q, ksize=ksize or 31,
                                                return_aux=True)
     mat, pooled, thresh = mat.cpu().numpy(), pooled.cpu().numpy(), thresh.cpu().numpy()
+    independent = 0
     for i in range(maps.shape[0]):
         ref_mask, ref_pooled, ref_thresh = op.generate_mask_conv_ff(maps[i].numpy(), bs, q, ksize=ksize, route="fp64")
         # fp64 accumulation on both sides, one rounding: equal except for double-rounding ties
@@ -28,8 +33,13 @@ def _check_maps(maps, bs, q, ksize):
         t_gpu = op.quantile_linear(pooled[i], q)[0]
         assert abs(float(thresh[i]) - float(t_gpu)) <= np.spacing(np.float32(abs(t_gpu)))
         assert np.array_equal(mat[i].astype(np.int8), op.mask_from_pooled(pooled[i], np.float32(thresh[i])))
-        if np.array_equal(pooled[i], ref_pooled) and thresh[i] == ref_thresh:
-            assert np.array_equal(mat[i].astype(np.int8), ref_mask)
+        nz = ref_pooled != 0
+        err = float(np.max(np.abs(pooled[i][nz].astype(np.float64) - ref_pooled[nz]) / np.abs(ref_pooled[nz]))) if nz.any() else 0.0
+        margin = op.decision_margin(ref_pooled, q)
+        if np.array_equal(pooled[i], ref_pooled) or margin > 8 * err:
+            independent += 1
+            assert np.array_equal(mat[i].astype(np.int8), ref_mask), (i, margin, err)
+    assert independent > 0, "no map of this case could be compared with the independent float64 route"
     return mat, pooled, thresh
 
 

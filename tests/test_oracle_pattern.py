@@ -159,3 +159,54 @@ def test_generators_and_margin():
     assert mc.sum() >= k and (np.diag(mc) == 1).all()
     mf, _, _ = op.generate_mask_conv_ff(A, 32, 0.9, ksize=0)
     assert mf.shape == (8, 8)
+
+
+@pytest.mark.parametrize("nb,density,seed", [(8, 0.3, 0), (16, 0.2, 1), (32, 0.1, 2), (32, 0.5, 3), (12, 0.9, 4)])
+def test_topk_generator_matches_torch_topk(nb, density, seed):
+    """SPION-C (main_conv.py:246-255): the k = int(nb*nb*density - nb) LARGEST pooled values plus the diagonal.
+    Pinned against torch.topk on maps without a tie at the k-th value, where topk's result is unique as a set.
+    Selecting the smallest k, an off-by-one k or a transposed index fails."""
+    bs = 4
+    rng = np.random.default_rng(seed)
+    k_expected = int(nb * nb * density - nb)
+    for _ in range(64):
+        A = rng.random((nb * bs, nb * bs)).astype(np.float32)
+        pooled = op.pooled_map(A, bs, 31, "fp64")
+        desc = np.sort(pooled.ravel())[::-1]
+        if desc[k_expected - 1] > desc[k_expected]:
+            break
+    else:  # pragma: no cover
+        pytest.fail("no tie-free map found")
+    mask, pooled2, k = op.generate_mask_conv(A, bs, density)
+    assert np.array_equal(pooled, pooled2)
+    assert k == k_expected
+    flat = torch.from_numpy(pooled).view(-1)
+    idx = torch.topk(flat, k)[1]
+    ref = torch.zeros(nb * nb)
+    ref[idx] = 1
+    ref = ref.reshape(nb, nb)
+    for i in range(nb):
+        ref[i, i] = 1
+    assert np.array_equal(mask, ref.numpy().astype(np.int8))
+    # the selection is of the largest values: every selected off-diagonal value >= every unselected one
+    off = ~np.eye(nb, dtype=bool)
+    sel = np.zeros(nb * nb, bool)
+    sel[idx.numpy()] = True
+    sel = sel.reshape(nb, nb)
+    assert pooled[sel].min() > pooled[~sel].max()
+    assert (mask[off & ~sel] == 0).all()
+    # and not of the smallest (which the count / diagonal checks alone would accept)
+    small = torch.topk(flat, k, largest=False)[1]
+    wrong = torch.zeros(nb * nb)
+    wrong[small] = 1
+    wrong = wrong.reshape(nb, nb).numpy().astype(np.int8)
+    wrong[np.arange(nb), np.arange(nb)] = 1
+    assert not np.array_equal(mask, wrong)
+
+
+def test_topk_generator_k_not_positive():
+    """density * nb*nb <= nb: torch.topk with k = 0 selects nothing, only the diagonal remains."""
+    rng = np.random.default_rng(5)
+    A = rng.random((32, 32)).astype(np.float32)
+    mask, _, k = op.generate_mask_conv(A, 4, 1.0 / 8)
+    assert k == 0 and np.array_equal(mask, np.eye(8, dtype=np.int8))
