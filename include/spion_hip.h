@@ -248,6 +248,24 @@ void spion_attn_backward_rowmajor(void* handle, const float* Q, const float* K, 
                                   float* dQ, float* dK, float* dV,
                                   const int* Offsets, const int* Columns, const int* SumMat, int nnz);
 
+/* spion_attn_backward_rowmajor for callers that cannot allocate.  No counterpart in the reference; it is for
+ * callers that cannot call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation.  Same arguments and results (bit for bit) as spion_attn_backward_rowmajor with Out given, minus the
+ * dS scratch; it calls no hipMalloc / hipFree and no allocating library routine.  The row sums the row pass
+ * leaves for the column pass go to a built-in device array of spion_noalloc_max_rows() floats (2^20 = 4 MiB,
+ * held by every GPU the library runs on until the process ends) instead of the handle's workspace.
+ * Limits, each reported through the error slot with nothing launched:
+ *   num_batches * seq_len <= spion_noalloc_max_rows();  emb_dim 32;  Out required;
+ *   the pattern must be a union of aligned 32x32 tiles and must already be analysed on this handle
+ *   (by an earlier forward with the same Offsets / Columns / nnz, or by spion_register_pattern).
+ * All calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads, two handles)
+ * race.  Nothing in it needs clearing between calls: the row pass writes every row sum the column pass reads. */
+void spion_attn_backward_noalloc(void* handle, const float* Q, const float* K, const float* V, const float* P,
+                                 const float* Out, const float* dO,
+                                 float* dQ, float* dK, float* dV,
+                                 const int* Offsets, const int* Columns, const int* SumMat, int nnz);
+long long spion_noalloc_max_rows(void);
+
 /* The same for heads that are views of other memory: the reference's layer produces Q, K and V as
  * [B][L][H*d] projections and views them as [B][H][L][d] (models/attention.py:84-96 and split_heads :136-139),
  * then copies each into a contiguous [NB][L][d] buffer before the call (models/attention_blockcuda.py:48,80;

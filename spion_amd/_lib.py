@@ -78,6 +78,10 @@ def core() -> ctypes.CDLL:
     lib.spion_attn_forward_rowmajor.restype = None
     lib.spion_attn_backward_rowmajor.argtypes = [_P] * 14 + [c_int]
     lib.spion_attn_backward_rowmajor.restype = None
+    lib.spion_attn_backward_noalloc.argtypes = [_P] * 13 + [c_int]
+    lib.spion_attn_backward_noalloc.restype = None
+    lib.spion_noalloc_max_rows.argtypes = []
+    lib.spion_noalloc_max_rows.restype = ctypes.c_longlong
     lib.spion_attn_forward_strided.argtypes = [_P] * 10 + [c_int, c_int, _P, _P]
     lib.spion_attn_forward_strided.restype = None
     lib.spion_attn_backward_strided.argtypes = [_P] * 13 + [c_int, c_int, _P, _P, _P]

@@ -63,6 +63,9 @@ void dense_backward_strided(void*, const float*, const float*, const float*, con
 void sparse_invalidate(void*);
 int sparse_register_pattern(void*, const int*, const int*, int, const int*, const int*);
 void sparse_forget_pattern(void*, const int*, const int*);
+void sparse_backward_noalloc(void*, const float*, const float*, const float*, const float*, const float*, const float*,
+                             float*, float*, float*, const int*, const int*, int);
+size_t sparse_noalloc_max_rows();
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
@@ -248,6 +251,13 @@ void spion_attn_backward_rowmajor(void* h, const float* Q, const float* K, const
     (void)SumMat;
     sparse_backward(h, Q, K, V, P, dO, nullptr, dS, dQ, dK, dV, Offsets, Columns, nnz, Out, true);
 }
+void spion_attn_backward_noalloc(void* h, const float* Q, const float* K, const float* V, const float* P,
+                                 const float* Out, const float* dO, float* dQ, float* dK, float* dV,
+                                 const int* Offsets, const int* Columns, const int* SumMat, int nnz) {
+    (void)SumMat;
+    sparse_backward_noalloc(h, Q, K, V, P, Out, dO, dQ, dK, dV, Offsets, Columns, nnz);
+}
+long long spion_noalloc_max_rows(void) { return (long long)sparse_noalloc_max_rows(); }
 static spion::HeadLayout to_layout(const spion_head_layout* y) {
     return spion::HeadLayout{y->batch_stride, y->head_stride, y->row_stride};
 }

@@ -394,6 +394,8 @@ static SparseAttn* as_sparse(void* h, const char* who) {
 static bool tile_supported(int d) { return d == 32 || d == 64; }
 static bool elem_supported(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 
+static float* noalloc_scratch(bool report);
+
 void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, bool has_mask) {
     if (emb_dim <= 0 || seq_len <= 0 || num_batches <= 0) {
         set_error("init: emb_dim, seq_len and num_batches must be positive (got %d, %d, %d)", emb_dim, seq_len,
@@ -418,6 +420,7 @@ void* sparse_init(int emb_dim, int seq_len, int num_batches, int block_size, boo
     a->bs = block_size;
     a->has_mask = has_mask;
     a->scale = 1.0f / sqrtf((float)emb_dim);  // models/block_attn.cu:420
+    (void)noalloc_scratch(false);  // per-device address of the built-in scratch array, looked up once
     return a;
 }
 
@@ -1038,6 +1041,94 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         default: launch_elem_bwd<128>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;
     }
     check_launch("elem_bwd kernels");
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward for callers that must not allocate (code under HIP graph capture, serving loops, harnesses that
+// forbid hipMalloc): the row sums -g [NB][L] that the row pass leaves for the column pass go to a file-scope
+// device array instead of the handle's workspace.  Every GPU holds its own copy of the array at its own
+// address, looked up once per device with hipGetSymbolAddress; host code never uses the array's name as an
+// address.  All calls on one GPU share the array: calls that overlap on one GPU race.
+// -------------------------------------------------------------------------------------------------
+constexpr size_t NOALLOC_MAX_ROWS = size_t(1) << 20;  // num_batches * seq_len; 4 MiB per GPU
+static __device__ __align__(256) float scratch[NOALLOC_MAX_ROWS];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+static float* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+// Address of `scratch` on the current device (nullptr and, if `report`, an error when it cannot be had).
+static float* noalloc_scratch(bool report) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= NOALLOC_MAX_DEVICES) {
+        (void)hipGetLastError();
+        if (report) set_error("spion_attn_backward_noalloc: no current device (or device index >= %d)", NOALLOC_MAX_DEVICES);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            (void)hipGetLastError();
+            if (report) set_error("spion_attn_backward_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = static_cast<float*>(p);
+    }
+    return g_scratch_ptr[dev];
+}
+
+size_t sparse_noalloc_max_rows() { return NOALLOC_MAX_ROWS; }
+
+void sparse_backward_noalloc(void* h, const float* Q, const float* K, const float* V, const float* P, const float* Out,
+                             const float* dO, float* dQ, float* dK, float* dV, const int* Offsets, const int* Columns,
+                             int nnz) {
+    const char* who = "spion_attn_backward_noalloc";
+    SparseAttn* a = as_sparse(h, who);
+    if (!a) return;
+    if (a->is_bf16) {
+        set_error("%s: handle was created by the bf16 init", who);
+        return;
+    }
+    if (!Q || !K || !V || !P || !Out || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("%s: null pointer argument (Out is required)", who);
+        return;
+    }
+    if ((size_t)a->NB * (size_t)a->L > NOALLOC_MAX_ROWS) {
+        set_error("%s: num_batches * seq_len = %lld exceeds the %lld rows of the built-in scratch array", who,
+                  (long long)a->NB * a->L, (long long)NOALLOC_MAX_ROWS);
+        return;
+    }
+    if (a->d != 32) {
+        set_error("%s: emb_dim %d unsupported (32 only: other sizes need workspace the library would have to allocate)",
+                  who, a->d);
+        return;
+    }
+    // the analysed pattern must be on file: analysing one allocates
+    bool known = a->pat.valid && a->pat.key_off == Offsets && a->pat.key_col == Columns && a->pat.key_nnz == nnz;
+    for (int i = 0; i < SparseAttn::PAT_SLOTS && !known; ++i) {
+        const PatternIndex& pi = a->pats[i];
+        if (pi.valid && pi.key_off == Offsets && pi.key_col == Columns && pi.key_nnz == nnz) {
+            a->pat_stamp[i] = ++a->pat_clock;
+            a->pat = pi;
+            known = true;
+        }
+    }
+    if (!known) {
+        set_error("%s: this (Offsets, Columns, nnz) has not been analysed on this handle yet; run a forward or "
+                  "spion_register_pattern first", who);
+        return;
+    }
+    if (!a->pat.tiled) {
+        set_error("%s: the pattern is not a union of aligned 32x32 tiles (the element kernels need a scratch of "
+                  "num_batches * nnz floats from the caller: use spion_attn_backward_rowmajor)", who);
+        return;
+    }
+    float* rowsum = noalloc_scratch(true);
+    if (!rowsum) return;
+    a->last_path = 1;
+    launch_tile_bwd<32, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, Layouts{}, rowsum);
+    check_launch("tile_bwd kernels");
 }
 
 // Heads that are views of other memory (the [B][L][H*d] output of a projection seen as [B][H][L][d]): the tile
