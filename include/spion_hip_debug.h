@@ -18,6 +18,10 @@ void spion_force_element_path(void* handle, int on);
  * needs the row sums of an earlier row pass).  Default 3 = both. */
 void spion_set_backward_passes(void* handle, int mask);
 
+/* Counters of a sparse handle: which = 0 -> pattern analyses that copied the index back from the device (and
+ * waited for the stream), which = 1 -> analyses made from host arrays (spion_register_pattern).  -1 otherwise. */
+int spion_debug_counter(void* handle, int which);
+
 #ifdef __cplusplus
 }
 #endif

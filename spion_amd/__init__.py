@@ -10,6 +10,7 @@ from .attention_cuda_mask import CUDAMaskAttention
 from .attention_blockcuda import CUDABlockAttention
 from .attention_blockcuda_mask import CUDABlockMaskAttention
 from .attention_blockbf16 import BlockAttentionBF16
+from .inference import attach_mask_sidecars, load_masks_for_inference, timed_eval
 from .masks import TransitionDetector, load_mask_list, save_mask_list, stack_for_replicas
 from .pattern import (
     discover_block_masks,
@@ -28,6 +29,9 @@ __all__ = [
     "CUDABlockAttention",
     "CUDABlockMaskAttention",
     "BlockAttentionBF16",
+    "attach_mask_sidecars",
+    "load_masks_for_inference",
+    "timed_eval",
     "TransitionDetector",
     "load_mask_list",
     "save_mask_list",

@@ -70,6 +70,8 @@ def core() -> ctypes.CDLL:
     lib.spion_force_element_path.restype = None
     lib.spion_set_backward_passes.argtypes = [_P, c_int]
     lib.spion_set_backward_passes.restype = None
+    lib.spion_debug_counter.argtypes = [_P, c_int]
+    lib.spion_debug_counter.restype = c_int
     lib.spion_use_output_cache.argtypes = [_P, c_int]
     lib.spion_use_output_cache.restype = None
     lib.spion_attn_backward_with_out.argtypes = [_P] * 15 + [c_int]

@@ -69,6 +69,7 @@ size_t sparse_noalloc_max_rows();
 int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
+int sparse_debug_counter(void*, int);
 void sparse_use_ocache(void*, int);
 void* sparse_bf16_init(int, int, int, int);
 void sparse_bf16_forward(void*, const void*, const void*, const void*, const float*, void*, float*, const int*,
@@ -232,6 +233,7 @@ void spion_forget_pattern(void* h, const int* Offsets, const int* Columns) { spa
 int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
+int spion_debug_counter(void* h, int which) { return sparse_debug_counter(h, which); }
 void spion_use_output_cache(void* h, int on) { sparse_use_ocache(h, on); }
 void spion_attn_backward_with_out(void* h, const float* Q, const float* K, const float* Vt, const float* P,
                                   const float* Out, const float* dO, float* dP, float* dS, float* dQ, float* dK,

@@ -353,6 +353,7 @@ struct SparseAttn {
     PatternIndex pats[PAT_SLOTS];
     uint64_t pat_stamp[PAT_SLOTS] = {};
     uint64_t pat_clock = 0;
+    int analyses_from_device = 0, analyses_from_host = 0;  // counted for tests
     PatternIndex pat;
     void release_patterns() {
         for (auto& p : pats) p.release();
@@ -501,6 +502,9 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
         host_off = off_copy.data();
         host_col = col_copy.data();
+        a->analyses_from_device++;
+    } else {
+        a->analyses_from_host++;
     }
     const int* off = host_off;
     const int* col = host_col;
@@ -1432,6 +1436,11 @@ void sparse_invalidate(void* h) {
 int sparse_last_path(void* h) {
     SparseAttn* a = as_sparse(h, "spion_last_path");
     return a ? a->last_path : 0;
+}
+int sparse_debug_counter(void* h, int which) {
+    SparseAttn* a = as_sparse(h, "spion_debug_counter");
+    if (!a) return -1;
+    return which == 0 ? a->analyses_from_device : which == 1 ? a->analyses_from_host : -1;
 }
 void sparse_set_bwd_passes(void* h, int mask) {
     SparseAttn* a = as_sparse(h, "spion_set_backward_passes");

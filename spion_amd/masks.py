@@ -32,7 +32,9 @@ def save_mask_list(mat_lst: torch.Tensor, path: str) -> None:
 
 
 def _storage_from_bytes(b: bytes):
-    return torch.load(io.BytesIO(b), weights_only=True)
+    # the reference pickles the tensor as it lies on the GPU (main_conv_ff.py:298-306): bring the bytes to the host,
+    # whatever device tag they carry
+    return torch.load(io.BytesIO(b), weights_only=True, map_location="cpu")
 
 
 class _TensorOnlyUnpickler(pickle.Unpickler):

@@ -96,7 +96,13 @@ class EncoderForSC(nn.Module):
         pooled = X.mean(dim=1)
         scores = self.head(pooled)
         loss = nn.functional.cross_entropy(scores, label, reduction="none")
+        self.last_accu = (scores.argmax(dim=-1) == label).to(torch.float32)  # models/model_LRA.py:62-63
         return loss, attn_lst
+
+    def outputs(self, input_ids, mask, label, mat_lst=None):
+        """The dict the reference's task model returns (models/model_LRA.py:52-71): per-sample loss and accuracy."""
+        loss, _ = self.forward(input_ids, mask, label, mat_lst)
+        return {"loss": loss, "accu": self.last_accu}
 
 
 def model_config(L=1024, batch=256, block_size=32, key_mask=False, threshold=0.96):
