@@ -175,6 +175,27 @@ int spion_score_map_mean(const float* Attn, int batch, int heads, int seq_len, i
                          float* Mean, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
+ * Dense-to-sparse transition test on the device (main_conv_ff.py:211-242; the reference runs it on the host
+ * with one synchronising torch reduction per layer).  Call once per evaluation with the averaged score maps of all
+ * layers; the decision accumulates in State and is read back by the caller as one float.
+ *   Cur     [layers][elems_per_layer]  this evaluation's maps;
+ *   Prev    [layers][elems_per_layer]  in/out: the maps kept for comparison (contents need not be initialised);
+ *   State   [2*layers + 3] floats, in/out, zero-initialised by the caller before the first call:
+ *           [0, layers)            Frobenius distance of the previous comparison, per layer
+ *           [layers, 2*layers)     last change of the distance in per cent, per layer
+ *           [2*layers]             stage: 0 no map kept yet, 1 maps kept, 2 maps and distances kept
+ *           [2*layers + 1]         1 once the change stayed below `percent` (truncated to an integer, as the
+ *                                  reference's int(diff) < 15) in every layer; later calls change nothing
+ *           [2*layers + 2]         scratch
+ *   Partial [layers][partial_blocks] doubles: workspace.
+ * First call: the maps are kept.  Second call: the first distances are taken, the kept maps stay.  Later calls:
+ * the distance to the kept maps is compared with the previous distance; if not every layer has settled, the kept
+ * maps are replaced by the current ones.  Differences are formed in fp32 as torch does, summed in fp64 in a fixed
+ * order.  Returns 0 on success. */
+int spion_transition_update(const float* Cur, float* Prev, int layers, long long elems_per_layer,
+                            float* State, double* Partial, int partial_blocks, int percent, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
  * Additions with no counterpart in the reference (which reports no errors at all).
  * ---------------------------------------------------------------------------------------------- */
 
@@ -310,6 +331,17 @@ void spion_dense_backward_strided(void* handle, const float* Q, const float* K, 
                                   float* dQ, float* dK, float* dV,
                                   int heads, const spion_head_layout* in, const spion_head_layout* out,
                                   const spion_head_layout* grad);
+
+/* The dense forward on [B][H][L][d] views (spion_dense_forward_strided) that also leaves the mean of all
+ * num_batches maps in Mean [seq_len][seq_len] (queries x keys, the Score input of spion_pattern_generate):
+ * models/model_transformer.py:136-137 takes that mean with two torch.mean passes over the [B,H,L,L] tensor the
+ * forward has just written; here every map tile is added to a partial sum while it is on its way to memory, and
+ * one reduction over a few partial maps finishes the mean, so the maps are not read back.  The handle keeps the
+ * partial maps (at most max(1, 512*32/seq_len) * seq_len^2 floats).  All other arguments and results as in
+ * spion_dense_forward_strided (Attn is still written: the API returns it). */
+void spion_dense_forward_strided_mean(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
+                                      float* Attn, float* Out, float* Mean,
+                                      int heads, const spion_head_layout* in, const spion_head_layout* out);
 
 /* Host-side helper: out[b][c][r] = in[b][r][c] (fp32), for the transposed K / V / Q / dO operands the
  * attention entry points take.  Returns 0 on success. */

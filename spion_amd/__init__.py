@@ -11,7 +11,7 @@ from .attention_blockcuda import CUDABlockAttention
 from .attention_blockcuda_mask import CUDABlockMaskAttention
 from .attention_blockbf16 import BlockAttentionBF16
 from .inference import attach_mask_sidecars, load_masks_for_inference, timed_eval
-from .masks import TransitionDetector, load_mask_list, save_mask_list, stack_for_replicas
+from .masks import DeviceTransitionDetector, TransitionDetector, load_mask_list, save_mask_list, stack_for_replicas
 from .pattern import (
     discover_block_masks,
     generate_pattern_conv,
@@ -33,6 +33,7 @@ __all__ = [
     "load_masks_for_inference",
     "timed_eval",
     "TransitionDetector",
+    "DeviceTransitionDetector",
     "load_mask_list",
     "save_mask_list",
     "stack_for_replicas",

@@ -90,6 +90,10 @@ def core() -> ctypes.CDLL:
     lib.spion_attn_backward_strided.restype = None
     lib.spion_dense_forward_strided.argtypes = [_P] * 7 + [c_int, _P, _P]
     lib.spion_dense_forward_strided.restype = None
+    lib.spion_dense_forward_strided_mean.argtypes = [_P] * 8 + [c_int, _P, _P]
+    lib.spion_dense_forward_strided_mean.restype = None
+    lib.spion_transition_update.argtypes = [_P, _P, c_int, ctypes.c_longlong, _P, _P, c_int, c_int, _P]
+    lib.spion_transition_update.restype = c_int
     lib.spion_dense_backward_strided.argtypes = [_P] * 10 + [c_int, _P, _P, _P]
     lib.spion_dense_backward_strided.restype = None
     lib.spion_transpose_last2.argtypes = [_P, _P, c_int, c_int, c_int, _P]

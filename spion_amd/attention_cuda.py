@@ -58,9 +58,18 @@ class _DenseAttnFunction(torch.autograd.Function):
             if m.with_mask:
                 pen = (1e6 * (1.0 - mask.repeat(1, H))).to(torch.float32).contiguous()
                 pen_ptr = pen.data_ptr()
-            _lib.core().spion_dense_forward_strided(
-                m.attn_handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pen_ptr, attn.data_ptr(),
-                out.data_ptr(), H, ctypes.addressof(lay), ctypes.addressof(lout))
+            if m.emit_score_map:
+                # models/model_transformer.py:136-137 averages the returned maps over batch and heads; the kernel
+                # does it while it writes them
+                mean = torch.empty((L, L), dtype=torch.float32, device=dev)
+                _lib.core().spion_dense_forward_strided_mean(
+                    m.attn_handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pen_ptr, attn.data_ptr(),
+                    out.data_ptr(), mean.data_ptr(), H, ctypes.addressof(lay), ctypes.addressof(lout))
+                m.score_map = mean
+            else:
+                _lib.core().spion_dense_forward_strided(
+                    m.attn_handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pen_ptr, attn.data_ptr(),
+                    out.data_ptr(), H, ctypes.addressof(lay), ctypes.addressof(lout))
             _lib.check_error("attn_forward")
             ctx.save_for_backward(query, key, value, attn, out)
             ctx.set_materialize_grads(False)
@@ -80,6 +89,9 @@ class _DenseAttnFunction(torch.autograd.Function):
             m.attn_cpp.attn_forward(m.attn_handle, qt.data_ptr(), k.data_ptr(), vt.data_ptr(), attn.data_ptr(),
                                     out_t.data_ptr())
         _lib.check_error("attn_forward")
+        if m.emit_score_map:  # shapes the fused kernel does not serve: one pass over the maps just written
+            from .pattern import mean_score_map
+            m.score_map = mean_score_map(attn.permute(0, 1, 3, 2))
         ctx.save_for_backward(qt, key, value, attn)
         ctx.set_materialize_grads(False)  # the gradient of the returned map is ignored (as in the reference)
         ctx.module = m
@@ -149,6 +161,10 @@ class _DenseAttentionBase(nn.Module):
         self.attn_func = _DenseAttnFunction
         # shapes the strided entry points serve; everything else goes through the reference's ABI
         self.reads_views = self.emb_dim == 32 and self.seq_len <= 16384
+        # When set, every forward also leaves ``self.score_map`` [L, L]: the mean of the returned maps over batch and
+        # heads (what models/model_transformer.py:136-137 computes from them), taken while the maps are written.
+        self.emit_score_map = False
+        self.score_map = None
 
     def forward(self, query, key, value, mask):
         return self.attn_func.apply(query, key, value, mask, self)

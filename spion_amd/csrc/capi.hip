@@ -77,13 +77,16 @@ void sparse_bf16_forward(void*, const void*, const void*, const void*, const flo
 void sparse_bf16_backward(void*, const void*, const void*, const void*, const float*, const void*, const float*,
                           const void*, void*, void*, void*, const int*, const int*, int);
 int transpose_last2(const float*, float*, int, int, int, hipStream_t);
+int transition_update(const float*, float*, int, long long, float*, double*, int, int, hipStream_t);
 void* dense_init(int, int, int, bool);
 void dense_destroy(void*);
 void dense_forward(void*, const float*, const float*, const float*, const float*, float*, float*, bool);
 void dense_backward(void*, const float*, const float*, const float*, const float*, const float*, float*, float*,
                     float*);
 int pattern_generate(const float*, int, int, int, int, int, double, float*, float*, float*, hipStream_t);
-int score_map_mean(const float*, int, int, int, int, float*, hipStream_t);
+int score_map_mean(const float*, int, int, int, int, float*, hipStream_t, float post = 1.0f);
+void dense_forward_strided_mean(void*, const float*, const float*, const float*, const float*, float*, float*, float*, int,
+                                const HeadLayout&, const HeadLayout&);
 
 }  // namespace spion
 
@@ -196,6 +199,13 @@ int spion_score_map_mean(const float* Attn, int batch, int heads, int seq_len, i
     return score_map_mean(Attn, batch, heads, seq_len, key_major, Mean, static_cast<hipStream_t>(stream));
 }
 
+int spion_transition_update(const float* Cur, float* Prev, int layers, long long elems_per_layer, float* State,
+                            double* Partial, int partial_blocks, int percent, void* stream) {
+    note_current_handle(nullptr);
+    return transition_update(Cur, Prev, layers, elems_per_layer, State, Partial, partial_blocks, percent,
+                             static_cast<hipStream_t>(stream));
+}
+
 // ---- additions -----------------------------------------------------------------------------------
 const char* spion_last_error(void) {
     static thread_local std::string copy;
@@ -293,6 +303,15 @@ void spion_dense_forward_strided(void* h, const float* Q, const float* K, const 
         return;
     }
     dense_forward_strided(h, Q, K, V, Mask, Attn, Out, heads, to_layout(in), to_layout(out));
+}
+void spion_dense_forward_strided_mean(void* h, const float* Q, const float* K, const float* V, const float* Mask,
+                                      float* Attn, float* Out, float* Mean, int heads, const spion_head_layout* in,
+                                      const spion_head_layout* out) {
+    if (!in || !out) {
+        set_error("dense attn_forward_strided_mean: null layout argument");
+        return;
+    }
+    dense_forward_strided_mean(h, Q, K, V, Mask, Attn, Out, Mean, heads, to_layout(in), to_layout(out));
 }
 void spion_dense_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P,
                                   const float* Out, const float* dO, float* dQ, float* dK, float* dV, int heads,

@@ -11,6 +11,7 @@
 #include "../../include/spion_hip.h"
 
 #include <cmath>
+#include <cstdlib>
 
 namespace spion {
 
@@ -224,12 +225,12 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     }
     if constexpr (RM) {
         reduce_store_rows<WAVES>(o[0], Out + ob, I * 32, w, li, h, lds, old_);
-        return;
-    }
-    reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
-    if (OutCopy) {
-        __syncthreads();
-        reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+    } else {
+        reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+        if (OutCopy) {
+            __syncthreads();
+            reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+        }
     }
 }
 
@@ -239,17 +240,26 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
 // accumulates O^T.  Tiles are fetched linearly one tile ahead and re-laid out in wave-private LDS tiles, as in
 // the kernels above.  48 MFMA per tile against the 32 of the register-resident kernel, which is why that one is
 // used whenever a strip's logits fit in the registers of four wavefronts.
-template <bool MASK, bool RM = false>
+// MEAN (row-major operands only): the launch also accumulates the sum of the maps over the heads.  The grid is
+// nbr x C work-groups instead of nbr x NB: work-group (c, I) walks the heads c, c + C, c + 2C, ... one after the
+// other and adds every map tile it writes to its own [L][32] slab of Part[c] (key-major like the map; plain
+// read-modify-write, nobody else touches the slab), so the mean over batch and heads is one small reduction of the
+// C partial maps afterwards instead of a second pass over all NB maps.
+template <bool MASK, bool RM = false, bool MEAN = false>
 SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
-    int L, int nbr, int NB, float scale, Layouts ly) {
+    int L, int nbr, int NB, float scale, Layouts ly, float* __restrict__ Part = nullptr, int C = 0) {
+    static_assert(!MEAN || RM, "the mean-emitting forward takes row-major operands");
     constexpr int D = 32, KH = 16, WAVES = 4;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
+    const int item = xcd_remap(blockIdx.x, nbr * (MEAN ? C : NB));
+    const int bh0 = item / nbr, I = item % nbr;
+    const int bh_step = MEAN ? C : NB;
+    int bh = bh0;
+    do {  // one head, or (MEAN) the heads bh0, bh0 + C, ...
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
     const size_t hb = (size_t)bh * L * D;
@@ -259,6 +269,7 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
     head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
     const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes);
     const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const rsrc_t rS = make_rsrc(MEAN ? Part + (size_t)bh0 * L * L : Part, MEAN ? (size_t)L * L * 4 : 0);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     float* T = lds_t[w];          // map tile on its way to memory
     float* Tk = T + 32 * TS;
@@ -355,6 +366,10 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
             },
             [&](Pre2& c, int i) {
                 const int J = w + i * WAVES;
+                f32x4 sum4[4];
+                if constexpr (MEAN) {
+                    if (bh != bh0) ldr_tile_lin_l2(rS, alin, (J * 32 * L + I * 32) * 4, L, sum4);
+                }
                 lds_put_lin(Tk, l, c.k);
                 lds_put_lin(Tv, l, c.v);
                 float kf[KH], vb[16];
@@ -377,17 +392,32 @@ SPION_TILE_KERNEL(4) void dense_fwd_sweep32_kernel(
 #pragma unroll
                 for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
                 str_tile_lin(rA, alin, (J * 32 * L + I * 32) * 4, L, pl);
+                if constexpr (MEAN) {
+                    if (bh != bh0) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) pl[k] += sum4[k];
+                    }
+                    str_tile_lin_cached(rS, alin, (J * 32 * L + I * 32) * 4, L, pl);
+                }
             });
     }
     if constexpr (RM) {
         reduce_store_rows<WAVES>(o[0], Out + ob, I * 32, w, li, h, lds, old_);
-        return;
+    } else {
+        reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
+        if (OutCopy) {
+            __syncthreads();
+            reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+        }
     }
-    reduce_store<D, WAVES, true>(o, Out + hb, I * 32, w, li, h, lds, L);
-    if (OutCopy) {
+    if constexpr (MEAN) {
+        // this wavefront's slab stores are complete before its loads of the next head; the barrier also frees the
+        // shared arrays for the next head
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
     }
+    bh += bh_step;
+    } while (MEAN && bh < NB);
 }
 
 // Row pass: g_i = sum_j dP_ij P_ij (kept in G), dS = (dP*P - P*g)*scale, dQ^T = K^T-tiles . dS^T.
@@ -687,6 +717,8 @@ struct DenseAttn {
     // takes its row sums g_i = dO_i . O_i from it instead of a sweep over the whole map.
     float* ws_out = nullptr;      // [NB][d][L]
     const float* out_key = nullptr;
+    float* ws_mean = nullptr;     // [C][L][L] partial sums of the maps (mean-emitting forward)
+    size_t ws_mean_floats = 0;
 };
 
 static DenseAttn* as_dense(void* h, const char* who) {
@@ -726,6 +758,7 @@ void dense_destroy(void* h) {
     if (!a) return;
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_out) (void)hipFree(a->ws_out);
+    if (a->ws_mean) (void)hipFree(a->ws_mean);
     a->hdr.magic = 0;
     note_current_handle(nullptr);
     delete a;
@@ -850,9 +883,14 @@ static DenseAttn* dense_strided_handle(void* h, const char* who, int heads, cons
 }
 static bool dense_aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-void dense_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
-                           float* Out, int heads, const HeadLayout& in, const HeadLayout& out) {
-    const char* who = "dense attn_forward_strided";
+int score_map_mean(const float* Attn, int batch, int heads, int L, int key_major, float* Mean, hipStream_t stream,
+                   float post);
+
+// Mean != nullptr: the launch also leaves the mean of all NB maps (queries x keys) in Mean, accumulated while the
+// maps are written (see dense_fwd_reg_kernel) and finished by one reduction over the partial maps.
+static void dense_forward_strided_impl(void* h, const float* Q, const float* K, const float* V, const float* Mask,
+                                       float* Attn, float* Out, float* Mean, int heads, const HeadLayout& in,
+                                       const HeadLayout& out, const char* who) {
     const HeadLayout* lays[2] = {&in, &out};
     DenseAttn* a = dense_strided_handle(h, who, heads, lays, 2);
     if (!a) return;
@@ -880,6 +918,38 @@ void dense_forward_strided(void* h, const float* Q, const float* K, const float*
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB), block4(64 * 4);
     a->out_key = nullptr;  // no kept copy: the strided backward is handed Out
+    if (Mean) {
+        // C partial maps: the smallest divisor of NB that gives the launch two work-groups per CU
+        int C = a->NB;
+        for (int c = 1; c <= a->NB; ++c)
+            if (a->NB % c == 0 && (long long)c * nbr >= 512) {
+                C = c;
+                break;
+            }
+        const size_t need = (size_t)C * a->L * a->L;
+        if (need > a->ws_mean_floats) {
+            if (a->ws_mean) {
+                if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return;
+                (void)hipFree(a->ws_mean);
+                a->ws_mean = nullptr;
+                a->ws_mean_floats = 0;
+            }
+            if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_mean, sizeof(float) * need))) return;
+            a->ws_mean_floats = need;
+        }
+        const dim3 grid_m(nbr * C);
+#define SPION_LAUNCH(KERNEL, MM)                                                                                     \
+    hipLaunchKernelGGL((KERNEL<MM, true, true>), grid_m, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out, nullptr, \
+                       a->L, nbr, a->NB, a->scale, ly, a->ws_mean, C)
+        // the two-sweep kernel for every length: the register-resident one has no registers left for the partial sums
+        if (a->has_mask) SPION_LAUNCH(dense_fwd_sweep32_kernel, true);
+        else SPION_LAUNCH(dense_fwd_sweep32_kernel, false);
+#undef SPION_LAUNCH
+        if (!check_launch("dense_fwd kernels")) return;
+        // mean over the C partial sums, times C / NB: the mean of all maps, transposed to queries x keys
+        (void)score_map_mean(a->ws_mean, C, 1, a->L, 1, Mean, a->hdr.stream, (float)C / (float)a->NB);
+        return;
+    }
     if (nbr <= 32) {
         if (a->has_mask)
             hipLaunchKernelGGL((dense_fwd_reg_kernel<true, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn,
@@ -896,6 +966,20 @@ void dense_forward_strided(void* h, const float* Q, const float* K, const float*
                                Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
     }
     check_launch("dense_fwd kernels");
+}
+
+void dense_forward_strided(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                           float* Out, int heads, const HeadLayout& in, const HeadLayout& out) {
+    dense_forward_strided_impl(h, Q, K, V, Mask, Attn, Out, nullptr, heads, in, out, "dense attn_forward_strided");
+}
+void dense_forward_strided_mean(void* h, const float* Q, const float* K, const float* V, const float* Mask, float* Attn,
+                                float* Out, float* Mean, int heads, const HeadLayout& in, const HeadLayout& out) {
+    if (!Mean) {
+        as_dense(h, "dense attn_forward_strided_mean");
+        set_error("dense attn_forward_strided_mean: null Mean");
+        return;
+    }
+    dense_forward_strided_impl(h, Q, K, V, Mask, Attn, Out, Mean, heads, in, out, "dense attn_forward_strided_mean");
 }
 
 void dense_backward_strided(void* h, const float* Q, const float* K, const float* V, const float* P, const float* Out,

@@ -280,7 +280,7 @@ static size_t g_pool_ws_count = 0;
 // reference's column-major map) and the mean is written queries x keys, transposed through LDS.
 template <bool KEY_MAJOR>
 __global__ __launch_bounds__(256) void score_map_mean_kernel(const float* __restrict__ A, int batch, int heads, int L,
-                                                             float* __restrict__ Mean) {
+                                                             float* __restrict__ Mean, float post) {
     __shared__ float tile[32][33];
     const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
     const int r0 = blockIdx.y * 32, c0 = blockIdx.x * 32;
@@ -301,17 +301,20 @@ __global__ __launch_bounds__(256) void score_map_mean_kernel(const float* __rest
     }
     if (KEY_MAJOR) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) tile[ty + 8 * j][tx] = hs[j] / (float)heads;
+        for (int j = 0; j < 4; ++j) tile[ty + 8 * j][tx] = hs[j] / (float)heads * post;
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < 4; ++j) Mean[(size_t)(c0 + ty + 8 * j) * L + r0 + tx] = tile[tx][ty + 8 * j];
     } else {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) Mean[(size_t)(r0 + ty + 8 * j) * L + c0 + tx] = hs[j] / (float)heads;
+        for (int j = 0; j < 4; ++j) Mean[(size_t)(r0 + ty + 8 * j) * L + c0 + tx] = hs[j] / (float)heads * post;
     }
 }
 
-int score_map_mean(const float* Attn, int batch, int heads, int L, int key_major, float* Mean, hipStream_t stream) {
+// post: factor applied to the result (1 for a plain mean; sums of several maps each are turned into the mean of all
+// maps by batch / number of maps summed).
+int score_map_mean(const float* Attn, int batch, int heads, int L, int key_major, float* Mean, hipStream_t stream,
+                   float post) {
     if (!Attn || !Mean || batch <= 0 || heads <= 0 || L <= 0 || L % 32) {
         set_error("spion_score_map_mean: need Attn, Mean, batch > 0, heads > 0 and seq_len a positive multiple of 32 "
                   "(got %d, %d, %d)", batch, heads, L);
@@ -323,9 +326,103 @@ int score_map_mean(const float* Attn, int batch, int heads, int L, int key_major
     }
     const dim3 grid(L / 32, L / 32), block(256);
     if (key_major)
-        hipLaunchKernelGGL(score_map_mean_kernel<true>, grid, block, 0, stream, Attn, batch, heads, L, Mean);
+        hipLaunchKernelGGL(score_map_mean_kernel<true>, grid, block, 0, stream, Attn, batch, heads, L, Mean, post);
     else
-        hipLaunchKernelGGL(score_map_mean_kernel<false>, grid, block, 0, stream, Attn, batch, heads, L, Mean);
+        hipLaunchKernelGGL(score_map_mean_kernel<false>, grid, block, 0, stream, Attn, batch, heads, L, Mean, post);
+    return SPION_HIP_OK(hipGetLastError()) ? 0 : 1;
+}
+
+// -------------------------------------------------------------------------------------------------
+// Dense-to-sparse transition test on the device (main_conv_ff.py:211-242).  After every evaluation the averaged
+// score map of each layer is compared with the map kept from an earlier evaluation; the Frobenius distance of the
+// two is compared with the previous distance, and once it changed by less than `percent` per cent (after
+// truncation to an integer) in every layer the pattern counts as settled.  All state lives in device memory:
+//   Prev  [layers][n]  the kept maps;
+//   State [2*layers+3] floats: before_distance per layer, change in per cent per layer, then stage
+//         (0 = no map kept yet, 1 = a map but no distance yet, 2 = map and distance), the transition flag and a
+//         scratch word (whether this call replaces the kept maps).
+// The host reads State[2*layers+1] once per evaluation; nothing else comes back.
+// -------------------------------------------------------------------------------------------------
+constexpr int TRANS_BLOCK = 256;
+__global__ __launch_bounds__(TRANS_BLOCK) void transition_partial_kernel(const float* __restrict__ Prev,
+                                                                         const float* __restrict__ Cur, long long n,
+                                                                         double* __restrict__ Partial) {
+    __shared__ double red[TRANS_BLOCK];
+    const int layer = blockIdx.y, nblk = gridDim.x;
+    const float* a = Prev + (size_t)layer * n;
+    const float* b = Cur + (size_t)layer * n;
+    double s = 0.0;
+    for (long long i = (long long)blockIdx.x * TRANS_BLOCK + threadIdx.x; i < n; i += (long long)nblk * TRANS_BLOCK) {
+        const float dlt = a[i] - b[i];  // float difference, as torch computes it
+        s += (double)dlt * (double)dlt;
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = TRANS_BLOCK / 2; o > 0; o >>= 1) {  // fixed order: the result does not depend on timing
+        if ((int)threadIdx.x < o) red[threadIdx.x] += red[threadIdx.x + o];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) Partial[(size_t)layer * nblk + blockIdx.x] = red[0];
+}
+
+__global__ void transition_decide_kernel(const double* __restrict__ Partial, int nblk, int layers, int percent,
+                                         float* __restrict__ State) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    float* before = State;
+    float* diff = State + layers;
+    float& stage = State[2 * layers];
+    float& flag = State[2 * layers + 1];
+    float& replace = State[2 * layers + 2];
+    replace = 0.f;
+    if (flag != 0.f) return;
+    if (stage == 0.f) {  // first evaluation: keep the maps, nothing to compare with
+        stage = 1.f;
+        replace = 1.f;
+        return;
+    }
+    int settled = 0;
+    for (int l = 0; l < layers; ++l) {
+        double s = 0.0;
+        for (int k = 0; k < nblk; ++k) s += Partial[(size_t)l * nblk + k];
+        const float dist = (float)sqrt(s);
+        if (stage == 1.f) {  // second evaluation: the first distance; the kept maps stay
+            before[l] = dist;
+            diff[l] = 0.f;
+        } else {
+            diff[l] = (fabsf(dist - before[l]) / before[l]) * 100.f;
+            before[l] = dist;
+            if ((int)diff[l] < percent) ++settled;
+        }
+    }
+    if (stage == 1.f) {
+        stage = 2.f;
+        return;
+    }
+    if (settled == layers) flag = 1.f;
+    else replace = 1.f;
+}
+
+__global__ __launch_bounds__(256) void transition_replace_kernel(float* __restrict__ Prev, const float* __restrict__ Cur,
+                                                                 long long total, const float* __restrict__ State,
+                                                                 int layers) {
+    if (State[2 * layers + 2] == 0.f) return;
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long long)gridDim.x * 256)
+        Prev[i] = Cur[i];
+}
+
+int transition_update(const float* Cur, float* Prev, int layers, long long n, float* State, double* Partial,
+                      int partial_blocks, int percent, hipStream_t stream) {
+    if (!Cur || !Prev || !State || !Partial || layers <= 0 || n <= 0 || partial_blocks <= 0 || layers > 65535) {
+        set_error("spion_transition_update: bad arguments");
+        return 1;
+    }
+    hipLaunchKernelGGL(transition_partial_kernel, dim3(partial_blocks, layers), dim3(TRANS_BLOCK), 0, stream, Prev, Cur,
+                       n, Partial);
+    hipLaunchKernelGGL(transition_decide_kernel, dim3(1), dim3(64), 0, stream, Partial, partial_blocks, layers, percent,
+                       State);
+    const long long total = n * layers;
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 2048);
+    hipLaunchKernelGGL(transition_replace_kernel, dim3(blocks), dim3(256), 0, stream, Prev, Cur, total, State, layers);
     return SPION_HIP_OK(hipGetLastError()) ? 0 : 1;
 }
 

@@ -179,6 +179,17 @@ __device__ __forceinline__ void str_tile_lin(rsrc_t r, int voff, int soff, int l
     for (int i = 0; i < 4; ++i)
         __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, raw[i]), r, voff, soff + 32 * i * ld, 2);
 }
+// The same tile access for data a work-group reads back after writing it (partial sums kept in memory): loads are
+// served by the L2 (device-scope policy: the vector L1 is not consulted), stores use the default policy.
+__device__ __forceinline__ void ldr_tile_lin_l2(rsrc_t r, int voff, int soff, int ld, f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        raw[i] = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff + 32 * i * ld, 16));
+}
+__device__ __forceinline__ void str_tile_lin_cached(rsrc_t r, int voff, int soff, int ld, const f32x4 (&raw)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st4(r, voff, soff + 32 * i * ld, raw[i]);
+}
 __device__ __forceinline__ void lds_put_lin(float* T, int l, const f32x4 (&raw)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) *reinterpret_cast<f32x4*>(T + (8 * i + (l >> 3)) * TS + 4 * (l & 7)) = raw[i];

@@ -98,3 +98,59 @@ class TransitionDetector:
         else:
             self.before_attn = cur
         return self.transition
+
+
+class DeviceTransitionDetector:
+    """The same test with its state on the GPU (``spion_transition_update``): the distances, their comparison and
+    the replacement of the kept maps run as three small kernels, and one float comes back per evaluation, where
+    ``TransitionDetector`` synchronises on a reduction per layer.  ``update(attn_lst)`` takes the layers' averaged
+    score maps ([L, L] CUDA tensors, or one stacked [layers, L, L] tensor) and returns the decision; ``diff`` and
+    ``before_distance`` read the device state back for logging."""
+
+    PARTIAL_BLOCKS = 256
+
+    def __init__(self, num_layers: int, percent: int = 15):
+        self.num_layers = num_layers
+        self.percent = percent
+        self.transition = False
+        self._prev = None
+        self._state = None
+        self._partial = None
+
+    def _state_host(self):
+        return self._state.cpu().tolist() if self._state is not None else [0.0] * (2 * self.num_layers + 3)
+
+    @property
+    def before_distance(self):
+        return self._state_host()[: self.num_layers]
+
+    @property
+    def diff(self):
+        return self._state_host()[self.num_layers: 2 * self.num_layers]
+
+    def update(self, attn_lst) -> bool:
+        from . import _lib
+
+        if self.transition:
+            return True
+        if isinstance(attn_lst, torch.Tensor):
+            cur = attn_lst[: self.num_layers]
+        else:
+            cur = torch.stack([attn_lst[l].detach() for l in range(self.num_layers)], 0)
+        cur = cur.detach().to(torch.float32).contiguous()
+        if not cur.is_cuda:
+            raise _lib.SpionLibraryError("DeviceTransitionDetector runs on the GPU only; got CPU tensors")
+        if self._prev is None:
+            self._prev = torch.empty_like(cur)
+            self._state = torch.zeros(2 * self.num_layers + 3, dtype=torch.float32, device=cur.device)
+            self._partial = torch.empty(self.num_layers * self.PARTIAL_BLOCKS, dtype=torch.float64, device=cur.device)
+        elif self._prev.shape != cur.shape:
+            raise ValueError(f"score maps changed shape: {tuple(self._prev.shape)} -> {tuple(cur.shape)}")
+        stream = torch.cuda.current_stream(cur.device).cuda_stream
+        rc = _lib.core().spion_transition_update(cur.data_ptr(), self._prev.data_ptr(), self.num_layers,
+                                                 cur[0].numel(), self._state.data_ptr(), self._partial.data_ptr(),
+                                                 self.PARTIAL_BLOCKS, self.percent, stream)
+        if rc != 0:
+            _lib.check_error("spion_transition_update")
+        self.transition = bool(self._state[2 * self.num_layers + 1].item() != 0.0)  # the one read-back
+        return self.transition

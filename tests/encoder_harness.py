@@ -87,8 +87,15 @@ class EncoderForSC(nn.Module):
         attn_lst = []
         for idx, layer in enumerate(self.layers):
             if mat_lst is None:
+                core = getattr(layer.mha, "attn", None)
+                fused = is_attn and hasattr(core, "emit_score_map")  # the HIP modules average while they write the maps
+                if fused:
+                    core.emit_score_map = True
                 X, attn = layer(X, mask)
-                if is_attn:  # models/model_transformer.py:136-137: mean over batch, then over heads
+                if fused:
+                    core.emit_score_map = False
+                    attn_lst.append(core.score_map)
+                elif is_attn:  # models/model_transformer.py:136-137: mean over batch, then over heads
                     attn_lst.append(torch.mean(torch.mean(attn, dim=0), dim=0))
             else:
                 X, attn = layer(X, mask, mat_lst[0][idx])

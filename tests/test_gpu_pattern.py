@@ -136,3 +136,88 @@ def test_mean_score_map_matches_torch(B, H, L):
         assert p.stride() == (H * L * L, L * L, 1, L)
         ref = torch.mean(torch.mean(p.double(), dim=0), dim=0)
         assert torch.max(torch.abs(spion_amd.mean_score_map(p).double() - ref)).item() < 1e-6
+
+
+@pytest.mark.parametrize("B,H,L,with_mask", [(3, 2, 64, False), (16, 2, 256, True), (64, 2, 1024, False), (4, 2, 2048, True)])
+def test_fused_score_map_from_the_dense_forward(B, H, L, with_mask):
+    """The mean map the dense forward accumulates while it writes the maps (spion_dense_forward_strided_mean) against
+    the two torch.mean passes of models/model_transformer.py:136-137 over the returned maps, in float64; outputs and
+    maps of that forward agree with the plain forward's."""
+    import spion_amd
+    from spion_amd.attention import Attention
+
+    d = 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
+    if with_mask:
+        cpp = Attention._cuda_mask_compile_module()
+        mod = spion_amd.CUDAMaskAttention(cfg, cpp, cpp.init(d, L, B * H))
+    else:
+        cpp = Attention._cuda_compile_module()
+        mod = spion_amd.CUDAAttention(cfg, cpp, cpp.init(d, L, B * H))
+    g = torch.Generator().manual_seed(B + L)
+    q, k, v = (torch.randn(B, H, L, d, generator=g).cuda() for _ in range(3))
+    lens = torch.randint(L // 2, L + 1, (B, 1), generator=g)
+    key_mask = (torch.arange(L)[None, :] < lens).float().cuda()
+    out0, p0 = mod(q, k, v, key_mask)
+    assert mod.score_map is None
+    mod.emit_score_map = True
+    for rep in range(2):   # the second call reuses the partial maps the first one left
+        out1, p1 = mod(q, k, v, key_mask)
+        if L > 1024:   # the same two-sweep kernel with and without the mean
+            assert torch.equal(out0, out1) and torch.equal(p0, p1)
+        else:          # up to 1024 the plain forward keeps the logits in registers, the mean-emitting one sweeps twice
+            assert torch.allclose(out0, out1, rtol=1e-5, atol=1e-6) and torch.allclose(p0, p1, rtol=1e-5, atol=1e-9)
+        ref = torch.mean(torch.mean(p1.double(), dim=0), dim=0)
+        got = mod.score_map
+        assert got.shape == (L, L) and got.is_contiguous()
+        err = torch.max(torch.abs(got.double() - ref)).item()
+        assert err < 2e-7 * max(1.0, float(ref.abs().max()) * 1e3), err
+        assert torch.allclose(got.double(), ref, rtol=1e-5, atol=1e-9)
+    # the map feeds discovery as it is
+    m = spion_amd.discover_block_masks(mod.score_map[None], 32, mode="conv_ff", threshold=0.9)
+    assert m.shape == (1, L // 32, L // 32)
+
+
+def test_device_transition_detector_matches_host_detector():
+    """spion_transition_update against the host statement of main_conv_ff.py:211-242 on the hand-worked sequences
+    (1x1 maps: distances are absolute differences) and on random maps with a drift that settles."""
+    from spion_amd import DeviceTransitionDetector, TransitionDetector
+
+    def maps(*values):
+        return [torch.tensor([[float(v)]]).cuda() for v in values]
+
+    det = DeviceTransitionDetector(1)
+    assert det.update(maps(0.0)) is False
+    assert det.update(maps(10.0)) is False
+    assert det.update(maps(10.5)) is True           # distance to the FIRST map 10.5: change 5 %
+    assert det.update(maps(99.0)) is True
+    det = DeviceTransitionDetector(1)
+    det.update(maps(0.0)); det.update(maps(10.0))
+    assert det.update(maps(20.0)) is False          # change 100 %: the kept map becomes 20
+    assert det.update(maps(41.0)) is True           # distance 21: change 5 %
+    for last, want in ((115.9, False), (114.99, True)):   # 15.9 % truncates to 15 (not below), 14.99 % to 14
+        det = DeviceTransitionDetector(1)
+        det.update(maps(0.0)); det.update(maps(100.0))
+        assert det.update(maps(last)) is want
+    det = DeviceTransitionDetector(2)
+    det.update(maps(0.0, 0.0)); det.update(maps(10.0, 10.0))
+    assert det.update(maps(10.5, 30.0)) is False    # layer 1 changed by 200 %
+    assert abs(det.diff[0] - 5.0) < 1e-3 and abs(det.diff[1] - 200.0) < 1e-2
+
+    # random maps: identical decisions and distances as the host detector, evaluation by evaluation
+    g = torch.Generator().manual_seed(7)
+    L, layers = 256, 3
+    base = torch.rand(layers, L, L, generator=g)
+    host, dev = TransitionDetector(layers), DeviceTransitionDetector(layers)
+    decided = None
+    for step in range(12):
+        cur = base + torch.randn(layers, L, L, generator=g) * (0.5 / (1 + step) ** 2)
+        a = host.update([cur[l] for l in range(layers)])
+        b = dev.update(cur.cuda())
+        assert a == b, step
+        if host.before_distance:
+            for x, y in zip(host.before_distance, dev.before_distance):
+                assert abs(float(x) - y) <= 1e-5 * abs(float(x))
+        if a and decided is None:
+            decided = step
+    assert decided is not None and decided >= 2
