@@ -694,7 +694,11 @@ def bench_sparse_layer(args, dev, workload, full=True):
     alg_bytes = workloads.sparse_bytes(nnz, L, d, NB)
     third = alg_flops / 3.0  # forward, row pass and column pass carry 4*n*d*NB each
     names = {1: ("tile_fwd_kernel", "tile_bwd_row_kernel", "tile_bwd_col_kernel"),
-             2: ("elem_fwd_kernel", "elem_bwd_row_kernel", "elem_bwd_col_kernel")}[path]
+             2: ("elem_fwd_kernel", "elem_bwd_row_kernel", "elem_bwd_col_kernel"),
+             # hybrid: dense window tiles on the MFMA units + gathered remainder; each phase is two or three launches
+             3: ("hyb_rem_logits_kernel + hyb_tile_fwd_kernel + hyb_rem_pv_kernel",
+                 "hyb_tile_bwd_row_kernel + hyb_rem_bwd_row_kernel",
+                 "hyb_tile_bwd_col_kernel + hyb_rem_bwd_col_kernel")}[path]
     kernels = dict(zip(names, (t_fwd, t_row, t_col)))
     dom = max(kernels, key=kernels.get)
     dom_ms = kernels[dom]
@@ -745,7 +749,7 @@ def bench_sparse_layer(args, dev, workload, full=True):
         "config": {"workload": f"{wl['name']}: sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, "
                                f"block {bs}, nnz/head={nnz}, block density="
                                f"{wl['block_density'] if wl['block_density'] is None else round(wl['block_density'], 4)}",
-                   "kernel_path": {1: "mfma-tile", 2: "element"}[path]},
+                   "kernel_path": {1: "mfma-tile", 2: "element", 3: "hybrid (mfma tiles + gathered remainder)"}[path]},
         "rowmajor_abi_ms": {"attn_forward": round(t_fwd, 4), "attn_backward": round(t_bwd, 4),
                             "fwd_plus_bwd": round(t_fwd + t_bwd, 4), "fwd_then_bwd_sequence": round(t_seq, 4),
                             "what": "spion_attn_forward_rowmajor / spion_attn_backward_rowmajor, the entry points "

@@ -1,0 +1,612 @@
+// Hybrid kernels for element-sparse patterns (d = 32): the well-filled aligned 32 x 32 tiles of the pattern (the
+// local window of a "window + random columns" pattern, say) run as dense MFMA tiles with a bit mask for the entries
+// that are absent, the remaining entries as per-row gathers; the softmax statistics are merged across the two
+// parts, and P stays in CSR order exactly as the reference's kernels leave it (models/block_attn_mask.cu:88-140):
+// a tile's entries of one row are consecutive in that row's CSR run, so `first position + number of present
+// columns to the left` addresses them.
+//
+// Per pattern entry the gather path costs about as much machine time as 1/80 of a 32 x 32 MFMA tile, so a tile
+// with more than ~10 % of its entries present is cheaper dense.
+//
+// The two parts run as separate launches, each at the occupancy that suits it: the tile kernels (one work-group of
+// four wavefronts per strip of 32 rows or columns, wavefront w taking the strip's dense tiles w, w+4, ...) and the
+// gather kernels (one wavefront per row or column of the remainder, sixteen wavefronts per CU, because the gathers
+// are bound by the number of requests in flight).  Forward: remainder logits and their row statistics, then the
+// tiles (which merge the statistics and fix the row's maximum and denominator), then the remainder's probabilities
+// and share of O.  Backward: tile part then remainder part of the row pass, the same for the column pass; the
+// remainder kernels add to what the tile kernels wrote (each row or column has exactly one writer per launch).
+#pragma once
+#include "tile_kernels.h"
+
+namespace spion {
+
+// The analysed pattern as the kernels see it (device pointers, shared by all heads).
+struct HybIndex {
+    // dense tiles, by block row: tiles t_rp[I] .. t_rp[I+1]-1 of block row I; per tile its block column, its block
+    // row, and per row of the tile the position of the row's first entry inside a head's P and the 32-bit set of
+    // present columns
+    const int* t_rp;
+    const int* t_col;
+    const int* t_row;
+    const int* t_pos;        // [tiles][32]
+    const unsigned* t_bits;  // [tiles][32]
+    // the same tiles by block column: tile ids t_ct[t_cp[J]] .. of block column J
+    const int* t_cp;
+    const int* t_ct;
+    // remainder entries in CSR form (r_off [L+1], columns, positions inside a head's P) and in CSC form (c_ptr
+    // [L+1], rows ascending within a column, positions)
+    const int* r_off;
+    const int* r_col;
+    const int* r_pos;
+    const int* c_ptr;
+    const int* c_row;
+    const int* c_pos;
+};
+
+constexpr int HYB_WAVES = 4;
+constexpr int HYB_MAXT = 4;     // dense tiles per wavefront whose logits stay in registers (forward)
+constexpr int HYB_GWAVES = 4;    // wavefronts (rows / columns) per work-group of the gather kernels
+constexpr float HYB_ABSENT = -1.0e30f;  // logit of an entry that is not in the pattern: exp2 gives exactly 0
+// three work-groups per CU: these launches have few tiles per wavefront and live on latency
+#define SPION_HYB_KERNEL __global__ __launch_bounds__(64 * HYB_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3)))
+
+// Positions and present-column sets of the 16 tile rows acc_row(q, h), q = 0..15, of tile t.
+__device__ __forceinline__ void hyb_tile_rows(const HybIndex& ix, int t, int h, int (&pos)[16], unsigned (&bits)[16]) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const int4 p = *reinterpret_cast<const int4*>(ix.t_pos + (size_t)t * 32 + 8 * g + 4 * h);
+        const uint4 b = *reinterpret_cast<const uint4*>(ix.t_bits + (size_t)t * 32 + 8 * g + 4 * h);
+        pos[4 * g + 0] = p.x, pos[4 * g + 1] = p.y, pos[4 * g + 2] = p.z, pos[4 * g + 3] = p.w;
+        bits[4 * g + 0] = b.x, bits[4 * g + 1] = b.y, bits[4 * g + 2] = b.z, bits[4 * g + 3] = b.w;
+    }
+}
+// The tile of P in the col-owner layout (lane li = column of the tile, register q = row acc_row(q, h)); absent
+// entries read as 0.  A tile row's entries are consecutive in memory: every instruction touches one run per
+// half-wave.
+__device__ __forceinline__ void hyb_load_p_cols(const float* __restrict__ Ph, const int (&pos)[16],
+                                                const unsigned (&bits)[16], int li, float (&pc)[16]) {
+    const unsigned below = (1u << li) - 1u;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+        const bool on = (bits[q] >> li) & 1u;
+        pc[q] = on ? Ph[pos[q] + __popc(bits[q] & below)] : 0.f;
+    }
+}
+__device__ __forceinline__ void hyb_store_p_cols(float* __restrict__ Ph, const int (&pos)[16],
+                                                 const unsigned (&bits)[16], int li, const float (&pc)[16]) {
+    const unsigned below = (1u << li) - 1u;
+#pragma unroll
+    for (int q = 0; q < 16; ++q)
+        if ((bits[q] >> li) & 1u) Ph[pos[q] + __popc(bits[q] & below)] = pc[q];
+}
+
+// Sum of the four wavefronts' 32 x 32 accumulators (rows acc_row(r, h) of the strip, columns li) times `factor`,
+// in a fixed order.  `lds` (4096 floats) may alias tile space no wavefront uses any more: the caller has a barrier
+// between that use and this call.
+__device__ __forceinline__ void hyb_reduce_store(const f32x16& acc, float factor, float* __restrict__ out,
+                                                 float* __restrict__ out2, int row0, int w, int li, int h,
+                                                 float* __restrict__ lds) {
+    const int l = h * 32 + li;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) lds[(w * 16 + r) * 64 + l] = acc[r];
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        if ((r % HYB_WAVES) != w) continue;
+        float s = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < HYB_WAVES; ++ww) s += lds[(ww * 16 + r) * 64 + l];
+        s *= factor;
+        const size_t a = (size_t)(row0 + acc_row(r, h)) * 32 + li;
+        out[a] = s;
+        if (out2) out2[a] = s;
+    }
+}
+
+// =================================================================================================
+// gather helpers (one wavefront per row / column of the remainder)
+// =================================================================================================
+// The gather kernels hold a chunk of up to 64 entries one per lane and fetch the entries' 32-float rows eight lanes
+// to a row (16 bytes per lane, eight rows per load instruction).  Lane L owns entry (L % 8) * 8 + L / 8 of the chunk,
+// so that the eight entries group g = L / 8 fetches (entry j*8 + g in instruction j) are the entries its own eight
+// lanes own: every exchange stays inside a group of eight lanes, nothing goes through LDS memory, and the number of
+// wavefronts in flight -- what bounds these latency-bound kernels -- is not limited by LDS space.
+__device__ __forceinline__ int hyb_entry_of_lane(int lane) { return ((lane & 7) << 3) | (lane >> 3); }
+
+// sum over the eight lanes of a group (quad swaps, then the mirror image of the half row)
+__device__ __forceinline__ float hyb_group_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // xor 1
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // xor 2
+    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // 7 - i
+    return v;
+}
+
+// Dot products of the rows X[row_l] (row index of the lane's entry; nk entries in the chunk) with the vector whose
+// piece 4*(lane%8) .. +3 the lane holds in a4: one result per lane, for the lane's own entry.  Only the load
+// instructions that carry entries are issued; lanes whose entry is past nk get 0 or a partial value to ignore.
+__device__ __forceinline__ float hyb_gather_dot(const f32x4 a4, const float* __restrict__ X, int row_l, int nk,
+                                                int lane) {
+    constexpr int D = 32;
+    const int base = lane & ~7, cl = lane & 7;
+    f32x4 x[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int rr = __shfl(row_l, base + j, 64);
+        if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * D)[cl];
+    }
+    float r = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if (j * 8 < nk) {
+            float sj = x[j].x * a4.x;
+            sj = fmaf(x[j].y, a4.y, sj);
+            sj = fmaf(x[j].z, a4.z, sj);
+            sj = fmaf(x[j].w, a4.w, sj);
+            sj = hyb_group_sum(sj);
+            r = cl == j ? sj : r;
+        }
+    }
+    return r;
+}
+
+// acc += sum over the chunk's entries (weight w_l and row index row_l of the lane's entry; nk entries) of
+// w * X[row][:]; the lane accumulates the piece 4*(lane%8) .. +3 of the rows its group fetches.
+struct HybRowAcc {
+    f32x4 acc;
+    __device__ __forceinline__ void clear() { acc = (f32x4){0.f, 0.f, 0.f, 0.f}; }
+    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int lane) {
+        constexpr int D = 32;
+        const int base = lane & ~7, cl = lane & 7;
+        float w[8];
+        f32x4 x[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            w[j] = __shfl(w_l, base + j, 64);
+            const int rr = __shfl(row_l, base + j, 64);
+            if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * D)[cl];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (j * 8 < nk) acc += w[j] * x[j];  // entries past nk inside a carried instruction have weight 0
+    }
+    // sum over the eight groups; every lane then holds the four floats 4*(lane%8) .. of the result row
+    __device__ __forceinline__ f32x4 total() const {
+        f32x4 a = acc;
+#pragma unroll
+        for (int o = 8; o < 64; o <<= 1)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] += __shfl_xor(a[e], o, 64);
+        return a;
+    }
+};
+#define SPION_HYB_GATHER_KERNEL __global__ __launch_bounds__(64 * HYB_GWAVES) __attribute__((amdgpu_waves_per_eu(6, 8)))
+
+// -------------------------------------------------------------------------------------------------
+// Forward, step 1: raw logits (log2 domain) of the remainder entries into P, and per row their maximum and the sum
+// of their exponentials relative to it: Stats[bh][row] = {m, z} ({HYB_ABSENT, 0} for a row without remainder).
+// -------------------------------------------------------------------------------------------------
+template <bool MASK>
+SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+                                                   const float* __restrict__ pen, float* __restrict__ P,
+                                                   float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz,
+                                                   float scale) {
+    const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
+    const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
+    if (wrow >= (long long)NB * L) return;
+    const int bh = (int)(wrow / L), row = (int)(wrow % L);
+    const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
+    const size_t hb = (size_t)bh * L * 32;
+    float* Ph = P + (size_t)bh * nnz;
+    const float c2 = scale * LOG2E;
+    f32x4 q4 = reinterpret_cast<const f32x4*>(Q + hb + (size_t)row * 32)[lane & 7];
+    q4 *= c2;
+    // the logits of the first chunks stay in registers; longer rows go back to what they stored in P
+    constexpr int KEEP = 2;
+    float vk[KEEP];
+    float mx = HYB_ABSENT;
+    for (int c0 = 0; c0 < rc; c0 += 64) {
+        const int k = c0 + ent;
+        const int col = k < rc ? ix.r_col[r0 + k] : 0;
+        const int pp = k < rc ? ix.r_pos[r0 + k] : 0;
+        float v = hyb_gather_dot(q4, K + hb, col, min(64, rc - c0), lane);
+        if (k < rc) {
+            if (MASK) v -= pen[(size_t)bh * L + col] * LOG2E;
+            Ph[pp] = v;
+            mx = fmaxf(mx, v);
+        } else {
+            v = HYB_ABSENT;
+        }
+#pragma unroll
+        for (int c = 0; c < KEEP; ++c)
+            if (c0 == 64 * c) vk[c] = v;
+    }
+    mx = wave_max(mx);
+    float z = 0.f;
+#pragma unroll
+    for (int c = 0; c < KEEP; ++c)
+        if (64 * c < rc) z += __builtin_amdgcn_exp2f(vk[c] - mx);
+    for (int k = 64 * KEEP + lane; k < rc; k += 64) z += __builtin_amdgcn_exp2f(Ph[ix.r_pos[r0 + k]] - mx);
+    z = wave_sum(z);
+    if (lane == 0) Stats[(size_t)bh * L + row] = make_float2(mx, z);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward, step 2: the dense tiles of a strip.  Logits in the log2 domain as in tile_fwd_kernel; the row's
+// maximum and denominator take in the remainder's statistics (Stats in: {m, z} of the remainder; out: {row
+// maximum, 1 / denominator} for step 3).  Writes the tiles' probabilities to their CSR positions and O = P.V of the
+// tile part (step 3 adds the remainder's share).
+// -------------------------------------------------------------------------------------------------
+template <bool MASK>
+SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+                                          const float* __restrict__ V, const float* __restrict__ pen,
+                                          float* __restrict__ P, float* __restrict__ O, float2* __restrict__ Stats,
+                                          const int* __restrict__ offs, HybIndex ix, int L, int nbr, int NB, int nnz,
+                                          float scale) {
+    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES, MAXT = HYB_MAXT;
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];  // two 32-row tiles per wavefront
+    float* lds = &lds_t[0][0];  // the final reduction reuses the tile space
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const rsrc_t rQ = make_rsrc(Q + hb, (size_t)L * D * 4), rK = make_rsrc(K + hb, (size_t)L * D * 4);
+    const rsrc_t rV = make_rsrc(V + hb, (size_t)L * D * 4);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    float* Ph = P + (size_t)bh * nnz;
+    float* T = lds_t[w];
+    float* Tx = T + 32 * TS;
+    const float c2 = scale * LOG2E;
+    const int lin = lin_voff(l, D);
+
+    float q[KH];
+    ldr_rows<D>(rQ, (li * D + h * KH) * 4, I * 32 * D * 4, q);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) q[s] *= c2;
+    const float2 rem = Stats[(size_t)bh * L + I * 32 + li];  // the remainder of row li
+
+    // ---- logits of this wavefront's tiles, own maximum ----------------------------------------------
+    const int t0 = ix.t_rp[I], cnt = ix.t_rp[I + 1] - t0;
+    const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;
+    float m = MASK ? 0.f : -100.f * LOG2E, z = 0.f;
+    f32x16 S[MAXT];
+    int Js[MAXT];
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) Js[u] = u < nu ? ix.t_col[t0 + w + u * WAVES] : 0;
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u < nu) {
+            const int t = t0 + w + u * WAVES;
+            f32x4 kraw[4];
+            ldr_tile_lin(rK, lin, Js[u] * 32 * D * 4, D, kraw);
+            const unsigned mybits = ix.t_bits[(size_t)t * 32 + li];  // present columns of this lane's row
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+                float pj[16];
+                ldr_4x4(rM, 16 * h, Js[u] * 128, pj);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = -LOG2E * pj[r];
+            }
+            lds_put_lin(Tx, l, kraw);
+            float kf[KH];
+            lds_get_feat32(Tx, li, h, kf);
+            S[u] = mma_feat_init<D>(kf, q, init);  // register = key acc_row(r, h), lane = query li
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (!((mybits >> acc_row(r, h)) & 1u)) S[u][r] = HYB_ABSENT;
+            m = max16(S[u], m);
+        }
+    }
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u < nu) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = __builtin_amdgcn_exp2f(S[u][r] - m);
+                S[u][r] = e;
+                z += e;
+            }
+        }
+    }
+    const float m_own = m;
+    z += __shfl_xor(z, 32, 64);
+    if (h == 0) {
+        lds_m[w][li] = m;
+        lds_z[w][li] = z;
+    }
+    __syncthreads();
+
+    // ---- merge: row maximum and denominator over the tiles of all wavefronts and the remainder ----
+    float Mx = rem.x;
+#pragma unroll
+    for (int ww = 0; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+    float Z = rem.y * __builtin_amdgcn_exp2f(rem.x - Mx);
+#pragma unroll
+    for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+    {
+        const int row = I * 32 + li;
+        const int n_i = offs[row + 1] - offs[row];
+        Z += (float)(L - n_i) * __builtin_amdgcn_exp2f(-Mx);
+    }
+    const float zinv = 1.0f / Z;  // +inf denominator -> 0 -> P = 0, as in the reference
+    const float rinv = __builtin_amdgcn_exp2f(m_own - Mx) * zinv;
+
+    // ---- probabilities, O += P.V, P to its CSR positions --------------------------------------------
+    f32x16 o[1] = {splat16(0.f)};
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u < nu) {
+            const int t = t0 + w + u * WAVES;
+            f32x4 vraw[4];
+            ldr_tile_lin(rV, lin, Js[u] * 32 * D * 4, D, vraw);
+            int pos[16];
+            unsigned bits[16];
+            hyb_tile_rows(ix, t, h, pos, bits);
+            lds_put_lin(Tx, l, vraw);
+            float p[16], vb[1][16], pc[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+            lds_put_rows(T, li, h, p);
+            lds_get_cols(Tx, li, h, vb[0]);
+            lds_get_cols(T, li, h, pc);
+            mma_b<D>(p, vb, o);
+            hyb_store_p_cols(Ph, pos, bits, li, pc);
+        }
+    }
+    __syncthreads();
+    // every wavefront has consumed the remainder's statistics by now: replace them by the row's final ones
+    if (w == 0 && h == 0) Stats[(size_t)bh * L + I * 32 + li] = make_float2(Mx, zinv);
+    hyb_reduce_store(o[0], 1.0f, O + hb, nullptr, I * 32, w, li, h, lds);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward, step 3: probabilities of the remainder entries from their raw logits and the row's {maximum,
+// 1 / denominator}; their share of O is added to what step 2 wrote.  Ocache (optional): second copy of O.
+// -------------------------------------------------------------------------------------------------
+SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, float* __restrict__ P,
+                                               float* __restrict__ O, float* __restrict__ Ocache,
+                                               const float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz) {
+    const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
+    const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
+    if (wrow >= (long long)NB * L) return;
+    const int bh = (int)(wrow / L), row = (int)(wrow % L);
+    const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
+    const size_t hb = (size_t)bh * L * 32;
+    float* Ph = P + (size_t)bh * nnz;
+    const float2 st = Stats[(size_t)bh * L + row];
+    HybRowAcc acc;
+    acc.clear();
+    for (int c0 = 0; c0 < rc; c0 += 64) {
+        const int k = c0 + ent;
+        float wgt = 0.f;
+        int col = 0;
+        if (k < rc) {
+            const int pp = ix.r_pos[r0 + k];
+            wgt = __builtin_amdgcn_exp2f(Ph[pp] - st.x) * st.y;
+            col = ix.r_col[r0 + k];
+            Ph[pp] = wgt;
+        }
+        acc.chunk(wgt, col, min(64, rc - c0), V + hb, lane);
+    }
+    const f32x4 tot = acc.total();
+    if (lane < 8) {
+        f32x4* orow = reinterpret_cast<f32x4*>(O + hb + (size_t)row * 32) + lane;
+        const f32x4 sum = *orow + tot;
+        *orow = sum;
+        if (Ocache) reinterpret_cast<f32x4*>(Ocache + hb + (size_t)row * 32)[lane] = sum;
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, row pass, dense tiles: g_i = dO_i . O_i (G receives -g for the other kernels); dP^T - g = V_J.dO_I^T
+// chain started from -g, dS' = (dP - g)*P, dQ = sum dS'.K_J / sqrt(d).
+// -------------------------------------------------------------------------------------------------
+SPION_HYB_KERNEL void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
+                                              const float* __restrict__ P, const float* __restrict__ dO,
+                                              const float* __restrict__ Out, float* __restrict__ G,
+                                              float* __restrict__ dQ, HybIndex ix, int L, int nbr, int NB, int nnz,
+                                              float scale) {
+    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES;
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
+    float* lds = &lds_t[0][0];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const rsrc_t rK = make_rsrc(K + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
+    const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4), rO = make_rsrc(Out + hb, (size_t)L * D * 4);
+    const float* Ph = P + (size_t)bh * nnz;
+    float* T = lds_t[w];
+    float* Tx = T + 32 * TS;
+    const int lin = lin_voff(l, D);
+
+    float go[KH], oo[KH];
+    ldr_rows<D>(rdO, (li * D + h * KH) * 4, I * 32 * D * 4, go);
+    ldr_rows<D>(rO, (li * D + h * KH) * 4, I * 32 * D * 4, oo);
+    float g = 0.f;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
+    g += __shfl_xor(g, 32, 64);
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;
+    const f32x16 gneg = splat16(-g);
+
+    const int t0 = ix.t_rp[I], cnt = ix.t_rp[I + 1] - t0;
+    f32x16 acc[1] = {splat16(0.f)};
+    for (int t = t0 + w; t < t0 + cnt; t += WAVES) {
+        const int J = ix.t_col[t];
+        f32x4 vraw[4], kraw[4];
+        ldr_tile_lin(rV, lin, J * 32 * D * 4, D, vraw);
+        ldr_tile_lin(rK, lin, J * 32 * D * 4, D, kraw);
+        int pos[16];
+        unsigned bits[16];
+        hyb_tile_rows(ix, t, h, pos, bits);
+        float pc[16], pr[16], vt[KH], kb[1][16];
+        hyb_load_p_cols(Ph, pos, bits, li, pc);
+        lds_put_lin(Tx, l, vraw);
+        lds_get_feat32(Tx, li, h, vt);
+        lds_put_cols(T, li, h, pc);
+        lds_get_rows(T, li, h, pr);                        // pr[r] = P[query li][key acc_row(r, h)]
+        const f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
+        lds_put_lin(Tx, l, kraw);
+        lds_get_cols(Tx, li, h, kb[0]);
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
+        mma_b<D>(ds, kb, acc);
+    }
+    __syncthreads();
+    hyb_reduce_store(acc[0], scale, dQ + hb, nullptr, I * 32, w, li, h, lds);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, row pass, remainder: dS = (dO_i . v_j - g_i) * P / sqrt(d) into the caller's dS scratch (for the
+// column pass), dQ_i += sum dS . K[col].
+// -------------------------------------------------------------------------------------------------
+SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
+                                                    const float* __restrict__ P, const float* __restrict__ dO,
+                                                    const float* __restrict__ G, float* __restrict__ dS,
+                                                    float* __restrict__ dQ, HybIndex ix, int L, int NB, int nnz,
+                                                    float scale) {
+    const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
+    const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
+    if (wrow >= (long long)NB * L) return;
+    const int bh = (int)(wrow / L), row = (int)(wrow % L);
+    const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
+    if (rc == 0) return;
+    const size_t hb = (size_t)bh * L * 32;
+    const f32x4 go4 = reinterpret_cast<const f32x4*>(dO + hb + (size_t)row * 32)[lane & 7];
+    const float* Ph = P + (size_t)bh * nnz;
+    float* dSh = dS + (size_t)bh * nnz;
+    const float gneg = G[(size_t)bh * L + row];
+    HybRowAcc acc;
+    acc.clear();
+    for (int c0 = 0; c0 < rc; c0 += 64) {
+        const int k = c0 + ent;
+        const int col = k < rc ? ix.r_col[r0 + k] : 0;
+        const int pp = k < rc ? ix.r_pos[r0 + k] : 0;
+        const float pv = k < rc ? Ph[pp] : 0.f;
+        const int nk = min(64, rc - c0);
+        const float dp = hyb_gather_dot(go4, V + hb, col, nk, lane);
+        float dsv = 0.f;
+        if (k < rc) {
+            dsv = (dp + gneg) * pv * scale;
+            dSh[pp] = dsv;
+        }
+        acc.chunk(dsv, col, nk, K + hb, lane);
+    }
+    const f32x4 tot = acc.total();
+    if (lane < 8) {
+        f32x4* qrow = reinterpret_cast<f32x4*>(dQ + hb + (size_t)row * 32) + lane;
+        *qrow = *qrow + tot;
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, column pass, dense tiles: dK_J = sum_I dS_IJ^T Q_I / sqrt(d), dV_J = sum_I P_IJ^T dO_I; dP - g is
+// recomputed per tile by a chain started from the stored -g.
+// -------------------------------------------------------------------------------------------------
+SPION_HYB_KERNEL void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const float* __restrict__ V,
+                                              const float* __restrict__ P, const float* __restrict__ dO,
+                                              const float* __restrict__ G, float* __restrict__ dK,
+                                              float* __restrict__ dV, HybIndex ix, int L, int nbr, int NB, int nnz,
+                                              float scale) {
+    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES;
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
+    float* lds = &lds_t[0][0];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const size_t hb = (size_t)bh * L * D;
+    const rsrc_t rQ = make_rsrc(Q + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
+    const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4);
+    const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
+    const float* Ph = P + (size_t)bh * nnz;
+    float* Tq = lds_t[w];
+    float* To = Tq + 32 * TS;
+    const int lin = lin_voff(l, D);
+
+    float vt[KH];
+    ldr_rows<D>(rV, (li * D + h * KH) * 4, J * 32 * D * 4, vt);
+
+    f32x16 ak[1] = {splat16(0.f)}, av[1] = {splat16(0.f)};
+    const int e0 = ix.t_cp[J], ecnt = ix.t_cp[J + 1] - e0;
+    for (int e = e0 + w; e < e0 + ecnt; e += WAVES) {
+        const int t = ix.t_ct[e];
+        const int I = ix.t_row[t];
+        f32x4 qraw[4], oraw[4];
+        ldr_tile_lin(rQ, lin, I * 32 * D * 4, D, qraw);
+        ldr_tile_lin(rdO, lin, I * 32 * D * 4, D, oraw);
+        float gn[16];
+        ldr_4x4(rG, 16 * h, I * 128, gn);
+        int pos[16];
+        unsigned bits[16];
+        hyb_tile_rows(ix, t, h, pos, bits);
+        float p[16], go[KH], qb[1][16], ob[1][16];
+        hyb_load_p_cols(Ph, pos, bits, li, p);  // p[r] = P[query acc_row(r, h)][key li]
+        lds_put_lin(Tq, l, qraw);
+        lds_put_lin(To, l, oraw);
+        lds_get_feat32(To, li, h, go);
+        lds_get_cols(Tq, li, h, qb[0]);
+        lds_get_cols(To, li, h, ob[0]);
+        f32x16 init;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) init[r] = gn[r];
+        const f32x16 dp = mma_feat_init<D>(go, vt, init);  // dO_i . v_j - g_i, i = acc_row(r, h), j = li
+        float ds[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * p[r];
+        mma_b<D>(ds, qb, ak);
+        mma_b<D>(p, ob, av);
+    }
+    __syncthreads();
+    hyb_reduce_store(ak[0], scale, dK + hb, nullptr, J * 32, w, li, h, lds);
+    __syncthreads();
+    hyb_reduce_store(av[0], 1.0f, dV + hb, nullptr, J * 32, w, li, h, lds);
+}
+
+// -------------------------------------------------------------------------------------------------
+// Backward, column pass, remainder: dK_j += sum_i dS_ij Q_i, dV_j += sum_i P_ij dO_i over the remainder's
+// transposed index (dS already carries the 1/sqrt(d)).
+// -------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // two gathers in flight per entry: four waves per SIMD
+    const float* __restrict__ Q, const float* __restrict__ dO,
+                                                    const float* __restrict__ P, const float* __restrict__ dS,
+                                                    float* __restrict__ dK, float* __restrict__ dV, HybIndex ix, int L,
+                                                    int NB, int nnz) {
+    const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
+    const long long wcol = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
+    if (wcol >= (long long)NB * L) return;
+    const int bh = (int)(wcol / L), colj = (int)(wcol % L);
+    const int c0p = ix.c_ptr[colj], cnt = ix.c_ptr[colj + 1] - c0p;
+    if (cnt == 0) return;
+    const size_t hb = (size_t)bh * L * 32;
+    const float* Ph = P + (size_t)bh * nnz;
+    const float* dSh = dS + (size_t)bh * nnz;
+    HybRowAcc ak, av;
+    ak.clear();
+    av.clear();
+    for (int c0 = 0; c0 < cnt; c0 += 64) {
+        const int e = c0 + ent;
+        float wk = 0.f, wv = 0.f;
+        int row = 0;
+        if (e < cnt) {
+            const int pp = ix.c_pos[c0p + e];
+            row = ix.c_row[c0p + e];
+            wk = dSh[pp];
+            wv = Ph[pp];
+        }
+        const int nk = min(64, cnt - c0);
+        ak.chunk(wk, row, nk, Q + hb, lane);
+        av.chunk(wv, row, nk, dO + hb, lane);
+    }
+    const f32x4 tk = ak.total(), tv = av.total();
+    if (lane < 8) {
+        f32x4* kr = reinterpret_cast<f32x4*>(dK + hb + (size_t)colj * 32) + lane;
+        f32x4* vr = reinterpret_cast<f32x4*>(dV + hb + (size_t)colj * 32) + lane;
+        *kr = *kr + tk;
+        *vr = *vr + tv;
+    }
+}
+
+}  // namespace spion

@@ -15,6 +15,7 @@
 #include "common.h"
 #include "tile_kernels.h"
 #include "bf16_kernels.h"
+#include "hybrid_kernels.h"
 #include "../../include/spion_hip.h"
 
 #include <algorithm>
@@ -328,6 +329,10 @@ struct PatternIndex {
     // per strip in launch order, {strip, first tile, tiles, P offset}: row pass, forward, column pass
     int *d_rdesc = nullptr, *d_fdesc = nullptr, *d_cdesc = nullptr;
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
+    // element-sparse pattern whose well-filled 32x32 tiles run on the MFMA units (hybrid_kernels.h)
+    bool hybrid = false;
+    int hyb_tiles = 0;
+    HybIndex hyb{};
     // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
     // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
     int *d_wg_row = nullptr, *d_wg_col = nullptr;
@@ -374,6 +379,7 @@ struct SparseAttn {
     uint64_t ostamp = 0;
     bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
+    float* ws_stats = nullptr;   // [NB][L][2] softmax row statistics handed between the hybrid forward's launches
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
     size_t ws_part_floats = 0;
     int last_path = 0;
@@ -431,6 +437,7 @@ void sparse_destroy(void* h) {
     a->release_patterns();
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
+    if (a->ws_stats) (void)hipFree(a->ws_stats);
     if (a->ws_part) (void)hipFree(a->ws_part);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
@@ -563,6 +570,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
     size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0;
+    size_t hyb_off[13] = {};
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -654,6 +662,101 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.max_row_tiles = mr;
         pi.max_col_tiles = mc;
     } else {
+        // ---- hybrid split: aligned 32x32 tiles with at least HYB_MIN_FILL entries become dense tiles (at most
+        // HYB_WAVES * HYB_MAXT per block row, the fullest first), everything else stays with the gather kernels
+        if (!a->force_element && a->d == 32 && L % 32 == 0 && nnz > 0) {
+            constexpr int HYB_MIN_FILL = 128;
+            const int nbr = L / 32;
+            std::vector<int> t_rp(nbr + 1, 0), t_col, t_row, cnt(nbr);
+            std::vector<std::vector<int>> dense_of(nbr);
+            long long dense_entries = 0;
+            for (int I = 0; I < nbr; ++I) {
+                std::fill(cnt.begin(), cnt.end(), 0);
+                for (int r = I * 32; r < I * 32 + 32; ++r)
+                    for (int k = off[r]; k < off[r + 1]; ++k) cnt[col[k] >> 5]++;
+                std::vector<int> cand;
+                for (int J = 0; J < nbr; ++J)
+                    if (cnt[J] >= HYB_MIN_FILL) cand.push_back(J);
+                if ((int)cand.size() > HYB_WAVES * HYB_MAXT) {
+                    std::stable_sort(cand.begin(), cand.end(), [&](int x, int y) { return cnt[x] > cnt[y]; });
+                    cand.resize(HYB_WAVES * HYB_MAXT);
+                    std::sort(cand.begin(), cand.end());
+                }
+                for (int J : cand) {
+                    t_col.push_back(J);
+                    t_row.push_back(I);
+                    dense_entries += cnt[J];
+                }
+                dense_of[I] = cand;
+                t_rp[I + 1] = (int)t_col.size();
+            }
+            const int nt = (int)t_col.size();
+            if (nt > 0 && dense_entries * 4 >= (long long)nnz) {
+                std::vector<int> t_pos((size_t)nt * 32, 0), r_off(L + 1, 0), r_col, r_pos;
+                std::vector<unsigned> t_bits((size_t)nt * 32, 0u);
+                std::vector<int> slot(nbr);
+                for (int I = 0; I < nbr; ++I) {
+                    std::fill(slot.begin(), slot.end(), -1);
+                    for (size_t e = 0; e < dense_of[I].size(); ++e) slot[dense_of[I][e]] = t_rp[I] + (int)e;
+                    for (int rr = 0; rr < 32; ++rr) {
+                        const int r = I * 32 + rr;
+                        for (int k = off[r]; k < off[r + 1]; ++k) {
+                            const int t = slot[col[k] >> 5];
+                            if (t < 0) {
+                                r_col.push_back(col[k]);
+                                r_pos.push_back(k);
+                            } else {
+                                if (!t_bits[(size_t)t * 32 + rr]) t_pos[(size_t)t * 32 + rr] = k;
+                                t_bits[(size_t)t * 32 + rr] |= 1u << (col[k] & 31);
+                            }
+                        }
+                        r_off[r + 1] = (int)r_col.size();
+                    }
+                }
+                const int nr = (int)r_col.size();
+                // transposed lists: dense tiles by block column, remainder entries column after column
+                std::vector<int> t_cp(nbr + 1, 0), t_ct(std::max(nt, 1));
+                for (int t = 0; t < nt; ++t) t_cp[t_col[t] + 1]++;
+                for (int J = 0; J < nbr; ++J) t_cp[J + 1] += t_cp[J];
+                {
+                    std::vector<int> fill(t_cp.begin(), t_cp.end() - 1);
+                    for (int t = 0; t < nt; ++t) t_ct[fill[t_col[t]]++] = t;
+                }
+                std::vector<int> c_ptr(L + 1, 0), c_row(std::max(nr, 1), 0), c_pos(std::max(nr, 1), 0);
+                for (int e = 0; e < nr; ++e) c_ptr[r_col[e] + 1]++;
+                for (int j = 0; j < L; ++j) c_ptr[j + 1] += c_ptr[j];
+                {
+                    std::vector<int> fill(c_ptr.begin(), c_ptr.end() - 1);
+                    for (int i = 0; i < L; ++i)  // rows ascend: every column's entries end up ordered by row
+                        for (int e = r_off[i]; e < r_off[i + 1]; ++e) {
+                            const int x = fill[r_col[e]]++;
+                            c_row[x] = i;
+                            c_pos[x] = r_pos[e];
+                        }
+                }
+                if (r_col.empty()) {
+                    r_col.push_back(0);
+                    r_pos.push_back(0);
+                }
+                std::vector<int> bits_as_int(t_bits.size());
+                memcpy(bits_as_int.data(), t_bits.data(), t_bits.size() * sizeof(int));
+                hyb_off[0] = append(t_rp);
+                hyb_off[1] = append(t_col);
+                hyb_off[2] = append(t_row);
+                hyb_off[3] = append(t_pos);
+                hyb_off[4] = append(bits_as_int);
+                hyb_off[5] = append(t_cp);
+                hyb_off[6] = append(t_ct);
+                hyb_off[7] = append(r_off);
+                hyb_off[8] = append(r_col);
+                hyb_off[9] = append(r_pos);
+                hyb_off[10] = append(c_ptr);
+                hyb_off[11] = append(c_row);
+                hyb_off[12] = append(c_pos);
+                pi.hybrid = true;
+                pi.hyb_tiles = nt;
+            }
+        }
         std::vector<int> ccp(L + 1, 0), crow(std::max(nnz, 1)), cpos(std::max(nnz, 1));
         for (int k = 0; k < nnz; ++k) ccp[col[k] + 1]++;
         for (int j = 0; j < L; ++j) ccp[j + 1] += ccp[j];
@@ -689,6 +792,13 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_ccp = pi.d_blob + o_ccp;
         pi.d_crow = pi.d_blob + o_crow;
         pi.d_cpos = pi.d_blob + o_cpos;
+        if (pi.hybrid) {
+            const int* b = pi.d_blob;
+            pi.hyb = HybIndex{b + hyb_off[0], b + hyb_off[1], b + hyb_off[2], b + hyb_off[3],
+                              reinterpret_cast<const unsigned*>(b + hyb_off[4]), b + hyb_off[5], b + hyb_off[6],
+                              b + hyb_off[7], b + hyb_off[8], b + hyb_off[9], b + hyb_off[10], b + hyb_off[11],
+                              b + hyb_off[12]};
+        }
     }
     pi.tiled = tiled;
     pi.key_off = Offsets;
@@ -977,12 +1087,37 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
         return;
     }
     a->last_path = 2;
-    ocache_drop(a, Attn);
+    float* hyb_ocopy = a->pat.hybrid ? ocache_for_forward(a, Attn) : nullptr;
+    if (!hyb_ocopy) ocache_drop(a, Attn);
     const float* Krm = Kt;  // the element kernels read K row-major
     if (!krow) {
         if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
         launch_transpose(a, Kt, a->ws_trans);
         Krm = a->ws_trans;
+    }
+    if (a->pat.hybrid) {
+        if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
+        a->last_path = 3;
+        const int nbr = a->L / 32;
+        const long long rows = (long long)a->NB * a->L;
+        const dim3 grid_t(nbr * a->NB), block_t(64 * HYB_WAVES);
+        const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
+        float2* stats = reinterpret_cast<float2*>(a->ws_stats);
+        if (a->has_mask) {
+            hipLaunchKernelGGL(hyb_rem_logits_kernel<true>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn, stats,
+                               a->pat.hyb, a->L, a->NB, nnz, a->scale);
+            hipLaunchKernelGGL(hyb_tile_fwd_kernel<true>, grid_t, block_t, 0, a->hdr.stream, Q, Krm, V, Mask, Attn, Out,
+                               stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+        } else {
+            hipLaunchKernelGGL(hyb_rem_logits_kernel<false>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn,
+                               stats, a->pat.hyb, a->L, a->NB, nnz, a->scale);
+            hipLaunchKernelGGL(hyb_tile_fwd_kernel<false>, grid_t, block_t, 0, a->hdr.stream, Q, Krm, V, Mask, Attn,
+                               Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+        }
+        hipLaunchKernelGGL(hyb_rem_pv_kernel, grid_g, block_g, 0, a->hdr.stream, V, Attn, Out, hyb_ocopy,
+                           (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz);
+        check_launch("hybrid forward kernels");
+        return;
     }
     switch (a->d) {
         case 16: launch_elem_fwd<16>(a, Q, Krm, V, Mask, Attn, Out, Offsets, Columns, nnz); break;
@@ -1037,6 +1172,33 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         if (!ensure_ws(&a->ws_trans, (size_t)a->NB * a->L * a->d)) return;
         launch_transpose(a, Vt, a->ws_trans);
         Vrm = a->ws_trans;
+    }
+    if (a->pat.hybrid) {
+        // the hybrid kernels take the row sums from the forward's output (the caller's, or the handle's kept copy);
+        // without it the gather kernels below serve the same P
+        const float* o = Out ? Out : ocache_for_backward(a, P);
+        if (o) {
+            if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+            a->last_path = 3;
+            const int nbr = a->L / 32;
+            const long long rows = (long long)a->NB * a->L;
+            const dim3 grid_t(nbr * a->NB), block_t(64 * HYB_WAVES);
+            const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
+            if (a->bwd_passes & 1) {
+                hipLaunchKernelGGL(hyb_tile_bwd_row_kernel, grid_t, block_t, 0, a->hdr.stream, K, Vrm, P, dO, o,
+                                   a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+                hipLaunchKernelGGL(hyb_rem_bwd_row_kernel, grid_g, block_g, 0, a->hdr.stream, K, Vrm, P, dO,
+                                   (const float*)a->ws_rowsum, dS, dQ, a->pat.hyb, a->L, a->NB, nnz, a->scale);
+            }
+            if (a->bwd_passes & 2) {
+                hipLaunchKernelGGL(hyb_tile_bwd_col_kernel, grid_t, block_t, 0, a->hdr.stream, Q, Vrm, P, dO,
+                                   (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+                hipLaunchKernelGGL(hyb_rem_bwd_col_kernel, grid_g, block_g, 0, a->hdr.stream, Q, dO, P,
+                                   (const float*)dS, dK, dV, a->pat.hyb, a->L, a->NB, nnz);
+            }
+            check_launch("hyb_bwd kernels");
+            return;
+        }
     }
     switch (a->d) {
         case 16: launch_elem_bwd<16>(a, Q, K, Vrm, P, dO, dS, dQ, dK, dV, Offsets, Columns, nnz); break;

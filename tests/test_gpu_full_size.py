@@ -33,6 +33,7 @@ def test_config4_full_batch_properties():
     O, P = abi.forward(Q, K, V, pen)
     dQ, dK, dV = abi.backward(Q, K, V, P, dO)
     torch.cuda.synchronize()
+    assert abi.last_path() == 3   # window tiles on the MFMA units, random columns gathered
     # (a) the oracle on the first and the last head of the full-size launch
     for hsel in (0, NB - 1):
         s = slice(hsel, hsel + 1)

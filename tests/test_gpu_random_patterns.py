@@ -91,7 +91,7 @@ def test_random_element_patterns(seed):
     g = torch.Generator().manual_seed(seed)
     Q, K, V, dO = (torch.randn(NB, L, d, generator=g).cuda() for _ in range(4))
     run_and_check(abi, Q, K, V, dO, pen, tag=f"seed {seed}: element L={L} d={d} NB={NB} p={p} mask={with_mask}")
-    assert abi.last_path() == 2
+    assert abi.last_path() in (2, 3)   # gather kernels, or the hybrid kernels when enough 32x32 tiles are well filled
     abi.close()
 
 

@@ -74,7 +74,7 @@ def test_noalloc_backward_refuses_unknown_patterns_and_element_patterns():
     sm2[0] -= 1
     abi.set_pattern(sm2, off2, col2)
     O, P = abi.forward_rowmajor(Q, K, V)
-    assert abi.last_path() == 2
+    assert abi.last_path() in (2, 3)
     with pytest.raises(_lib.SpionLibraryError, match="aligned 32x32 tiles"):
         _noalloc_backward(abi, Q, K, V, P, O, dO)
     abi.close()
