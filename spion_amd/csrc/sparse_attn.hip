@@ -1331,8 +1331,8 @@ static SparseAttn* strided_handle(void* h, const char* who, const int* Offsets, 
         return nullptr;
     }
     if (!ensure_pattern(a, Offsets, Columns, nnz)) return nullptr;
-    if (!a->pat.tiled || a->d != 32) {
-        set_error("%s: strided heads are read in place only by the tile kernels for emb_dim 32 (pattern of aligned "
+    if (!a->pat.tiled || !tile_supported(a->d)) {
+        set_error("%s: strided heads are read in place only by the tile kernels (emb_dim 32 or 64, pattern of aligned "
                   "32x32 tiles); make the operands contiguous and use the row-major entry points", who);
         return nullptr;
     }
@@ -1368,8 +1368,13 @@ void sparse_forward_strided(void* h, const float* Q, const float* K, const float
     ly.grad = out;
     ly.H = heads;
     a->last_path = 1;
-    if (a->has_mask) launch_tile_fwd<32, true, true, true>(a, Q, K, V, Mask, Attn, Out, Offsets, nnz, ly);
-    else launch_tile_fwd<32, false, true, true>(a, Q, K, V, nullptr, Attn, Out, Offsets, nnz, ly);
+    if (a->d == 32) {
+        if (a->has_mask) launch_tile_fwd<32, true, true, true>(a, Q, K, V, Mask, Attn, Out, Offsets, nnz, ly);
+        else launch_tile_fwd<32, false, true, true>(a, Q, K, V, nullptr, Attn, Out, Offsets, nnz, ly);
+    } else {
+        if (a->has_mask) launch_tile_fwd<64, true, true, true>(a, Q, K, V, Mask, Attn, Out, Offsets, nnz, ly);
+        else launch_tile_fwd<64, false, true, true>(a, Q, K, V, nullptr, Attn, Out, Offsets, nnz, ly);
+    }
     check_launch("tile_fwd_kernel");
 }
 
@@ -1402,7 +1407,8 @@ void sparse_backward_strided(void* h, const float* Q, const float* K, const floa
     ly.grad = grad;
     ly.H = heads;
     a->last_path = 1;
-    launch_tile_bwd<32, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);
+    if (a->d == 32) launch_tile_bwd<32, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);
+    else launch_tile_bwd<64, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);
     check_launch("tile_bwd kernels");
 }
 

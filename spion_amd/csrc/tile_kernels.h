@@ -333,14 +333,16 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // recomputing the logits (any row length).  Ocache (optional): second copy of O for the backward.
 // -------------------------------------------------------------------------------------------------
 // KROW: the K operand is row-major [NB][L][D] (what a caller has before it makes the transposed copy the
-// reference's ABI asks for) instead of feature-major [NB][D][L]; d = 32 only.
+// reference's ABI asks for) instead of feature-major [NB][D][L].  For d = 64 every lane then reads 128 bytes of
+// its own row (one cache line per lane), which is slower than the feature-major form: the row-major entry points
+// for contiguous heads therefore still transpose once; only the strided entry points use it.
 template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
     const int* __restrict__ rdesc, const int* __restrict__ tcol, int L, int nbr,
     int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
-    static_assert(!ST || (KROW && D == 32), "strided heads: row-major operands, d = 32");
+    static_assert(!ST || KROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
@@ -587,15 +589,14 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
 // dP^T - g = V_J.dO_I^T chain started from -g, dS' = (dP - g)*P, dQ += dS'.K_J; the 1/sqrt(d) is applied to
 // the 32 x d result.  G receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------
-// VROW: the V operand is row-major [NB][L][D] instead of feature-major [NB][D][L]; d = 32 only.
+// VROW: the V operand is row-major [NB][L][D] instead of feature-major [NB][D][L].
 template <int D, int WAVES, bool HAVE_O, bool VROW = false, bool ST = false>
 SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
     float* __restrict__ dQ, const int* __restrict__ rdesc, const int* __restrict__ tcol,
     int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
-    static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, d = 32, Out given");
-    static_assert(!VROW || D == 32, "row-major V operand: d = 32 only");
+    static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, Out given");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_g[WAVES][32];
@@ -732,16 +733,17 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             [&](Pre& x, int i) {
                 const int t = w + min(i, nu - 1) * WAVES;
                 x.J = tcol[t0 + t];
-                ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
+                if constexpr (VROW) ldr_rows<D>(rV, r_voff, x.J * 32 * ild * 4, x.vt);
+                else ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
                 // the P tile straight in the layout dP^T comes in (every lane pieces of its own row): measured
                 // twice as fast here as full rows plus an LDS transpose, which costs this path its registers
                 // (not non-temporal: a lane reads its 128-byte row in four instructions)
                 ldr_4x4(rP, (li * rn + 4 * h) * 4, p_base + t * 128, x.pv);
-                if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * D * 4, x.kb);
+                if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * ild * 4, x.kb, ild);
             },
             [&](Pre& c, int) {
                 float kb2[D / 32][16];
-                if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * D * 4, kb2);
+                if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * ild * 4, kb2, ild);
                 const float (&pr)[16] = c.pv;
                 f32x16 dp = mma_feat_init<D>(c.vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
@@ -768,7 +770,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
     const int* __restrict__ cdesc, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
     int hc, Layouts ly) {
-    static_assert(!ST || VROW, "strided heads: row-major operands, d = 32");
+    static_assert(!ST || VROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];

@@ -556,14 +556,15 @@ def _head_views(B, H, L, d, layout, n, seed, fill=None):
     return bufs, views
 
 
+@pytest.mark.parametrize("d", [32, 64])
 @pytest.mark.parametrize("layout,kind,with_mask", [("proj", "tile", False), ("fused", "tile", True), ("plain", "tile", False),
                                                    ("proj", "tile_rows", False), ("fused", "many_rows", False)])
-def test_strided_entry_points(layout, kind, with_mask):
+def test_strided_entry_points(layout, kind, with_mask, d):
     """spion_attn_forward_strided / spion_attn_backward_strided: heads read and written in place in the memory of
     [B, L, H*d] projections.  Same kernels, same arithmetic as the row-major entry points on contiguous copies:
     bit-identical results; padding between the heads' rows is left alone."""
-    d, H, bs = 32, 2, 32
-    B, L = {"tile": (2, 256), "tile_rows": (1, 2048), "many_rows": (8, 4096)}[kind]
+    H, bs = 2, 32
+    B, L = {"tile": (2, 256), "tile_rows": (1, 2048), "many_rows": (8 if d == 32 else 4, 4096)}[kind]
     NB = B * H
     mat = _random_block_mask(L // bs, 0.3 if kind != "many_rows" else 0.05, seed=7)
     if kind == "tile_rows":
@@ -618,12 +619,12 @@ def test_strided_entry_points_refuse_what_they_cannot_serve():
             abi.offsets.data_ptr(), abi.columns.data_ptr(), abi.sum_mat.data_ptr(), abi.nnz, heads,
             ctypes.addressof(lin), ctypes.addressof(lout))
 
-    abi64 = SparseABI(64, L, B * H, bs, with_mask=False)
-    abi64.set_pattern(sm, off, col)
+    abi64 = SparseABI(64, L, B * H, bs, with_mask=False)   # d = 64 is served, but not on an element-sparse pattern
+    abi64.set_pattern(sm - (np.arange(L) == 0), off - (np.arange(L + 1) > 0), col[1:])
     q64 = torch.zeros(B, H, L, 64, device="cuda")
     call(abi64, q64, torch.zeros_like(q64))
-    with pytest.raises(RuntimeError, match="emb_dim 32"):
-        _lib.check_error("d=64")
+    with pytest.raises(RuntimeError, match="aligned"):
+        _lib.check_error("element pattern")
     abi64.close()
     abi = SparseABI(32, L, B * H, bs, with_mask=False)
     abi.set_pattern(sm, off, col)
