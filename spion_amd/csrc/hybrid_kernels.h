@@ -30,77 +30,146 @@ struct HybIndex {
     const int* t_row;
     const int* t_pos;        // [tiles][32]
     const unsigned* t_bits;  // [tiles][32]
-    // the same tiles by block column: tile ids t_ct[t_cp[J]] .. of block column J
+    // the same tiles by block column: tile ids t_ct[t_cp[J]] .. of block column J and their block rows t_ci
     const int* t_cp;
     const int* t_ct;
+    const int* t_ci;
     // remainder entries in CSR form (r_off [L+1], columns, positions inside a head's P) and in CSC form (c_ptr
-    // [L+1], rows ascending within a column, positions)
+    // [L+1], rows ascending within a column, index of the entry in the CSR list); nr entries per head
     const int* r_off;
     const int* r_col;
     const int* r_pos;
     const int* c_ptr;
     const int* c_row;
-    const int* c_pos;
+    const int* c_src;
+    int nr;
+    int nt;  // dense tiles in all
 };
 
-constexpr int HYB_WAVES = 4;
-constexpr int HYB_MAXT = 4;     // dense tiles per wavefront whose logits stay in registers (forward)
+// Tile kernels come in two shapes: one wavefront per strip (strips of up to HYB_MAXT1 dense tiles: the window
+// patterns this path is for have about five; the wavefront walks them one after the other, nothing is shared and
+// nothing waits at a barrier) and four wavefronts per strip (up to 4 * HYB_MAXT4 dense tiles).  With a handful of
+// tiles per strip these launches live on latency, and a strip handled by one wavefront costs a quarter of the
+// wavefront start-ups, index look-ups and final reductions.
+constexpr int HYB_MAXT1 = 6;    // dense tiles whose logits a single wavefront keeps in registers (forward)
+constexpr int HYB_MAXT4 = 4;    // the same per wavefront when four share a strip
+constexpr int HYB_MAX_ROW_TILES = 4 * HYB_MAXT4;
 constexpr int HYB_GWAVES = 4;    // wavefronts (rows / columns) per work-group of the gather kernels
 constexpr float HYB_ABSENT = -1.0e30f;  // logit of an entry that is not in the pattern: exp2 gives exactly 0
-// three work-groups per CU: these launches have few tiles per wavefront and live on latency
-#define SPION_HYB_KERNEL __global__ __launch_bounds__(64 * HYB_WAVES) __attribute__((amdgpu_waves_per_eu(3, 3)))
+// two wavefronts per SIMD, each with the next tile's operands in flight while it works on one
+#define SPION_HYB_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2, 2)))
 
-// Positions and present-column sets of the 16 tile rows acc_row(q, h), q = 0..15, of tile t.
-__device__ __forceinline__ void hyb_tile_rows(const HybIndex& ix, int t, int h, int (&pos)[16], unsigned (&bits)[16]) {
+// What the tile kernels request ahead of a tile: two operand tiles (raw 16-byte pieces, linear), the tile of P in the
+// col-owner layout, and -- one tile further ahead, because the addresses of P come out of it -- the tile's index:
+// block column (or row), and position and present-column set of tile row li (lane li and lane 32 + li hold the same).
+struct HybPre {
+    f32x4 a[4], b[4];
+    float p[16];
+    float g_l;
+    int pos_l, blk;
+    unsigned bits_l;
+};
+
+__device__ __forceinline__ void hyb_fetch_index(const HybIndex& ix, int t, int li, HybPre& x) {
+    x.pos_l = ix.t_pos[(size_t)t * 32 + li];
+    x.bits_l = ix.t_bits[(size_t)t * 32 + li];
+}
+
+// One value per tile row, held by lane li (and 32 + li) for row li, to the 16 rows acc_row(q, h), q = 0..15, a lane
+// works on: through 32 words of the wavefront's own LDS space.
+__device__ __forceinline__ void hyb_rows_from_lanes(int* xs, int l, int h, int v, int (&out)[16]) {
+    xs[l] = v;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-        const int4 p = *reinterpret_cast<const int4*>(ix.t_pos + (size_t)t * 32 + 8 * g + 4 * h);
-        const uint4 b = *reinterpret_cast<const uint4*>(ix.t_bits + (size_t)t * 32 + 8 * g + 4 * h);
-        pos[4 * g + 0] = p.x, pos[4 * g + 1] = p.y, pos[4 * g + 2] = p.z, pos[4 * g + 3] = p.w;
-        bits[4 * g + 0] = b.x, bits[4 * g + 1] = b.y, bits[4 * g + 2] = b.z, bits[4 * g + 3] = b.w;
+        const int4 p = *reinterpret_cast<const int4*>(xs + 8 * g + 4 * h);
+        out[4 * g + 0] = p.x, out[4 * g + 1] = p.y, out[4 * g + 2] = p.z, out[4 * g + 3] = p.w;
     }
 }
+__device__ __forceinline__ void hyb_tile_rows(int* xs, int l, int h, const HybPre& x, int (&pos)[16],
+                                              unsigned (&bits)[16]) {
+    int b[16];
+    hyb_rows_from_lanes(xs, l, h, x.pos_l, pos);
+    hyb_rows_from_lanes(xs + 64, l, h, (int)x.bits_l, b);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) bits[q] = (unsigned)b[q];
+}
 // The tile of P in the col-owner layout (lane li = column of the tile, register q = row acc_row(q, h)); absent
-// entries read as 0.  A tile row's entries are consecutive in memory: every instruction touches one run per
-// half-wave.
-__device__ __forceinline__ void hyb_load_p_cols(const float* __restrict__ Ph, const int (&pos)[16],
-                                                const unsigned (&bits)[16], int li, float (&pc)[16]) {
+// entries read as 0 (their offset lies past the end of the buffer).  A tile row's entries are consecutive in memory:
+// every instruction touches one run per half-wave.
+__device__ __forceinline__ void hyb_load_p_cols(rsrc_t rP, const int (&pos)[16], const unsigned (&bits)[16], int li,
+                                                float (&pc)[16]) {
     const unsigned below = (1u << li) - 1u;
 #pragma unroll
     for (int q = 0; q < 16; ++q) {
         const bool on = (bits[q] >> li) & 1u;
-        pc[q] = on ? Ph[pos[q] + __popc(bits[q] & below)] : 0.f;
+        pc[q] = ld1(rP, on ? 4 * (pos[q] + __popc(bits[q] & below)) : -1, 0);
     }
 }
 __device__ __forceinline__ void hyb_store_p_cols(float* __restrict__ Ph, const int (&pos)[16],
-                                                 const unsigned (&bits)[16], int li, const float (&pc)[16]) {
+                                                 const int (&bits)[16], int li, const float (&pc)[16]) {
     const unsigned below = (1u << li) - 1u;
 #pragma unroll
-    for (int q = 0; q < 16; ++q)
-        if ((bits[q] >> li) & 1u) Ph[pos[q] + __popc(bits[q] & below)] = pc[q];
+    for (int q = 0; q < 16; ++q) {
+        const unsigned b = (unsigned)bits[q];
+        if ((b >> li) & 1u) Ph[pos[q] + __popc(b & below)] = pc[q];
+    }
 }
 
-// Sum of the four wavefronts' 32 x 32 accumulators (rows acc_row(r, h) of the strip, columns li) times `factor`,
-// in a fixed order.  `lds` (4096 floats) may alias tile space no wavefront uses any more: the caller has a barrier
-// between that use and this call.
+// Sum of the wavefronts' 32 x 32 accumulators (rows acc_row(r, h) of the strip, columns li) times `factor`, in a
+// fixed order.  `lds` (WAVES * 1024 floats, unused for one wavefront) may alias tile space no wavefront uses any
+// more: the caller has a barrier between that use and this call.
+template <int WAVES>
 __device__ __forceinline__ void hyb_reduce_store(const f32x16& acc, float factor, float* __restrict__ out,
                                                  float* __restrict__ out2, int row0, int w, int li, int h,
                                                  float* __restrict__ lds) {
     const int l = h * 32 + li;
+    if constexpr (WAVES > 1) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) lds[(w * 16 + r) * 64 + l] = acc[r];
-    __syncthreads();
+        for (int r = 0; r < 16; ++r) lds[(w * 16 + r) * 64 + l] = acc[r];
+        __syncthreads();
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        if ((r % HYB_WAVES) != w) continue;
-        float s = 0.f;
+        if (WAVES > 1 && (r % WAVES) != w) continue;
+        float s = acc[r];
+        if constexpr (WAVES > 1) {
+            s = 0.f;
 #pragma unroll
-        for (int ww = 0; ww < HYB_WAVES; ++ww) s += lds[(ww * 16 + r) * 64 + l];
+            for (int ww = 0; ww < WAVES; ++ww) s += lds[(ww * 16 + r) * 64 + l];
+        }
         s *= factor;
         const size_t a = (size_t)(row0 + acc_row(r, h)) * 32 + li;
         out[a] = s;
         if (out2) out2[a] = s;
     }
+}
+
+// Two-deep software pipeline over n tiles with two register sets: while tile i is computed, the operands and P of
+// tile i + 1 are in flight and so is the index of tile i + 2 (requested first, so that waiting for it leaves the
+// younger requests outstanding).  Positions past the end are clamped by the callers (valid, redundant requests).
+template <class FetchIdx, class FetchData, class Compute>
+__device__ __forceinline__ void hyb_pipeline(int n, HybPre& a, HybPre& b, FetchIdx fetch_idx, FetchData fetch_data,
+                                             Compute compute) {
+    if (n <= 0) return;
+    fetch_idx(a, 0);
+    fetch_idx(b, 1);
+    fetch_data(a, 0);
+    int i = 0;
+    for (; i + 1 < n; i += 2) {
+        fetch_idx(a, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_data(b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(a, i);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_idx(b, i + 3);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_data(a, i + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(b, i + 1);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (i < n) compute(a, i);
 }
 
 // =================================================================================================
@@ -236,15 +305,16 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
 // maximum, 1 / denominator} for step 3).  Writes the tiles' probabilities to their CSR positions and O = P.V of the
 // tile part (step 3 adds the remainder's share).
 // -------------------------------------------------------------------------------------------------
-template <bool MASK>
-SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
+template <bool MASK, int WAVES, int MAXT>
+SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                           const float* __restrict__ V, const float* __restrict__ pen,
                                           float* __restrict__ P, float* __restrict__ O, float2* __restrict__ Stats,
                                           const int* __restrict__ offs, HybIndex ix, int L, int nbr, int NB, int nnz,
                                           float scale) {
-    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES, MAXT = HYB_MAXT;
+    constexpr int D = 32, KH = 16;
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];  // two 32-row tiles per wavefront
+    __shared__ __attribute__((aligned(16))) int lds_x[WAVES][128];
     float* lds = &lds_t[0][0];  // the final reduction reuses the tile space
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
@@ -256,6 +326,7 @@ SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const flo
     float* Ph = P + (size_t)bh * nnz;
     float* T = lds_t[w];
     float* Tx = T + 32 * TS;
+    int* X = lds_x[w];
     const float c2 = scale * LOG2E;
     const int lin = lin_voff(l, D);
 
@@ -265,37 +336,51 @@ SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const flo
     for (int s = 0; s < KH; ++s) q[s] *= c2;
     const float2 rem = Stats[(size_t)bh * L + I * 32 + li];  // the remainder of row li
 
-    // ---- logits of this wavefront's tiles, own maximum ----------------------------------------------
+    // ---- index of this wavefront's tiles (positions past the end repeat the last one: valid, redundant) -----
     const int t0 = ix.t_rp[I], cnt = ix.t_rp[I + 1] - t0;
     const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;
-    float m = MASK ? 0.f : -100.f * LOG2E, z = 0.f;
-    f32x16 S[MAXT];
-    int Js[MAXT];
-#pragma unroll
-    for (int u = 0; u < MAXT; ++u) Js[u] = u < nu ? ix.t_col[t0 + w + u * WAVES] : 0;
+    int Js[MAXT], pos_l[MAXT];
+    unsigned bits_l[MAXT];  // present columns / first position of tile row li
 #pragma unroll
     for (int u = 0; u < MAXT; ++u) {
+        const int t = min(t0 + w + min(u, max(nu, 1) - 1) * WAVES, ix.nt - 1);
+        Js[u] = ix.t_col[t];
+        pos_l[u] = ix.t_pos[(size_t)t * 32 + li];
+        bits_l[u] = ix.t_bits[(size_t)t * 32 + li];
+    }
+
+    // ---- logits of the tiles, own maximum; the next tile of K is in flight while one is worked on --------
+    float m = MASK ? 0.f : -100.f * LOG2E, z = 0.f;
+    f32x16 S[MAXT];
+    f32x4 raw[2][4];
+    float pj[2][16];
+    ldr_tile_lin(rK, lin, Js[0] * 32 * D * 4, D, raw[0]);
+    if constexpr (MASK) ldr_4x4(rM, 16 * h, Js[0] * 128, pj[0]);
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u + 1 < MAXT) {
+            ldr_tile_lin(rK, lin, Js[u + 1] * 32 * D * 4, D, raw[(u + 1) & 1]);
+            if constexpr (MASK) ldr_4x4(rM, 16 * h, Js[u + 1] * 128, pj[(u + 1) & 1]);
+        } else {
+            ldr_tile_lin(rV, lin, Js[0] * 32 * D * 4, D, raw[(u + 1) & 1]);  // first tile of V for the last step
+        }
+        __builtin_amdgcn_sched_barrier(0);
         if (u < nu) {
-            const int t = t0 + w + u * WAVES;
-            f32x4 kraw[4];
-            ldr_tile_lin(rK, lin, Js[u] * 32 * D * 4, D, kraw);
-            const unsigned mybits = ix.t_bits[(size_t)t * 32 + li];  // present columns of this lane's row
             f32x16 init = splat16(0.f);
             if constexpr (MASK) {
-                float pj[16];
-                ldr_4x4(rM, 16 * h, Js[u] * 128, pj);
 #pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] = -LOG2E * pj[r];
+                for (int r = 0; r < 16; ++r) init[r] = -LOG2E * pj[u & 1][r];
             }
-            lds_put_lin(Tx, l, kraw);
+            lds_put_lin(Tx, l, raw[u & 1]);
             float kf[KH];
             lds_get_feat32(Tx, li, h, kf);
             S[u] = mma_feat_init<D>(kf, q, init);  // register = key acc_row(r, h), lane = query li
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                if (!((mybits >> acc_row(r, h)) & 1u)) S[u][r] = HYB_ABSENT;
+                if (!((bits_l[u] >> acc_row(r, h)) & 1u)) S[u][r] = HYB_ABSENT;
             m = max16(S[u], m);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
     m = fmaxf(m, __shfl_xor(m, 32, 64));
 #pragma unroll
@@ -311,19 +396,24 @@ SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const flo
     }
     const float m_own = m;
     z += __shfl_xor(z, 32, 64);
-    if (h == 0) {
-        lds_m[w][li] = m;
-        lds_z[w][li] = z;
-    }
-    __syncthreads();
 
     // ---- merge: row maximum and denominator over the tiles of all wavefronts and the remainder ----
-    float Mx = rem.x;
-#pragma unroll
-    for (int ww = 0; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+    float Mx = fmaxf(rem.x, m);
     float Z = rem.y * __builtin_amdgcn_exp2f(rem.x - Mx);
+    if constexpr (WAVES > 1) {
+        if (h == 0) {
+            lds_m[w][li] = m;
+            lds_z[w][li] = z;
+        }
+        __syncthreads();
 #pragma unroll
-    for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+        for (int ww = 0; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        Z = rem.y * __builtin_amdgcn_exp2f(rem.x - Mx);
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+    } else {
+        Z += z * __builtin_amdgcn_exp2f(m - Mx);
+    }
     {
         const int row = I * 32 + li;
         const int n_i = offs[row + 1] - offs[row];
@@ -332,18 +422,15 @@ SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const flo
     const float zinv = 1.0f / Z;  // +inf denominator -> 0 -> P = 0, as in the reference
     const float rinv = __builtin_amdgcn_exp2f(m_own - Mx) * zinv;
 
-    // ---- probabilities, O += P.V, P to its CSR positions --------------------------------------------
+    // ---- probabilities, O += P.V, P to its CSR positions; V of the next tile in flight ------------------
     f32x16 o[1] = {splat16(0.f)};
 #pragma unroll
     for (int u = 0; u < MAXT; ++u) {
+        constexpr int FIRST = MAXT & 1;  // the set the first tile of V went to
+        if (u + 1 < MAXT) ldr_tile_lin(rV, lin, Js[u + 1] * 32 * D * 4, D, raw[(FIRST + u + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
         if (u < nu) {
-            const int t = t0 + w + u * WAVES;
-            f32x4 vraw[4];
-            ldr_tile_lin(rV, lin, Js[u] * 32 * D * 4, D, vraw);
-            int pos[16];
-            unsigned bits[16];
-            hyb_tile_rows(ix, t, h, pos, bits);
-            lds_put_lin(Tx, l, vraw);
+            lds_put_lin(Tx, l, raw[(FIRST + u) & 1]);
             float p[16], vb[1][16], pc[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
@@ -351,13 +438,17 @@ SPION_HYB_KERNEL void hyb_tile_fwd_kernel(const float* __restrict__ Q, const flo
             lds_get_cols(Tx, li, h, vb[0]);
             lds_get_cols(T, li, h, pc);
             mma_b<D>(p, vb, o);
+            int pos[16], bits[16];
+            hyb_rows_from_lanes(X, l, h, pos_l[u], pos);
+            hyb_rows_from_lanes(X + 64, l, h, (int)bits_l[u], bits);
             hyb_store_p_cols(Ph, pos, bits, li, pc);
         }
+        __builtin_amdgcn_sched_barrier(0);
     }
-    __syncthreads();
+    if constexpr (WAVES > 1) __syncthreads();
     // every wavefront has consumed the remainder's statistics by now: replace them by the row's final ones
     if (w == 0 && h == 0) Stats[(size_t)bh * L + I * 32 + li] = make_float2(Mx, zinv);
-    hyb_reduce_store(o[0], 1.0f, O + hb, nullptr, I * 32, w, li, h, lds);
+    hyb_reduce_store<WAVES>(o[0], 1.0f, O + hb, nullptr, I * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -402,13 +493,15 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, floa
 // Backward, row pass, dense tiles: g_i = dO_i . O_i (G receives -g for the other kernels); dP^T - g = V_J.dO_I^T
 // chain started from -g, dS' = (dP - g)*P, dQ = sum dS'.K_J / sqrt(d).
 // -------------------------------------------------------------------------------------------------
-SPION_HYB_KERNEL void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
+template <int WAVES>
+SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
                                               const float* __restrict__ P, const float* __restrict__ dO,
                                               const float* __restrict__ Out, float* __restrict__ G,
                                               float* __restrict__ dQ, HybIndex ix, int L, int nbr, int NB, int nnz,
                                               float scale) {
-    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES;
+    constexpr int D = 32, KH = 16;
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
+    __shared__ __attribute__((aligned(16))) int lds_x[WAVES][128];
     float* lds = &lds_t[0][0];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
@@ -416,9 +509,10 @@ SPION_HYB_KERNEL void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const
     const size_t hb = (size_t)bh * L * D;
     const rsrc_t rK = make_rsrc(K + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
     const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4), rO = make_rsrc(Out + hb, (size_t)L * D * 4);
-    const float* Ph = P + (size_t)bh * nnz;
+    const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     float* T = lds_t[w];
     float* Tx = T + 32 * TS;
+    int* X = lds_x[w];
     const int lin = lin_voff(l, D);
 
     float go[KH], oo[KH];
@@ -432,40 +526,52 @@ SPION_HYB_KERNEL void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const
     const f32x16 gneg = splat16(-g);
 
     const int t0 = ix.t_rp[I], cnt = ix.t_rp[I + 1] - t0;
+    const int n = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;
     f32x16 acc[1] = {splat16(0.f)};
-    for (int t = t0 + w; t < t0 + cnt; t += WAVES) {
-        const int J = ix.t_col[t];
-        f32x4 vraw[4], kraw[4];
-        ldr_tile_lin(rV, lin, J * 32 * D * 4, D, vraw);
-        ldr_tile_lin(rK, lin, J * 32 * D * 4, D, kraw);
-        int pos[16];
-        unsigned bits[16];
-        hyb_tile_rows(ix, t, h, pos, bits);
-        float pc[16], pr[16], vt[KH], kb[1][16];
-        hyb_load_p_cols(Ph, pos, bits, li, pc);
-        lds_put_lin(Tx, l, vraw);
-        lds_get_feat32(Tx, li, h, vt);
-        lds_put_cols(T, li, h, pc);
-        lds_get_rows(T, li, h, pr);                        // pr[r] = P[query li][key acc_row(r, h)]
-        const f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
-        lds_put_lin(Tx, l, kraw);
-        lds_get_cols(Tx, li, h, kb[0]);
-        float ds[16];
+    HybPre xa, xb;
+    hyb_pipeline(
+        n, xa, xb,
+        [&](HybPre& x, int i) {
+            const int t = t0 + w + min(i, n - 1) * WAVES;
+            x.blk = ix.t_col[t];
+            hyb_fetch_index(ix, t, li, x);
+        },
+        [&](HybPre& x, int) {
+            int pos[16];
+            unsigned bits[16];
+            hyb_tile_rows(X, l, h, x, pos, bits);
+            ldr_tile_lin(rV, lin, x.blk * 32 * D * 4, D, x.a);
+            hyb_load_p_cols(rP, pos, bits, li, x.p);
+            ldr_tile_lin(rK, lin, x.blk * 32 * D * 4, D, x.b);
+        },
+        [&](HybPre& x, int) {
+            float pr[16], vt[KH], kb[1][16];
+            lds_put_lin(Tx, l, x.a);
+            lds_get_feat32(Tx, li, h, vt);
+            lds_put_cols(T, li, h, x.p);
+            lds_get_rows(T, li, h, pr);                        // pr[r] = P[query li][key acc_row(r, h)]
+            const f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
+            lds_put_lin(Tx, l, x.b);
+            lds_get_cols(Tx, li, h, kb[0]);
+            float ds[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
-        mma_b<D>(ds, kb, acc);
-    }
-    __syncthreads();
-    hyb_reduce_store(acc[0], scale, dQ + hb, nullptr, I * 32, w, li, h, lds);
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
+            mma_b<D>(ds, kb, acc);
+        });
+    if constexpr (WAVES > 1) __syncthreads();
+    hyb_reduce_store<WAVES>(acc[0], scale, dQ + hb, nullptr, I * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
-// Backward, row pass, remainder: dS = (dO_i . v_j - g_i) * P / sqrt(d) into the caller's dS scratch (for the
-// column pass), dQ_i += sum dS . K[col].
+// Backward, row pass, remainder: dS = (dO_i . v_j - g_i) * P / sqrt(d), dQ_i += sum dS . K[col].  The column pass
+// walks the same entries column after column; looking P and dS up there inside a head's full P and dS (two arrays
+// of nnz floats, more than the L2 cache holds per head) would fetch a memory sector for every four bytes, so this
+// kernel leaves the pairs {dS, P} of the remainder alone in one compact list (Pairs [NB][nr], row order, inside the
+// caller's dS scratch), small enough per head for the column pass to find in the L2 cache.
 // -------------------------------------------------------------------------------------------------
 SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
                                                     const float* __restrict__ P, const float* __restrict__ dO,
-                                                    const float* __restrict__ G, float* __restrict__ dS,
+                                                    const float* __restrict__ G, float2* __restrict__ Pairs,
                                                     float* __restrict__ dQ, HybIndex ix, int L, int NB, int nnz,
                                                     float scale) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
@@ -477,7 +583,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K,
     const size_t hb = (size_t)bh * L * 32;
     const f32x4 go4 = reinterpret_cast<const f32x4*>(dO + hb + (size_t)row * 32)[lane & 7];
     const float* Ph = P + (size_t)bh * nnz;
-    float* dSh = dS + (size_t)bh * nnz;
+    float2* pairs = Pairs + (size_t)bh * ix.nr;
     const float gneg = G[(size_t)bh * L + row];
     HybRowAcc acc;
     acc.clear();
@@ -491,7 +597,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K,
         float dsv = 0.f;
         if (k < rc) {
             dsv = (dp + gneg) * pv * scale;
-            dSh[pp] = dsv;
+            pairs[r0 + k] = make_float2(dsv, pv);
         }
         acc.chunk(dsv, col, nk, K + hb, lane);
     }
@@ -506,13 +612,15 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K,
 // Backward, column pass, dense tiles: dK_J = sum_I dS_IJ^T Q_I / sqrt(d), dV_J = sum_I P_IJ^T dO_I; dP - g is
 // recomputed per tile by a chain started from the stored -g.
 // -------------------------------------------------------------------------------------------------
-SPION_HYB_KERNEL void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const float* __restrict__ V,
+template <int WAVES>
+SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const float* __restrict__ V,
                                               const float* __restrict__ P, const float* __restrict__ dO,
                                               const float* __restrict__ G, float* __restrict__ dK,
                                               float* __restrict__ dV, HybIndex ix, int L, int nbr, int NB, int nnz,
                                               float scale) {
-    constexpr int D = 32, KH = 16, WAVES = HYB_WAVES;
+    constexpr int D = 32, KH = 16;
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
+    __shared__ __attribute__((aligned(16))) int lds_x[WAVES][128];
     float* lds = &lds_t[0][0];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, J = item % nbr;
@@ -521,9 +629,10 @@ SPION_HYB_KERNEL void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const
     const rsrc_t rQ = make_rsrc(Q + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
     const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4);
     const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
-    const float* Ph = P + (size_t)bh * nnz;
+    const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     float* Tq = lds_t[w];
     float* To = Tq + 32 * TS;
+    int* X = lds_x[w];
     const int lin = lin_voff(l, D);
 
     float vt[KH];
@@ -531,49 +640,58 @@ SPION_HYB_KERNEL void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const
 
     f32x16 ak[1] = {splat16(0.f)}, av[1] = {splat16(0.f)};
     const int e0 = ix.t_cp[J], ecnt = ix.t_cp[J + 1] - e0;
-    for (int e = e0 + w; e < e0 + ecnt; e += WAVES) {
-        const int t = ix.t_ct[e];
-        const int I = ix.t_row[t];
-        f32x4 qraw[4], oraw[4];
-        ldr_tile_lin(rQ, lin, I * 32 * D * 4, D, qraw);
-        ldr_tile_lin(rdO, lin, I * 32 * D * 4, D, oraw);
-        float gn[16];
-        ldr_4x4(rG, 16 * h, I * 128, gn);
-        int pos[16];
-        unsigned bits[16];
-        hyb_tile_rows(ix, t, h, pos, bits);
-        float p[16], go[KH], qb[1][16], ob[1][16];
-        hyb_load_p_cols(Ph, pos, bits, li, p);  // p[r] = P[query acc_row(r, h)][key li]
-        lds_put_lin(Tq, l, qraw);
-        lds_put_lin(To, l, oraw);
-        lds_get_feat32(To, li, h, go);
-        lds_get_cols(Tq, li, h, qb[0]);
-        lds_get_cols(To, li, h, ob[0]);
-        f32x16 init;
+    const int n = ecnt > w ? (ecnt - w + WAVES - 1) / WAVES : 0;
+    HybPre xa, xb;
+    hyb_pipeline(
+        n, xa, xb,
+        [&](HybPre& x, int i) {
+            const int e = e0 + w + min(i, n - 1) * WAVES;
+            x.blk = ix.t_ci[e];
+            hyb_fetch_index(ix, ix.t_ct[e], li, x);
+        },
+        [&](HybPre& x, int) {
+            int pos[16];
+            unsigned bits[16];
+            hyb_tile_rows(X, l, h, x, pos, bits);
+            ldr_tile_lin(rQ, lin, x.blk * 32 * D * 4, D, x.a);
+            ldr_tile_lin(rdO, lin, x.blk * 32 * D * 4, D, x.b);
+            hyb_load_p_cols(rP, pos, bits, li, x.p);  // p[r] = P[query acc_row(r, h)][key li]
+            x.g_l = ld1(rG, li * 4, x.blk * 128);
+        },
+        [&](HybPre& x, int) {
+            float go[KH], qb[1][16], ob[1][16];
+            int gn[16];
+            lds_put_lin(Tq, l, x.a);
+            lds_put_lin(To, l, x.b);
+            hyb_rows_from_lanes(X, l, h, __builtin_bit_cast(int, x.g_l), gn);
+            lds_get_feat32(To, li, h, go);
+            lds_get_cols(Tq, li, h, qb[0]);
+            lds_get_cols(To, li, h, ob[0]);
+            f32x16 init;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) init[r] = gn[r];
-        const f32x16 dp = mma_feat_init<D>(go, vt, init);  // dO_i . v_j - g_i, i = acc_row(r, h), j = li
-        float ds[16];
+            for (int r = 0; r < 16; ++r) init[r] = __builtin_bit_cast(float, gn[r]);
+            const f32x16 dp = mma_feat_init<D>(go, vt, init);  // dO_i . v_j - g_i, i = acc_row(r, h), j = li
+            float ds[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = dp[r] * p[r];
-        mma_b<D>(ds, qb, ak);
-        mma_b<D>(p, ob, av);
-    }
-    __syncthreads();
-    hyb_reduce_store(ak[0], scale, dK + hb, nullptr, J * 32, w, li, h, lds);
-    __syncthreads();
-    hyb_reduce_store(av[0], 1.0f, dV + hb, nullptr, J * 32, w, li, h, lds);
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * x.p[r];
+            mma_b<D>(ds, qb, ak);
+            mma_b<D>(x.p, ob, av);
+        });
+    if constexpr (WAVES > 1) __syncthreads();
+    hyb_reduce_store<WAVES>(ak[0], scale, dK + hb, nullptr, J * 32, w, li, h, lds);
+    if constexpr (WAVES > 1) __syncthreads();
+    hyb_reduce_store<WAVES>(av[0], 1.0f, dV + hb, nullptr, J * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass, remainder: dK_j += sum_i dS_ij Q_i, dV_j += sum_i P_ij dO_i over the remainder's
-// transposed index (dS already carries the 1/sqrt(d)).
+// transposed index, from the compact {dS, P} pairs of the row pass (dS already carries the 1/sqrt(d)).
 // -------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // two gathers in flight per entry: four waves per SIMD
     const float* __restrict__ Q, const float* __restrict__ dO,
-                                                    const float* __restrict__ P, const float* __restrict__ dS,
+                                                    const float2* __restrict__ Pairs,
                                                     float* __restrict__ dK, float* __restrict__ dV, HybIndex ix, int L,
-                                                    int NB, int nnz) {
+                                                    int NB) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wcol = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
     if (wcol >= (long long)NB * L) return;
@@ -581,8 +699,7 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
     const int c0p = ix.c_ptr[colj], cnt = ix.c_ptr[colj + 1] - c0p;
     if (cnt == 0) return;
     const size_t hb = (size_t)bh * L * 32;
-    const float* Ph = P + (size_t)bh * nnz;
-    const float* dSh = dS + (size_t)bh * nnz;
+    const float2* pairs = Pairs + (size_t)bh * ix.nr;
     HybRowAcc ak, av;
     ak.clear();
     av.clear();
@@ -591,10 +708,10 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
         float wk = 0.f, wv = 0.f;
         int row = 0;
         if (e < cnt) {
-            const int pp = ix.c_pos[c0p + e];
             row = ix.c_row[c0p + e];
-            wk = dSh[pp];
-            wv = Ph[pp];
+            const float2 pr = pairs[ix.c_src[c0p + e]];
+            wk = pr.x;
+            wv = pr.y;
         }
         const int nk = min(64, cnt - c0);
         ak.chunk(wk, row, nk, Q + hb, lane);

@@ -331,7 +331,7 @@ struct PatternIndex {
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // element-sparse pattern whose well-filled 32x32 tiles run on the MFMA units (hybrid_kernels.h)
     bool hybrid = false;
-    int hyb_tiles = 0;
+    int hyb_tiles = 0, hyb_nr = 0;
     HybIndex hyb{};
     // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
     // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
@@ -570,7 +570,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
     size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0;
-    size_t hyb_off[13] = {};
+    size_t hyb_off[14] = {};
     if (tiled) {
         const int nt = (int)tcol.size();
         std::vector<int> tcp(nbr + 1, 0), tcdesc(4 * (size_t)std::max(nt, 1), 0);
@@ -663,7 +663,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.max_col_tiles = mc;
     } else {
         // ---- hybrid split: aligned 32x32 tiles with at least HYB_MIN_FILL entries become dense tiles (at most
-        // HYB_WAVES * HYB_MAXT per block row, the fullest first), everything else stays with the gather kernels
+        // HYB_MAX_ROW_TILES per block row, the fullest first), everything else stays with the gather kernels
         if (!a->force_element && a->d == 32 && L % 32 == 0 && nnz > 0) {
             constexpr int HYB_MIN_FILL = 128;
             const int nbr = L / 32;
@@ -677,9 +677,9 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                 std::vector<int> cand;
                 for (int J = 0; J < nbr; ++J)
                     if (cnt[J] >= HYB_MIN_FILL) cand.push_back(J);
-                if ((int)cand.size() > HYB_WAVES * HYB_MAXT) {
+                if ((int)cand.size() > HYB_MAX_ROW_TILES) {
                     std::stable_sort(cand.begin(), cand.end(), [&](int x, int y) { return cnt[x] > cnt[y]; });
-                    cand.resize(HYB_WAVES * HYB_MAXT);
+                    cand.resize(HYB_MAX_ROW_TILES);
                     std::sort(cand.begin(), cand.end());
                 }
                 for (int J : cand) {
@@ -691,7 +691,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                 t_rp[I + 1] = (int)t_col.size();
             }
             const int nt = (int)t_col.size();
-            if (nt > 0 && dense_entries * 4 >= (long long)nnz) {
+            if (nt > 0 && dense_entries * 2 >= (long long)nnz) {
                 std::vector<int> t_pos((size_t)nt * 32, 0), r_off(L + 1, 0), r_col, r_pos;
                 std::vector<unsigned> t_bits((size_t)nt * 32, 0u);
                 std::vector<int> slot(nbr);
@@ -722,7 +722,9 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                     std::vector<int> fill(t_cp.begin(), t_cp.end() - 1);
                     for (int t = 0; t < nt; ++t) t_ct[fill[t_col[t]]++] = t;
                 }
-                std::vector<int> c_ptr(L + 1, 0), c_row(std::max(nr, 1), 0), c_pos(std::max(nr, 1), 0);
+                std::vector<int> t_ci(t_ct.size());
+                for (size_t e = 0; e < t_ct.size(); ++e) t_ci[e] = t_row[t_ct[e]];
+                std::vector<int> c_ptr(L + 1, 0), c_row(std::max(nr, 1), 0), c_src(std::max(nr, 1), 0);
                 for (int e = 0; e < nr; ++e) c_ptr[r_col[e] + 1]++;
                 for (int j = 0; j < L; ++j) c_ptr[j + 1] += c_ptr[j];
                 {
@@ -731,7 +733,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                         for (int e = r_off[i]; e < r_off[i + 1]; ++e) {
                             const int x = fill[r_col[e]]++;
                             c_row[x] = i;
-                            c_pos[x] = r_pos[e];
+                            c_src[x] = e;
                         }
                 }
                 if (r_col.empty()) {
@@ -752,9 +754,15 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                 hyb_off[9] = append(r_pos);
                 hyb_off[10] = append(c_ptr);
                 hyb_off[11] = append(c_row);
-                hyb_off[12] = append(c_pos);
+                hyb_off[12] = append(c_src);
+                hyb_off[13] = append(t_ci);
+                pi.hyb_nr = nr;
                 pi.hybrid = true;
                 pi.hyb_tiles = nt;
+                for (int I = 0; I < nbr; ++I) {
+                    pi.max_row_tiles = std::max(pi.max_row_tiles, t_rp[I + 1] - t_rp[I]);
+                    pi.max_col_tiles = std::max(pi.max_col_tiles, t_cp[I + 1] - t_cp[I]);
+                }
             }
         }
         std::vector<int> ccp(L + 1, 0), crow(std::max(nnz, 1)), cpos(std::max(nnz, 1));
@@ -796,8 +804,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             const int* b = pi.d_blob;
             pi.hyb = HybIndex{b + hyb_off[0], b + hyb_off[1], b + hyb_off[2], b + hyb_off[3],
                               reinterpret_cast<const unsigned*>(b + hyb_off[4]), b + hyb_off[5], b + hyb_off[6],
-                              b + hyb_off[7], b + hyb_off[8], b + hyb_off[9], b + hyb_off[10], b + hyb_off[11],
-                              b + hyb_off[12]};
+                              b + hyb_off[13], b + hyb_off[7], b + hyb_off[8], b + hyb_off[9], b + hyb_off[10],
+                              b + hyb_off[11], b + hyb_off[12], pi.hyb_nr, pi.hyb_tiles};
         }
     }
     pi.tiled = tiled;
@@ -1100,20 +1108,27 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
         a->last_path = 3;
         const int nbr = a->L / 32;
         const long long rows = (long long)a->NB * a->L;
-        const dim3 grid_t(nbr * a->NB), block_t(64 * HYB_WAVES);
+        // strips of few dense tiles: one wavefront walks the whole strip; else four share it
+        const bool one = a->pat.max_row_tiles <= HYB_MAXT1;
+        const dim3 grid_t(nbr * a->NB), block_t(one ? 64 : 256);
         const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
         float2* stats = reinterpret_cast<float2*>(a->ws_stats);
-        if (a->has_mask) {
-            hipLaunchKernelGGL(hyb_rem_logits_kernel<true>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn, stats,
-                               a->pat.hyb, a->L, a->NB, nnz, a->scale);
-            hipLaunchKernelGGL(hyb_tile_fwd_kernel<true>, grid_t, block_t, 0, a->hdr.stream, Q, Krm, V, Mask, Attn, Out,
-                               stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
-        } else {
-            hipLaunchKernelGGL(hyb_rem_logits_kernel<false>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn,
-                               stats, a->pat.hyb, a->L, a->NB, nnz, a->scale);
-            hipLaunchKernelGGL(hyb_tile_fwd_kernel<false>, grid_t, block_t, 0, a->hdr.stream, Q, Krm, V, Mask, Attn,
-                               Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
-        }
+#define SPION_HYB_FWD(MASKED)                                                                                         \
+    do {                                                                                                              \
+        hipLaunchKernelGGL(hyb_rem_logits_kernel<MASKED>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn,      \
+                           stats, a->pat.hyb, a->L, a->NB, nnz, a->scale);                                            \
+        if (one)                                                                                                      \
+            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 1, HYB_MAXT1>), grid_t, block_t, 0, a->hdr.stream, Q,     \
+                               Krm, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale); \
+        else                                                                                                          \
+            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 4, HYB_MAXT4>), grid_t, block_t, 0, a->hdr.stream, Q,     \
+                               Krm, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale); \
+    } while (0)
+        if (a->has_mask)
+            SPION_HYB_FWD(true);
+        else
+            SPION_HYB_FWD(false);
+#undef SPION_HYB_FWD
         hipLaunchKernelGGL(hyb_rem_pv_kernel, grid_g, block_g, 0, a->hdr.stream, V, Attn, Out, hyb_ocopy,
                            (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz);
         check_launch("hybrid forward kernels");
@@ -1182,19 +1197,33 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
             a->last_path = 3;
             const int nbr = a->L / 32;
             const long long rows = (long long)a->NB * a->L;
-            const dim3 grid_t(nbr * a->NB), block_t(64 * HYB_WAVES);
+            const bool one_r = a->pat.max_row_tiles <= 2 * HYB_MAXT1, one_c = a->pat.max_col_tiles <= 2 * HYB_MAXT1;
+            const dim3 grid_t(nbr * a->NB);
             const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
+            // the remainder's {dS, P} pairs, [NB][nr] inside the caller's dS scratch (NB*nnz floats:
+            // a hybrid pattern keeps at most half of its entries in the remainder)
+            float2* pairs = reinterpret_cast<float2*>(dS);
             if (a->bwd_passes & 1) {
-                hipLaunchKernelGGL(hyb_tile_bwd_row_kernel, grid_t, block_t, 0, a->hdr.stream, K, Vrm, P, dO, o,
-                                   a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+                if (one_r)
+                    hipLaunchKernelGGL(hyb_tile_bwd_row_kernel<1>, grid_t, dim3(64), 0, a->hdr.stream, K, Vrm, P, dO, o,
+                                       a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
+                else
+                    hipLaunchKernelGGL(hyb_tile_bwd_row_kernel<4>, grid_t, dim3(256), 0, a->hdr.stream, K, Vrm, P, dO,
+                                       o, a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
                 hipLaunchKernelGGL(hyb_rem_bwd_row_kernel, grid_g, block_g, 0, a->hdr.stream, K, Vrm, P, dO,
-                                   (const float*)a->ws_rowsum, dS, dQ, a->pat.hyb, a->L, a->NB, nnz, a->scale);
+                                   (const float*)a->ws_rowsum, pairs, dQ, a->pat.hyb, a->L, a->NB, nnz, a->scale);
             }
             if (a->bwd_passes & 2) {
-                hipLaunchKernelGGL(hyb_tile_bwd_col_kernel, grid_t, block_t, 0, a->hdr.stream, Q, Vrm, P, dO,
-                                   (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
-                hipLaunchKernelGGL(hyb_rem_bwd_col_kernel, grid_g, block_g, 0, a->hdr.stream, Q, dO, P,
-                                   (const float*)dS, dK, dV, a->pat.hyb, a->L, a->NB, nnz);
+                if (one_c)
+                    hipLaunchKernelGGL(hyb_tile_bwd_col_kernel<1>, grid_t, dim3(64), 0, a->hdr.stream, Q, Vrm, P, dO,
+                                       (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz,
+                                       a->scale);
+                else
+                    hipLaunchKernelGGL(hyb_tile_bwd_col_kernel<4>, grid_t, dim3(256), 0, a->hdr.stream, Q, Vrm, P, dO,
+                                       (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz,
+                                       a->scale);
+                hipLaunchKernelGGL(hyb_rem_bwd_col_kernel, grid_g, block_g, 0, a->hdr.stream, Q, dO,
+                                   (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB);
             }
             check_launch("hyb_bwd kernels");
             return;
