@@ -259,8 +259,8 @@ void spion_attn_backward_with_out(void* handle, const float* Q, const float* K, 
  * (backward) are read as they are: no transposed copy is made by anyone (d = 32 and the element kernels; the
  * d = 64 tile kernels make one internally).  Mask: NULL for a handle of spion_block_init, the [NB][L] penalty
  * for a handle of spion_blockmask_init.  Out in the backward: the forward's output (may be NULL: the kept copy,
- * or one more sweep, is used).  dS: scratch [NB][nnz], needed by the element kernels only (may be NULL for
- * tile patterns). */
+ * or one more sweep, is used).  dS: scratch [NB][nnz] floats, needed for patterns that are not made of aligned
+ * 32x32 tiles (element and hybrid kernels; contents unspecified on return); may be NULL for tile patterns. */
 void spion_attn_forward_rowmajor(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
                                  float* Attn, float* Out,
                                  const int* Offsets, const int* Columns, const int* SumMat, int nnz);

@@ -8,13 +8,14 @@
 // Per pattern entry the gather path costs about as much machine time as 1/80 of a 32 x 32 MFMA tile, so a tile
 // with more than ~10 % of its entries present is cheaper dense.
 //
-// The two parts run as separate launches, each at the occupancy that suits it: the tile kernels (one work-group of
-// four wavefronts per strip of 32 rows or columns, wavefront w taking the strip's dense tiles w, w+4, ...) and the
-// gather kernels (one wavefront per row or column of the remainder, sixteen wavefronts per CU, because the gathers
-// are bound by the number of requests in flight).  Forward: remainder logits and their row statistics, then the
-// tiles (which merge the statistics and fix the row's maximum and denominator), then the remainder's probabilities
-// and share of O.  Backward: tile part then remainder part of the row pass, the same for the column pass; the
-// remainder kernels add to what the tile kernels wrote (each row or column has exactly one writer per launch).
+// The two parts run as separate launches, each at the occupancy that suits it: the tile kernels (one wavefront per
+// strip of 32 rows or columns when strips hold few dense tiles, else a work-group of four wavefronts, wavefront w
+// taking the strip's dense tiles w, w+4, ...) and the gather kernels (one wavefront per row or column of the
+// remainder, sixteen wavefronts per CU, because the gathers are bound by the number of requests in flight).
+// Forward: remainder logits and their row statistics, then the tiles (which merge the statistics and fix the row's
+// maximum and denominator), then the remainder's probabilities and share of O.  Backward: tile part then remainder
+// part of the row pass, the same for the column pass; the remainder kernels add to what the tile kernels wrote
+// (each row or column has exactly one writer per launch).
 #pragma once
 #include "tile_kernels.h"
 
