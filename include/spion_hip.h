@@ -202,6 +202,9 @@ int spion_transition_update(const float* Cur, float* Prev, int layers, long long
 /* Message of the most recent failure in this process, or "" if none since spion_clear_error(). */
 const char* spion_last_error(void);
 void spion_clear_error(void);
+/* 1 if spion_last_error() would return a message, else 0: the cheap check for a caller that polls after every
+ * call. */
+int spion_error_pending(void);
 
 /* Launch this handle's work on `stream` (a hipStream_t; NULL = null stream).  Any family. */
 void spion_set_stream(void* handle, void* stream);

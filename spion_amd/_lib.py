@@ -52,6 +52,8 @@ def core() -> ctypes.CDLL:
     lib.spion_last_error.argtypes = []
     lib.spion_clear_error.argtypes = []
     lib.spion_clear_error.restype = None
+    lib.spion_error_pending.argtypes = []
+    lib.spion_error_pending.restype = c_int
     lib.spion_set_stream.argtypes = [_P, _P]
     lib.spion_set_stream.restype = None
     lib.spion_invalidate_pattern.argtypes = [_P]
@@ -187,18 +189,30 @@ def empty_adjacent_heads(B, H, L, d, device):
 def use_current_stream(module, device) -> None:
     """Point the module's handle at torch's current stream on ``device`` (the reference runs on the legacy
     default stream only): what makes the modules usable on side streams and under HIP graph capture.  One
-    ctypes call per forward / backward; not cached, since handles can be shared or their addresses reused."""
-    core().spion_set_stream(module.attn_handle, torch.cuda.current_stream(device).cuda_stream)
+    ctypes call per forward / backward; not cached, since handles can be shared or their addresses reused.
+    (The raw-stream query is the one torch's own compiled code uses; ``torch.cuda.current_stream`` builds a Python
+    stream object per call, 15 us on a slow host.)"""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    core().spion_set_stream(module.attn_handle, _raw_stream(index))
+
+
+def _raw_stream_fallback(index: int) -> int:
+    return torch.cuda.current_stream(index).cuda_stream
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", _raw_stream_fallback)
 
 
 def check_error(where: str = "") -> None:
     """Raise if the library recorded a failure since the last check (the C entry points return void)."""
     lib = core()
-    msg = lib.spion_last_error()
-    if msg:
-        text = msg.decode("utf-8", "replace")
-        lib.spion_clear_error()
-        raise SpionLibraryError(f"{where}: {text}" if where else text)
+    if not lib.spion_error_pending():
+        return
+    text = lib.spion_last_error().decode("utf-8", "replace")
+    lib.spion_clear_error()
+    raise SpionLibraryError(f"{where}: {text}" if where else text)
 
 
 def load_dropin(name: str, n_init: int, n_fwd: int, n_bwd: int, trailing_int: bool) -> ctypes.CDLL:

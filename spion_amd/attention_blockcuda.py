@@ -38,14 +38,11 @@ class _BlockAttnFunction(torch.autograd.Function):
         m = module
         _lib.use_current_stream(m, query.device)
         idx = m.csr_cache.get(mat, m.block_size)
-        nb_, L, d = m.num_batches, m.seq_len, m.emb_dim
-        if tuple(query.shape) != (m.batch_size, m.num_heads, L, d):
-            raise ValueError(
-                f"query shape {tuple(query.shape)} does not match the handle "
-                f"({m.batch_size}, {m.num_heads}, {L}, {d})"
-            )
+        nb_ = m.num_batches
+        shape = m.head_shape
+        if query.shape != shape:
+            raise ValueError(f"query shape {tuple(query.shape)} does not match the handle {shape}")
         dev = query.device
-        shape = (m.batch_size, m.num_heads, L, d)
         p_flat = torch.empty(nb_ * idx.nnz, dtype=torch.float32, device=dev)
         pen_ptr = None
         if m.with_mask:
@@ -63,19 +60,18 @@ class _BlockAttnFunction(torch.autograd.Function):
             lout = _lib.head_layout(out)
             _lib.core().spion_attn_forward_strided(
                 m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr, p_flat.data_ptr(), out.data_ptr(),
-                idx.offsets.data_ptr(), idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz, m.num_heads,
-                ctypes.addressof(lay), ctypes.addressof(lout))
+                *idx.tail, m.num_heads, ctypes.addressof(lay), ctypes.addressof(lout))
         else:
             q, k, v = query.contiguous(), key.contiguous(), value.contiguous()
             out = torch.empty(shape, dtype=torch.float32, device=dev)
             _lib.core().spion_attn_forward_rowmajor(m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
-                                                    p_flat.data_ptr(), out.data_ptr(), idx.offsets.data_ptr(),
-                                                    idx.columns.data_ptr(), idx.sum_mat.data_ptr(), idx.nnz)
+                                                    p_flat.data_ptr(), out.data_ptr(), *idx.tail)
         _lib.check_error("attn_forward")
         ctx.save_for_backward(q, k, v, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
         ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
         ctx.nnz = idx.nnz
+        ctx.tail = idx.tail  # the index tensors themselves are among the saved tensors
         ctx.strided = lay is not None
         if m.with_mask:
             ctx.mark_non_differentiable(p_flat)
@@ -104,9 +100,8 @@ class _BlockAttnFunction(torch.autograd.Function):
             lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
             core.spion_attn_backward_strided(
                 m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), p_flat.data_ptr(), out.data_ptr(),
-                go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), offsets.data_ptr(), columns.data_ptr(),
-                sum_mat.data_ptr(), ctx.nnz, m.num_heads, ctypes.addressof(lin), ctypes.addressof(lout),
-                ctypes.addressof(lgrad))
+                go.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), *ctx.tail, m.num_heads,
+                ctypes.addressof(lin), ctypes.addressof(lout), ctypes.addressof(lgrad))
             _lib.check_error("attn_backward")
             return dq, dk, dv, None, None, None
         go = grad_output.contiguous()
@@ -115,14 +110,14 @@ class _BlockAttnFunction(torch.autograd.Function):
         scratch_ds = None
         if core.spion_last_path(m.attn_handle) != 1:
             scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
-        shape = (m.batch_size, m.num_heads, m.seq_len, m.emb_dim)
+        shape = m.head_shape
         dq = torch.empty(shape, dtype=torch.float32, device=dev)
         dk = torch.empty(shape, dtype=torch.float32, device=dev)
         dv = torch.empty(shape, dtype=torch.float32, device=dev)
         core.spion_attn_backward_rowmajor(
             m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), p_flat.data_ptr(), out.data_ptr(), go.data_ptr(),
             scratch_ds.data_ptr() if scratch_ds is not None else None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-            offsets.data_ptr(), columns.data_ptr(), sum_mat.data_ptr(), ctx.nnz)
+            *ctx.tail)
         _lib.check_error("attn_backward")
         return dq, dk, dv, None, None, None
 
@@ -156,6 +151,7 @@ class _BlockAttentionBase(nn.Module):
         self.attn_handle = attn_handle
         self.csr_cache = CsrCache(handle=attn_handle)
         self.attn_func = _BlockAttnFunction
+        self.head_shape = (self.batch_size, self.num_heads, self.seq_len, self.emb_dim)
         _lib.core().spion_use_output_cache(attn_handle, 0)  # the backward is handed the output instead
         # block masks whose blocks are unions of 32x32 tiles run on the tile kernels, which take views
         self.reads_views = self.emb_dim in (32, 64) and self.block_size % 32 == 0 and self.seq_len % 32 == 0

@@ -32,6 +32,10 @@ class CsrIndex:
     nnz: int
     keepalive: object = None
 
+    def __post_init__(self):
+        # (Offsets, Columns, SumMat, nnz) as the C entry points take them; the tensors never change or move
+        self.tail = (self.offsets.data_ptr(), self.columns.data_ptr(), self.sum_mat.data_ptr(), self.nnz)
+
 
 def block_mask_to_csr_host(mat: np.ndarray, block_size: int):
     """numpy arrays (sum_mat, offsets, columns) for a [nb, nb] block mask (non-zero = kept)."""
@@ -96,7 +100,7 @@ class CsrCache:
 
     def put(self, mat: torch.Tensor, block_size: int, entry: CsrIndex) -> None:
         """File a prebuilt index (a sidecar built when the masks were loaded) under ``mat``."""
-        key = (mat.data_ptr(), mat._version, tuple(mat.shape), tuple(mat.stride()), int(block_size), str(mat.device))
+        key = (mat.data_ptr(), mat._version, mat.shape, mat.stride(), block_size, mat.device)
         old = self._entries.pop(key, None)
         if old is not None and old is not entry:
             self._forget(old)
@@ -110,7 +114,7 @@ class CsrCache:
             self._forget(old)
 
     def get(self, mat: torch.Tensor, block_size: int) -> CsrIndex:
-        key = (mat.data_ptr(), mat._version, tuple(mat.shape), tuple(mat.stride()), int(block_size), str(mat.device))
+        key = (mat.data_ptr(), mat._version, mat.shape, mat.stride(), block_size, mat.device)
         hit = self._entries.get(key)
         if hit is not None:
             self._entries.move_to_end(key)

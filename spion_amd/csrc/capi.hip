@@ -217,6 +217,10 @@ void spion_clear_error(void) {
     std::lock_guard<std::mutex> lock(g_err_mutex);
     g_err.clear();
 }
+int spion_error_pending(void) {
+    std::lock_guard<std::mutex> lock(g_err_mutex);
+    return g_err.empty() ? 0 : 1;
+}
 const char* spion_handle_error(void* h) {
     HandleHeader* hd = static_cast<HandleHeader*>(h);
     if (!hd || (hd->magic != KIND_SPARSE && hd->magic != KIND_DENSE)) return "not a spion handle";

@@ -76,6 +76,44 @@ def test_pattern_config2_bit_exact_against_both_routes():
         assert np.array_equal(mat[i].astype(np.int8), m32)
 
 
+def test_discovery_repeats_on_any_stream_and_under_capture():
+    """The result must not depend on how often, on which stream, or whether inside a graph the call is made.  The
+    reference for every variant is the first eager call, itself checked against the oracle."""
+    g = torch.Generator().manual_seed(5)
+    maps = torch.softmax(torch.randn(5, 512, 512, generator=g) * 2, -1)
+    ref_mat, ref_pooled, ref_thresh = _check_maps(maps, 32, 0.9, 31)
+    dev_maps = maps.cuda()
+
+    def same(out):
+        mat, pooled, thresh = (t.cpu().numpy() for t in out)
+        assert np.array_equal(mat, ref_mat) and np.array_equal(pooled, ref_pooled) and np.array_equal(thresh, ref_thresh)
+
+    for _ in range(3):
+        same(discover_block_masks(dev_maps, 32, mode="conv_ff", threshold=0.9, return_aux=True))
+    for _ in range(2):  # two side streams
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                out = discover_block_masks(dev_maps, 32, mode="conv_ff", threshold=0.9, return_aux=True)
+        side.synchronize()
+        same(out)
+    # recorded into a graph and replayed, with eager calls in between
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            out_g = discover_block_masks(dev_maps, 32, mode="conv_ff", threshold=0.9, return_aux=True)
+    for _ in range(3):
+        for t in out_g:
+            t.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        same(out_g)
+        same(discover_block_masks(dev_maps, 32, mode="conv_ff", threshold=0.9, return_aux=True))
+
+
 @pytest.mark.parametrize("density", [0.2, 0.45, 0.8])
 def test_pattern_topk_with_ties(density):
     """Maps of few exact levels (multiples of 1/4): pooled values are exact in both routes and tie massively, so
