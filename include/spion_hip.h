@@ -299,10 +299,12 @@ long long spion_noalloc_max_rows(void);
  * the gradients dQ, dK, dV.  heads = H (num_batches of the handle = B*H, head index fastest).  Strides are
  * multiples of 4 floats, pointers 16-byte aligned, seq_len * row_stride < 2^29; the layouts of tensors that are
  * written (out, grad) must not map two elements to one address, those of inputs may (head_stride 0: one K / V
- * head shared by all query heads).  Served by the tile kernels
- * for emb_dim 32 (patterns of aligned 32x32 tiles); otherwise an error is recorded and the caller makes
- * contiguous copies for the row-major entry points above.  Attn / P stay [NB][nnz] as everywhere.  The kept
- * copies of Out are not used: the backward takes Out (required). */
+ * head shared by all query heads).  Served by every kernel family: the tile kernels (emb_dim 32 or 64, patterns
+ * of aligned 32x32 tiles), the hybrid kernels (emb_dim 32) and the element kernels (emb_dim 16, 32, 64, 128);
+ * the results equal those of the row-major entry points bit for bit.  Attn / P stay [NB][nnz] as everywhere.
+ * The kept copies of Out are not used: the backward takes Out (required).  On patterns without tile structure
+ * the backward's dS scratch ([NB][nnz] floats) belongs to the handle and is allocated by the first such call
+ * (not under HIP graph capture). */
 typedef struct spion_head_layout {
     long long batch_stride;
     int head_stride;

@@ -26,12 +26,12 @@ class _BlockAttnFunction(torch.autograd.Function):
     ``attn_cpp`` (the drop-in with the reference's four symbols) is still what created the handle.
 
     The reference also starts with ``.contiguous()`` copies of query, key and value (models/attention_blockcuda.py:
-    36-48), which arrive as [B,H,L,d] views of [B,L,H*d] projections (models/attention.py:136-139).  For head
-    dimension 32 and block sizes that are multiples of 32 (the tile kernels) the strided entry points read the
-    views in place, write ``out`` in the same interleaved layout (so that combine_heads, models/attention.py:131-134,
-    is a view as well) and the gradients likewise: no copy on either side of the kernels.  (Head dimension 64 is served
-    the same way; its kernels read row-major K and V a cache line per lane, slower than the transposed form the
-    contiguous entry points use, but still cheaper than the copies.)"""
+    36-48), which arrive as [B,H,L,d] views of [B,L,H*d] projections (models/attention.py:136-139).  The strided
+    entry points read the views in place, write ``out`` in the same interleaved layout (so that combine_heads,
+    models/attention.py:131-134, is a view as well) and the gradients likewise: no copy on either side of the
+    kernels.  (Head dimension 64 on tile patterns is served the same way; its kernels read row-major K and V a cache
+    line per lane, slower than the transposed form the contiguous entry points use, but still cheaper than the
+    copies.)"""
 
     @staticmethod
     def forward(ctx, query, key, value, mask, mat, module):
@@ -153,8 +153,8 @@ class _BlockAttentionBase(nn.Module):
         self.attn_func = _BlockAttnFunction
         self.head_shape = (self.batch_size, self.num_heads, self.seq_len, self.emb_dim)
         _lib.core().spion_use_output_cache(attn_handle, 0)  # the backward is handed the output instead
-        # block masks whose blocks are unions of 32x32 tiles run on the tile kernels, which take views
-        self.reads_views = self.emb_dim in (32, 64) and self.block_size % 32 == 0 and self.seq_len % 32 == 0
+        # every kernel family (tile, hybrid, element) reads [B,H,L,d] views of projections in place
+        self.reads_views = self.emb_dim in (16, 32, 64, 128)
 
 
 class CUDABlockAttention(_BlockAttentionBase):

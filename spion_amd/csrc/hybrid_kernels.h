@@ -117,12 +117,11 @@ __device__ __forceinline__ void hyb_store_p_cols(float* __restrict__ Ph, const i
 }
 
 // Sum of the wavefronts' 32 x 32 accumulators (rows acc_row(r, h) of the strip, columns li) times `factor`, in a
-// fixed order.  `lds` (WAVES * 1024 floats, unused for one wavefront) may alias tile space no wavefront uses any
+// fixed order, to rows of stride ld.  `lds` (WAVES * 1024 floats, unused for one wavefront) may alias tile space no wavefront uses any
 // more: the caller has a barrier between that use and this call.
 template <int WAVES>
-__device__ __forceinline__ void hyb_reduce_store(const f32x16& acc, float factor, float* __restrict__ out,
-                                                 float* __restrict__ out2, int row0, int w, int li, int h,
-                                                 float* __restrict__ lds) {
+__device__ __forceinline__ void hyb_reduce_store(const f32x16& acc, float factor, float* __restrict__ out, int ld,
+                                                 int row0, int w, int li, int h, float* __restrict__ lds) {
     const int l = h * 32 + li;
     if constexpr (WAVES > 1) {
 #pragma unroll
@@ -139,9 +138,7 @@ __device__ __forceinline__ void hyb_reduce_store(const f32x16& acc, float factor
             for (int ww = 0; ww < WAVES; ++ww) s += lds[(ww * 16 + r) * 64 + l];
         }
         s *= factor;
-        const size_t a = (size_t)(row0 + acc_row(r, h)) * 32 + li;
-        out[a] = s;
-        if (out2) out2[a] = s;
+        out[(size_t)(row0 + acc_row(r, h)) * ld + li] = s;
     }
 }
 
@@ -191,18 +188,25 @@ __device__ __forceinline__ float hyb_group_sum(float v) {
     return v;
 }
 
-// Dot products of the rows X[row_l] (row index of the lane's entry; nk entries in the chunk) with the vector whose
+// Start (in floats) and row stride of head bh in a tensor group: contiguous [NB][L][32] heads (ST = false, compile-time
+// figures) or [B][H][L][32] views given by a layout.
+template <bool ST>
+__device__ __forceinline__ void hyb_head(const HeadLayout& y, int H, int bh, int L, size_t& base, int& ld) {
+    size_t bytes;
+    head_slice<ST, 32>(y, H, bh, L, base, ld, bytes);
+}
+
+// Dot products of the rows X[row_l] (row stride ld) (row index of the lane's entry; nk entries in the chunk) with the vector whose
 // piece 4*(lane%8) .. +3 the lane holds in a4: one result per lane, for the lane's own entry.  Only the load
 // instructions that carry entries are issued; lanes whose entry is past nk get 0 or a partial value to ignore.
-__device__ __forceinline__ float hyb_gather_dot(const f32x4 a4, const float* __restrict__ X, int row_l, int nk,
-                                                int lane) {
-    constexpr int D = 32;
+__device__ __forceinline__ float hyb_gather_dot(const f32x4 a4, const float* __restrict__ X, int ld, int row_l,
+                                                int nk, int lane) {
     const int base = lane & ~7, cl = lane & 7;
     f32x4 x[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int rr = __shfl(row_l, base + j, 64);
-        if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * D)[cl];
+        if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * ld)[cl];
     }
     float r = 0.f;
 #pragma unroll
@@ -224,8 +228,8 @@ __device__ __forceinline__ float hyb_gather_dot(const f32x4 a4, const float* __r
 struct HybRowAcc {
     f32x4 acc;
     __device__ __forceinline__ void clear() { acc = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int lane) {
-        constexpr int D = 32;
+    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int ld,
+                                          int lane) {
         const int base = lane & ~7, cl = lane & 7;
         float w[8];
         f32x4 x[8];
@@ -233,7 +237,7 @@ struct HybRowAcc {
         for (int j = 0; j < 8; ++j) {
             w[j] = __shfl(w_l, base + j, 64);
             const int rr = __shfl(row_l, base + j, 64);
-            if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * D)[cl];
+            if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * ld)[cl];
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j)
@@ -255,20 +259,22 @@ struct HybRowAcc {
 // Forward, step 1: raw logits (log2 domain) of the remainder entries into P, and per row their maximum and the sum
 // of their exponentials relative to it: Stats[bh][row] = {m, z} ({HYB_ABSENT, 0} for a row without remainder).
 // -------------------------------------------------------------------------------------------------
-template <bool MASK>
+template <bool MASK, bool ST>
 SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                                    const float* __restrict__ pen, float* __restrict__ P,
                                                    float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz,
-                                                   float scale) {
+                                                   float scale, Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
-    const size_t hb = (size_t)bh * L * 32;
+    size_t ib;
+    int ild;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
     float* Ph = P + (size_t)bh * nnz;
     const float c2 = scale * LOG2E;
-    f32x4 q4 = reinterpret_cast<const f32x4*>(Q + hb + (size_t)row * 32)[lane & 7];
+    f32x4 q4 = reinterpret_cast<const f32x4*>(Q + ib + (size_t)row * ild)[lane & 7];
     q4 *= c2;
     // the logits of the first chunks stay in registers; longer rows go back to what they stored in P
     constexpr int KEEP = 2;
@@ -278,7 +284,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
         const int k = c0 + ent;
         const int col = k < rc ? ix.r_col[r0 + k] : 0;
         const int pp = k < rc ? ix.r_pos[r0 + k] : 0;
-        float v = hyb_gather_dot(q4, K + hb, col, min(64, rc - c0), lane);
+        float v = hyb_gather_dot(q4, K + ib, ild, col, min(64, rc - c0), lane);
         if (k < rc) {
             if (MASK) v -= pen[(size_t)bh * L + col] * LOG2E;
             Ph[pp] = v;
@@ -306,12 +312,12 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
 // maximum, 1 / denominator} for step 3).  Writes the tiles' probabilities to their CSR positions and O = P.V of the
 // tile part (step 3 adds the remainder's share).
 // -------------------------------------------------------------------------------------------------
-template <bool MASK, int WAVES, int MAXT>
+template <bool MASK, int WAVES, int MAXT, bool ST>
 SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, const float* __restrict__ K,
                                           const float* __restrict__ V, const float* __restrict__ pen,
                                           float* __restrict__ P, float* __restrict__ O, float2* __restrict__ Stats,
                                           const int* __restrict__ offs, HybIndex ix, int L, int nbr, int NB, int nnz,
-                                          float scale) {
+                                          float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];  // two 32-row tiles per wavefront
@@ -320,19 +326,21 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, co
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const size_t hb = (size_t)bh * L * D;
-    const rsrc_t rQ = make_rsrc(Q + hb, (size_t)L * D * 4), rK = make_rsrc(K + hb, (size_t)L * D * 4);
-    const rsrc_t rV = make_rsrc(V + hb, (size_t)L * D * 4);
+    size_t ib, ob, ibytes, obytes;
+    int ild, old_;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     float* Ph = P + (size_t)bh * nnz;
     float* T = lds_t[w];
     float* Tx = T + 32 * TS;
     int* X = lds_x[w];
     const float c2 = scale * LOG2E;
-    const int lin = lin_voff(l, D);
+    const int lin = lin_voff(l, ild), tile_bytes = 32 * ild * 4;
 
     float q[KH];
-    ldr_rows<D>(rQ, (li * D + h * KH) * 4, I * 32 * D * 4, q);
+    ldr_rows<D>(rQ, (li * ild + h * KH) * 4, I * tile_bytes, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
     const float2 rem = Stats[(size_t)bh * L + I * 32 + li];  // the remainder of row li
@@ -355,15 +363,15 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, co
     f32x16 S[MAXT];
     f32x4 raw[2][4];
     float pj[2][16];
-    ldr_tile_lin(rK, lin, Js[0] * 32 * D * 4, D, raw[0]);
+    ldr_tile_lin(rK, lin, Js[0] * tile_bytes, ild, raw[0]);
     if constexpr (MASK) ldr_4x4(rM, 16 * h, Js[0] * 128, pj[0]);
 #pragma unroll
     for (int u = 0; u < MAXT; ++u) {
         if (u + 1 < MAXT) {
-            ldr_tile_lin(rK, lin, Js[u + 1] * 32 * D * 4, D, raw[(u + 1) & 1]);
+            ldr_tile_lin(rK, lin, Js[u + 1] * tile_bytes, ild, raw[(u + 1) & 1]);
             if constexpr (MASK) ldr_4x4(rM, 16 * h, Js[u + 1] * 128, pj[(u + 1) & 1]);
         } else {
-            ldr_tile_lin(rV, lin, Js[0] * 32 * D * 4, D, raw[(u + 1) & 1]);  // first tile of V for the last step
+            ldr_tile_lin(rV, lin, Js[0] * tile_bytes, ild, raw[(u + 1) & 1]);  // first tile of V for the last step
         }
         __builtin_amdgcn_sched_barrier(0);
         if (u < nu) {
@@ -428,7 +436,7 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, co
 #pragma unroll
     for (int u = 0; u < MAXT; ++u) {
         constexpr int FIRST = MAXT & 1;  // the set the first tile of V went to
-        if (u + 1 < MAXT) ldr_tile_lin(rV, lin, Js[u + 1] * 32 * D * 4, D, raw[(FIRST + u + 1) & 1]);
+        if (u + 1 < MAXT) ldr_tile_lin(rV, lin, Js[u + 1] * tile_bytes, ild, raw[(FIRST + u + 1) & 1]);
         __builtin_amdgcn_sched_barrier(0);
         if (u < nu) {
             lds_put_lin(Tx, l, raw[(FIRST + u) & 1]);
@@ -449,22 +457,27 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, co
     if constexpr (WAVES > 1) __syncthreads();
     // every wavefront has consumed the remainder's statistics by now: replace them by the row's final ones
     if (w == 0 && h == 0) Stats[(size_t)bh * L + I * 32 + li] = make_float2(Mx, zinv);
-    hyb_reduce_store<WAVES>(o[0], 1.0f, O + hb, nullptr, I * 32, w, li, h, lds);
+    hyb_reduce_store<WAVES>(o[0], 1.0f, O + ob, old_, I * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Forward, step 3: probabilities of the remainder entries from their raw logits and the row's {maximum,
 // 1 / denominator}; their share of O is added to what step 2 wrote.  Ocache (optional): second copy of O.
 // -------------------------------------------------------------------------------------------------
+template <bool ST>
 SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, float* __restrict__ P,
                                                float* __restrict__ O, float* __restrict__ Ocache,
-                                               const float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz) {
+                                               const float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz,
+                                               Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
-    const size_t hb = (size_t)bh * L * 32;
+    size_t ib, ob;
+    int ild, old_;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
     float* Ph = P + (size_t)bh * nnz;
     const float2 st = Stats[(size_t)bh * L + row];
     HybRowAcc acc;
@@ -479,14 +492,14 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, floa
             col = ix.r_col[r0 + k];
             Ph[pp] = wgt;
         }
-        acc.chunk(wgt, col, min(64, rc - c0), V + hb, lane);
+        acc.chunk(wgt, col, min(64, rc - c0), V + ib, ild, lane);
     }
     const f32x4 tot = acc.total();
     if (lane < 8) {
-        f32x4* orow = reinterpret_cast<f32x4*>(O + hb + (size_t)row * 32) + lane;
+        f32x4* orow = reinterpret_cast<f32x4*>(O + ob + (size_t)row * old_) + lane;
         const f32x4 sum = *orow + tot;
         *orow = sum;
-        if (Ocache) reinterpret_cast<f32x4*>(Ocache + hb + (size_t)row * 32)[lane] = sum;
+        if (Ocache) reinterpret_cast<f32x4*>(Ocache + ((size_t)bh * L + row) * 32)[lane] = sum;  // own copy: contiguous
     }
 }
 
@@ -494,12 +507,12 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, floa
 // Backward, row pass, dense tiles: g_i = dO_i . O_i (G receives -g for the other kernels); dP^T - g = V_J.dO_I^T
 // chain started from -g, dS' = (dP - g)*P, dQ = sum dS'.K_J / sqrt(d).
 // -------------------------------------------------------------------------------------------------
-template <int WAVES>
+template <int WAVES, bool ST>
 SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
                                               const float* __restrict__ P, const float* __restrict__ dO,
                                               const float* __restrict__ Out, float* __restrict__ G,
                                               float* __restrict__ dQ, HybIndex ix, int L, int nbr, int NB, int nnz,
-                                              float scale) {
+                                              float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
     __shared__ __attribute__((aligned(16))) int lds_x[WAVES][128];
@@ -507,18 +520,22 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const size_t hb = (size_t)bh * L * D;
-    const rsrc_t rK = make_rsrc(K + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
-    const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4), rO = make_rsrc(Out + hb, (size_t)L * D * 4);
+    size_t ib, ob, gb, ibytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rdO = make_rsrc(dO + ob, obytes), rO = make_rsrc(Out + ob, obytes);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     float* T = lds_t[w];
     float* Tx = T + 32 * TS;
     int* X = lds_x[w];
-    const int lin = lin_voff(l, D);
+    const int lin = lin_voff(l, ild), tile_bytes = 32 * ild * 4;
 
     float go[KH], oo[KH];
-    ldr_rows<D>(rdO, (li * D + h * KH) * 4, I * 32 * D * 4, go);
-    ldr_rows<D>(rO, (li * D + h * KH) * 4, I * 32 * D * 4, oo);
+    ldr_rows<D>(rdO, (li * old_ + h * KH) * 4, I * 32 * old_ * 4, go);
+    ldr_rows<D>(rO, (li * old_ + h * KH) * 4, I * 32 * old_ * 4, oo);
     float g = 0.f;
 #pragma unroll
     for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
@@ -541,9 +558,9 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K
             int pos[16];
             unsigned bits[16];
             hyb_tile_rows(X, l, h, x, pos, bits);
-            ldr_tile_lin(rV, lin, x.blk * 32 * D * 4, D, x.a);
+            ldr_tile_lin(rV, lin, x.blk * tile_bytes, ild, x.a);
             hyb_load_p_cols(rP, pos, bits, li, x.p);
-            ldr_tile_lin(rK, lin, x.blk * 32 * D * 4, D, x.b);
+            ldr_tile_lin(rK, lin, x.blk * tile_bytes, ild, x.b);
         },
         [&](HybPre& x, int) {
             float pr[16], vt[KH], kb[1][16];
@@ -560,7 +577,7 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K
             mma_b<D>(ds, kb, acc);
         });
     if constexpr (WAVES > 1) __syncthreads();
-    hyb_reduce_store<WAVES>(acc[0], scale, dQ + hb, nullptr, I * 32, w, li, h, lds);
+    hyb_reduce_store<WAVES>(acc[0], scale, dQ + gb, gld, I * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -570,19 +587,24 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_row_kernel(const float* __restrict__ K
 // kernel leaves the pairs {dS, P} of the remainder alone in one compact list (Pairs [NB][nr], row order, inside the
 // caller's dS scratch), small enough per head for the column pass to find in the L2 cache.
 // -------------------------------------------------------------------------------------------------
+template <bool ST>
 SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K, const float* __restrict__ V,
                                                     const float* __restrict__ P, const float* __restrict__ dO,
                                                     const float* __restrict__ G, float2* __restrict__ Pairs,
                                                     float* __restrict__ dQ, HybIndex ix, int L, int NB, int nnz,
-                                                    float scale) {
+                                                    float scale, Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = ix.r_off[row], rc = ix.r_off[row + 1] - r0;
     if (rc == 0) return;
-    const size_t hb = (size_t)bh * L * 32;
-    const f32x4 go4 = reinterpret_cast<const f32x4*>(dO + hb + (size_t)row * 32)[lane & 7];
+    size_t ib, ob, gb;
+    int ild, old_, gld;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
+    hyb_head<ST>(ly.grad, ly.H, bh, L, gb, gld);
+    const f32x4 go4 = reinterpret_cast<const f32x4*>(dO + ob + (size_t)row * old_)[lane & 7];
     const float* Ph = P + (size_t)bh * nnz;
     float2* pairs = Pairs + (size_t)bh * ix.nr;
     const float gneg = G[(size_t)bh * L + row];
@@ -594,17 +616,17 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K,
         const int pp = k < rc ? ix.r_pos[r0 + k] : 0;
         const float pv = k < rc ? Ph[pp] : 0.f;
         const int nk = min(64, rc - c0);
-        const float dp = hyb_gather_dot(go4, V + hb, col, nk, lane);
+        const float dp = hyb_gather_dot(go4, V + ib, ild, col, nk, lane);
         float dsv = 0.f;
         if (k < rc) {
             dsv = (dp + gneg) * pv * scale;
             pairs[r0 + k] = make_float2(dsv, pv);
         }
-        acc.chunk(dsv, col, nk, K + hb, lane);
+        acc.chunk(dsv, col, nk, K + ib, ild, lane);
     }
     const f32x4 tot = acc.total();
     if (lane < 8) {
-        f32x4* qrow = reinterpret_cast<f32x4*>(dQ + hb + (size_t)row * 32) + lane;
+        f32x4* qrow = reinterpret_cast<f32x4*>(dQ + gb + (size_t)row * gld) + lane;
         *qrow = *qrow + tot;
     }
 }
@@ -613,12 +635,12 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_bwd_row_kernel(const float* __restrict__ K,
 // Backward, column pass, dense tiles: dK_J = sum_I dS_IJ^T Q_I / sqrt(d), dV_J = sum_I P_IJ^T dO_I; dP - g is
 // recomputed per tile by a chain started from the stored -g.
 // -------------------------------------------------------------------------------------------------
-template <int WAVES>
+template <int WAVES, bool ST>
 SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_col_kernel(const float* __restrict__ Q, const float* __restrict__ V,
                                               const float* __restrict__ P, const float* __restrict__ dO,
                                               const float* __restrict__ G, float* __restrict__ dK,
                                               float* __restrict__ dV, HybIndex ix, int L, int nbr, int NB, int nnz,
-                                              float scale) {
+                                              float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][64 * TS];
     __shared__ __attribute__((aligned(16))) int lds_x[WAVES][128];
@@ -626,18 +648,22 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_col_kernel(const float* __restrict__ Q
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, J = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const size_t hb = (size_t)bh * L * D;
-    const rsrc_t rQ = make_rsrc(Q + hb, (size_t)L * D * 4), rV = make_rsrc(V + hb, (size_t)L * D * 4);
-    const rsrc_t rdO = make_rsrc(dO + hb, (size_t)L * D * 4);
+    size_t ib, ob, gb, ibytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rdO = make_rsrc(dO + ob, obytes);
     const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
     const rsrc_t rP = make_rsrc(P + (size_t)bh * nnz, (size_t)nnz * 4);
     float* Tq = lds_t[w];
     float* To = Tq + 32 * TS;
     int* X = lds_x[w];
-    const int lin = lin_voff(l, D);
+    const int lin_i = lin_voff(l, ild), lin_o = lin_voff(l, old_);
 
     float vt[KH];
-    ldr_rows<D>(rV, (li * D + h * KH) * 4, J * 32 * D * 4, vt);
+    ldr_rows<D>(rV, (li * ild + h * KH) * 4, J * 32 * ild * 4, vt);
 
     f32x16 ak[1] = {splat16(0.f)}, av[1] = {splat16(0.f)};
     const int e0 = ix.t_cp[J], ecnt = ix.t_cp[J + 1] - e0;
@@ -654,8 +680,8 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_col_kernel(const float* __restrict__ Q
             int pos[16];
             unsigned bits[16];
             hyb_tile_rows(X, l, h, x, pos, bits);
-            ldr_tile_lin(rQ, lin, x.blk * 32 * D * 4, D, x.a);
-            ldr_tile_lin(rdO, lin, x.blk * 32 * D * 4, D, x.b);
+            ldr_tile_lin(rQ, lin_i, x.blk * 32 * ild * 4, ild, x.a);
+            ldr_tile_lin(rdO, lin_o, x.blk * 32 * old_ * 4, old_, x.b);
             hyb_load_p_cols(rP, pos, bits, li, x.p);  // p[r] = P[query acc_row(r, h)][key li]
             x.g_l = ld1(rG, li * 4, x.blk * 128);
         },
@@ -679,27 +705,32 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_bwd_col_kernel(const float* __restrict__ Q
             mma_b<D>(x.p, ob, av);
         });
     if constexpr (WAVES > 1) __syncthreads();
-    hyb_reduce_store<WAVES>(ak[0], scale, dK + hb, nullptr, J * 32, w, li, h, lds);
+    hyb_reduce_store<WAVES>(ak[0], scale, dK + gb, gld, J * 32, w, li, h, lds);
     if constexpr (WAVES > 1) __syncthreads();
-    hyb_reduce_store<WAVES>(av[0], 1.0f, dV + hb, nullptr, J * 32, w, li, h, lds);
+    hyb_reduce_store<WAVES>(av[0], 1.0f, dV + gb, gld, J * 32, w, li, h, lds);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass, remainder: dK_j += sum_i dS_ij Q_i, dV_j += sum_i P_ij dO_i over the remainder's
 // transposed index, from the compact {dS, P} pairs of the row pass (dS already carries the 1/sqrt(d)).
 // -------------------------------------------------------------------------------------------------
+template <bool ST>
 __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // two gathers in flight per entry: four waves per SIMD
     const float* __restrict__ Q, const float* __restrict__ dO,
                                                     const float2* __restrict__ Pairs,
                                                     float* __restrict__ dK, float* __restrict__ dV, HybIndex ix, int L,
-                                                    int NB) {
+                                                    int NB, Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wcol = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
     if (wcol >= (long long)NB * L) return;
     const int bh = (int)(wcol / L), colj = (int)(wcol % L);
     const int c0p = ix.c_ptr[colj], cnt = ix.c_ptr[colj + 1] - c0p;
     if (cnt == 0) return;
-    const size_t hb = (size_t)bh * L * 32;
+    size_t ib, ob, gb;
+    int ild, old_, gld;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
+    hyb_head<ST>(ly.grad, ly.H, bh, L, gb, gld);
     const float2* pairs = Pairs + (size_t)bh * ix.nr;
     HybRowAcc ak, av;
     ak.clear();
@@ -715,13 +746,13 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
             wv = pr.y;
         }
         const int nk = min(64, cnt - c0);
-        ak.chunk(wk, row, nk, Q + hb, lane);
-        av.chunk(wv, row, nk, dO + hb, lane);
+        ak.chunk(wk, row, nk, Q + ib, ild, lane);
+        av.chunk(wv, row, nk, dO + ob, old_, lane);
     }
     const f32x4 tk = ak.total(), tv = av.total();
     if (lane < 8) {
-        f32x4* kr = reinterpret_cast<f32x4*>(dK + hb + (size_t)colj * 32) + lane;
-        f32x4* vr = reinterpret_cast<f32x4*>(dV + hb + (size_t)colj * 32) + lane;
+        f32x4* kr = reinterpret_cast<f32x4*>(dK + gb + (size_t)colj * gld) + lane;
+        f32x4* vr = reinterpret_cast<f32x4*>(dV + gb + (size_t)colj * gld) + lane;
         *kr = *kr + tk;
         *vr = *vr + tv;
     }

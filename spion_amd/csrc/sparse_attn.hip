@@ -75,7 +75,7 @@ struct GatherDot {
     static constexpr int RS = D + 4;
     static constexpr int FLOATS = 64 * RS;
     static __device__ __forceinline__ float run(float* T, const float* __restrict__ a, const float* __restrict__ X,
-                                                int row_l, int nk, int lane) {
+                                                int ld, int row_l, int nk, int lane) {
         const int grp = lane / LPR, cl = lane % LPR;
         constexpr int UN = 8;
         for (int kb = 0; kb < nk; kb += UN * G) {
@@ -83,7 +83,7 @@ struct GatherDot {
 #pragma unroll
             for (int j = 0; j < UN; ++j) {
                 const int rr = __shfl(row_l, (kb + j * G + grp) & 63, 64);
-                x[j] = reinterpret_cast<const float4*>(X + (size_t)rr * D)[cl];
+                x[j] = reinterpret_cast<const float4*>(X + (size_t)rr * ld)[cl];
             }
 #pragma unroll
             for (int j = 0; j < UN; ++j)
@@ -117,7 +117,8 @@ struct RowAcc {
     static constexpr int G = 64 / LPR;
     vec_t acc;
     __device__ __forceinline__ void clear() { acc = (vec_t)(0.f); }
-    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int lane) {
+    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int ld,
+                                          int lane) {
         const int grp = lane / LPR, cl = lane % LPR;
         // Uniform trip count: every lane takes part in every shuffle.  Slots past nk carry w = 0
         // and row 0 (set by the caller), so they add nothing.
@@ -131,7 +132,7 @@ struct RowAcc {
                 w[j] = __shfl(w_l, kk & 63, 64);
                 const int rr = __shfl(row_l, kk & 63, 64);
                 if (kb + j * G >= 64) w[j] = 0.f;
-                xr[j] = reinterpret_cast<const vec_t*>(X + (size_t)rr * D) + cl;
+                xr[j] = reinterpret_cast<const vec_t*>(X + (size_t)rr * ld) + cl;
             }
             vec_t x[UN];
 #pragma unroll
@@ -152,20 +153,24 @@ struct RowAcc {
     }
 };
 
-// One wavefront per (head, row).  K is row-major here ([NB][L][D], transposed copy in the workspace).
-template <int D, bool MASK>
+// One wavefront per (head, row).  K is row-major here ([NB][L][D], transposed copy in the workspace).  ST: the heads
+// are [B][H][L][D] views located by `ly` (head_slice) instead of contiguous slices.
+template <int D, bool MASK, bool ST>
 __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
-    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
+    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale, Layouts ly) {
     const int lane = threadIdx.x & 63;
     // consecutive rows (which gather overlapping K/V rows and share lines of P) on the same XCD
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * ELEM_WAVES + (threadIdx.x >> 6);
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = offs[row], cnt = offs[row + 1] - r0;
-    const size_t hb = (size_t)bh * L * D;
-    const float* q = Q + hb + (size_t)row * D;
+    size_t ib, ob, bytes;
+    int ild, old_;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, bytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, bytes);
+    const float* q = Q + ib + (size_t)row * ild;
     float* p = P + (size_t)bh * nnz + r0;
     const int* cj = cols + r0;
 
@@ -176,7 +181,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
         for (int c0 = 0; c0 < cnt; c0 += 64) {
             const int k = c0 + lane;
             const int col = k < cnt ? cj[k] : 0;
-            float v = GatherDot<D>::run(T, q, K + hb, col, min(64, cnt - c0), lane) * scale;
+            float v = GatherDot<D>::run(T, q, K + ib, ild, col, min(64, cnt - c0), lane) * scale;
             if (k < cnt) {
                 if (MASK) v -= pen[(size_t)bh * L + col];
                 p[k] = v;
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
     } else {
         for (int k = lane; k < cnt; k += 64) {
             int col = cj[k];
-            float v = row_dot<D>(q, K + hb + (size_t)col * D) * scale;
+            float v = row_dot<D>(q, K + ib + (size_t)col * ild) * scale;
             if (MASK) v -= pen[(size_t)bh * L + col];
             p[k] = v;
             m = fmaxf(m, v);
@@ -210,26 +215,30 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
             col = cj[k];
             p[k] = w;
         }
-        acc.chunk(w, col, min(64, cnt - c0), V + hb, lane);
+        acc.chunk(w, col, min(64, cnt - c0), V + ib, ild, lane);
     }
-    acc.finish(O + hb + (size_t)row * D, lane);
+    acc.finish(O + ob + (size_t)row * old_, lane);
 }
 
 // Row pass of the backward: dP = dO.V^T on the pattern, g = sum_row dP*P, dS = (dP*P - P*g)*scale
 // (written to the caller's dS scratch for the column pass), dQ = dS.K.
-template <int D>
+template <int D, bool ST>
 __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ P,
     const float* __restrict__ dO, float* __restrict__ dS, float* __restrict__ dQ,
-    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale) {
+    const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale, Layouts ly) {
     const int lane = threadIdx.x & 63;
     // consecutive rows (which gather overlapping K/V rows and share lines of P) on the same XCD
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * ELEM_WAVES + (threadIdx.x >> 6);
     if (wrow >= (long long)NB * L) return;
     const int bh = (int)(wrow / L), row = (int)(wrow % L);
     const int r0 = offs[row], cnt = offs[row + 1] - r0;
-    const size_t hb = (size_t)bh * L * D;
-    const float* go = dO + hb + (size_t)row * D;
+    size_t ib, ob, gb, bytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, bytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, bytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, bytes);
+    const float* go = dO + ob + (size_t)row * old_;
     const float* p = P + (size_t)bh * nnz + r0;
     float* ds = dS + (size_t)bh * nnz + r0;
     const int* cj = cols + r0;
@@ -241,7 +250,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
         for (int c0 = 0; c0 < cnt; c0 += 64) {
             const int k = c0 + lane;
             const int col = k < cnt ? cj[k] : 0;
-            const float dp = GatherDot<D>::run(T, go, V + hb, col, min(64, cnt - c0), lane);
+            const float dp = GatherDot<D>::run(T, go, V + ib, ild, col, min(64, cnt - c0), lane);
             if (k < cnt) {
                 const float t = dp * p[k];
                 ds[k] = t;
@@ -250,7 +259,7 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
         }
     } else {
         for (int k = lane; k < cnt; k += 64) {
-            float t = row_dot<D>(go, V + hb + (size_t)cj[k] * D) * p[k];
+            float t = row_dot<D>(go, V + ib + (size_t)cj[k] * ild) * p[k];
             ds[k] = t;
             g += t;
         }
@@ -268,18 +277,18 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
             col = cj[k];
             ds[k] = w;
         }
-        acc.chunk(w, col, min(64, cnt - c0), K + hb, lane);
+        acc.chunk(w, col, min(64, cnt - c0), K + ib, ild, lane);
     }
-    acc.finish(dQ + hb + (size_t)row * D, lane);
+    acc.finish(dQ + gb + (size_t)row * gld, lane);
 }
 
 // Column pass of the backward: dK_j = sum_i dS_ij Q_i, dV_j = sum_i P_ij dO_i over the transposed index.
-template <int D>
+template <int D, bool ST>
 __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ dO, const float* __restrict__ P,
     const float* __restrict__ dS, float* __restrict__ dK, float* __restrict__ dV,
     const int* __restrict__ colptr, const int* __restrict__ crow, const int* __restrict__ cpos, int L, int NB,
-    int nnz) {
+    int nnz, Layouts ly) {
     const int lane = threadIdx.x & 63;
     // consecutive columns on the same XCD: the 32 columns whose entries in a row share a 128-byte line of P and
     // dS then share it in one L2 instead of fetching it into eight
@@ -287,7 +296,11 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
     if (wcol >= (long long)NB * L) return;
     const int bh = (int)(wcol / L), col = (int)(wcol % L);
     const int c0p = colptr[col], cnt = colptr[col + 1] - c0p;
-    const size_t hb = (size_t)bh * L * D;
+    size_t ib, ob, gb, bytes;
+    int ild, old_, gld;
+    head_slice<ST, D>(ly.in, ly.H, bh, L, ib, ild, bytes);
+    head_slice<ST, D>(ly.out, ly.H, bh, L, ob, old_, bytes);
+    head_slice<ST, D>(ly.grad, ly.H, bh, L, gb, gld, bytes);
     const float* p = P + (size_t)bh * nnz;
     const float* ds = dS + (size_t)bh * nnz;
 
@@ -305,11 +318,11 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
             wv = p[pos];
         }
         const int nk = min(64, cnt - c0);
-        ak.chunk(wk, row, nk, Q + hb, lane);
-        av.chunk(wv, row, nk, dO + hb, lane);
+        ak.chunk(wk, row, nk, Q + ib, ild, lane);
+        av.chunk(wv, row, nk, dO + ob, old_, lane);
     }
-    ak.finish(dK + hb + (size_t)col * D, lane);
-    av.finish(dV + hb + (size_t)col * D, lane);
+    ak.finish(dK + gb + (size_t)col * gld, lane);
+    av.finish(dV + gb + (size_t)col * gld, lane);
 }
 
 // =================================================================================================
@@ -380,6 +393,8 @@ struct SparseAttn {
     bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
     float* ws_stats = nullptr;   // [NB][L][2] softmax row statistics handed between the hybrid forward's launches
+    float* ws_ds = nullptr;      // [NB][nnz] dS scratch of the strided backward on patterns without tile structure
+    size_t ws_ds_count = 0;
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
     size_t ws_part_floats = 0;
     int last_path = 0;
@@ -438,6 +453,7 @@ void sparse_destroy(void* h) {
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
     if (a->ws_stats) (void)hipFree(a->ws_stats);
+    if (a->ws_ds) (void)hipFree(a->ws_ds);
     if (a->ws_part) (void)hipFree(a->ws_part);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
@@ -1025,37 +1041,112 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 #undef SPION_LAUNCH
 }
 
+// Hybrid patterns (dense tiles + remainder, d = 32).  Every operand row-major; ST: heads located by `ly`.
+// ocopy (contiguous heads only): where a second copy of O goes, or null.
+template <bool ST>
+static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const float* V, const float* Mask,
+                           float* Attn, float* Out, float* ocopy, const int* Offsets, int nnz, const Layouts& ly) {
+    if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
+    a->last_path = 3;
+    const int nbr = a->L / 32;
+    const long long rows = (long long)a->NB * a->L;
+    // strips of few dense tiles: one wavefront walks the whole strip; else four share it
+    const bool one = a->pat.max_row_tiles <= HYB_MAXT1;
+    const dim3 grid_t(nbr * a->NB), block_t(one ? 64 : 256);
+    const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
+    float2* stats = reinterpret_cast<float2*>(a->ws_stats);
+#define SPION_HYB_FWD(MASKED)                                                                                        \
+    do {                                                                                                             \
+        hipLaunchKernelGGL((hyb_rem_logits_kernel<MASKED, ST>), grid_g, block_g, 0, a->hdr.stream, Q, K, Mask, Attn, \
+                           stats, a->pat.hyb, a->L, a->NB, nnz, a->scale, ly);                                       \
+        if (one)                                                                                                     \
+            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 1, HYB_MAXT1, ST>), grid_t, block_t, 0, a->hdr.stream,   \
+                               Q, K, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz,          \
+                               a->scale, ly);                                                                        \
+        else                                                                                                         \
+            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 4, HYB_MAXT4, ST>), grid_t, block_t, 0, a->hdr.stream,   \
+                               Q, K, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz,          \
+                               a->scale, ly);                                                                        \
+    } while (0)
+    if (a->has_mask)
+        SPION_HYB_FWD(true);
+    else
+        SPION_HYB_FWD(false);
+#undef SPION_HYB_FWD
+    hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, Attn, Out, ocopy,
+                       (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
+    check_launch("hybrid forward kernels");
+}
+
+// o: the forward's output (same layout as dO).  dS: the caller's [NB][nnz] scratch, which receives the remainder's
+// {dS, P} pairs, [NB][nr] (a hybrid pattern keeps at most half of its entries in the remainder).
+template <bool ST>
+static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const float* V, const float* P,
+                           const float* dO, const float* o, float* dS, float* dQ, float* dK, float* dV, int nnz,
+                           const Layouts& ly) {
+    if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+    a->last_path = 3;
+    const int nbr = a->L / 32;
+    const long long rows = (long long)a->NB * a->L;
+    const bool one_r = a->pat.max_row_tiles <= 2 * HYB_MAXT1, one_c = a->pat.max_col_tiles <= 2 * HYB_MAXT1;
+    const dim3 grid_t(nbr * a->NB);
+    const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
+    float2* pairs = reinterpret_cast<float2*>(dS);
+    if (a->bwd_passes & 1) {
+        if (one_r)
+            hipLaunchKernelGGL((hyb_tile_bwd_row_kernel<1, ST>), grid_t, dim3(64), 0, a->hdr.stream, K, V, P, dO, o,
+                               a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
+        else
+            hipLaunchKernelGGL((hyb_tile_bwd_row_kernel<4, ST>), grid_t, dim3(256), 0, a->hdr.stream, K, V, P, dO, o,
+                               a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
+        hipLaunchKernelGGL(hyb_rem_bwd_row_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, K, V, P, dO,
+                           (const float*)a->ws_rowsum, pairs, dQ, a->pat.hyb, a->L, a->NB, nnz, a->scale, ly);
+    }
+    if (a->bwd_passes & 2) {
+        if (one_c)
+            hipLaunchKernelGGL((hyb_tile_bwd_col_kernel<1, ST>), grid_t, dim3(64), 0, a->hdr.stream, Q, V, P, dO,
+                               (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
+        else
+            hipLaunchKernelGGL((hyb_tile_bwd_col_kernel<4, ST>), grid_t, dim3(256), 0, a->hdr.stream, Q, V, P, dO,
+                               (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
+        hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO, (const float2*)pairs,
+                           dK, dV, a->pat.hyb, a->L, a->NB, ly);
+    }
+    check_launch("hyb_bwd kernels");
+}
+
 static void launch_transpose(SparseAttn* a, const float* Xt, float* X) {
     dim3 grid((a->L + 31) / 32, (a->d + 31) / 32, a->NB);
     hipLaunchKernelGGL(transpose_dl_kernel, grid, dim3(256), 0, a->hdr.stream, Xt, X, a->d, a->L);
 }
 
-template <int D>
+template <int D, bool ST = false>
 static void launch_elem_fwd(SparseAttn* a, const float* Q, const float* Krm, const float* V, const float* pen,
-                            float* P, float* O, const int* offs, const int* cols, int nnz) {
+                            float* P, float* O, const int* offs, const int* cols, int nnz,
+                            const Layouts& ly = Layouts{}) {
     const long long rows = (long long)a->NB * a->L;
     dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
     if (a->has_mask)
-        hipLaunchKernelGGL((elem_fwd_kernel<D, true>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V, pen,
-                           P, O, offs, cols, a->L, a->NB, nnz, a->scale);
+        hipLaunchKernelGGL((elem_fwd_kernel<D, true, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V,
+                           pen, P, O, offs, cols, a->L, a->NB, nnz, a->scale, ly);
     else
-        hipLaunchKernelGGL((elem_fwd_kernel<D, false>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V, pen,
-                           P, O, offs, cols, a->L, a->NB, nnz, a->scale);
+        hipLaunchKernelGGL((elem_fwd_kernel<D, false, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, Krm, V,
+                           pen, P, O, offs, cols, a->L, a->NB, nnz, a->scale, ly);
 }
 
-template <int D>
+template <int D, bool ST = false>
 static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vrm, const float* P,
                             const float* dO, float* dS, float* dQ, float* dK, float* dV, const int* offs,
-                            const int* cols, int nnz) {
+                            const int* cols, int nnz, const Layouts& ly = Layouts{}) {
     const PatternIndex& pi = a->pat;
     const long long rows = (long long)a->NB * a->L;
     dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
     if (a->bwd_passes & 1)
-        hipLaunchKernelGGL((elem_bwd_row_kernel<D>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, K, Vrm, P, dO, dS,
-                           dQ, offs, cols, a->L, a->NB, nnz, a->scale);
+        hipLaunchKernelGGL((elem_bwd_row_kernel<D, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, K, Vrm, P, dO,
+                           dS, dQ, offs, cols, a->L, a->NB, nnz, a->scale, ly);
     if (a->bwd_passes & 2)
-        hipLaunchKernelGGL((elem_bwd_col_kernel<D>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, dO, P, dS, dK,
-                           dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz);
+        hipLaunchKernelGGL((elem_bwd_col_kernel<D, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, dO, P, dS,
+                           dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz, ly);
 }
 
 // krow: Kt is K itself, row-major [NB][L][d], not the transposed copy of the reference's ABI.
@@ -1104,34 +1195,7 @@ void sparse_forward(void* h, const float* Q, const float* Kt, const float* V, co
         Krm = a->ws_trans;
     }
     if (a->pat.hybrid) {
-        if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
-        a->last_path = 3;
-        const int nbr = a->L / 32;
-        const long long rows = (long long)a->NB * a->L;
-        // strips of few dense tiles: one wavefront walks the whole strip; else four share it
-        const bool one = a->pat.max_row_tiles <= HYB_MAXT1;
-        const dim3 grid_t(nbr * a->NB), block_t(one ? 64 : 256);
-        const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
-        float2* stats = reinterpret_cast<float2*>(a->ws_stats);
-#define SPION_HYB_FWD(MASKED)                                                                                         \
-    do {                                                                                                              \
-        hipLaunchKernelGGL(hyb_rem_logits_kernel<MASKED>, grid_g, block_g, 0, a->hdr.stream, Q, Krm, Mask, Attn,      \
-                           stats, a->pat.hyb, a->L, a->NB, nnz, a->scale);                                            \
-        if (one)                                                                                                      \
-            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 1, HYB_MAXT1>), grid_t, block_t, 0, a->hdr.stream, Q,     \
-                               Krm, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale); \
-        else                                                                                                          \
-            hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 4, HYB_MAXT4>), grid_t, block_t, 0, a->hdr.stream, Q,     \
-                               Krm, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale); \
-    } while (0)
-        if (a->has_mask)
-            SPION_HYB_FWD(true);
-        else
-            SPION_HYB_FWD(false);
-#undef SPION_HYB_FWD
-        hipLaunchKernelGGL(hyb_rem_pv_kernel, grid_g, block_g, 0, a->hdr.stream, V, Attn, Out, hyb_ocopy,
-                           (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz);
-        check_launch("hybrid forward kernels");
+        launch_hyb_fwd<false>(a, Q, Krm, V, Mask, Attn, Out, hyb_ocopy, Offsets, nnz, Layouts{});
         return;
     }
     switch (a->d) {
@@ -1193,39 +1257,7 @@ void sparse_backward(void* h, const float* Q, const float* K, const float* Vt, c
         // without it the gather kernels below serve the same P
         const float* o = Out ? Out : ocache_for_backward(a, P);
         if (o) {
-            if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
-            a->last_path = 3;
-            const int nbr = a->L / 32;
-            const long long rows = (long long)a->NB * a->L;
-            const bool one_r = a->pat.max_row_tiles <= 2 * HYB_MAXT1, one_c = a->pat.max_col_tiles <= 2 * HYB_MAXT1;
-            const dim3 grid_t(nbr * a->NB);
-            const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
-            // the remainder's {dS, P} pairs, [NB][nr] inside the caller's dS scratch (NB*nnz floats:
-            // a hybrid pattern keeps at most half of its entries in the remainder)
-            float2* pairs = reinterpret_cast<float2*>(dS);
-            if (a->bwd_passes & 1) {
-                if (one_r)
-                    hipLaunchKernelGGL(hyb_tile_bwd_row_kernel<1>, grid_t, dim3(64), 0, a->hdr.stream, K, Vrm, P, dO, o,
-                                       a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
-                else
-                    hipLaunchKernelGGL(hyb_tile_bwd_row_kernel<4>, grid_t, dim3(256), 0, a->hdr.stream, K, Vrm, P, dO,
-                                       o, a->ws_rowsum, dQ, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale);
-                hipLaunchKernelGGL(hyb_rem_bwd_row_kernel, grid_g, block_g, 0, a->hdr.stream, K, Vrm, P, dO,
-                                   (const float*)a->ws_rowsum, pairs, dQ, a->pat.hyb, a->L, a->NB, nnz, a->scale);
-            }
-            if (a->bwd_passes & 2) {
-                if (one_c)
-                    hipLaunchKernelGGL(hyb_tile_bwd_col_kernel<1>, grid_t, dim3(64), 0, a->hdr.stream, Q, Vrm, P, dO,
-                                       (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz,
-                                       a->scale);
-                else
-                    hipLaunchKernelGGL(hyb_tile_bwd_col_kernel<4>, grid_t, dim3(256), 0, a->hdr.stream, Q, Vrm, P, dO,
-                                       (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz,
-                                       a->scale);
-                hipLaunchKernelGGL(hyb_rem_bwd_col_kernel, grid_g, block_g, 0, a->hdr.stream, Q, dO,
-                                   (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB);
-            }
-            check_launch("hyb_bwd kernels");
+            launch_hyb_bwd<false>(a, Q, K, Vrm, P, dO, o, dS, dQ, dK, dV, nnz, Layouts{});
             return;
         }
     }
@@ -1360,9 +1392,8 @@ static SparseAttn* strided_handle(void* h, const char* who, const int* Offsets, 
         return nullptr;
     }
     if (!ensure_pattern(a, Offsets, Columns, nnz)) return nullptr;
-    if (!a->pat.tiled || !tile_supported(a->d)) {
-        set_error("%s: strided heads are read in place only by the tile kernels (emb_dim 32 or 64, pattern of aligned "
-                  "32x32 tiles); make the operands contiguous and use the row-major entry points", who);
+    if (a->pat.tiled && !tile_supported(a->d)) {  // cannot happen: tile patterns are only recognised for 32 and 64
+        set_error("%s: emb_dim %d has no tile kernels", who, a->d);
         return nullptr;
     }
     return a;
@@ -1396,6 +1427,22 @@ void sparse_forward_strided(void* h, const float* Q, const float* K, const float
     ly.out = out;
     ly.grad = out;
     ly.H = heads;
+    if (!a->pat.tiled) {
+        ocache_drop(a, Attn);  // the backward of these entry points is handed Out
+        if (a->pat.hybrid) {
+            launch_hyb_fwd<true>(a, Q, K, V, Mask, Attn, Out, nullptr, Offsets, nnz, ly);
+            return;
+        }
+        a->last_path = 2;
+        switch (a->d) {
+            case 16: launch_elem_fwd<16, true>(a, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, ly); break;
+            case 32: launch_elem_fwd<32, true>(a, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, ly); break;
+            case 64: launch_elem_fwd<64, true>(a, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, ly); break;
+            default: launch_elem_fwd<128, true>(a, Q, K, V, Mask, Attn, Out, Offsets, Columns, nnz, ly); break;
+        }
+        check_launch("elem_fwd_kernel");
+        return;
+    }
     a->last_path = 1;
     if (a->d == 32) {
         if (a->has_mask) launch_tile_fwd<32, true, true, true>(a, Q, K, V, Mask, Attn, Out, Offsets, nnz, ly);
@@ -1435,6 +1482,36 @@ void sparse_backward_strided(void* h, const float* Q, const float* K, const floa
     ly.out = out;
     ly.grad = grad;
     ly.H = heads;
+    if (!a->pat.tiled) {
+        // these entry points have no dS argument: the scratch is the handle's (grown outside graph capture only)
+        const size_t need = (size_t)a->NB * (size_t)std::max(nnz, 1);
+        if (a->ws_ds_count < need) {
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+            if (cap != hipStreamCaptureStatusNone) {
+                set_error("%s: the scratch for this pattern is not allocated yet; run one step outside the capture", who);
+                return;
+            }
+            if (a->ws_ds) (void)hipFree(a->ws_ds);
+            a->ws_ds = nullptr;
+            a->ws_ds_count = 0;
+            if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_ds, sizeof(float) * need))) return;
+            a->ws_ds_count = need;
+        }
+        if (a->pat.hybrid) {
+            launch_hyb_bwd<true>(a, Q, K, V, P, dO, Out, a->ws_ds, dQ, dK, dV, nnz, ly);
+            return;
+        }
+        a->last_path = 2;
+        switch (a->d) {
+            case 16: launch_elem_bwd<16, true>(a, Q, K, V, P, dO, a->ws_ds, dQ, dK, dV, Offsets, Columns, nnz, ly); break;
+            case 32: launch_elem_bwd<32, true>(a, Q, K, V, P, dO, a->ws_ds, dQ, dK, dV, Offsets, Columns, nnz, ly); break;
+            case 64: launch_elem_bwd<64, true>(a, Q, K, V, P, dO, a->ws_ds, dQ, dK, dV, Offsets, Columns, nnz, ly); break;
+            default: launch_elem_bwd<128, true>(a, Q, K, V, P, dO, a->ws_ds, dQ, dK, dV, Offsets, Columns, nnz, ly); break;
+        }
+        check_launch("elem_bwd kernels");
+        return;
+    }
     a->last_path = 1;
     if (a->d == 32) launch_tile_bwd<32, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);
     else launch_tile_bwd<64, true, true>(a, Q, K, V, P, dO, dQ, dK, dV, Offsets, nnz, Out, ly);

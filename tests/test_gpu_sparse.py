@@ -603,6 +603,59 @@ def test_strided_entry_points(layout, kind, with_mask, d):
     abi.close()
 
 
+@pytest.mark.parametrize("kind,d,layout,with_mask", [("hybrid", 32, "proj", False), ("hybrid", 32, "fused", True),
+                                                     ("hybrid4", 32, "proj", False),
+                                                     ("element", 16, "proj", False), ("element", 32, "fused", True),
+                                                     ("element", 64, "proj", False), ("element", 128, "fused", False)])
+def test_strided_entry_points_on_element_sparse_patterns(kind, d, layout, with_mask):
+    """The strided entry points on patterns that are not made of 32x32 tiles: the hybrid kernels (window + random
+    entries; "hybrid4": strips of more than six dense tiles, four wavefronts per strip) and the element kernels
+    (any head size) read the heads in place too.  Bit-identical to the row-major entry points on contiguous
+    copies, both against the oracle."""
+    B, H = 2, 2
+    NB = B * H
+    if kind == "hybrid":
+        L = 512
+        sm, off, col = workloads.window_random_csr(L, 48, 150, seed=9)
+    elif kind == "hybrid4":
+        L = 512
+        sm, off, col = workloads.window_random_csr(L, 150, 330, seed=4)
+    else:
+        L = 256
+        sm, off, col = workloads.window_random_csr(L, 2, 23, seed=5)
+    abi = SparseABI(d, L, NB, 1, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    _, (q, k, v) = _head_views(B, H, L, d, layout, 3, seed=51)
+    _, (dout,) = _head_views(B, H, L, d, "proj", 1, seed=52)
+    _, (out,) = _head_views(B, H, L, d, "proj", 1, seed=0, fill=float("nan"))
+    gbufs, (dq, dk, dv) = _head_views(B, H, L, d, layout, 3, seed=0, fill=-7.0)
+    pen = None
+    if with_mask:
+        valid = torch.tensor([L, L - 40, L // 2, L - 1][:NB])
+        pen = (1e6 * (torch.arange(L)[None, :] >= valid[:, None]).float()).contiguous().cuda()
+    P = abi.forward_strided(q, k, v, out, pen)
+    path = abi.last_path()
+    abi.backward_strided(q, k, v, P, out, dout, dq, dk, dv)
+    torch.cuda.synchronize()
+    assert path == abi.last_path() == (2 if kind == "element" else 3)
+    flat = lambda t: t.reshape(NB, L, d).contiguous()
+    Qc, Kc, Vc, dOc = flat(q), flat(k), flat(v), flat(dout)
+    O2, P2 = abi.forward_rowmajor(Qc, Kc, Vc, pen)
+    g2 = abi.backward_rowmajor(Qc, Kc, Vc, P2, O2, dOc)
+    torch.cuda.synchronize()
+    assert torch.equal(P, P2) and torch.equal(flat(out), O2)
+    for name, a, b in zip(("dQ", "dK", "dV"), (dq, dk, dv), g2):
+        assert torch.equal(flat(a), b), name
+    if layout == "fused":
+        assert (gbufs[0][..., d:] == -7.0).all(), "padding between the heads' rows was written"
+    ref = oracle_fwd_bwd(Qc, Kc, Vc, dOc, sm, off, col, pen)
+    assert_close(P.cpu().numpy(), ref["P"], what=f"strided {kind} P")
+    assert_close(flat(out).cpu().numpy(), ref["O"], what=f"strided {kind} O")
+    for name, a in zip(("dQ", "dK", "dV"), (dq, dk, dv)):
+        assert_close(flat(a).cpu().numpy(), ref[name], what=f"strided {kind} {name}")
+    abi.close()
+
+
 def test_strided_entry_points_refuse_what_they_cannot_serve():
     import ctypes
     from spion_amd import _lib
@@ -619,13 +672,6 @@ def test_strided_entry_points_refuse_what_they_cannot_serve():
             abi.offsets.data_ptr(), abi.columns.data_ptr(), abi.sum_mat.data_ptr(), abi.nnz, heads,
             ctypes.addressof(lin), ctypes.addressof(lout))
 
-    abi64 = SparseABI(64, L, B * H, bs, with_mask=False)   # d = 64 is served, but not on an element-sparse pattern
-    abi64.set_pattern(sm - (np.arange(L) == 0), off - (np.arange(L + 1) > 0), col[1:])
-    q64 = torch.zeros(B, H, L, 64, device="cuda")
-    call(abi64, q64, torch.zeros_like(q64))
-    with pytest.raises(RuntimeError, match="aligned"):
-        _lib.check_error("element pattern")
-    abi64.close()
     abi = SparseABI(32, L, B * H, bs, with_mask=False)
     abi.set_pattern(sm, off, col)
     q = torch.zeros(B, H, L, 32, device="cuda")
