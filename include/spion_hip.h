@@ -321,6 +321,21 @@ void spion_attn_backward_strided(void* handle, const float* Q, const float* K, c
                                  int heads, const spion_head_layout* in, const spion_head_layout* out,
                                  const spion_head_layout* grad);
 
+/* The bf16 family on the same kind of views (no counterpart in the reference; models/attention.py:136-139 is where
+ * its fp32 layer makes them): Q, K, V / Out, dO / dQ, dK, dV as [B][H][L][d] views located by one layout per group,
+ * strides in bf16 elements and multiples of 8, pointers 16-byte aligned; Lse and Mask stay [NB][L].  Same kernels
+ * and arithmetic as the contiguous entry points: bit-identical results. */
+void spion_block_bf16_attn_forward_strided(void* handle, const void* Q, const void* K, const void* V, const float* Mask,
+                                           void* Out, float* Lse,
+                                           const int* Offsets, const int* Columns, const int* SumMat, int nnz,
+                                           int heads, const spion_head_layout* in, const spion_head_layout* out);
+void spion_block_bf16_attn_backward_strided(void* handle, const void* Q, const void* K, const void* V, const float* Mask,
+                                            const void* Out, const float* Lse, const void* dO,
+                                            void* dQ, void* dK, void* dV,
+                                            const int* Offsets, const int* Columns, const int* SumMat, int nnz,
+                                            int heads, const spion_head_layout* in, const spion_head_layout* out,
+                                            const spion_head_layout* grad);
+
 /* The dense phase on the same views: the reference's dense modules transpose Q and V before the forward and K
  * and grad_output before the backward (models/attention_cuda.py:22-31,52-62) because its GEMM calls
  * (models/attn.cu:179-262) take feature-major operands, and hand Out and the gradients back feature-major.

@@ -121,6 +121,10 @@ def core() -> ctypes.CDLL:
     lib.spion_block_bf16_attn_forward.restype = None
     lib.spion_block_bf16_attn_backward.argtypes = [_P] * 14 + [c_int]
     lib.spion_block_bf16_attn_backward.restype = None
+    lib.spion_block_bf16_attn_forward_strided.argtypes = [_P] * 10 + [c_int, c_int, _P, _P]
+    lib.spion_block_bf16_attn_forward_strided.restype = None
+    lib.spion_block_bf16_attn_backward_strided.argtypes = [_P] * 14 + [c_int, c_int, _P, _P, _P]
+    lib.spion_block_bf16_attn_backward_strided.restype = None
     lib.spion_block_bf16_destroy.argtypes = [_P]
     lib.spion_block_bf16_destroy.restype = None
     for fam, extra in (("dense", 0), ("densemask", 1)):
@@ -160,11 +164,12 @@ class HeadLayout(ctypes.Structure):
 
 def head_layout(t: "torch.Tensor") -> HeadLayout | None:
     """Layout of a 4-D [B, H, L, d] tensor or view for the strided entry points; None when they cannot take it
-    (last dimension not unit-stride, strides not multiples of 4 floats, storage offset not 16-byte aligned)."""
+    (last dimension not unit-stride, strides not multiples of 16 bytes, storage offset not 16-byte aligned)."""
     sb, sh, sl, sf = t.stride()
     if t.dim() != 4 or sf != 1 or t.data_ptr() % 16:
         return None
-    if sb % 4 or sh % 4 or sl % 4 or sl < t.shape[3] or min(sb, sh) < 0:
+    unit = 16 // t.element_size()  # strides in elements, 16-byte granularity: 4 floats, 8 bf16
+    if sb % unit or sh % unit or sl % unit or sl < t.shape[3] or min(sb, sh) < 0:
         return None
     if t.shape[2] * sl >= 1 << 29:
         return None

@@ -55,10 +55,29 @@ __device__ __forceinline__ void ldb_rows(rsrc_t r, int voff, int soff, bf16x8 (&
 // the 64 lanes read 1 KB of consecutive addresses: 8 cache lines per instruction.  (Reading it directly in the
 // operand layout -- every lane 16 bytes of its own row -- costs one tag lookup per lane and was measured to
 // keep the texture path busy 84 % of the time.)  Lane l, instruction i holds 16-byte piece 64i + l of the tile.
+// With rows ld elements apart (a head that is a view of a wider buffer) the same pieces come from 512 / D rows per
+// instruction: lane offset bf16_tile_voff, `step` = bf16_tile_step bytes from one instruction to the next.
 template <int D>
-__device__ __forceinline__ void ldb_tile(rsrc_t r, int l16, int soff, u32x4 (&raw)[D / 16]) {
+__device__ __forceinline__ void ldb_tile(rsrc_t r, int lvoff, int soff, int step, u32x4 (&raw)[D / 16]) {
 #pragma unroll
-    for (int i = 0; i < D / 16; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(r, l16, soff + 1024 * i, 0);
+    for (int i = 0; i < D / 16; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lvoff, soff + step * i, 0);
+}
+template <int D>
+__device__ __forceinline__ int bf16_tile_voff(int l, int ld) {
+    constexpr int PPR = D / 8;  // 16-byte pieces per row
+    return ((l / PPR) * ld + (l % PPR) * 8) * 2;
+}
+template <int D>
+__device__ __forceinline__ int bf16_tile_step(int ld) {
+    return (512 / D) * ld * 2;
+}
+// Start (in elements), row stride and size in bytes of head bh: contiguous [NB][L][D] heads (ST = false, compile-time
+// figures) or [B][H][L][D] views given by a layout (strides in elements).
+template <bool ST, int D>
+__device__ __forceinline__ void bf16_head(const HeadLayout& y, int H, int bh, int L, size_t& base, int& ld,
+                                          size_t& bytes) {
+    head_slice<ST, D>(y, H, bh, L, base, ld, bytes);
+    bytes >>= 1;  // head_slice counts four bytes an element
 }
 
 template <int D>
@@ -155,8 +174,8 @@ __device__ __forceinline__ float half_swap_sum(float x) {
 // part (chunk of a long strip only): the work-group's sum goes there as fp32, register (c, r) of lane l at
 // [(16c + r)*64 + l], instead of to the tensor.
 template <int D>
-__device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO, int row0, bool coop, int w, int li, int h,
-                                                float* lds, float* part = nullptr) {
+__device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO, int ld, int row0, bool coop, int w,
+                                                int li, int h, float* lds, float* part = nullptr) {
     const int l = li + 32 * h;
     if (coop) {
         __syncthreads();  // lds is the memory of the wave-private tiles: every wavefront is done with them
@@ -182,7 +201,7 @@ __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO
             return;
         }
     }
-    const int voff = (li * D + 4 * h) * 2;
+    const int voff = (li * ld + 4 * h) * 2;
 #pragma unroll
     for (int c = 0; c < D / 32; ++c)
 #pragma unroll
@@ -190,7 +209,7 @@ __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO
             bf16x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = (__bf16)acc[c][4 * g + e];
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rO, voff, row0 * D * 2 + (32 * c + 8 * g) * 2, 0);
+            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rO, voff, row0 * ld * 2 + (32 * c + 8 * g) * 2, 0);
         }
 }
 
@@ -219,12 +238,12 @@ constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
 // -------------------------------------------------------------------------------------------------
 // Forward: one sweep per block row with a lazily raised running maximum.
 // -------------------------------------------------------------------------------------------------
-template <int D, bool MASK>
+template <int D, bool MASK, bool ST>
 SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk) {
+    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     __shared__ float lds_m[BF16_WAVES][32], lds_z[BF16_WAVES][32];
@@ -240,18 +259,22 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
     const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
     float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
-    const rsrc_t rO = make_rsrc(O + hb, hbytes);
+    size_t ib, ob, ibytes, obytes;
+    int ild, old_;
+    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rO = make_rsrc(O + ob, obytes);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int r_voff = li * D * 2 + h * D;
+    const int r_voff = li * ild * 2 + h * D;
+    const int t_voff = bf16_tile_voff<D>(l, ild), t_step = bf16_tile_step<D>(ild), t_bytes = 32 * ild * 2;
     char* Tk = lds_t[w][0];
     char* Tv = lds_t[w][1];
     const int tbase = LT::lane_base(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
     bf16x8 q[D / 16];
-    ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, q);
+    ldb_rows<D>(rQ, r_voff, I * t_bytes, q);
 
     // Floor of the running maximum (the reference's max(-100, .) / max(0, .), models/block_attn.cu:52): any
     // value gives the same probabilities; 2^-100 keeps (L - n) * 2^-m finite in fp32 for empty rows.
@@ -269,8 +292,8 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_tile<D>(rK, l * 16, J * 32 * D * 2, x.k);
-            ldb_tile<D>(rV, l * 16, J * 32 * D * 2, x.v);
+            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
+            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
             if constexpr (MASK) {
                 float pj[16];
                 ldr_4x4(rM, 16 * h, J * 128, pj);
@@ -336,7 +359,7 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
             part[2 * 32 * D + li] = m;
             part[2 * 32 * D + 32 + li] = z;
         }
-        store_rows_bf16<D>(o, rO, I * 32, true, w, li, h, lds_o, part);
+        store_rows_bf16<D>(o, rO, old_, I * 32, true, w, li, h, lds_o, part);
         return;
     }
     const int off_pattern = L - cnt_all * 32;
@@ -345,20 +368,20 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
 #pragma unroll
     for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
     if (sa.rank == 0 && h == 0) Lse[(size_t)bh * L + I * 32 + li] = m + __builtin_amdgcn_logf(z);
-    store_rows_bf16<D>(o, rO, I * 32, sa.coop, w, li, h, lds_o);
+    store_rows_bf16<D>(o, rO, old_, I * 32, sa.coop, w, li, h, lds_o);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, row pass: g_i = dO_i . O_i, P and dP recomputed per tile, dS' = P*(dP - g), dQ += dS'.K_J;
 // the 1/sqrt(d) is applied to the 32 x d result.  Gneg receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------
-template <int D, bool MASK>
+template <int D, bool MASK, bool ST>
 SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
     const float* __restrict__ pen, float* __restrict__ Gneg, __bf16* __restrict__ dQ, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk) {
+    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
@@ -373,23 +396,28 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
     const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
     float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
-    const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rO = make_rsrc(O + hb, hbytes), rdQ = make_rsrc(dQ + hb, hbytes);
+    size_t ib, ob, gb, ibytes, obytes, gbytes;
+    int ild, old_, gld;
+    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rdO = make_rsrc(dO + ob, obytes), rO = make_rsrc(O + ob, obytes), rdQ = make_rsrc(dQ + gb, gbytes);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int r_voff = li * D * 2 + h * D;
+    const int r_voff = li * ild * 2 + h * D, ro_voff = li * old_ * 2 + h * D;
+    const int t_voff = bf16_tile_voff<D>(l, ild), t_step = bf16_tile_step<D>(ild), t_bytes = 32 * ild * 2;
     char* Tk = lds_t[w][0];
     char* Tv = lds_t[w][1];
     const int tbase = LT::lane_base(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
     bf16x8 q[D / 16], go[D / 16];
-    ldb_rows<D>(rQ, r_voff, I * 32 * D * 2, q);
-    ldb_rows<D>(rdO, r_voff, I * 32 * D * 2, go);
+    ldb_rows<D>(rQ, r_voff, I * t_bytes, q);
+    ldb_rows<D>(rdO, ro_voff, I * 32 * old_ * 2, go);
     float g = 0.f;
     {
         bf16x8 oo[D / 16];
-        ldb_rows<D>(rO, r_voff, I * 32 * D * 2, oo);
+        ldb_rows<D>(rO, ro_voff, I * 32 * old_ * 2, oo);
 #pragma unroll
         for (int t = 0; t < D / 16; ++t)
 #pragma unroll
@@ -412,8 +440,8 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_tile<D>(rK, l * 16, J * 32 * D * 2, x.k);
-            ldb_tile<D>(rV, l * 16, J * 32 * D * 2, x.v);
+            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
+            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
             if constexpr (MASK) {
                 float pj[16];
                 ldr_4x4(rM, 16 * h, J * 128, pj);
@@ -445,19 +473,19 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
         });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
-    store_rows_bf16<D>(acc, rdQ, I * 32, sa.coop, w, li, h, lds_o, part);
+    store_rows_bf16<D>(acc, rdQ, gld, I * 32, sa.coop, w, li, h, lds_o, part);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
 // -------------------------------------------------------------------------------------------------
-template <int D, bool MASK>
+template <int D, bool MASK, bool ST>
 SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const float* __restrict__ Lse, const float* __restrict__ Gneg,
     const float* __restrict__ pen, __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcp,
     const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk) {
+    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
     typedef LdsTile<D> LT;
     __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
     float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
@@ -472,19 +500,25 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
     const int e0 = tcp[J] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
     const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
     float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
-    const rsrc_t rdO = make_rsrc(dO + hb, hbytes), rdK = make_rsrc(dK + hb, hbytes), rdV = make_rsrc(dV + hb, hbytes);
+    size_t ib, ob, gb, ibytes, obytes, gbytes;
+    int ild, old_, gld;
+    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
+    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rdO = make_rsrc(dO + ob, obytes), rdK = make_rsrc(dK + gb, gbytes), rdV = make_rsrc(dV + gb, gbytes);
     const rsrc_t rL = make_rsrc(Lse + (size_t)bh * L, (size_t)L * 4), rG = make_rsrc(Gneg + (size_t)bh * L, (size_t)L * 4);
-    const int r_voff = li * D * 2 + h * D;
+    const int r_voff = li * ild * 2 + h * D;
+    const int q_voff = bf16_tile_voff<D>(l, ild), q_step = bf16_tile_step<D>(ild);
+    const int o_voff = bf16_tile_voff<D>(l, old_), o_step = bf16_tile_step<D>(old_);
     char* Tq = lds_t[w][0];
     char* Tg = lds_t[w][1];
     const int tbase = LT::lane_base(l);
     const float c2 = scale * LOG2E;
 
     bf16x8 k[D / 16], v[D / 16];
-    ldb_rows<D>(rK, r_voff, J * 32 * D * 2, k);
-    ldb_rows<D>(rV, r_voff, J * 32 * D * 2, v);
+    ldb_rows<D>(rK, r_voff, J * 32 * ild * 2, k);
+    ldb_rows<D>(rV, r_voff, J * 32 * ild * 2, v);
     f32x16 sinit = splat16(0.f);
     if constexpr (MASK) sinit = splat16(-pen[(size_t)bh * L + J * 32 + li] / scale);
 
@@ -511,8 +545,8 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
         nu, xa, xb,
         [&](Pre& x, int i) {
             const int I = desc[sa.rank + min(i, nu - 1) * sa.step].x;
-            ldb_tile<D>(rQ, l * 16, I * 32 * D * 2, x.q);
-            ldb_tile<D>(rdO, l * 16, I * 32 * D * 2, x.go);
+            ldb_tile<D>(rQ, q_voff, I * 32 * ild * 2, q_step, x.q);
+            ldb_tile<D>(rdO, o_voff, I * 32 * old_ * 2, o_step, x.go);
             x.lse = ld1(rL, li * 4, I * 128);
             x.gneg = ld1(rG, li * 4, I * 128);
         },
@@ -554,9 +588,9 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
         });
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
-    store_rows_bf16<D>(ak, rdK, J * 32, sa.coop, w, li, h, lds_o, part);
+    store_rows_bf16<D>(ak, rdK, gld, J * 32, sa.coop, w, li, h, lds_o, part);
     if (sa.coop) __syncthreads();
-    store_rows_bf16<D>(av, rdV, J * 32, sa.coop, w, li, h, lds_o, part ? part + 32 * D : nullptr);
+    store_rows_bf16<D>(av, rdV, gld, J * 32, sa.coop, w, li, h, lds_o, part ? part + 32 * D : nullptr);
 }
 
 // -------------------------------------------------------------------------------------------------
@@ -565,10 +599,10 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
 // up to eight chunks in flight at a time.  Element e of a slot is register (c, r) = (e / 1024, e / 64 % 16) of lane
 // l = e % 64: row l % 32 of the strip, feature 32c + acc_row(r, l / 32).
 // -------------------------------------------------------------------------------------------------
-template <int D>
+template <int D, bool ST>
 __global__ __launch_bounds__(256) void bf16_merge_fwd_kernel(const float* __restrict__ Part, const int* __restrict__ desc,
                                                              int n_long, int n_slots, __bf16* __restrict__ O,
-                                                             float* __restrict__ Lse, int L) {
+                                                             float* __restrict__ Lse, int L, HeadLayout lay, int H) {
     constexpr int PSZ = bf16_slot_floats<D>(), EB = 32 * D / 256;
     const int eb = blockIdx.x % EB, item = blockIdx.x / EB;
     const int bh = item / n_long;
@@ -619,15 +653,18 @@ __global__ __launch_bounds__(256) void bf16_merge_fwd_kernel(const float* __rest
         for (int k = 0; k < 8; ++k)
             if (c0 + k < d.z) v += x[k] * __builtin_amdgcn_exp2f(mm[k] - sm[row]);
     }
-    O[((size_t)bh * L + d.x * 32 + row) * D + 32 * c + acc_row(r, l >> 5)] = (__bf16)(v * sr[row]);
+    size_t ob, obytes;
+    int old_;
+    bf16_head<ST, D>(lay, H, bh, L, ob, old_, obytes);
+    O[ob + (size_t)(d.x * 32 + row) * old_ + 32 * c + acc_row(r, l >> 5)] = (__bf16)(v * sr[row]);
 }
 
 // Plain sums (backward): out0 from the first 32 x D block of the slots, out1 (column pass: dV; grid twice as
 // large) from the second.
-template <int D>
+template <int D, bool ST>
 __global__ __launch_bounds__(256) void bf16_merge_sum_kernel(const float* __restrict__ Part, const int* __restrict__ desc,
                                                              int n_long, int n_slots, __bf16* __restrict__ out0,
-                                                             __bf16* __restrict__ out1, int L) {
+                                                             __bf16* __restrict__ out1, int L, HeadLayout lay, int H) {
     constexpr int PSZ = bf16_slot_floats<D>();
     const int EB = (out1 ? 2 : 1) * 32 * D / 256;
     const int eb = blockIdx.x % EB, item = blockIdx.x / EB;
@@ -646,7 +683,10 @@ __global__ __launch_bounds__(256) void bf16_merge_sum_kernel(const float* __rest
         for (int k = 0; k < 8; ++k)
             if (c0 + k < d.z) v += x[k];
     }
-    (which ? out1 : out0)[((size_t)bh * L + d.x * 32 + row) * D + 32 * c + acc_row(r, l >> 5)] = (__bf16)v;
+    size_t gb, gbytes;
+    int gld;
+    bf16_head<ST, D>(lay, H, bh, L, gb, gld, gbytes);
+    (which ? out1 : out0)[gb + (size_t)(d.x * 32 + row) * gld + 32 * c + acc_row(r, l >> 5)] = (__bf16)v;
 }
 
 }  // namespace spion

@@ -76,6 +76,11 @@ void sparse_bf16_forward(void*, const void*, const void*, const void*, const flo
                          const int*, int);
 void sparse_bf16_backward(void*, const void*, const void*, const void*, const float*, const void*, const float*,
                           const void*, void*, void*, void*, const int*, const int*, int);
+void sparse_bf16_forward_strided(void*, const void*, const void*, const void*, const float*, void*, float*, const int*,
+                                 const int*, int, int, const HeadLayout&, const HeadLayout&);
+void sparse_bf16_backward_strided(void*, const void*, const void*, const void*, const float*, const void*, const float*,
+                                  const void*, void*, void*, void*, const int*, const int*, int, int, const HeadLayout&,
+                                  const HeadLayout&, const HeadLayout&);
 int transpose_last2(const float*, float*, int, int, int, hipStream_t);
 int transition_update(const float*, float*, int, long long, float*, double*, int, int, hipStream_t);
 void* dense_init(int, int, int, bool);
@@ -111,6 +116,31 @@ void spion_block_bf16_attn_backward(void* h, const void* Q, const void* K, const
     sparse_bf16_backward(h, Q, K, V, Mask, Out, Lse, dO, dQ, dK, dV, Offsets, Columns, nnz);
 }
 void spion_block_bf16_destroy(void* h) { sparse_destroy(h); }
+static spion::HeadLayout to_layout(const spion_head_layout* y);
+void spion_block_bf16_attn_forward_strided(void* h, const void* Q, const void* K, const void* V, const float* Mask,
+                                           void* Out, float* Lse, const int* Offsets, const int* Columns,
+                                           const int* SumMat, int nnz, int heads, const spion_head_layout* in,
+                                           const spion_head_layout* out) {
+    (void)SumMat;
+    if (!in || !out) {
+        set_error("bf16 attn_forward_strided: null layout argument");
+        return;
+    }
+    sparse_bf16_forward_strided(h, Q, K, V, Mask, Out, Lse, Offsets, Columns, nnz, heads, to_layout(in), to_layout(out));
+}
+void spion_block_bf16_attn_backward_strided(void* h, const void* Q, const void* K, const void* V, const float* Mask,
+                                            const void* Out, const float* Lse, const void* dO, void* dQ, void* dK,
+                                            void* dV, const int* Offsets, const int* Columns, const int* SumMat,
+                                            int nnz, int heads, const spion_head_layout* in,
+                                            const spion_head_layout* out, const spion_head_layout* grad) {
+    (void)SumMat;
+    if (!in || !out || !grad) {
+        set_error("bf16 attn_backward_strided: null layout argument");
+        return;
+    }
+    sparse_bf16_backward_strided(h, Q, K, V, Mask, Out, Lse, dO, dQ, dK, dV, Offsets, Columns, nnz, heads,
+                                 to_layout(in), to_layout(out), to_layout(grad));
+}
 
 // ---- sparse, no key mask -----------------------------------------------------------------------
 void* spion_block_init(int emb_dim, int seq_len, int num_batches, int block_size) {

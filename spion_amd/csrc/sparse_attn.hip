@@ -1566,14 +1566,9 @@ static bool ensure_part_ws(SparseAttn* a, int slots) {
     return true;
 }
 
-void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out, float* Lse,
-                         const int* Offsets, const int* Columns, int nnz) {
-    if (!Q || !K || !V || !Out || !Lse || !Offsets || (nnz > 0 && !Columns)) {
-        set_error("bf16 attn_forward: null pointer argument");
-        return;
-    }
-    SparseAttn* a = as_bf16(h, "bf16 attn_forward", Offsets, Columns, nnz);
-    if (!a) return;
+template <bool ST>
+static void bf16_forward_impl(SparseAttn* a, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
+                              float* Lse, const Layouts& ly) {
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
     if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
@@ -1582,12 +1577,12 @@ void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, c
     __bf16* o = static_cast<__bf16*>(Out);
 #define SPION_LAUNCH(DD, MM)                                                                                         \
     do {                                                                                                             \
-        hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,          \
+        hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,      \
                            pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,         \
-                           pi.slots_row, pi.chunk_row);                                                              \
+                           pi.slots_row, pi.chunk_row, ly);                                                          \
         if (pi.n_long_row)                                                                                           \
-            hipLaunchKernelGGL((bf16_merge_fwd_kernel<DD>), grid_m, dim3(256), 0, a->hdr.stream, a->ws_part,         \
-                               pi.d_long_row, pi.n_long_row, pi.slots_row, o, Lse, a->L);                            \
+            hipLaunchKernelGGL((bf16_merge_fwd_kernel<DD, ST>), grid_m, dim3(256), 0, a->hdr.stream, a->ws_part,     \
+                               pi.d_long_row, pi.n_long_row, pi.slots_row, o, Lse, a->L, ly.out, ly.H);              \
     } while (0)
     if (a->d == 32) {
         if (Mask) SPION_LAUNCH(32, true);
@@ -1600,15 +1595,10 @@ void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, c
     check_launch("bf16_fwd_kernel");
 }
 
-void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, const float* Mask, const void* Out,
-                          const float* Lse, const void* dO, void* dQ, void* dK, void* dV, const int* Offsets,
-                          const int* Columns, int nnz) {
-    if (!Q || !K || !V || !Out || !Lse || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
-        set_error("bf16 attn_backward: null pointer argument");
-        return;
-    }
-    SparseAttn* a = as_bf16(h, "bf16 attn_backward", Offsets, Columns, nnz);
-    if (!a) return;
+template <bool ST>
+static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, const void* V, const float* Mask,
+                               const void* Out, const float* Lse, const void* dO, void* dQ, void* dK, void* dV,
+                               const Layouts& ly) {
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
@@ -1621,20 +1611,21 @@ void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, 
 #define SPION_LAUNCH(DD, MM)                                                                                          \
     do {                                                                                                              \
         if (a->bwd_passes & 1) {                                                                                      \
-            hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o, Lse,   \
-                               Mask, a->ws_rowsum, dq, pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB,    \
-                               a->scale, a->ws_part, pi.slots_row, pi.chunk_row);                                     \
+            hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM, ST>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o,    \
+                               Lse, Mask, a->ws_rowsum, dq, pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L,      \
+                               a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row, ly);                          \
             if (pi.n_long_row)                                                                                        \
-                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD>), grid_mr, dim3(256), 0, a->hdr.stream, a->ws_part,     \
-                                   pi.d_long_row, pi.n_long_row, pi.slots_row, dq, (__bf16*)nullptr, a->L);           \
+                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD, ST>), grid_mr, dim3(256), 0, a->hdr.stream, a->ws_part, \
+                                   pi.d_long_row, pi.n_long_row, pi.slots_row, dq, (__bf16*)nullptr, a->L, ly.grad,   \
+                                   ly.H);                                                                             \
         }                                                                                                             \
         if (a->bwd_passes & 2) {                                                                                      \
-            hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM>), grid_c, block, 0, a->hdr.stream, q, k, v, go, Lse,      \
+            hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM, ST>), grid_c, block, 0, a->hdr.stream, q, k, v, go, Lse,  \
                                a->ws_rowsum, Mask, dk, dv, pi.d_tcp, pi.d_tcdesc, pi.d_wg_col, pi.n_wg_col, a->L,     \
-                               a->NB, a->scale, a->ws_part, pi.slots_col, pi.chunk_col);                              \
+                               a->NB, a->scale, a->ws_part, pi.slots_col, pi.chunk_col, ly);                          \
             if (pi.n_long_col)                                                                                        \
-                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD>), grid_mc, dim3(256), 0, a->hdr.stream, a->ws_part,     \
-                                   pi.d_long_col, pi.n_long_col, pi.slots_col, dk, dv, a->L);                         \
+                hipLaunchKernelGGL((bf16_merge_sum_kernel<DD, ST>), grid_mc, dim3(256), 0, a->hdr.stream, a->ws_part, \
+                                   pi.d_long_col, pi.n_long_col, pi.slots_col, dk, dv, a->L, ly.grad, ly.H);          \
         }                                                                                                             \
     } while (0)
     if (a->d == 32) {
@@ -1646,6 +1637,109 @@ void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, 
     }
 #undef SPION_LAUNCH
     check_launch("bf16_bwd kernels");
+}
+
+void sparse_bf16_forward(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out, float* Lse,
+                         const int* Offsets, const int* Columns, int nnz) {
+    if (!Q || !K || !V || !Out || !Lse || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("bf16 attn_forward: null pointer argument");
+        return;
+    }
+    SparseAttn* a = as_bf16(h, "bf16 attn_forward", Offsets, Columns, nnz);
+    if (!a) return;
+    bf16_forward_impl<false>(a, Q, K, V, Mask, Out, Lse, Layouts{});
+}
+
+void sparse_bf16_backward(void* h, const void* Q, const void* K, const void* V, const float* Mask, const void* Out,
+                          const float* Lse, const void* dO, void* dQ, void* dK, void* dV, const int* Offsets,
+                          const int* Columns, int nnz) {
+    if (!Q || !K || !V || !Out || !Lse || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("bf16 attn_backward: null pointer argument");
+        return;
+    }
+    SparseAttn* a = as_bf16(h, "bf16 attn_backward", Offsets, Columns, nnz);
+    if (!a) return;
+    bf16_backward_impl<false>(a, Q, K, V, Mask, Out, Lse, dO, dQ, dK, dV, Layouts{});
+}
+
+// The bf16 family on [B][H][L][d] views (strides in elements, multiples of 8; pointers 16-byte aligned).
+static bool check_layout_bf16(const char* who, const char* what, const SparseAttn* a, const HeadLayout& y) {
+    if (y.ld < a->d || y.ld % 8 || y.hstride % 8 || y.bstride % 8 || y.hstride < 0 || y.bstride < 0) {
+        set_error("%s: %s layout: strides must be non-negative multiples of 8 elements and the row stride >= emb_dim",
+                  who, what);
+        return false;
+    }
+    if ((long long)a->L * y.ld >= (1ll << 29)) {
+        set_error("%s: %s layout: seq_len * row stride = %lld elements exceeds 2^29", who, what, (long long)a->L * y.ld);
+        return false;
+    }
+    return true;
+}
+
+void sparse_bf16_forward_strided(void* h, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
+                                 float* Lse, const int* Offsets, const int* Columns, int nnz, int heads,
+                                 const HeadLayout& in, const HeadLayout& out) {
+    const char* who = "bf16 attn_forward_strided";
+    if (!Q || !K || !V || !Out || !Lse || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    SparseAttn* a = as_bf16(h, who, Offsets, Columns, nnz);
+    if (!a) return;
+    if (heads <= 0 || a->NB % heads) {
+        set_error("%s: heads = %d does not divide num_batches = %d", who, heads, a->NB);
+        return;
+    }
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Out)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!check_layout_bf16(who, "input", a, in) || !check_layout_bf16(who, "output", a, out)) return;
+    if (!layout_is_injective(out, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the output layout maps two elements to one address", who);
+        return;
+    }
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = out;
+    ly.H = heads;
+    bf16_forward_impl<true>(a, Q, K, V, Mask, Out, Lse, ly);
+}
+
+void sparse_bf16_backward_strided(void* h, const void* Q, const void* K, const void* V, const float* Mask,
+                                  const void* Out, const float* Lse, const void* dO, void* dQ, void* dK, void* dV,
+                                  const int* Offsets, const int* Columns, int nnz, int heads, const HeadLayout& in,
+                                  const HeadLayout& out, const HeadLayout& grad) {
+    const char* who = "bf16 attn_backward_strided";
+    if (!Q || !K || !V || !Out || !Lse || !dO || !dQ || !dK || !dV || !Offsets || (nnz > 0 && !Columns)) {
+        set_error("%s: null pointer argument", who);
+        return;
+    }
+    SparseAttn* a = as_bf16(h, who, Offsets, Columns, nnz);
+    if (!a) return;
+    if (heads <= 0 || a->NB % heads) {
+        set_error("%s: heads = %d does not divide num_batches = %d", who, heads, a->NB);
+        return;
+    }
+    if (!aligned16(Q) || !aligned16(K) || !aligned16(V) || !aligned16(Out) || !aligned16(dO) || !aligned16(dQ) ||
+        !aligned16(dK) || !aligned16(dV)) {
+        set_error("%s: operand pointers must be 16-byte aligned", who);
+        return;
+    }
+    if (!check_layout_bf16(who, "input", a, in) || !check_layout_bf16(who, "output", a, out) ||
+        !check_layout_bf16(who, "gradient", a, grad))
+        return;
+    if (!layout_is_injective(grad, a->NB / heads, heads, a->L, a->d)) {
+        set_error("%s: the gradient layout maps two elements to one address", who);
+        return;
+    }
+    Layouts ly{};
+    ly.in = in;
+    ly.out = out;
+    ly.grad = grad;
+    ly.H = heads;
+    bf16_backward_impl<true>(a, Q, K, V, Mask, Out, Lse, dO, dQ, dK, dV, ly);
 }
 
 // [batch][rows][cols] -> [batch][cols][rows], fp32.  Used by the host modules for the K^T / V^T operands

@@ -203,6 +203,108 @@ def test_bf16_long_strips_with_key_mask_and_large_logits(d):
     abi.close()
 
 
+def _bf16_head_views(B, H, L, d, layout, n, seed, fill=None):
+    """n bf16 tensors seen as [B, H, L, d]: "proj": each a [B, L, H*d] projection; "fused": slices of one
+    [B, L, n, H, d+8] buffer (padded rows)."""
+    g = torch.Generator().manual_seed(seed)
+    if layout == "proj":
+        bufs = [torch.randn(B, L, H * d, generator=g).to(torch.bfloat16).cuda() for _ in range(n)]
+        views = [b.view(B, L, H, d).transpose(1, 2) for b in bufs]
+    else:
+        buf = torch.randn(B, L, n, H, d + 8, generator=g).to(torch.bfloat16).cuda()
+        bufs = [buf]
+        views = [buf[:, :, i, :, :d].transpose(1, 2) for i in range(n)]
+    if fill is not None:
+        for b in bufs:
+            b.fill_(fill)
+    return bufs, views
+
+
+@pytest.mark.parametrize("d,layout,glob,with_mask", [(32, "proj", False, False), (64, "fused", False, True),
+                                                     (64, "proj", True, False), (32, "fused", True, True)])
+def test_bf16_strided_entry_points(d, layout, glob, with_mask):
+    """spion_block_bf16_attn_{forward,backward}_strided: bf16 heads read and written in place in the memory of
+    [B, L, H*d] projections (or of one fused, padded buffer).  Same kernels and arithmetic as the contiguous entry
+    points on contiguous copies -- long strips cut into chunks and merged included: bit-identical results; the
+    padding between the heads' rows is left alone."""
+    import ctypes
+    B, H, L, bs = 2, 2, 1024, 32
+    NB = B * H
+    mat = _mask(L // bs, 0.1, seed=21, global_block=glob)
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    _, (q, k, v) = _bf16_head_views(B, H, L, d, layout, 3, seed=71)
+    _, (dout,) = _bf16_head_views(B, H, L, d, "proj", 1, seed=72)
+    _, (out,) = _bf16_head_views(B, H, L, d, "proj", 1, seed=0, fill=float("nan"))
+    gbufs, (dq, dk, dv) = _bf16_head_views(B, H, L, d, layout, 3, seed=0, fill=-7.0)
+    pen = None
+    if with_mask:
+        valid = torch.tensor([L, L - 40, L // 2, L - 1])
+        pen = (1e6 * (torch.arange(L)[None, :] >= valid[:, None]).float()).contiguous().cuda()
+    pen_ptr = pen.data_ptr() if pen is not None else None
+    lse = torch.full((NB, L), float("nan"), device="cuda")
+    lin, lout, lgrad = _lib.head_layout(q), _lib.head_layout(out), _lib.head_layout(dq)
+    assert lin is not None and lout is not None and lgrad is not None
+    tail = (abi.offsets.data_ptr(), abi.columns.data_ptr(), abi.sum_mat.data_ptr(), abi.nnz)
+    abi.lib.spion_block_bf16_attn_forward_strided(abi.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
+                                                  out.data_ptr(), lse.data_ptr(), *tail, H, ctypes.addressof(lin),
+                                                  ctypes.addressof(lout))
+    _lib.check_error("bf16 forward strided")
+    abi.lib.spion_block_bf16_attn_backward_strided(abi.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
+                                                   out.data_ptr(), lse.data_ptr(), dout.data_ptr(), dq.data_ptr(),
+                                                   dk.data_ptr(), dv.data_ptr(), *tail, H, ctypes.addressof(lin),
+                                                   ctypes.addressof(lout), ctypes.addressof(lgrad))
+    _lib.check_error("bf16 backward strided")
+    torch.cuda.synchronize()
+    flat = lambda t: t.reshape(NB, L, d).contiguous()
+    Qc, Kc, Vc, dOc = flat(q), flat(k), flat(v), flat(dout)
+    O2, lse2 = abi.forward(Qc, Kc, Vc, pen)
+    g2 = abi.backward(Qc, Kc, Vc, O2, lse2, dOc, pen)
+    torch.cuda.synchronize()
+    assert torch.equal(flat(out), O2) and torch.equal(lse, lse2)
+    for name, a, b in zip(("dQ", "dK", "dV"), (dq, dk, dv), g2):
+        assert torch.equal(flat(a), b), name
+    if layout == "fused":
+        assert (gbufs[0][..., d:] == -7.0).all(), "padding between the heads' rows was written"
+    ref = _oracle(Qc, Kc, Vc, dOc, sm, off, col, pen)
+    for name, t in (("O", out), ("dQ", dq), ("dK", dk), ("dV", dv)):
+        assert_close_bf16(flat(t).float().cpu().numpy(), ref[name], f"bf16 strided {name}")
+    # a layout the kernels cannot take is refused
+    bad = _lib.HeadLayout(lin.batch_stride, lin.head_stride, lin.row_stride + 4)
+    abi.lib.spion_block_bf16_attn_forward_strided(abi.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
+                                                  out.data_ptr(), lse.data_ptr(), *tail, H, ctypes.addressof(bad),
+                                                  ctypes.addressof(lout))
+    with pytest.raises(RuntimeError, match="multiples of 8"):
+        _lib.check_error("bad layout")
+    abi.close()
+
+
+def test_bf16_module_reads_views_in_place():
+    """BlockAttentionBF16 on heads that are views of bf16 projections: same values and gradients as on contiguous
+    copies (bit-identical: same kernels), output and gradients laid out like the inputs."""
+    from spion_amd import BlockAttentionBF16
+    B, H, L, d, bs = 2, 2, 512, 64, 64
+    mat = torch.from_numpy(_mask(L // bs, 0.3, seed=5).astype(np.float32)).cuda()
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    mod = BlockAttentionBF16(cfg)
+    g = torch.Generator().manual_seed(9)
+    proj = [torch.randn(B, L, H * d, generator=g).to(torch.bfloat16).cuda().requires_grad_() for _ in range(3)]
+    views = [p.view(B, L, H, d).transpose(1, 2) for p in proj]
+    dout = torch.randn(B, L, H * d, generator=g).to(torch.bfloat16).cuda().view(B, L, H, d).transpose(1, 2)
+    out, _ = mod(*views, None, mat)
+    assert out.stride() == views[0].stride()
+    out.backward(dout)
+    grads = [p.grad.clone() for p in proj]
+    cont = [v.detach().contiguous().requires_grad_() for v in views]
+    out2, _ = mod(*cont, None, mat)
+    out2.backward(dout.contiguous())
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    for gp, c in zip(grads, cont):
+        assert torch.equal(gp.view(B, L, H, d).transpose(1, 2), c.grad)
+
+
 def test_bf16_rejects_element_patterns_and_fp32_handles():
     L, d, NB = 128, 32, 1
     sm, off, col = workloads.window_random_csr(L, 4, 12, seed=3)
