@@ -261,8 +261,8 @@ struct HybRowAcc {
 // -------------------------------------------------------------------------------------------------
 template <bool MASK, bool ST>
 SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, const float* __restrict__ K,
-                                                   const float* __restrict__ pen, float* __restrict__ P,
-                                                   float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz,
+                                                   const float* __restrict__ pen, float* __restrict__ Raw,
+                                                   float2* __restrict__ Stats, HybIndex ix, int L, int NB,
                                                    float scale, Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
     const long long wrow = (long long)xcd_remap((int)blockIdx.x, (int)gridDim.x) * HYB_GWAVES + wave_index();
@@ -272,7 +272,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
     size_t ib;
     int ild;
     hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
-    float* Ph = P + (size_t)bh * nnz;
+    float* raw = Raw + (size_t)bh * ix.nr + r0;  // this row's logits, in the order of the remainder's CSR list
     const float c2 = scale * LOG2E;
     f32x4 q4 = reinterpret_cast<const f32x4*>(Q + ib + (size_t)row * ild)[lane & 7];
     q4 *= c2;
@@ -283,11 +283,10 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
     for (int c0 = 0; c0 < rc; c0 += 64) {
         const int k = c0 + ent;
         const int col = k < rc ? ix.r_col[r0 + k] : 0;
-        const int pp = k < rc ? ix.r_pos[r0 + k] : 0;
         float v = hyb_gather_dot(q4, K + ib, ild, col, min(64, rc - c0), lane);
         if (k < rc) {
             if (MASK) v -= pen[(size_t)bh * L + col] * LOG2E;
-            Ph[pp] = v;
+            raw[k] = v;
             mx = fmaxf(mx, v);
         } else {
             v = HYB_ABSENT;
@@ -301,7 +300,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_logits_kernel(const float* __restrict__ Q, 
 #pragma unroll
     for (int c = 0; c < KEEP; ++c)
         if (64 * c < rc) z += __builtin_amdgcn_exp2f(vk[c] - mx);
-    for (int k = 64 * KEEP + lane; k < rc; k += 64) z += __builtin_amdgcn_exp2f(Ph[ix.r_pos[r0 + k]] - mx);
+    for (int k = 64 * KEEP + lane; k < rc; k += 64) z += __builtin_amdgcn_exp2f(raw[k] - mx);
     z = wave_sum(z);
     if (lane == 0) Stats[(size_t)bh * L + row] = make_float2(mx, z);
 }
@@ -465,8 +464,9 @@ SPION_HYB_KERNEL(WAVES) void hyb_tile_fwd_kernel(const float* __restrict__ Q, co
 // 1 / denominator}; their share of O is added to what step 2 wrote.  Ocache (optional): second copy of O.
 // -------------------------------------------------------------------------------------------------
 template <bool ST>
-SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, float* __restrict__ P,
-                                               float* __restrict__ O, float* __restrict__ Ocache,
+SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, const float* __restrict__ Raw,
+                                               float* __restrict__ P, float* __restrict__ O,
+                                               float* __restrict__ Ocache,
                                                const float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz,
                                                Layouts ly) {
     const int lane = threadIdx.x & 63, ent = hyb_entry_of_lane(lane);
@@ -479,6 +479,7 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, floa
     hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
     hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
     float* Ph = P + (size_t)bh * nnz;
+    const float* raw = Raw + (size_t)bh * ix.nr + r0;
     const float2 st = Stats[(size_t)bh * L + row];
     HybRowAcc acc;
     acc.clear();
@@ -488,9 +489,9 @@ SPION_HYB_GATHER_KERNEL void hyb_rem_pv_kernel(const float* __restrict__ V, floa
         int col = 0;
         if (k < rc) {
             const int pp = ix.r_pos[r0 + k];
-            wgt = __builtin_amdgcn_exp2f(Ph[pp] - st.x) * st.y;
+            wgt = __builtin_amdgcn_exp2f(raw[k] - st.x) * st.y;
             col = ix.r_col[r0 + k];
-            Ph[pp] = wgt;
+            __builtin_nontemporal_store(wgt, Ph + pp);  // written once, not read again before the backward
         }
         acc.chunk(wgt, col, min(64, rc - c0), V + ib, ild, lane);
     }

@@ -393,6 +393,8 @@ struct SparseAttn {
     bool use_ocache = true;
     float* ws_trans = nullptr;   // [NB][L][d] row-major copy of the transposed operand (element path)
     float* ws_stats = nullptr;   // [NB][L][2] softmax row statistics handed between the hybrid forward's launches
+    float* ws_raw = nullptr;     // [NB][nr] raw logits of a hybrid pattern's remainder, forward only
+    size_t ws_raw_count = 0;
     float* ws_ds = nullptr;      // [NB][nnz] dS scratch of the strided backward on patterns without tile structure
     size_t ws_ds_count = 0;
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
@@ -454,6 +456,7 @@ void sparse_destroy(void* h) {
     if (a->ws_trans) (void)hipFree(a->ws_trans);
     if (a->ws_stats) (void)hipFree(a->ws_stats);
     if (a->ws_ds) (void)hipFree(a->ws_ds);
+    if (a->ws_raw) (void)hipFree(a->ws_raw);
     if (a->ws_part) (void)hipFree(a->ws_part);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
@@ -1047,6 +1050,22 @@ template <bool ST>
 static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const float* V, const float* Mask,
                            float* Attn, float* Out, float* ocopy, const int* Offsets, int nnz, const Layouts& ly) {
     if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
+    // the remainder's raw logits between the first and the third launch: a compact list of their own (written and
+    // read in full lines) rather than their places inside P, where every four-byte store would pull in a line
+    const size_t raw_need = (size_t)a->NB * (size_t)std::max(a->pat.hyb_nr, 1);
+    if (a->ws_raw_count < raw_need) {
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+        if (cap != hipStreamCaptureStatusNone) {
+            set_error("attn_forward: the workspace for this pattern is not allocated yet; run one step outside the capture");
+            return;
+        }
+        if (a->ws_raw) (void)hipFree(a->ws_raw);
+        a->ws_raw = nullptr;
+        a->ws_raw_count = 0;
+        if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_raw, sizeof(float) * raw_need))) return;
+        a->ws_raw_count = raw_need;
+    }
     a->last_path = 3;
     const int nbr = a->L / 32;
     const long long rows = (long long)a->NB * a->L;
@@ -1057,8 +1076,8 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
     float2* stats = reinterpret_cast<float2*>(a->ws_stats);
 #define SPION_HYB_FWD(MASKED)                                                                                        \
     do {                                                                                                             \
-        hipLaunchKernelGGL((hyb_rem_logits_kernel<MASKED, ST>), grid_g, block_g, 0, a->hdr.stream, Q, K, Mask, Attn, \
-                           stats, a->pat.hyb, a->L, a->NB, nnz, a->scale, ly);                                       \
+        hipLaunchKernelGGL((hyb_rem_logits_kernel<MASKED, ST>), grid_g, block_g, 0, a->hdr.stream, Q, K, Mask,       \
+                           a->ws_raw, stats, a->pat.hyb, a->L, a->NB, a->scale, ly);                                 \
         if (one)                                                                                                     \
             hipLaunchKernelGGL((hyb_tile_fwd_kernel<MASKED, 1, HYB_MAXT1, ST>), grid_t, block_t, 0, a->hdr.stream,   \
                                Q, K, V, Mask, Attn, Out, stats, Offsets, a->pat.hyb, a->L, nbr, a->NB, nnz,          \
@@ -1073,7 +1092,8 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
     else
         SPION_HYB_FWD(false);
 #undef SPION_HYB_FWD
-    hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, Attn, Out, ocopy,
+    hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, (const float*)a->ws_raw, Attn, Out,
+                       ocopy,
                        (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
     check_launch("hybrid forward kernels");
 }
