@@ -95,6 +95,61 @@ def test_random_element_patterns(seed):
     abi.close()
 
 
+@pytest.mark.parametrize("seed", range(500, 512))
+def test_random_hybrid_patterns(seed):
+    """Element-sparse patterns with dense structure, drawn at random: a band of random width (sometimes shifted off
+    the diagonal or doubled), a few full blocks, random scattered entries, empty rows and columns, key masks.  Through
+    the reference's ABI (kept copy of Out) and the row-major entries (Out handed over): both against the oracle and
+    equal to each other bit for bit."""
+    from tests.abi_utils import assert_close, oracle_fwd_bwd
+    rng = np.random.default_rng(seed)
+    L = 32 * int(rng.integers(4, 25))
+    NB = int(rng.integers(1, 5))
+    keep = np.zeros((L, L), dtype=bool)
+    i = np.arange(L)
+    w = int(rng.choice([8, 24, 48, 100]))
+    shift = int(rng.choice([0, 0, 37]))
+    keep |= np.abs(i[:, None] - i[None, :] - shift) <= w
+    if rng.random() < 0.4:
+        keep |= np.abs(i[:, None] - i[None, :] + L // 3) <= w // 2      # a second band
+    for _ in range(int(rng.integers(0, 4))):                            # full blocks anywhere
+        a, b, n = int(rng.integers(0, L - 64)), int(rng.integers(0, L - 64)), int(rng.choice([32, 64]))
+        keep[a:a + n, b:b + n] = True
+    keep |= rng.random((L, L)) < float(rng.choice([0.0, 0.01, 0.04]))   # scattered entries
+    if rng.random() < 0.5:
+        keep[int(rng.integers(L)), :] = False
+    if rng.random() < 0.5:
+        keep[:, int(rng.integers(L))] = False
+    if rng.random() < 0.3:
+        r0 = 32 * int(rng.integers(L // 32))
+        keep[r0:r0 + 32, :] = False                                      # an empty strip
+    sm = keep.sum(1).astype(np.int32)
+    off = np.concatenate([[0], np.cumsum(sm)]).astype(np.int32)
+    col = np.nonzero(keep)[1].astype(np.int32)
+    with_mask = bool(rng.random() < 0.5)
+    pen = None
+    if with_mask:
+        valid = rng.integers(1, L + 1, size=NB)
+        pen = torch.from_numpy((1e6 * (np.arange(L)[None, :] >= valid[:, None])).astype(np.float32)).cuda()
+    tag = f"seed {seed}: hybrid L={L} NB={NB} band={w} shift={shift} nnz={int(off[-1])} mask={with_mask}"
+    abi = SparseABI(32, L, NB, 1, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    g = torch.Generator().manual_seed(seed)
+    scale = float(rng.choice([0.5, 1.5]))
+    Q, K, V, dO = (torch.randn(NB, L, 32, generator=g).cuda() * s for s in (scale, scale, 1, 1))
+    got, ref = run_and_check(abi, Q, K, V, dO, pen, tag=tag)
+    path = abi.last_path()
+    assert path in (2, 3), tag
+    O2, P2 = abi.forward_rowmajor(Q, K, V, pen)
+    g2 = abi.backward_rowmajor(Q, K, V, P2, O2, dO)
+    torch.cuda.synchronize()
+    assert abi.last_path() == path, tag
+    assert torch.equal(P2, got["P"]) and torch.equal(O2, got["O"]), tag
+    for name, a in zip(("dQ", "dK", "dV"), g2):
+        assert torch.equal(a, got[name]), f"{tag} {name}"
+    abi.close()
+
+
 @pytest.mark.parametrize("seed", range(400, 408))
 def test_random_dense_shapes(seed):
     from oracle import dense_attention as oda
