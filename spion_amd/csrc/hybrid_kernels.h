@@ -23,12 +23,10 @@ namespace spion {
 
 // The analysed pattern as the kernels see it (device pointers, shared by all heads).
 struct HybIndex {
-    // dense tiles, by block row: tiles t_rp[I] .. t_rp[I+1]-1 of block row I; per tile its block column, its block
-    // row, and per row of the tile the position of the row's first entry inside a head's P and the 32-bit set of
-    // present columns
+    // dense tiles, by block row: tiles t_rp[I] .. t_rp[I+1]-1 of block row I; per tile its block column and, per
+    // row of the tile, the position of the row's first entry inside a head's P and the 32-bit set of present columns
     const int* t_rp;
     const int* t_col;
-    const int* t_row;
     const int* t_pos;        // [tiles][32]
     const unsigned* t_bits;  // [tiles][32]
     // the same tiles by block column: tile ids t_ct[t_cp[J]] .. of block column J and their block rows t_ci

@@ -763,7 +763,6 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                 memcpy(bits_as_int.data(), t_bits.data(), t_bits.size() * sizeof(int));
                 hyb_off[0] = append(t_rp);
                 hyb_off[1] = append(t_col);
-                hyb_off[2] = append(t_row);
                 hyb_off[3] = append(t_pos);
                 hyb_off[4] = append(bits_as_int);
                 hyb_off[5] = append(t_cp);
@@ -821,7 +820,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_cpos = pi.d_blob + o_cpos;
         if (pi.hybrid) {
             const int* b = pi.d_blob;
-            pi.hyb = HybIndex{b + hyb_off[0], b + hyb_off[1], b + hyb_off[2], b + hyb_off[3],
+            pi.hyb = HybIndex{b + hyb_off[0], b + hyb_off[1], b + hyb_off[3],
                               reinterpret_cast<const unsigned*>(b + hyb_off[4]), b + hyb_off[5], b + hyb_off[6],
                               b + hyb_off[13], b + hyb_off[7], b + hyb_off[8], b + hyb_off[9], b + hyb_off[10],
                               b + hyb_off[11], b + hyb_off[12], pi.hyb_nr, pi.hyb_tiles};
@@ -896,6 +895,25 @@ void sparse_forget_pattern(void* h, const int* Offsets, const int* Columns) {
 static bool ensure_ws(float** p, size_t count) {
     if (*p) return true;
     return SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * count));
+}
+
+// A workspace whose size follows the pattern: grown (never under HIP graph capture, where an allocation would
+// invalidate the capture) to the largest size asked for.  hipFree waits for the device, so no launch still uses the
+// old buffer.
+static bool ensure_ws_grow(SparseAttn* a, float** p, size_t* have, size_t need, const char* who) {
+    if (*have >= need) return true;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+    if (cap != hipStreamCaptureStatusNone) {
+        set_error("%s: the workspace for this pattern is not allocated yet; run one step outside the capture", who);
+        return false;
+    }
+    if (*p) (void)hipFree(*p);
+    *p = nullptr;
+    *have = 0;
+    if (!SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * need))) return false;
+    *have = need;
+    return true;
 }
 
 int transpose_last2(const float* in, float* out, int batch, int rows, int cols, hipStream_t stream);
@@ -1052,20 +1070,9 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
     if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
     // the remainder's raw logits between the first and the third launch: a compact list of their own (written and
     // read in full lines) rather than their places inside P, where every four-byte store would pull in a line
-    const size_t raw_need = (size_t)a->NB * (size_t)std::max(a->pat.hyb_nr, 1);
-    if (a->ws_raw_count < raw_need) {
-        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(a->hdr.stream, &cap);
-        if (cap != hipStreamCaptureStatusNone) {
-            set_error("attn_forward: the workspace for this pattern is not allocated yet; run one step outside the capture");
-            return;
-        }
-        if (a->ws_raw) (void)hipFree(a->ws_raw);
-        a->ws_raw = nullptr;
-        a->ws_raw_count = 0;
-        if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_raw, sizeof(float) * raw_need))) return;
-        a->ws_raw_count = raw_need;
-    }
+    if (!ensure_ws_grow(a, &a->ws_raw, &a->ws_raw_count, (size_t)a->NB * (size_t)std::max(a->pat.hyb_nr, 1),
+                        "attn_forward"))
+        return;
     a->last_path = 3;
     const int nbr = a->L / 32;
     const long long rows = (long long)a->NB * a->L;
@@ -1504,20 +1511,7 @@ void sparse_backward_strided(void* h, const float* Q, const float* K, const floa
     ly.H = heads;
     if (!a->pat.tiled) {
         // these entry points have no dS argument: the scratch is the handle's (grown outside graph capture only)
-        const size_t need = (size_t)a->NB * (size_t)std::max(nnz, 1);
-        if (a->ws_ds_count < need) {
-            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-            (void)hipStreamIsCapturing(a->hdr.stream, &cap);
-            if (cap != hipStreamCaptureStatusNone) {
-                set_error("%s: the scratch for this pattern is not allocated yet; run one step outside the capture", who);
-                return;
-            }
-            if (a->ws_ds) (void)hipFree(a->ws_ds);
-            a->ws_ds = nullptr;
-            a->ws_ds_count = 0;
-            if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_ds, sizeof(float) * need))) return;
-            a->ws_ds_count = need;
-        }
+        if (!ensure_ws_grow(a, &a->ws_ds, &a->ws_ds_count, (size_t)a->NB * (size_t)std::max(nnz, 1), who)) return;
         if (a->pat.hybrid) {
             launch_hyb_bwd<true>(a, Q, K, V, P, dO, Out, a->ws_ds, dQ, dK, dV, nnz, ly);
             return;
