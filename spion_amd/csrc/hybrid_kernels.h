@@ -17,6 +17,7 @@
 // part of the row pass, the same for the column pass; the remainder kernels add to what the tile kernels wrote
 // (each row or column has exactly one writer per launch).
 #pragma once
+#include "gather_ops.h"
 #include "tile_kernels.h"
 
 namespace spion {
@@ -171,20 +172,8 @@ __device__ __forceinline__ void hyb_pipeline(int n, HybPre& a, HybPre& b, FetchI
 // =================================================================================================
 // gather helpers (one wavefront per row / column of the remainder)
 // =================================================================================================
-// The gather kernels hold a chunk of up to 64 entries one per lane and fetch the entries' 32-float rows eight lanes
-// to a row (16 bytes per lane, eight rows per load instruction).  Lane L owns entry (L % 8) * 8 + L / 8 of the chunk,
-// so that the eight entries group g = L / 8 fetches (entry j*8 + g in instruction j) are the entries its own eight
-// lanes own: every exchange stays inside a group of eight lanes, nothing goes through LDS memory, and the number of
-// wavefronts in flight -- what bounds these latency-bound kernels -- is not limited by LDS space.
-__device__ __forceinline__ int hyb_entry_of_lane(int lane) { return ((lane & 7) << 3) | (lane >> 3); }
-
-// sum over the eight lanes of a group (quad swaps, then the mirror image of the half row)
-__device__ __forceinline__ float hyb_group_sum(float v) {
-    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // xor 1
-    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // xor 2
-    v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // 7 - i
-    return v;
-}
+// The gather primitives (gather_ops.h) with eight lanes to a 32-float row.
+__device__ __forceinline__ int hyb_entry_of_lane(int lane) { return gather_entry_of_lane<8>(lane); }
 
 // Start (in floats) and row stride of head bh in a tensor group: contiguous [NB][L][32] heads (ST = false, compile-time
 // figures) or [B][H][L][32] views given by a layout.
@@ -194,63 +183,11 @@ __device__ __forceinline__ void hyb_head(const HeadLayout& y, int H, int bh, int
     head_slice<ST, 32>(y, H, bh, L, base, ld, bytes);
 }
 
-// Dot products of the rows X[row_l] (row stride ld) (row index of the lane's entry; nk entries in the chunk) with the vector whose
-// piece 4*(lane%8) .. +3 the lane holds in a4: one result per lane, for the lane's own entry.  Only the load
-// instructions that carry entries are issued; lanes whose entry is past nk get 0 or a partial value to ignore.
 __device__ __forceinline__ float hyb_gather_dot(const f32x4 a4, const float* __restrict__ X, int ld, int row_l,
                                                 int nk, int lane) {
-    const int base = lane & ~7, cl = lane & 7;
-    f32x4 x[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const int rr = __shfl(row_l, base + j, 64);
-        if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * ld)[cl];
-    }
-    float r = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        if (j * 8 < nk) {
-            float sj = x[j].x * a4.x;
-            sj = fmaf(x[j].y, a4.y, sj);
-            sj = fmaf(x[j].z, a4.z, sj);
-            sj = fmaf(x[j].w, a4.w, sj);
-            sj = hyb_group_sum(sj);
-            r = cl == j ? sj : r;
-        }
-    }
-    return r;
+    return gather_dot<8>(a4, X, ld, row_l, nk, lane);
 }
-
-// acc += sum over the chunk's entries (weight w_l and row index row_l of the lane's entry; nk entries) of
-// w * X[row][:]; the lane accumulates the piece 4*(lane%8) .. +3 of the rows its group fetches.
-struct HybRowAcc {
-    f32x4 acc;
-    __device__ __forceinline__ void clear() { acc = (f32x4){0.f, 0.f, 0.f, 0.f}; }
-    __device__ __forceinline__ void chunk(float w_l, int row_l, int nk, const float* __restrict__ X, int ld,
-                                          int lane) {
-        const int base = lane & ~7, cl = lane & 7;
-        float w[8];
-        f32x4 x[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            w[j] = __shfl(w_l, base + j, 64);
-            const int rr = __shfl(row_l, base + j, 64);
-            if (j * 8 < nk) x[j] = reinterpret_cast<const f32x4*>(X + (size_t)rr * ld)[cl];
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            if (j * 8 < nk) acc += w[j] * x[j];  // entries past nk inside a carried instruction have weight 0
-    }
-    // sum over the eight groups; every lane then holds the four floats 4*(lane%8) .. of the result row
-    __device__ __forceinline__ f32x4 total() const {
-        f32x4 a = acc;
-#pragma unroll
-        for (int o = 8; o < 64; o <<= 1)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) a[e] += __shfl_xor(a[e], o, 64);
-        return a;
-    }
-};
+typedef GatherRowAcc<8> HybRowAcc;
 #define SPION_HYB_GATHER_KERNEL __global__ __launch_bounds__(64 * HYB_GWAVES) __attribute__((amdgpu_waves_per_eu(6, 8)))
 
 // -------------------------------------------------------------------------------------------------

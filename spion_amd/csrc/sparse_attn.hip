@@ -64,47 +64,7 @@ __device__ __forceinline__ float row_dot(const float* __restrict__ a, const floa
     return s;
 }
 
-// Dot products of one vector a (the same for all lanes) with up to 64 gathered rows X[row_l], one result per
-// lane.  The rows are fetched D/4 lanes to a row, 16 bytes per lane -- 256/D rows per instruction instead of the
-// 64 cache lines a lane-per-row gather touches -- into a wave-private LDS tile (row stride D + 4 floats), from
-// which every lane then reads its own row.  D <= 64.
-template <int D>
-struct GatherDot {
-    static constexpr int LPR = D / 4;   // 16 bytes per lane
-    static constexpr int G = 64 / LPR;  // rows per load instruction
-    static constexpr int RS = D + 4;
-    static constexpr int FLOATS = 64 * RS;
-    static __device__ __forceinline__ float run(float* T, const float* __restrict__ a, const float* __restrict__ X,
-                                                int ld, int row_l, int nk, int lane) {
-        const int grp = lane / LPR, cl = lane % LPR;
-        constexpr int UN = 8;
-        for (int kb = 0; kb < nk; kb += UN * G) {
-            float4 x[UN];
-#pragma unroll
-            for (int j = 0; j < UN; ++j) {
-                const int rr = __shfl(row_l, (kb + j * G + grp) & 63, 64);
-                x[j] = reinterpret_cast<const float4*>(X + (size_t)rr * ld)[cl];
-            }
-#pragma unroll
-            for (int j = 0; j < UN; ++j)
-                *reinterpret_cast<float4*>(T + ((kb + j * G + grp) & 63) * RS + 4 * cl) = x[j];
-        }
-        // same-wave LDS accesses complete in order: no barrier
-        const float4* t4 = reinterpret_cast<const float4*>(T + lane * RS);
-        const float4* a4 = reinterpret_cast<const float4*>(a);
-        float s = 0.f;
-#pragma unroll
-        for (int t = 0; t < D / 4; ++t) {
-            const float4 x = t4[t], y = a4[t];
-            s = fmaf(x.x, y.x, s);
-            s = fmaf(x.y, y.y, s);
-            s = fmaf(x.z, y.z, s);
-            s = fmaf(x.w, y.w, s);
-        }
-        return s;
-    }
-};
-
+// (Head size 128 only; smaller heads use the LDS-free primitives of gather_ops.h.)
 // acc += sum_k w_k * X[col_k][:] over the entries of one CSR row, the entries being held one per lane in chunks
 // of 64 (w_l, col_l).  VEC floats per lane: D/VEC lanes cover one X row and 64*VEC/D entries are processed per load
 // instruction.  16-byte loads (eight entries per instruction at d = 32) because the vector-memory path charges per
@@ -156,7 +116,7 @@ struct RowAcc {
 // One wavefront per (head, row).  K is row-major here ([NB][L][D], transposed copy in the workspace).  ST: the heads
 // are [B][H][L][D] views located by `ly` (head_slice) instead of contiguous slices.
 template <int D, bool MASK, bool ST>
-__global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
+__global__ __launch_bounds__(64 * ELEM_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 6 : D == 64 ? 3 : 2, 8))) void elem_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O,
     const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale, Layouts ly) {
@@ -176,18 +136,57 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
 
     float m = MASK ? 0.f : -100.f;
     if constexpr (D <= 64) {
-        __shared__ __attribute__((aligned(16))) float lds_rows[ELEM_WAVES][GatherDot<D>::FLOATS];
-        float* T = lds_rows[threadIdx.x >> 6];
+        // LDS-free gathers (gather_ops.h): the chunk's entries follow the lane order of the gather groups
+        constexpr int LPR = D / 4, KEEP = 2;
+        const int ent = gather_entry_of_lane<LPR>(lane);
+        const f32x4 q4 = reinterpret_cast<const f32x4*>(q)[lane % LPR];
+        float vk[KEEP];  // the logits of the first chunks stay in registers; longer rows go back to what they stored
         for (int c0 = 0; c0 < cnt; c0 += 64) {
-            const int k = c0 + lane;
+            const int k = c0 + ent;
             const int col = k < cnt ? cj[k] : 0;
-            float v = GatherDot<D>::run(T, q, K + ib, ild, col, min(64, cnt - c0), lane) * scale;
+            float v = gather_dot<LPR>(q4, K + ib, ild, col, min(64, cnt - c0), lane) * scale;
             if (k < cnt) {
                 if (MASK) v -= pen[(size_t)bh * L + col];
                 p[k] = v;
                 m = fmaxf(m, v);
             }
+#pragma unroll
+            for (int c = 0; c < KEEP; ++c)
+                if (c0 == 64 * c) vk[c] = v;
         }
+        m = wave_max(m);
+        float z = 0.f;
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + ent;
+            float v = 0.f;
+#pragma unroll
+            for (int c = 0; c < KEEP; ++c)
+                if (c0 == 64 * c) v = vk[c];
+            if (c0 >= 64 * KEEP && k < cnt) v = p[k];
+            if (k < cnt) z += __expf(v - m);
+        }
+        z = wave_sum(z);
+        z += (float)(L - cnt) * __expf(-m);
+        const float r = 1.0f / z;
+        GatherRowAcc<LPR> acc;
+        acc.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + ent;
+            float v = 0.f, w = 0.f;
+#pragma unroll
+            for (int c = 0; c < KEEP; ++c)
+                if (c0 == 64 * c) v = vk[c];
+            int col = 0;
+            if (k < cnt) {
+                if (c0 >= 64 * KEEP) v = p[k];
+                w = __expf(v - m) * r;
+                col = cj[k];
+                p[k] = w;
+            }
+            acc.chunk(w, col, min(64, cnt - c0), V + ib, ild, lane);
+        }
+        const f32x4 tot = acc.total();
+        if (lane < LPR) reinterpret_cast<f32x4*>(O + ob + (size_t)row * old_)[lane] = tot;
     } else {
         for (int k = lane; k < cnt; k += 64) {
             int col = cj[k];
@@ -196,34 +195,34 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_fwd_kernel(
             p[k] = v;
             m = fmaxf(m, v);
         }
-    }
-    m = wave_max(m);
-    float z = 0.f;
-    for (int k = lane; k < cnt; k += 64) z += __expf(p[k] - m);
-    z = wave_sum(z);
-    z += (float)(L - cnt) * __expf(-m);
-    const float r = 1.0f / z;
+        m = wave_max(m);
+        float z = 0.f;
+        for (int k = lane; k < cnt; k += 64) z += __expf(p[k] - m);
+        z = wave_sum(z);
+        z += (float)(L - cnt) * __expf(-m);
+        const float r = 1.0f / z;
 
-    RowAcc<D> acc;
-    acc.clear();
-    for (int c0 = 0; c0 < cnt; c0 += 64) {
-        const int k = c0 + lane;
-        float w = 0.f;
-        int col = 0;
-        if (k < cnt) {
-            w = __expf(p[k] - m) * r;
-            col = cj[k];
-            p[k] = w;
+        RowAcc<D> acc;
+        acc.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + lane;
+            float w = 0.f;
+            int col = 0;
+            if (k < cnt) {
+                w = __expf(p[k] - m) * r;
+                col = cj[k];
+                p[k] = w;
+            }
+            acc.chunk(w, col, min(64, cnt - c0), V + ib, ild, lane);
         }
-        acc.chunk(w, col, min(64, cnt - c0), V + ib, ild, lane);
+        acc.finish(O + ob + (size_t)row * old_, lane);
     }
-    acc.finish(O + ob + (size_t)row * old_, lane);
 }
 
 // Row pass of the backward: dP = dO.V^T on the pattern, g = sum_row dP*P, dS = (dP*P - P*g)*scale
 // (written to the caller's dS scratch for the column pass), dQ = dS.K.
 template <int D, bool ST>
-__global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
+__global__ __launch_bounds__(64 * ELEM_WAVES) __attribute__((amdgpu_waves_per_eu(D <= 32 ? 6 : D == 64 ? 3 : 2, 8))) void elem_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ P,
     const float* __restrict__ dO, float* __restrict__ dS, float* __restrict__ dQ,
     const int* __restrict__ offs, const int* __restrict__ cols, int L, int NB, int nnz, float scale, Layouts ly) {
@@ -245,41 +244,77 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_row_kernel(
 
     float g = 0.f;
     if constexpr (D <= 64) {
-        __shared__ __attribute__((aligned(16))) float lds_rows[ELEM_WAVES][GatherDot<D>::FLOATS];
-        float* T = lds_rows[threadIdx.x >> 6];
+        constexpr int LPR = D / 4, KEEP = 2;
+        const int ent = gather_entry_of_lane<LPR>(lane);
+        const f32x4 go4 = reinterpret_cast<const f32x4*>(go)[lane % LPR];
+        float tk[KEEP], pk[KEEP];  // dP*P and P of the first chunks stay in registers
         for (int c0 = 0; c0 < cnt; c0 += 64) {
-            const int k = c0 + lane;
+            const int k = c0 + ent;
             const int col = k < cnt ? cj[k] : 0;
-            const float dp = GatherDot<D>::run(T, go, V + ib, ild, col, min(64, cnt - c0), lane);
+            const float dp = gather_dot<LPR>(go4, V + ib, ild, col, min(64, cnt - c0), lane);
+            float t = 0.f, pv = 0.f;
             if (k < cnt) {
-                const float t = dp * p[k];
-                ds[k] = t;
+                pv = p[k];
+                t = dp * pv;
+                if (c0 >= 64 * KEEP) ds[k] = t;
                 g += t;
             }
+#pragma unroll
+            for (int c = 0; c < KEEP; ++c)
+                if (c0 == 64 * c) {
+                    tk[c] = t;
+                    pk[c] = pv;
+                }
         }
+        g = wave_sum(g);
+        GatherRowAcc<LPR> acc;
+        acc.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + ent;
+            float t = 0.f, pv = 0.f, w = 0.f;
+#pragma unroll
+            for (int c = 0; c < KEEP; ++c)
+                if (c0 == 64 * c) {
+                    t = tk[c];
+                    pv = pk[c];
+                }
+            int col = 0;
+            if (k < cnt) {
+                if (c0 >= 64 * KEEP) {
+                    t = ds[k];
+                    pv = p[k];
+                }
+                w = (t - pv * g) * scale;
+                col = cj[k];
+                ds[k] = w;
+            }
+            acc.chunk(w, col, min(64, cnt - c0), K + ib, ild, lane);
+        }
+        const f32x4 tot = acc.total();
+        if (lane < LPR) reinterpret_cast<f32x4*>(dQ + gb + (size_t)row * gld)[lane] = tot;
     } else {
         for (int k = lane; k < cnt; k += 64) {
             float t = row_dot<D>(go, V + ib + (size_t)cj[k] * ild) * p[k];
             ds[k] = t;
             g += t;
         }
-    }
-    g = wave_sum(g);
+        g = wave_sum(g);
 
-    RowAcc<D> acc;
-    acc.clear();
-    for (int c0 = 0; c0 < cnt; c0 += 64) {
-        const int k = c0 + lane;
-        float w = 0.f;
-        int col = 0;
-        if (k < cnt) {
-            w = (ds[k] - p[k] * g) * scale;
-            col = cj[k];
-            ds[k] = w;
+        RowAcc<D> acc;
+        acc.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int k = c0 + lane;
+            float w = 0.f;
+            int col = 0;
+            if (k < cnt) {
+                w = (ds[k] - p[k] * g) * scale;
+                col = cj[k];
+                ds[k] = w;
+            }
+            acc.chunk(w, col, min(64, cnt - c0), K + ib, ild, lane);
         }
-        acc.chunk(w, col, min(64, cnt - c0), K + ib, ild, lane);
+        acc.finish(dQ + gb + (size_t)row * gld, lane);
     }
-    acc.finish(dQ + gb + (size_t)row * gld, lane);
 }
 
 // Column pass of the backward: dK_j = sum_i dS_ij Q_i, dV_j = sum_i P_ij dO_i over the transposed index.
@@ -304,25 +339,52 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
     const float* p = P + (size_t)bh * nnz;
     const float* ds = dS + (size_t)bh * nnz;
 
-    RowAcc<D> ak, av;
-    ak.clear();
-    av.clear();
-    for (int c0 = 0; c0 < cnt; c0 += 64) {
-        const int e = c0 + lane;
-        float wk = 0.f, wv = 0.f;
-        int row = 0;
-        if (e < cnt) {
-            int pos = cpos[c0p + e];
-            row = crow[c0p + e];
-            wk = ds[pos];
-            wv = p[pos];
+    if constexpr (D <= 64) {
+        constexpr int LPR = D / 4;
+        const int ent = gather_entry_of_lane<LPR>(lane);
+        GatherRowAcc<LPR> ak, av;
+        ak.clear();
+        av.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int e = c0 + ent;
+            float wk = 0.f, wv = 0.f;
+            int row = 0;
+            if (e < cnt) {
+                int pos = cpos[c0p + e];
+                row = crow[c0p + e];
+                wk = ds[pos];
+                wv = p[pos];
+            }
+            const int nk = min(64, cnt - c0);
+            ak.chunk(wk, row, nk, Q + ib, ild, lane);
+            av.chunk(wv, row, nk, dO + ob, old_, lane);
         }
-        const int nk = min(64, cnt - c0);
-        ak.chunk(wk, row, nk, Q + ib, ild, lane);
-        av.chunk(wv, row, nk, dO + ob, old_, lane);
+        const f32x4 tk = ak.total(), tv = av.total();
+        if (lane < LPR) {
+            reinterpret_cast<f32x4*>(dK + gb + (size_t)col * gld)[lane] = tk;
+            reinterpret_cast<f32x4*>(dV + gb + (size_t)col * gld)[lane] = tv;
+        }
+    } else {
+        RowAcc<D> ak, av;
+        ak.clear();
+        av.clear();
+        for (int c0 = 0; c0 < cnt; c0 += 64) {
+            const int e = c0 + lane;
+            float wk = 0.f, wv = 0.f;
+            int row = 0;
+            if (e < cnt) {
+                int pos = cpos[c0p + e];
+                row = crow[c0p + e];
+                wk = ds[pos];
+                wv = p[pos];
+            }
+            const int nk = min(64, cnt - c0);
+            ak.chunk(wk, row, nk, Q + ib, ild, lane);
+            av.chunk(wv, row, nk, dO + ob, old_, lane);
+        }
+        ak.finish(dK + gb + (size_t)col * gld, lane);
+        av.finish(dV + gb + (size_t)col * gld, lane);
     }
-    ak.finish(dK + gb + (size_t)col * gld, lane);
-    av.finish(dV + gb + (size_t)col * gld, lane);
 }
 
 // =================================================================================================
