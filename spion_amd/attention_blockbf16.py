@@ -116,6 +116,7 @@ class BlockAttentionBF16(nn.Module):
             _lib.check_error("spion_block_bf16_init")
         self.attn_handle = attn_handle
         self.csr_cache = CsrCache(handle=attn_handle)
+        self.reads_views = True  # bf16 heads that are views of projections are read in place
 
     def forward(self, query, key, value, mask, mat):
         return _BlockBF16Function.apply(query, key, value, mask, mat, self), 0

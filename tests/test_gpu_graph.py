@@ -41,13 +41,23 @@ def _eager_step(module, args, q, k, v, do):
     return out.detach().clone(), [t.grad.clone() for t in (q, k, v)]
 
 
-@pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16", "block_views", "blockmask_views", "dense_views"])
+@pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16", "block_views", "blockmask_views", "dense_views",
+                                  "bf16_views", "hybrid", "hybrid_views", "hybridmask_views"])
 def test_whole_step_graph_replays_match_eager(kind):
     views = kind.endswith("_views")  # heads as views of [B, L, H*d] projections: the strided entry points
     kind = kind.split("_")[0]
     B, H, L, d, bs = 2, 2, 256, 32, 32
+    hybrid = kind.startswith("hybrid")  # element-sparse pattern (window + scattered entries): seven launches a step
+    if hybrid:
+        bs = 1
+        sm, off, col = workloads.window_random_csr(L, 40, 100, seed=3)
+        pattern = np.zeros((L, L), dtype=np.float32)
+        pattern[np.repeat(np.arange(L), sm), col] = 1.0
+        mat = torch.from_numpy(pattern).cuda()
+        kind = "blockmask" if kind == "hybridmask" else "block"
+    else:
+        mat = torch.from_numpy(workloads.band_random_block_mask(L // bs, 1, extra_frac=0.1, seed=3)).cuda()
     cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
-    mat = torch.from_numpy(workloads.band_random_block_mask(L // bs, 1, extra_frac=0.1, seed=3)).cuda()
     key_mask = torch.ones(B, L)
     key_mask[1, 200:] = 0
     key_mask = key_mask.cuda()
@@ -70,6 +80,9 @@ def test_whole_step_graph_replays_match_eager(kind):
     for t in (q, k, v):
         t.requires_grad_()
     ref_out, ref_grads = _eager_step(module, args, q, k, v, do)
+    if hybrid:
+        from spion_amd import _lib
+        assert _lib.core().spion_last_path(module.attn_handle) == 3
     graph, out, static_grads = _capture_step(module, args, q, k, v, do)
     for replay in range(4):
         out.detach().zero_()
