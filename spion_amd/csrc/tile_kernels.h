@@ -336,17 +336,23 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // reference's ABI asks for) instead of feature-major [NB][D][L].  For d = 64 every lane then reads 128 bytes of
 // its own row (one cache line per lane), which is slower than the feature-major form: the row-major entry points
 // for contiguous heads therefore still transpose once; only the strided entry points use it.
+// MAXT == 4 at d = 32 (at most four logit tiles per wavefront) fits three wavefronts per SIMD: the buffer of the
+// final reduction then shares the space of the wave-private tiles (a barrier in between).
 template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false>
-SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(D == 32 && MAXT == 4 ? 3 : 2, D == 32 && MAXT == 4 ? 3 : 2)))
+void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
     const int* __restrict__ rdesc, const int* __restrict__ tcol, int L, int nbr,
     int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
     static_assert(!ST || KROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
+    constexpr bool SHARE = D == 32 && MAXT == 4 && WAVES > 1;  // reduction buffer inside the tile space
+    __shared__ float lds_own[!SHARE && WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 && MAXT > 0 ? 2 : 1) * 32 * TS];
+    static_assert(!SHARE || WAVES * 2 * 32 * TS >= WAVES * 16 * 64, "the reduction fits in the tile space");
+    float* lds = SHARE ? &lds_t[0][0] : lds_own;
     // this launch covers strips s0 .. s0+ns-1 of the longest-first order of every head
     const int item = xcd_remap(blockIdx.x, ns * NB);
     int bh, pos;
@@ -579,6 +585,7 @@ SPION_TILE_KERNEL(WAVES) void tile_fwd_kernel(
                 });
         }
     }
+    if constexpr (SHARE) __syncthreads();  // every wavefront is done with its tiles
     if (!ST && Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);
     else reduce_store<D, WAVES>(o, O + ob, I * 32, w, li, h, lds, old_);
 }
