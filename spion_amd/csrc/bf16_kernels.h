@@ -372,6 +372,119 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
 }
 
 // -------------------------------------------------------------------------------------------------
+// Forward, two strips per wavefront: for masks of 64 x 64 blocks and larger, strips 2p and 2p+1 hold the same block
+// columns, so one wavefront takes both: every K and V tile is fetched, copied to LDS and read back as an operand
+// once for the two strips' chains, and the two softmax updates are independent instruction streams.  pair_list:
+// four pair indices per work-group (-1: none); pairs whose strips are long enough to be cut into chunks stay with
+// bf16_fwd_kernel.
+// -------------------------------------------------------------------------------------------------
+template <int D, bool MASK>
+SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ pair_list, int n_wg, int L, int NB, float scale) {
+    typedef LdsTile<D> LT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int pr = pair_list[(item % n_wg) * 4 + w];
+    if (pr < 0) return;
+    const int I = 2 * pr;
+    const int t0 = trp[I], cnt = trp[I + 1] - t0;
+    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rO = make_rsrc(O + hb, hbytes);
+    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int r_voff = li * D * 2 + h * D;
+    const int t_voff = l * 16, t_step = 1024, t_bytes = 32 * D * 2;
+    char* Tk = lds_t[w][0];
+    char* Tv = lds_t[w][1];
+    const int tbase = LT::lane_base(l);
+    const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+
+    bf16x8 q0[D / 16], q1[D / 16];
+    ldb_rows<D>(rQ, r_voff, I * t_bytes, q0);
+    ldb_rows<D>(rQ, r_voff, (I + 1) * t_bytes, q1);
+    float m0 = MASK ? 0.f : -100.f, z0 = 0.f, m1 = m0, z1 = 0.f;
+    f32x16 o0[D / 32], o1[D / 32];
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c) {
+        o0[c] = splat16(0.f);
+        o1[c] = splat16(0.f);
+    }
+    auto update = [&](const f32x16& s, float& m, float& z, f32x16 (&o)[D / 32], bf16x8 (&pb)[2]) {
+        const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
+        if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
+            const float mn = t2 > m + BF16_LAZY ? t2 : m;
+            const float f = __builtin_amdgcn_exp2f(m - mn);
+            z *= f;
+#pragma unroll
+            for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
+            m = mn;
+        }
+        float p[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
+            z += p[r];
+        }
+        pack16(p, pb);
+    };
+    struct Pre {
+        u32x4 k[D / 16], v[D / 16];
+        float pj[MASK ? 16 : 1];
+    };
+    Pre xa, xb;
+    tile_pipeline(
+        cnt, xa, xb,
+        [&](Pre& x, int i) {
+            const int J = tcol[t0 + min(i, cnt - 1)];
+            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
+            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
+            if constexpr (MASK) {
+                float pj[16];
+                ldr_4x4(rM, 16 * h, J * 128, pj);
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
+            }
+        },
+        [&](Pre& c, int) {
+            LT::put_raw(Tk, l, c.k);
+            LT::put_raw(Tv, l, c.v);
+            bf16x8 kr[D / 16], vt[D / 32][2];
+            LT::get_rows(Tk, li, h, kr);
+            LT::get_tile_t(Tv, tbase, vt);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
+            }
+            const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
+            const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
+            bf16x8 pb0[2], pb1[2];
+            update(s0, m0, z0, o0, pb0);
+            update(s1, m1, z1, o1, pb1);
+            mma_tile_bf16<D>(vt, pb0, o0);
+            mma_tile_bf16<D>(vt, pb1, o1);
+        });
+    const int off_pattern = L - cnt * 32;
+    float* lds_unused = nullptr;
+    auto finish = [&](float m, float z, f32x16 (&o)[D / 32], int strip) {
+        z = half_swap_sum(z);
+        if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);
+        const float rinv = 1.0f / z;
+#pragma unroll
+        for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
+        if (h == 0) Lse[(size_t)bh * L + strip * 32 + li] = m + __builtin_amdgcn_logf(z);
+        store_rows_bf16<D>(o, rO, D, strip * 32, false, w, li, h, lds_unused);
+    };
+    finish(m0, z0, o0, I);
+    finish(m1, z1, o1, I + 1);
+}
+
+// -------------------------------------------------------------------------------------------------
 // Backward, row pass: g_i = dO_i . O_i, P and dP recomputed per tile, dS' = P*(dP - g), dQ += dS'.K_J;
 // the 1/sqrt(d) is applied to the 32 x d result.  Gneg receives -g for the column pass.
 // -------------------------------------------------------------------------------------------------

@@ -404,6 +404,9 @@ struct PatternIndex {
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     // per strip in launch order, {strip, first tile, tiles, P offset}: row pass, forward, column pass
     int *d_rdesc = nullptr, *d_fdesc = nullptr, *d_cdesc = nullptr;
+    int *d_pair_list = nullptr, *d_wg_long = nullptr;  // bf16 forward by strip pairs
+    int n_wg_pair = 0, n_wg_long = 0;
+    bool bf16_pairs = false;
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // element-sparse pattern whose well-filled 32x32 tiles run on the MFMA units (hybrid_kernels.h)
     bool hybrid = false;
@@ -651,7 +654,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         return o;
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
-    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0;
+    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0, o_plist = 0, o_longwg = 0;
     size_t hyb_off[14] = {};
     if (tiled) {
         const int nt = (int)tcol.size();
@@ -725,6 +728,32 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         o_rdesc = append(rdesc);
         o_fdesc = append(fdesc);
         o_cdesc = append(cdesc);
+        {
+            // strips 2k and 2k+1 with the same block columns (masks of 64 x 64 blocks and larger): lists for the bf16
+            // forward that gives one wavefront both strips of a pair -- four short pairs per work-group, and the
+            // work-groups of the chunked long strips on their own
+            bool pairs = nbr % 2 == 0 && nt > 0;
+            for (int k = 0; pairs && k < nbr / 2; ++k) {
+                const int a0 = trp[2 * k], a1 = trp[2 * k + 1], n0 = a1 - a0, n1 = trp[2 * k + 2] - a1;
+                pairs = n0 == n1 && std::equal(tcol.begin() + a0, tcol.begin() + a1, tcol.begin() + a1);
+            }
+            if (pairs) {
+                std::vector<int> plist, longwg;
+                for (int k = 0; k < nbr / 2; ++k)
+                    if (trp[2 * k + 1] - trp[2 * k] <= wgr.chunk) plist.push_back(k);
+                while (plist.size() % 4) plist.push_back(-1);
+                for (size_t g = 0; g + 3 < wgr.wg.size(); g += 4)
+                    if (wgr.wg[g] == wgr.wg[g + 1] && wgr.wg[g] >= 0)
+                        longwg.insert(longwg.end(), wgr.wg.begin() + g, wgr.wg.begin() + g + 4);
+                pi.n_wg_pair = (int)plist.size() / 4;
+                pi.n_wg_long = (int)longwg.size() / 4;
+                if (plist.empty()) plist.push_back(-1);
+                if (longwg.empty()) longwg.push_back(-1);
+                o_plist = append(plist);
+                o_longwg = append(longwg);
+                pi.bf16_pairs = pi.n_wg_pair > 0;
+            }
+        }
         pi.n_wg_row = (int)wgr.wg.size() / 4;
         pi.n_wg_col = (int)wgc.wg.size() / 4;
         pi.chunk_row = wgr.chunk;
@@ -873,6 +902,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcp = pi.d_blob + o_tcp;
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
         pi.d_rdesc = pi.d_blob + o_rdesc;
+        pi.d_pair_list = pi.d_blob + o_plist;
+        pi.d_wg_long = pi.d_blob + o_longwg;
         pi.d_fdesc = pi.d_blob + o_fdesc;
         pi.d_cdesc = pi.d_blob + o_cdesc;
         pi.d_wg_row = pi.d_blob + o_wgr;
@@ -1671,11 +1702,23 @@ static void bf16_forward_impl(SparseAttn* a, const void* Q, const void* K, const
     const dim3 grid(pi.n_wg_row * a->NB), block(64 * BF16_WAVES), grid_m(pi.n_long_row * a->NB * (32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
     __bf16* o = static_cast<__bf16*>(Out);
+    static const bool no_pairs = getenv("SPION_BF16_NO_PAIRS") != nullptr;
+    // (with the key mask at d = 64 the pair kernel would spill 56 registers: one strip per wavefront there)
+    const bool by_pairs = !ST && pi.bf16_pairs && !no_pairs && !(a->d == 64 && Mask);
 #define SPION_LAUNCH(DD, MM)                                                                                         \
     do {                                                                                                             \
-        hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,      \
-                           pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,         \
-                           pi.slots_row, pi.chunk_row, ly);                                                          \
+        if (by_pairs) {                                                                                              \
+            if (pi.n_wg_long)                                                                                        \
+                hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), dim3(pi.n_wg_long * a->NB), block, 0,              \
+                                   a->hdr.stream, q, k, v, Mask, o, Lse, pi.d_trp, pi.d_tcol, pi.d_wg_long,          \
+                                   pi.n_wg_long, a->L, a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row, ly); \
+            hipLaunchKernelGGL((bf16_fwd_pair_kernel<DD, MM>), dim3(pi.n_wg_pair * a->NB), block, 0, a->hdr.stream,  \
+                               q, k, v, Mask, o, Lse, pi.d_trp, pi.d_tcol, pi.d_pair_list, pi.n_wg_pair, a->L,       \
+                               a->NB, a->scale);                                                                     \
+        } else                                                                                                       \
+            hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,  \
+                               pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,     \
+                               pi.slots_row, pi.chunk_row, ly);                                                      \
         if (pi.n_long_row)                                                                                           \
             hipLaunchKernelGGL((bf16_merge_fwd_kernel<DD, ST>), grid_m, dim3(256), 0, a->hdr.stream, a->ws_part,     \
                                pi.d_long_row, pi.n_long_row, pi.slots_row, o, Lse, a->L, ly.out, ly.H);              \

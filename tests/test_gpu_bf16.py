@@ -220,15 +220,19 @@ def _bf16_head_views(B, H, L, d, layout, n, seed, fill=None):
     return bufs, views
 
 
-@pytest.mark.parametrize("d,layout,glob,with_mask", [(32, "proj", False, False), (64, "fused", False, True),
-                                                     (64, "proj", True, False), (32, "fused", True, True)])
-def test_bf16_strided_entry_points(d, layout, glob, with_mask):
+@pytest.mark.parametrize("d,layout,glob,with_mask,bs", [(32, "proj", False, False, 32), (64, "fused", False, True, 32),
+                                                        (64, "proj", True, False, 32), (32, "fused", True, True, 32),
+                                                        (64, "proj", True, False, 64), (32, "fused", False, True, 64),
+                                                        (32, "proj", True, False, 128)])
+def test_bf16_strided_entry_points(d, layout, glob, with_mask, bs):
     """spion_block_bf16_attn_{forward,backward}_strided: bf16 heads read and written in place in the memory of
     [B, L, H*d] projections (or of one fused, padded buffer).  Same kernels and arithmetic as the contiguous entry
     points on contiguous copies -- long strips cut into chunks and merged included: bit-identical results; the
-    padding between the heads' rows is left alone."""
+    padding between the heads' rows is left alone.  With blocks of 64 x 64 and larger the contiguous forward takes two
+    strips per wavefront and the strided one a strip per wavefront: two kernels, the same arithmetic in the same
+    order."""
     import ctypes
-    B, H, L, bs = 2, 2, 1024, 32
+    B, H, L = 2, 2, 1024
     NB = B * H
     mat = _mask(L // bs, 0.1, seed=21, global_block=glob)
     sm, off, col = osa.build_csr_from_block_mask(mat, bs)
