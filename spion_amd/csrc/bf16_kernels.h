@@ -238,22 +238,29 @@ constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
 // -------------------------------------------------------------------------------------------------
 // Forward: one sweep per block row with a lazily raised running maximum.
 // -------------------------------------------------------------------------------------------------
-template <int D, bool MASK, bool ST>
-SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
-    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
+// The LDS space of a forward work-group: two wave-private tiles per wavefront (reused for the partial results of a
+// shared strip) and the row statistics the wavefronts of a shared strip exchange.
+template <int D>
+struct Bf16FwdLds {
     typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    __shared__ float lds_m[BF16_WAVES][32], lds_z[BF16_WAVES][32];
+    __attribute__((aligned(16))) char t[BF16_WAVES][2][LT::BYTES];
+    float m[BF16_WAVES][32], z[BF16_WAVES][32];
+};
+
+// One strip (or one chunk of a long strip, shared by the four wavefronts) per wavefront.
+template <int D, bool MASK, bool ST>
+__device__ __forceinline__ void bf16_fwd_strip(
+    Bf16FwdLds<D>& lds, const StripAssign sa, int bh, int w, const __bf16* __restrict__ Q,
+    const __bf16* __restrict__ K, const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O,
+    float* __restrict__ Lse, const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale,
+    float* __restrict__ Part, int n_slots, int chunk, const Layouts& ly) {
+    typedef LdsTile<D> LT;
+    auto& lds_t = lds.t;
+    auto& lds_m = lds.m;
+    auto& lds_z = lds.z;
     float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
     static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
-    if (sa.strip < 0) return;  // only in entries of independent strips: no barrier is skipped
+    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int I = sa.strip;
     const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
     const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
@@ -371,6 +378,21 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
     store_rows_bf16<D>(o, rO, old_, I * 32, sa.coop, w, li, h, lds_o);
 }
 
+template <int D, bool MASK, bool ST>
+SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
+    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
+    __shared__ Bf16FwdLds<D> lds;
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index();
+    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
+    if (sa.strip < 0) return;  // only in entries of independent strips: no barrier is skipped
+    bf16_fwd_strip<D, MASK, ST>(lds, sa, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale, Part, n_slots, chunk, ly);
+}
+
 // -------------------------------------------------------------------------------------------------
 // Forward, two strips per wavefront: for masks of 64 x 64 blocks and larger, strips 2p and 2p+1 hold the same block
 // columns, so one wavefront takes both: every K and V tile is fetched, copied to LDS and read back as an operand
@@ -379,17 +401,13 @@ SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
 // bf16_fwd_kernel.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK>
-SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
-    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ pair_list, int n_wg, int L, int NB, float scale) {
+__device__ __forceinline__ void bf16_fwd_pair(
+    Bf16FwdLds<D>& lds, int pr, int bh, int w, const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+    const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse,
+    const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale) {
     typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int pr = pair_list[(item % n_wg) * 4 + w];
-    if (pr < 0) return;
+    auto& lds_t = lds.t;
+    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int I = 2 * pr;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
@@ -482,6 +500,32 @@ SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
     };
     finish(m0, z0, o0, I);
     finish(m1, z1, o1, I + 1);
+}
+
+// Work-group list of the paired forward: entries {a, a, c, slot} are chunk c of long strip a, shared by the four
+// wavefronts (bf16_fwd_strip; these entries come first), entries {p0, p1, p2, p3} four pairs of strips, one per
+// wavefront (-1: none).  One launch for both kinds: the few work-groups of the long strips would otherwise set the
+// length of a launch of their own (32 us for configuration 5).
+template <int D, bool MASK>
+SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
+    const int* __restrict__ tcol, const int* __restrict__ list, int n_wg, int L, int NB, float scale,
+    float* __restrict__ Part, int n_slots, int chunk) {
+    __shared__ Bf16FwdLds<D> lds;
+    const int item = xcd_remap(blockIdx.x, n_wg * NB);
+    const int bh = item / n_wg;
+    const int w = wave_index();
+    const int4 e = reinterpret_cast<const int4*>(list)[item % n_wg];
+    if (e.x == e.y) {  // uniform over the work-group
+        const StripAssign sa = strip_of_wave(list, item % n_wg, w);
+        bf16_fwd_strip<D, MASK, false>(lds, sa, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale, Part, n_slots, chunk,
+                                       Layouts{});
+        return;
+    }
+    const int pr = w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w;
+    if (pr < 0) return;
+    bf16_fwd_pair<D, MASK>(lds, pr, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale);
 }
 
 // -------------------------------------------------------------------------------------------------

@@ -404,8 +404,8 @@ struct PatternIndex {
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     // per strip in launch order, {strip, first tile, tiles, P offset}: row pass, forward, column pass
     int *d_rdesc = nullptr, *d_fdesc = nullptr, *d_cdesc = nullptr;
-    int *d_pair_list = nullptr, *d_wg_long = nullptr;  // bf16 forward by strip pairs
-    int n_wg_pair = 0, n_wg_long = 0;
+    int* d_pair_list = nullptr;  // bf16 forward by strip pairs: chunks of long strips, then four pairs per work-group
+    int n_wg_pair = 0;
     bool bf16_pairs = false;
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // element-sparse pattern whose well-filled 32x32 tiles run on the MFMA units (hybrid_kernels.h)
@@ -654,7 +654,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         return o;
     };
     size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
-    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0, o_plist = 0, o_longwg = 0;
+    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0, o_plist = 0;
     size_t hyb_off[14] = {};
     if (tiled) {
         const int nt = (int)tcol.size();
@@ -745,13 +745,12 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
                 for (size_t g = 0; g + 3 < wgr.wg.size(); g += 4)
                     if (wgr.wg[g] == wgr.wg[g + 1] && wgr.wg[g] >= 0)
                         longwg.insert(longwg.end(), wgr.wg.begin() + g, wgr.wg.begin() + g + 4);
-                pi.n_wg_pair = (int)plist.size() / 4;
-                pi.n_wg_long = (int)longwg.size() / 4;
-                if (plist.empty()) plist.push_back(-1);
+                pi.bf16_pairs = !plist.empty();
+                // one list: the chunks of the long strips first, then the pairs, four to a work-group
+                longwg.insert(longwg.end(), plist.begin(), plist.end());
+                pi.n_wg_pair = (int)longwg.size() / 4;
                 if (longwg.empty()) longwg.push_back(-1);
-                o_plist = append(plist);
-                o_longwg = append(longwg);
-                pi.bf16_pairs = pi.n_wg_pair > 0;
+                o_plist = append(longwg);
             }
         }
         pi.n_wg_row = (int)wgr.wg.size() / 4;
@@ -903,7 +902,6 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
         pi.d_rdesc = pi.d_blob + o_rdesc;
         pi.d_pair_list = pi.d_blob + o_plist;
-        pi.d_wg_long = pi.d_blob + o_longwg;
         pi.d_fdesc = pi.d_blob + o_fdesc;
         pi.d_cdesc = pi.d_blob + o_cdesc;
         pi.d_wg_row = pi.d_blob + o_wgr;
@@ -1707,15 +1705,11 @@ static void bf16_forward_impl(SparseAttn* a, const void* Q, const void* K, const
     const bool by_pairs = !ST && pi.bf16_pairs && !no_pairs && !(a->d == 64 && Mask);
 #define SPION_LAUNCH(DD, MM)                                                                                         \
     do {                                                                                                             \
-        if (by_pairs) {                                                                                              \
-            if (pi.n_wg_long)                                                                                        \
-                hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), dim3(pi.n_wg_long * a->NB), block, 0,              \
-                                   a->hdr.stream, q, k, v, Mask, o, Lse, pi.d_trp, pi.d_tcol, pi.d_wg_long,          \
-                                   pi.n_wg_long, a->L, a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row, ly); \
+        if (by_pairs)                                                                                                \
             hipLaunchKernelGGL((bf16_fwd_pair_kernel<DD, MM>), dim3(pi.n_wg_pair * a->NB), block, 0, a->hdr.stream,  \
                                q, k, v, Mask, o, Lse, pi.d_trp, pi.d_tcol, pi.d_pair_list, pi.n_wg_pair, a->L,       \
-                               a->NB, a->scale);                                                                     \
-        } else                                                                                                       \
+                               a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row);                             \
+        else                                                                                                         \
             hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,  \
                                pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,     \
                                pi.slots_row, pi.chunk_row, ly);                                                      \
