@@ -22,6 +22,13 @@ void spion_set_backward_passes(void* handle, int mask);
  * waited for the stream), which = 1 -> analyses made from host arrays (spion_register_pattern).  -1 otherwise. */
 int spion_debug_counter(void* handle, int which);
 
+/* Environment switches read once per process, for A/B measurements only (results are the same either way):
+ *   SPION_NO_FWD_SPLIT   the fp32 tile forward runs all strips in one launch, eight logit tiles per wavefront
+ *                        (default: strips of at most 16 tiles in a launch of their own, three work-groups to a CU);
+ *   SPION_BF16_NO_PAIRS  the bf16 forward takes one strip per wavefront on every pattern (default: two strips per
+ *                        wavefront on masks of 64 x 64 blocks and larger).
+ * SPION_QUIET and SPION_ABORT_ON_ERROR (error reporting) are described in spion_hip.h. */
+
 #ifdef __cplusplus
 }
 #endif
