@@ -230,7 +230,9 @@ int spion_register_pattern(void* handle, const int* Offsets, const int* Columns,
                            const int* host_Offsets, const int* host_Columns);
 
 /* Which kernel family the last forward/backward of a sparse handle used:
- * 0 = none yet, 1 = MFMA 32x32 tile path, 2 = element (gather) path. */
+ * 0 = none yet, 1 = MFMA 32x32 tile path, 2 = element (gather) path, 3 = hybrid path (element-sparse pattern
+ * whose well-filled 32x32 tiles run on the MFMA units, the rest on the gather kernels).  For 2 and 3 the backward
+ * needs the dS scratch.  It describes the most recent call on the handle, not a particular pattern. */
 int spion_last_path(void* handle);
 
 /* Most recent failure recorded by a call on THIS handle ("" if none), besides the process-wide slot of
@@ -304,7 +306,9 @@ long long spion_noalloc_max_rows(void);
  * the results equal those of the row-major entry points bit for bit.  Attn / P stay [NB][nnz] as everywhere.
  * The kept copies of Out are not used: the backward takes Out (required).  On patterns without tile structure
  * the backward's dS scratch ([NB][nnz] floats) belongs to the handle and is allocated by the first such call
- * (not under HIP graph capture). */
+ * (not under HIP graph capture).  Workspaces that follow the pattern's size grow when a larger pattern arrives; the
+ * buffer a larger one replaces stays allocated until the handle is destroyed, so a HIP graph recorded earlier on
+ * the handle can still be replayed. */
 typedef struct spion_head_layout {
     long long batch_stride;
     int head_stride;
@@ -357,7 +361,8 @@ void spion_dense_backward_strided(void* handle, const float* Q, const float* K, 
  * models/model_transformer.py:136-137 takes that mean with two torch.mean passes over the [B,H,L,L] tensor the
  * forward has just written; here every map tile is added to a partial sum while it is on its way to memory, and
  * one reduction over a few partial maps finishes the mean, so the maps are not read back.  The handle keeps the
- * partial maps (at most max(1, 512*32/seq_len) * seq_len^2 floats).  All other arguments and results as in
+ * partial maps: C * seq_len^2 floats, C = the smallest divisor of num_batches with C * seq_len / 32 >= 512, or
+ * num_batches itself when it has none; allocated by the first such call (not under HIP graph capture).  All other arguments and results as in
  * spion_dense_forward_strided (Attn is still written: the API returns it). */
 void spion_dense_forward_strided_mean(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
                                       float* Attn, float* Out, float* Mean,

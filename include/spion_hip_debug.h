@@ -19,7 +19,9 @@ void spion_force_element_path(void* handle, int on);
 void spion_set_backward_passes(void* handle, int mask);
 
 /* Counters of a sparse handle: which = 0 -> pattern analyses that copied the index back from the device (and
- * waited for the stream), which = 1 -> analyses made from host arrays (spion_register_pattern).  -1 otherwise. */
+ * waited for the stream), which = 1 -> analyses made from host arrays (spion_register_pattern), which = 2 ->
+ * workspace buffers that a larger pattern has outgrown and that stay allocated until the handle is destroyed (a HIP
+ * graph recorded before the growth still points at them).  -1 otherwise. */
 int spion_debug_counter(void* handle, int which);
 
 /* Environment switches read once per process, for A/B measurements only (results are the same either way):

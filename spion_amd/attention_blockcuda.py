@@ -67,6 +67,8 @@ class _BlockAttnFunction(torch.autograd.Function):
             _lib.core().spion_attn_forward_rowmajor(m.attn_handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
                                                     p_flat.data_ptr(), out.data_ptr(), *idx.tail)
         _lib.check_error("attn_forward")
+        # which kernel family serves THIS pattern (the handle may run other patterns before the backward)
+        ctx.tiled = _lib.core().spion_last_path(m.attn_handle) == 1
         ctx.save_for_backward(q, k, v, p_flat, idx.offsets, idx.columns, idx.sum_mat, out)
         ctx.set_materialize_grads(False)  # the gradient of the returned probabilities is ignored anyway
         ctx.module = m
@@ -108,7 +110,7 @@ class _BlockAttnFunction(torch.autograd.Function):
         # Of the ABI's two [NB*nnz] scratch arguments (models/attention_blockcuda.py:83-84) the tile kernels use
         # neither and the element kernels only dS: nothing that size is allocated unless it is needed.
         scratch_ds = None
-        if core.spion_last_path(m.attn_handle) != 1:
+        if not ctx.tiled:
             scratch_ds = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
         shape = m.head_shape
         dq = torch.empty(shape, dtype=torch.float32, device=dev)

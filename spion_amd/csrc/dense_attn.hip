@@ -926,13 +926,16 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
                 C = c;
                 break;
             }
+        // C follows from the handle's shape alone, so the partial maps are allocated once per handle and their
+        // address never changes afterwards (a recorded HIP graph stays valid); never under capture, where an
+        // allocation would invalidate the capture
         const size_t need = (size_t)C * a->L * a->L;
         if (need > a->ws_mean_floats) {
-            if (a->ws_mean) {
-                if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return;
-                (void)hipFree(a->ws_mean);
-                a->ws_mean = nullptr;
-                a->ws_mean_floats = 0;
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            (void)hipStreamIsCapturing(a->hdr.stream, &cap);
+            if (cap != hipStreamCaptureStatusNone || a->ws_mean) {
+                set_error("%s: the partial maps are not allocated yet; run one call outside the capture", who);
+                return;
             }
             if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_mean, sizeof(float) * need))) return;
             a->ws_mean_floats = need;

@@ -389,9 +389,12 @@ __global__ void transition_decide_kernel(const double* __restrict__ Partial, int
             before[l] = dist;
             diff[l] = 0.f;
         } else {
-            diff[l] = (fabsf(dist - before[l]) / before[l]) * 100.f;
+            // a previous distance of 0 (two identical maps in a row) gives inf or NaN here, where the
+            // reference's int(diff) raises (main_conv_ff.py:228-233): such a layer counts as not settled
+            const float dl = (fabsf(dist - before[l]) / before[l]) * 100.f;
+            diff[l] = dl;
             before[l] = dist;
-            if ((int)diff[l] < percent) ++settled;
+            if (isfinite(dl) && dl < 2.0e9f && (int)dl < percent) ++settled;
         }
     }
     if (stage == 1.f) {

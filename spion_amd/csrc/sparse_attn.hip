@@ -465,6 +465,9 @@ struct SparseAttn {
     size_t ws_ds_count = 0;
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
     size_t ws_part_floats = 0;
+    // Buffers a grown workspace has replaced.  They stay allocated until the handle is destroyed: a HIP graph
+    // recorded earlier on this handle has their addresses in its kernel nodes and may still be replayed.
+    std::vector<void*> retired;
     int last_path = 0;
     bool is_bf16 = false;  // handle of the bf16 family: tile patterns only, P is never materialised
     bool force_element = false;
@@ -524,6 +527,7 @@ void sparse_destroy(void* h) {
     if (a->ws_ds) (void)hipFree(a->ws_ds);
     if (a->ws_raw) (void)hipFree(a->ws_raw);
     if (a->ws_part) (void)hipFree(a->ws_part);
+    for (void* p : a->retired) (void)hipFree(p);
     for (auto& sl : a->oslot)
         if (sl.buf) (void)hipFree(sl.buf);
     a->hdr.magic = 0;
@@ -992,8 +996,10 @@ static bool ensure_ws(float** p, size_t count) {
 }
 
 // A workspace whose size follows the pattern: grown (never under HIP graph capture, where an allocation would
-// invalidate the capture) to the largest size asked for.  hipFree waits for the device, so no launch still uses the
-// old buffer.
+// invalidate the capture) to at least the size asked for, by half of its size or more so that a series of slightly
+// larger patterns does not allocate every time.  The buffer it replaces is not freed but retired until the handle
+// is destroyed: a graph recorded before the growth keeps working on the old buffer, which is large enough for the
+// pattern it was recorded with.
 static bool ensure_ws_grow(SparseAttn* a, float** p, size_t* have, size_t need, const char* who) {
     if (*have >= need) return true;
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
@@ -1002,11 +1008,20 @@ static bool ensure_ws_grow(SparseAttn* a, float** p, size_t* have, size_t need, 
         set_error("%s: the workspace for this pattern is not allocated yet; run one step outside the capture", who);
         return false;
     }
-    if (*p) (void)hipFree(*p);
-    *p = nullptr;
-    *have = 0;
-    if (!SPION_HIP_OK(hipMalloc((void**)p, sizeof(float) * need))) return false;
-    *have = need;
+    const size_t want = std::max(need, *have + *have / 2);
+    float* fresh = nullptr;
+    if (hipMalloc((void**)&fresh, sizeof(float) * want) != hipSuccess) {
+        (void)hipGetLastError();
+        if (want == need || !SPION_HIP_OK(hipMalloc((void**)&fresh, sizeof(float) * need))) {
+            if (want == need) set_error("%s: hipMalloc of %zu bytes of workspace failed", who, sizeof(float) * need);
+            return false;
+        }
+        *have = need;
+    } else {
+        *have = want;
+    }
+    if (*p) a->retired.push_back(*p);
+    *p = fresh;
     return true;
 }
 
@@ -1676,19 +1691,10 @@ static SparseAttn* as_bf16(void* h, const char* who, const int* Offsets, const i
     return a;
 }
 
-// Workspace for the partial results of long strips: grows to the largest pattern seen.
+// Workspace for the partial results of long strips: grows to the largest pattern seen (see ensure_ws_grow).
 static bool ensure_part_ws(SparseAttn* a, int slots) {
     const size_t need = (size_t)a->NB * slots * (a->d == 32 ? bf16_slot_floats<32>() : bf16_slot_floats<64>());
-    if (need <= a->ws_part_floats) return true;
-    if (a->ws_part) {
-        if (!SPION_HIP_OK(hipStreamSynchronize(a->hdr.stream))) return false;
-        (void)hipFree(a->ws_part);
-        a->ws_part = nullptr;
-        a->ws_part_floats = 0;
-    }
-    if (!SPION_HIP_OK(hipMalloc((void**)&a->ws_part, sizeof(float) * need))) return false;
-    a->ws_part_floats = need;
-    return true;
+    return ensure_ws_grow(a, &a->ws_part, &a->ws_part_floats, need, "bf16 attention");
 }
 
 template <bool ST>
@@ -1941,7 +1947,8 @@ int sparse_last_path(void* h) {
 int sparse_debug_counter(void* h, int which) {
     SparseAttn* a = as_sparse(h, "spion_debug_counter");
     if (!a) return -1;
-    return which == 0 ? a->analyses_from_device : which == 1 ? a->analyses_from_host : -1;
+    return which == 0 ? a->analyses_from_device : which == 1 ? a->analyses_from_host
+         : which == 2 ? (int)a->retired.size() : -1;
 }
 void sparse_set_bwd_passes(void* h, int mask) {
     SparseAttn* a = as_sparse(h, "spion_set_backward_passes");

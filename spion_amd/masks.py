@@ -13,6 +13,7 @@
 from __future__ import annotations
 
 import io
+import math
 import pickle
 
 import torch
@@ -91,7 +92,9 @@ class TransitionDetector:
         for l in range(self.num_layers):
             self.diff[l] = float((abs(dist[l] - self.before_distance[l]) / self.before_distance[l]) * 100)
             self.before_distance[l] = dist[l]
-            if int(self.diff[l]) < self.percent:
+            # a previous distance of 0 (two identical maps in a row) makes the change inf or NaN, on which the
+            # reference's int(diff) raises: such a layer counts as not settled
+            if math.isfinite(self.diff[l]) and int(self.diff[l]) < self.percent:
                 settled += 1
         if settled == self.num_layers:
             self.transition = True

@@ -242,6 +242,14 @@ def test_device_transition_detector_matches_host_detector():
     assert det.update(maps(10.5, 30.0)) is False    # layer 1 changed by 200 %
     assert abs(det.diff[0] - 5.0) < 1e-3 and abs(det.diff[1] - 200.0) < 1e-2
 
+    # identical maps in a row: a previous distance of 0 never counts as settled (0/0, then 2/0)
+    det = DeviceTransitionDetector(1)
+    det.update(maps(5.0))
+    assert det.update(maps(5.0)) is False
+    assert det.update(maps(5.0)) is False
+    assert det.update(maps(7.0)) is False
+    assert det.update(maps(9.0)) is True
+
     # random maps: identical decisions and distances as the host detector, evaluation by evaluation
     g = torch.Generator().manual_seed(7)
     L, layers = 256, 3

@@ -161,3 +161,75 @@ def test_kept_output_copy_is_dropped_by_forwards_that_do_not_refresh_it():
     for name, got in (("dQ", dQ), ("dK", dK), ("dV", dV)):
         assert_close(got.cpu().numpy(), ref[name], what=f"backward after a forward that kept no copy: {name}")
     abi.close()
+
+
+def test_grown_workspaces_retire_the_buffers_they_replace():
+    """A workspace that follows the pattern's size is replaced, not freed, when a larger pattern arrives: a HIP graph
+    recorded with the smaller pattern still has the old address in its kernel nodes.  Checked through the handle's
+    bookkeeping (no stale graph is replayed here): the retired count rises by the number of grown buffers, stays put
+    when the smaller pattern comes back, and both patterns keep giving the oracle's results."""
+    L, d, B, H = 256, 32, 1, 2
+    NB = B * H
+    core = _lib.core()
+    abi = SparseABI(d, L, NB, 1, with_mask=False)
+    small = workloads.window_random_csr(L, 40, 60, seed=3)
+    large = workloads.window_random_csr(L, 40, 120, seed=4)
+    Q, K, V, dO = _inputs(NB, L, d, seed=21)
+    q, k, v, do = (t.view(B, H, L, d) for t in (Q, K, V, dO))
+
+    def step(pattern):
+        abi.set_pattern(*pattern)
+        out = torch.empty(B, H, L, d, device="cuda")
+        P = abi.forward_strided(q, k, v, out)
+        assert abi.last_path() == 3
+        dq, dk, dv = (torch.empty(B, H, L, d, device="cuda") for _ in range(3))
+        abi.backward_strided(q, k, v, P, out, do, dq, dk, dv)   # dS scratch and raw logits belong to the handle
+        torch.cuda.synchronize()
+        ref = oracle_fwd_bwd(Q, K, V, dO, *pattern)
+        for name, got in (("O", out), ("dQ", dq), ("dK", dk), ("dV", dv)):
+            assert_close(got.reshape(NB, L, d).cpu().numpy(), ref[name], what=name)
+        keep.append((abi.sum_mat, abi.offsets, abi.columns))    # the handle's keys must stay unique addresses
+
+    keep = []
+    step(small)
+    assert core.spion_debug_counter(abi.handle, 2) == 0
+    step(large)
+    retired = core.spion_debug_counter(abi.handle, 2)
+    assert retired >= 1, "the dS scratch of the smaller pattern must be retired, not freed"
+    step(small)
+    step(large)
+    assert core.spion_debug_counter(abi.handle, 2) == retired
+    abi.close()
+
+
+def test_module_backward_allocates_scratch_by_its_own_pattern():
+    """forward(hybrid mask), forward(tile mask), backward(tile), backward(hybrid) on one module: the second backward
+    needs the dS scratch although the handle's most recent call ran the tile kernels."""
+    B, H, L, d = 1, 2, 256, 32
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=1)
+    cpp = Attention._blockcuda_compile_module()
+    mod = spion_amd.CUDABlockAttention(cfg, cpp, cpp.init(d, L, B * H, 1))
+    sm, off, col = workloads.window_random_csr(L, 40, 100, seed=3)
+    hyb = np.zeros((L, L), dtype=np.float32)
+    hyb[np.repeat(np.arange(L), sm), col] = 1.0
+    blocks = workloads.band_random_block_mask(L // 32, 1, extra_frac=0.1, seed=3)
+    tile = np.repeat(np.repeat(blocks, 32, 0), 32, 1).astype(np.float32)
+    ones = torch.ones(B, L, device="cuda")
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=5, device="cuda")
+    outs, leaves = [], []
+    for pat in (hyb, tile):
+        qq, kk, vv = (t.detach().clone().requires_grad_() for t in (q, k, v))
+        out, _ = mod(qq, kk, vv, ones, torch.from_numpy(pat).cuda())
+        outs.append(out)
+        leaves.append((qq, kk, vv))
+    outs[1].backward(do)
+    outs[0].backward(do)          # used to fail: "the element path needs the dS scratch buffer"
+    torch.cuda.synchronize()
+    for pat, (qq, kk, vv) in zip((hyb, tile), leaves):
+        rows, cols = np.nonzero(pat)
+        sm_ = pat.sum(1).astype(np.int32)
+        off_ = np.concatenate([[0], np.cumsum(sm_)]).astype(np.int32)
+        ref = oracle_fwd_bwd(q.reshape(B * H, L, d), k.reshape(B * H, L, d), v.reshape(B * H, L, d),
+                             do.reshape(B * H, L, d), sm_, off_, cols.astype(np.int32))
+        for name, t in (("dQ", qq), ("dK", kk), ("dV", vv)):
+            assert_close(t.grad.reshape(B * H, L, d).cpu().numpy(), ref[name], what=name)

@@ -71,3 +71,13 @@ def test_transition_detector_truncates_and_needs_every_layer():
     det.update(_maps(10.0, 10.0))
     assert det.update(_maps(10.5, 30.0)) is False   # layer 1 changed by 200 %
     assert abs(det.diff[0] - 5.0) < 1e-4 and abs(det.diff[1] - 200.0) < 1e-3
+
+
+def test_transition_detector_identical_maps_do_not_settle():
+    # two identical maps in a row: the previous distance is 0 and the change is 0/0 or x/0; the layer is not settled
+    det = TransitionDetector(1)
+    det.update(_maps(5.0))
+    assert det.update(_maps(5.0)) is False          # distance 0 recorded
+    assert det.update(_maps(5.0)) is False          # 0/0: not settled, the kept map is replaced
+    assert det.update(_maps(7.0)) is False          # 2/0 = inf: not settled
+    assert det.update(_maps(9.0)) is True           # distance 2 after 2: change 0 %

@@ -59,6 +59,52 @@ def test_noalloc_backward_matches_rowmajor_backward_twice():
 
 
 @pytest.mark.gpu
+def test_noalloc_backward_allocates_nothing():
+    """What the entry point is for: the call analyses no pattern, leaves the device's free memory where it was and
+    can be recorded into a HIP graph (a hipMalloc on the capturing thread would invalidate the capture); every
+    replay equals the allocating entry point bit for bit."""
+    abi, _, (Q, K, V, dO), _ = _case(512, 32, 4, 0.2, 5, False)
+    core = _lib.core()
+    O, P = abi.forward_rowmajor(Q, K, V)
+    want = abi.backward_rowmajor(Q, K, V, P, O, dO)
+    P = P.contiguous()
+    dQ, dK, dV = (torch.full((abi.NB, abi.L, abi.d), float("nan"), device="cuda") for _ in range(3))
+
+    def call():
+        core.spion_attn_backward_noalloc(
+            abi.handle, Q.data_ptr(), K.data_ptr(), V.data_ptr(), P.data_ptr(), O.data_ptr(), dO.data_ptr(),
+            dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(), abi.offsets.data_ptr(), abi.columns.data_ptr(),
+            abi.sum_mat.data_ptr(), abi.nnz)
+        _lib.check_error("spion_attn_backward_noalloc")
+
+    torch.cuda.synchronize()
+    counters = [core.spion_debug_counter(abi.handle, w) for w in (0, 1, 2)]
+    free_before = torch.cuda.mem_get_info()[0]
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
+    assert [core.spion_debug_counter(abi.handle, w) for w in (0, 1, 2)] == counters, "the call analysed or grew something"
+    for name, g_, w_ in zip(("dQ", "dK", "dV"), (dQ, dK, dV), want):
+        assert torch.equal(g_, w_), name
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        core.spion_set_stream(abi.handle, torch.cuda.current_stream().cuda_stream)
+        call()
+    core.spion_set_stream(abi.handle, None)
+    for rep in range(3):
+        for t in (dQ, dK, dV):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, g_, w_ in zip(("dQ", "dK", "dV"), (dQ, dK, dV), want):
+            assert torch.equal(g_, w_), f"replay {rep}: {name}"
+    abi.close()
+
+
+@pytest.mark.gpu
 def test_noalloc_backward_refuses_unknown_patterns_and_element_patterns():
     abi, (sm, off, col), (Q, K, V, dO), _ = _case(128, 32, 2, 0.5, 3, False)
     P = torch.zeros(abi.NB * abi.nnz, device="cuda")
