@@ -149,6 +149,140 @@ struct LdsTile {
     }
 };
 
+// -------------------------------------------------------------------------------------------------
+// Tiles that go from global memory straight into LDS (buffer loads with the LDS modifier): no registers hold a
+// tile in flight and no ds_write is spent on it.  One instruction moves 64 x 16 bytes to 1 KB of consecutive LDS
+// addresses starting at M0 (+ the instruction's immediate offset, which is added to the global address as well);
+// which 16-byte piece of global memory a lane fetches is free, so the LDS image of a tile is unpadded rows with
+// the pieces of a row permuted: piece c of tile row r lies at position c ^ swz(r).  With that permutation both
+// kinds of LDS reads are free of bank conflicts: eight consecutive rows of one piece (operand over the head
+// dimension, ds_read_b128) and four consecutive rows of two adjacent pieces (transposing read).
+// The loads are inline assembly, so the compiler neither tracks them in its s_waitcnt bookkeeping nor knows that
+// they write LDS: the kernels wait for them with wait_vm<N> (N = loads issued after the ones waited for; loads
+// return in order, and the compiler's own counts can only wait longer than needed) and order them against their
+// LDS reads with wait_lgkm0; both carry a memory clobber, so no LDS access moves across them.
+// -------------------------------------------------------------------------------------------------
+__device__ __forceinline__ u32x4 rsrc_words(const void* p, size_t bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(p);
+    u32x4 r;
+    r.x = (unsigned)a;
+    r.y = (unsigned)(a >> 32);  // stride 0, no swizzle
+    r.z = bytes > 0xfffffff0ull ? 0xfffffff0u : (unsigned)bytes;
+    r.w = 0x00020000u;
+    // wave-uniform by construction; keep it in scalar registers
+    r.x = __builtin_amdgcn_readfirstlane(r.x);
+    r.y = __builtin_amdgcn_readfirstlane(r.y);
+    r.z = __builtin_amdgcn_readfirstlane(r.z);
+    return r;
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    typedef __attribute__((address_space(3))) const char* lds_ptr;
+    return __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<unsigned long long>((lds_ptr)p));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// An empty use of operand registers.  The compiler waits for the loads that fill them before this point -- else it
+// puts that wait at their first use inside the tile loop, as vmcnt(0), where it would also wait, on every
+// iteration, for the tile loads just issued (which it does not know of).
+template <int N>
+__device__ __forceinline__ void settle(const bf16x8 (&x)[N]) {
+#pragma unroll
+    for (int t = 0; t < N; ++t) asm volatile("" ::"v"(x[t]));
+}
+__device__ __forceinline__ void settle(float x) { asm volatile("" ::"v"(x)); }
+// 64 floats (lane l: 4 bytes at voff) to 256 bytes of LDS
+__device__ __forceinline__ void dma_b32(u32x4 r, unsigned lds, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds), "v"(voff), "s"(r),
+                 "s"(soff)
+                 : "memory");
+}
+
+template <int D>
+struct DmaTile {
+    static constexpr int ROW = D * 2;     // bytes per LDS row
+    static constexpr int TILE = 32 * ROW;  // 2 KB (D = 32) or 4 KB (D = 64)
+    static constexpr int CPR = D / 8;      // 16-byte pieces per row
+    static constexpr int NI = D / 16;      // instructions per tile, 64 / CPR rows each
+    __device__ static __forceinline__ int swz(int row) {
+        if constexpr (D == 64) return ((row & 3) << 1) | ((row >> 2) & 1);
+        else return (((row >> 1) & 1) << 1) | ((row >> 2) & 1);
+    }
+    // Lane offset into the head slice (bytes): lane l fills LDS piece l of every instruction's 1 KB, i.e. position
+    // l % CPR of row l / CPR (+ 64 / CPR rows per instruction), with the global piece that belongs there.
+    __device__ static __forceinline__ int voff(int l, int ld) {
+        const int r = l / CPR, c = (l % CPR) ^ swz(r);
+        return (r * ld + c * 8) * 2;
+    }
+    // what the scalar offset advances by from one instruction to the next, beyond the 1024 its immediate adds
+    __device__ static __forceinline__ int extra_step(int ld) { return (64 / CPR) * ld * 2 - 1024; }
+    __device__ static __forceinline__ void load(u32x4 r, unsigned lds, int lvoff, int soff, int xstep) {
+        if constexpr (D == 64)
+            asm volatile(
+                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %6 offen offset:3072 lds" ::"s"(lds),
+                "v"(lvoff), "s"(r), "s"(soff), "s"(soff + xstep), "s"(soff + 2 * xstep), "s"(soff + 3 * xstep)
+                : "memory");
+        else
+            asm volatile(
+                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds" ::"s"(lds),
+                "v"(lvoff), "s"(r), "s"(soff), "s"(soff + xstep)
+                : "memory");
+    }
+    // Byte offsets of lane (row li, half h) for its operand over the head dimension: features h*D/2 + 8t .. of row
+    // li, t = 0 .. D/16-1 (piece h*CPR/2 + t).
+    struct RowAddr {
+        int a[D / 16];
+    };
+    __device__ static __forceinline__ RowAddr row_addr(int li, int h) {
+        RowAddr x;
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) x.a[t] = li * ROW + 16 * ((h * (CPR / 2) + t) ^ swz(li));
+        return x;
+    }
+    __device__ static __forceinline__ void get_rows(const char* T, const RowAddr& ra, bf16x8 (&x)[D / 16]) {
+#pragma unroll
+        for (int t = 0; t < D / 16; ++t) x[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(T + ra.a[t]));
+    }
+    // Transposing reads (see LdsTile::get_tile_t): lane j of a group of 16 points at features F + 4(j%4) .. +3 of
+    // row R + j/4, R = 4h (+ 16t, + 8), F = 16*((l/16)%2) (+ 32c): 8 bytes inside piece 2*((l/16)%2) + (j%4)/2
+    // (+ 4c).  Rows 8 apart share their permutation, so the row steps stay immediate offsets.
+    struct TrAddr {
+        int a[D / 32];
+    };
+    __device__ static __forceinline__ TrAddr tr_addr(int l) {
+        const int h = l >> 5, gm = (l >> 4) & 1, j = l & 15, row = 4 * h + (j >> 2);
+        TrAddr x;
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+            x.a[c] = row * ROW + 16 * ((4 * c + 2 * gm + ((j & 3) >> 1)) ^ swz(row)) + 8 * (j & 1);
+        return x;
+    }
+    __device__ static __forceinline__ void get_tile_t(const char* T, const TrAddr& ta, bf16x8 (&xt)[D / 32][2]) {
+        typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + ta.a[c] + (16 * t) * ROW));
+                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + ta.a[c] + (16 * t + 8) * ROW));
+                xt[c][t] = __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1,
+                                                   2, 3, 4, 5, 6, 7);
+            }
+    }
+    // LDS of one wavefront: two buffers of two tiles and 256 bytes of per-tile scalars (key penalties or row
+    // statistics of the tile, 64 floats)
+    static constexpr int BUF = 2 * TILE + 256;
+    static constexpr int WAVE = 2 * BUF;
+};
+
 // x of the lower and of the upper half-wave lane with the same lane%32, by v_permlane32_swap (exchanges the
 // upper half of its first operand with the lower half of its second).  Written as inline assembly with two
 // read-write operands: they must be different registers for the exchange to mean anything.
@@ -238,12 +372,12 @@ constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
 // -------------------------------------------------------------------------------------------------
 // Forward: one sweep per block row with a lazily raised running maximum.
 // -------------------------------------------------------------------------------------------------
-// The LDS space of a forward work-group: two wave-private tiles per wavefront (reused for the partial results of a
-// shared strip) and the row statistics the wavefronts of a shared strip exchange.
+// The LDS space of a forward work-group: the tile buffers of each wavefront (DmaTile; reused for the partial results
+// of a shared strip) and the row statistics the wavefronts of a shared strip exchange.
 template <int D>
 struct Bf16FwdLds {
-    typedef LdsTile<D> LT;
-    __attribute__((aligned(16))) char t[BF16_WAVES][2][LT::BYTES];
+    typedef DmaTile<D> DT;
+    __attribute__((aligned(16))) char t[BF16_WAVES][DT::WAVE];
     float m[BF16_WAVES][32], z[BF16_WAVES][32];
 };
 
@@ -254,12 +388,11 @@ __device__ __forceinline__ void bf16_fwd_strip(
     const __bf16* __restrict__ K, const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O,
     float* __restrict__ Lse, const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale,
     float* __restrict__ Part, int n_slots, int chunk, const Layouts& ly) {
-    typedef LdsTile<D> LT;
-    auto& lds_t = lds.t;
+    typedef DmaTile<D> DT;
     auto& lds_m = lds.m;
     auto& lds_z = lds.z;
-    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
+    float* lds_o = reinterpret_cast<float*>(&lds.t[0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
     const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int I = sa.strip;
     const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
@@ -270,14 +403,17 @@ __device__ __forceinline__ void bf16_fwd_strip(
     int ild, old_;
     bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
     bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
-    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes);
     const rsrc_t rO = make_rsrc(O + ob, obytes);
-    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const u32x4 wK = rsrc_words(K + ib, ibytes), wV = rsrc_words(V + ib, ibytes);
+    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int r_voff = li * ild * 2 + h * D;
-    const int t_voff = bf16_tile_voff<D>(l, ild), t_step = bf16_tile_step<D>(ild), t_bytes = 32 * ild * 2;
-    char* Tk = lds_t[w][0];
-    char* Tv = lds_t[w][1];
-    const int tbase = LT::lane_base(l);
+    const int t_bytes = 32 * ild * 2;
+    const int d_voff = DT::voff(l, ild), d_xstep = DT::extra_step(ild);
+    const char* Tw = lds.t[w];
+    const unsigned lds_w = lds_address(Tw);
+    const typename DT::RowAddr ra = DT::row_addr(li, h);
+    const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
     bf16x8 q[D / 16];
@@ -290,58 +426,66 @@ __device__ __forceinline__ void bf16_fwd_strip(
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
 
-    struct Pre {
-        u32x4 k[D / 16], v[D / 16];
-        float pj[MASK ? 16 : 1];
+    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
+    auto tile_id = [&](int i) { return tcol[t0 + sa.rank + min(i, nu - 1) * sa.step]; };
+    auto issue = [&](int J, int par) {  // key tile J -> buffer par
+        const unsigned a = lds_w + par * DT::BUF;
+        DT::load(wK, a, d_voff, J * t_bytes, d_xstep);
+        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, d_xstep);
+        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
     };
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
-            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
-            if constexpr (MASK) {
-                float pj[16];
-                ldr_4x4(rM, 16 * h, J * 128, pj);
+    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
+    auto compute = [&](int par, int inext) {
+        const char* Tk = Tw + par * DT::BUF;
+        const char* Tv = Tk + DT::TILE;
+        bf16x8 kr[D / 16], vt[D / 32][2];
+        DT::get_rows(Tk, ra, kr);
+        DT::get_tile_t(Tv, ta, vt);
+        f32x16 init = splat16(0.f);
+        if constexpr (MASK) {
+            float pj[16];
+            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
 #pragma unroll
-                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
-            }
-        },
-        [&](Pre& c, int) {
-            LT::put_raw(Tk, l, c.k);
-            LT::put_raw(Tv, l, c.v);
-            // every LDS read is issued before the first chain starts (the compiler would otherwise sink each
-            // one next to its use and wait for it there)
-            bf16x8 kr[D / 16], vt[D / 32][2];
-            LT::get_rows(Tk, li, h, kr);
-            LT::get_tile_t(Tv, tbase, vt);
-            __builtin_amdgcn_sched_barrier(0);
-            f32x16 init = splat16(0.f);
-            if constexpr (MASK) {
+            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+        }
+        wait_lgkm0();  // the tile's operands are in registers: its buffer can take the tile after next
+        if (inext >= 0) issue(Jq, par);
+        Jq = tile_id(inext + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
+        const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
+        if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
+            const float mn = t2 > m + BF16_LAZY ? t2 : m;
+            const float f = __builtin_amdgcn_exp2f(m - mn);
+            z *= f;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
-            }
-            const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
-            const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
-            if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
-                const float mn = t2 > m + BF16_LAZY ? t2 : m;
-                const float f = __builtin_amdgcn_exp2f(m - mn);
-                z *= f;
+            for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
+            m = mn;
+        }
+        float p[16];
 #pragma unroll
-                for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
-                m = mn;
-            }
-            float p[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
-                z += p[r];
-            }
-            bf16x8 pb[2];
-            pack16(p, pb);
-            mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
-        });
+        for (int r = 0; r < 16; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
+            z += p[r];
+        }
+        bf16x8 pb[2];
+        pack16(p, pb);
+        mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    settle(q);
+    if (nu > 0) issue(tile_id(0), 0);
+    if (nu > 1) issue(tile_id(1), 1);
+    if (nu > 2) Jq = tile_id(2);
+    for (int i = 0; i < nu; i += 2) {
+        if (i + 1 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(0, i + 2 < nu ? i + 2 : -1);
+        if (i + 1 >= nu) break;
+        if (i + 2 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(1, i + 3 < nu ? i + 3 : -1);
+    }
     z = half_swap_sum(z);
     if (sa.coop) {
         if (h == 0) {
@@ -405,20 +549,22 @@ __device__ __forceinline__ void bf16_fwd_pair(
     Bf16FwdLds<D>& lds, int pr, int bh, int w, const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
     const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse,
     const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale) {
-    typedef LdsTile<D> LT;
-    auto& lds_t = lds.t;
+    typedef DmaTile<D> DT;
     const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int I = 2 * pr;
     const int t0 = trp[I], cnt = trp[I + 1] - t0;
     const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes), rK = make_rsrc(K + hb, hbytes), rV = make_rsrc(V + hb, hbytes);
+    const rsrc_t rQ = make_rsrc(Q + hb, hbytes);
     const rsrc_t rO = make_rsrc(O + hb, hbytes);
-    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const u32x4 wK = rsrc_words(K + hb, hbytes), wV = rsrc_words(V + hb, hbytes);
+    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int r_voff = li * D * 2 + h * D;
-    const int t_voff = l * 16, t_step = 1024, t_bytes = 32 * D * 2;
-    char* Tk = lds_t[w][0];
-    char* Tv = lds_t[w][1];
-    const int tbase = LT::lane_base(l);
+    const int t_bytes = 32 * D * 2;
+    const int d_voff = DT::voff(l, D);
+    const char* Tw = lds.t[w];
+    const unsigned lds_w = lds_address(Tw);
+    const typename DT::RowAddr ra = DT::row_addr(li, h);
+    const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
     bf16x8 q0[D / 16], q1[D / 16];
@@ -449,44 +595,55 @@ __device__ __forceinline__ void bf16_fwd_pair(
         }
         pack16(p, pb);
     };
-    struct Pre {
-        u32x4 k[D / 16], v[D / 16];
-        float pj[MASK ? 16 : 1];
+    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
+    auto tile_id = [&](int i) { return tcol[t0 + min(i, cnt - 1)]; };
+    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
+    auto issue = [&](int J, int par) {
+        const unsigned a = lds_w + par * DT::BUF;
+        DT::load(wK, a, d_voff, J * t_bytes, 0);
+        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, 0);
+        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
     };
-    Pre xa, xb;
-    tile_pipeline(
-        cnt, xa, xb,
-        [&](Pre& x, int i) {
-            const int J = tcol[t0 + min(i, cnt - 1)];
-            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
-            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
-            if constexpr (MASK) {
-                float pj[16];
-                ldr_4x4(rM, 16 * h, J * 128, pj);
+    auto compute = [&](int par, int inext) {
+        const char* Tk = Tw + par * DT::BUF;
+        const char* Tv = Tk + DT::TILE;
+        bf16x8 kr[D / 16], vt[D / 32][2];
+        DT::get_rows(Tk, ra, kr);
+        DT::get_tile_t(Tv, ta, vt);
+        f32x16 init = splat16(0.f);
+        if constexpr (MASK) {
+            float pj[16];
+            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);
 #pragma unroll
-                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
-            }
-        },
-        [&](Pre& c, int) {
-            LT::put_raw(Tk, l, c.k);
-            LT::put_raw(Tv, l, c.v);
-            bf16x8 kr[D / 16], vt[D / 32][2];
-            LT::get_rows(Tk, li, h, kr);
-            LT::get_tile_t(Tv, tbase, vt);
-            __builtin_amdgcn_sched_barrier(0);
-            f32x16 init = splat16(0.f);
-            if constexpr (MASK) {
-#pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
-            }
-            const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
-            const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
-            bf16x8 pb0[2], pb1[2];
-            update(s0, m0, z0, o0, pb0);
-            update(s1, m1, z1, o1, pb1);
-            mma_tile_bf16<D>(vt, pb0, o0);
-            mma_tile_bf16<D>(vt, pb1, o1);
-        });
+            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+        }
+        wait_lgkm0();
+        if (inext >= 0) issue(Jq, par);
+        Jq = tile_id(inext + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
+        const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
+        bf16x8 pb0[2], pb1[2];
+        update(s0, m0, z0, o0, pb0);
+        update(s1, m1, z1, o1, pb1);
+        mma_tile_bf16<D>(vt, pb0, o0);
+        mma_tile_bf16<D>(vt, pb1, o1);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    settle(q0);
+    settle(q1);
+    if (cnt > 0) issue(tile_id(0), 0);
+    if (cnt > 1) issue(tile_id(1), 1);
+    if (cnt > 2) Jq = tile_id(2);
+    for (int i = 0; i < cnt; i += 2) {
+        if (i + 1 < cnt) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(0, i + 2 < cnt ? i + 2 : -1);
+        if (i + 1 >= cnt) break;
+        if (i + 2 < cnt) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(1, i + 3 < cnt ? i + 3 : -1);
+    }
     const int off_pattern = L - cnt * 32;
     float* lds_unused = nullptr;
     auto finish = [&](float m, float z, f32x16 (&o)[D / 32], int strip) {
@@ -530,19 +687,22 @@ SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
 
 // -------------------------------------------------------------------------------------------------
 // Backward, row pass: g_i = dO_i . O_i, P and dP recomputed per tile, dS' = P*(dP - g), dQ += dS'.K_J;
-// the 1/sqrt(d) is applied to the 32 x d result.  Gneg receives -g for the column pass.
+// the 1/sqrt(d) is applied to the 32 x d result.  Stats receives {lse2, -g} of every strip (64 floats per strip:
+// the 32 lse2 values, then the 32 -g values) for the column pass.
+// K and V tiles go from global memory straight into one of two LDS buffers of the wavefront (DmaTile), two tiles
+// ahead of the one being worked on.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK, bool ST>
-SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
+SPION_BF16_KERNEL(D == 32 ? 3 : 2) void bf16_bwd_row_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
-    const float* __restrict__ pen, float* __restrict__ Gneg, __bf16* __restrict__ dQ, const int* __restrict__ trp,
+    const float* __restrict__ pen, float* __restrict__ Stats, __bf16* __restrict__ dQ, const int* __restrict__ trp,
     const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
     float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
-    typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
+    typedef DmaTile<D> DT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][DT::WAVE];
+    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -558,14 +718,17 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
     bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
     bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
     bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rQ = make_rsrc(Q + ib, ibytes);
     const rsrc_t rdO = make_rsrc(dO + ob, obytes), rO = make_rsrc(O + ob, obytes), rdQ = make_rsrc(dQ + gb, gbytes);
-    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const u32x4 wK = rsrc_words(K + ib, ibytes), wV = rsrc_words(V + ib, ibytes);
+    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
     const int r_voff = li * ild * 2 + h * D, ro_voff = li * old_ * 2 + h * D;
-    const int t_voff = bf16_tile_voff<D>(l, ild), t_step = bf16_tile_step<D>(ild), t_bytes = 32 * ild * 2;
-    char* Tk = lds_t[w][0];
-    char* Tv = lds_t[w][1];
-    const int tbase = LT::lane_base(l);
+    const int t_bytes = 32 * ild * 2;
+    const int d_voff = DT::voff(l, ild), d_xstep = DT::extra_step(ild);
+    const char* Tw = lds_t[w];
+    const unsigned lds_w = lds_address(Tw);
+    const typename DT::RowAddr ra = DT::row_addr(li, h);
+    const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
 
     bf16x8 q[D / 16], go[D / 16];
@@ -582,52 +745,65 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
         g = half_swap_sum(g);
     }
     const float lse = Lse[(size_t)bh * L + I * 32 + li];
-    if (sa.rank == 0 && h == 0) Gneg[(size_t)bh * L + I * 32 + li] = -g;
+    if (sa.rank == 0 && tb == 0) Stats[((size_t)bh * (L / 32) + I) * 64 + l] = h ? -g : lse;
     const f32x16 gneg = splat16(-g);
 
     f32x16 acc[D / 32];
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
-    struct Pre {
-        u32x4 k[D / 16], v[D / 16];
-        float pj[MASK ? 16 : 1];
+    // tile i of this wavefront -> buffer par
+    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
+    auto tile_id = [&](int i) { return tcol[t0 + sa.rank + min(i, nu - 1) * sa.step]; };
+    auto issue = [&](int J, int par) {
+        const unsigned a = lds_w + par * DT::BUF;
+        DT::load(wK, a, d_voff, J * t_bytes, d_xstep);
+        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, d_xstep);
+        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
     };
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int J = tcol[t0 + sa.rank + min(i, nu - 1) * sa.step];
-            ldb_tile<D>(rK, t_voff, J * t_bytes, t_step, x.k);
-            ldb_tile<D>(rV, t_voff, J * t_bytes, t_step, x.v);
-            if constexpr (MASK) {
-                float pj[16];
-                ldr_4x4(rM, 16 * h, J * 128, pj);
+    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
+    auto compute = [&](int par, int inext) {
+        const char* Tk = Tw + par * DT::BUF;
+        const char* Tv = Tk + DT::TILE;
+        bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
+        DT::get_rows(Tk, ra, kr);
+        DT::get_rows(Tv, ra, vr);
+        DT::get_tile_t(Tk, ta, kt);
+        f32x16 init = splat16(0.f);
+        if constexpr (MASK) {
+            float pj[16];
+            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
 #pragma unroll
-                for (int r = 0; r < 16; ++r) x.pj[r] = pj[r];
-            }
-        },
-        [&](Pre& c, int) {
-            LT::put_raw(Tk, l, c.k);
-            LT::put_raw(Tv, l, c.v);
-            bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
-            LT::get_rows(Tk, li, h, kr);
-            LT::get_rows(Tv, li, h, vr);
-            LT::get_tile_t(Tk, tbase, kt);
-            __builtin_amdgcn_sched_barrier(0);
-            f32x16 init = splat16(0.f);
-            if constexpr (MASK) {
+            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+        }
+        wait_lgkm0();  // the tile's operands are in registers: its buffer can take the tile after next
+        if (inext >= 0) issue(Jq, par);
+        Jq = tile_id(inext + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x16 s = mma_feat_bf16<D>(kr, q, init);
+        const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
+        float ds[16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] = c.pj[r] * pen_mul;
-            }
-            const f32x16 s = mma_feat_bf16<D>(kr, q, init);
-            const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
-            float ds[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
-            bf16x8 dsb[2];
-            pack16(ds, dsb);
-            mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
-        });
+        for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
+        bf16x8 dsb[2];
+        pack16(ds, dsb);
+        mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    settle(q);
+    settle(go);
+    settle(lse);
+    if (nu > 0) issue(tile_id(0), 0);
+    if (nu > 1) issue(tile_id(1), 1);
+    if (nu > 2) Jq = tile_id(2);
+    for (int i = 0; i < nu; i += 2) {
+        if (i + 1 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(0, i + 2 < nu ? i + 2 : -1);
+        if (i + 1 >= nu) break;
+        if (i + 2 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(1, i + 3 < nu ? i + 3 : -1);
+    }
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
     store_rows_bf16<D>(acc, rdQ, gld, I * 32, sa.coop, w, li, h, lds_o, part);
@@ -636,17 +812,19 @@ SPION_BF16_KERNEL(D == 32 && !MASK ? 3 : 2) void bf16_bwd_row_kernel(
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
 // -------------------------------------------------------------------------------------------------
+// Stats: {lse2, -g} of every strip as the row pass left them (64 floats per strip).  The Q and dO tiles and the
+// tile's 64 statistics go from global memory straight into one of two LDS buffers of the wavefront (DmaTile).
 template <int D, bool MASK, bool ST>
 SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const __bf16* __restrict__ dO, const float* __restrict__ Lse, const float* __restrict__ Gneg,
+    const __bf16* __restrict__ dO, const float* __restrict__ Stats,
     const float* __restrict__ pen, __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcp,
     const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
     float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
-    typedef LdsTile<D> LT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][2][LT::BYTES];
-    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * 2 * LT::BYTES, "partial results fit");
+    typedef DmaTile<D> DT;
+    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][DT::WAVE];
+    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0]);  // partial results of a shared strip, after the tiles
+    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
     const int item = xcd_remap(blockIdx.x, n_wg * NB);
     const int bh = item / n_wg;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -662,15 +840,17 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
     bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
     bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
     bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rQ = make_rsrc(Q + ib, ibytes), rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
-    const rsrc_t rdO = make_rsrc(dO + ob, obytes), rdK = make_rsrc(dK + gb, gbytes), rdV = make_rsrc(dV + gb, gbytes);
-    const rsrc_t rL = make_rsrc(Lse + (size_t)bh * L, (size_t)L * 4), rG = make_rsrc(Gneg + (size_t)bh * L, (size_t)L * 4);
+    const rsrc_t rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
+    const rsrc_t rdK = make_rsrc(dK + gb, gbytes), rdV = make_rsrc(dV + gb, gbytes);
+    const u32x4 wQ = rsrc_words(Q + ib, ibytes), wG = rsrc_words(dO + ob, obytes);
+    const u32x4 wS = rsrc_words(Stats + (size_t)bh * (L / 32) * 64, (size_t)(L / 32) * 256);
     const int r_voff = li * ild * 2 + h * D;
-    const int q_voff = bf16_tile_voff<D>(l, ild), q_step = bf16_tile_step<D>(ild);
-    const int o_voff = bf16_tile_voff<D>(l, old_), o_step = bf16_tile_step<D>(old_);
-    char* Tq = lds_t[w][0];
-    char* Tg = lds_t[w][1];
-    const int tbase = LT::lane_base(l);
+    const int q_voff = DT::voff(l, ild), q_xstep = DT::extra_step(ild);
+    const int o_voff = DT::voff(l, old_), o_xstep = DT::extra_step(old_);
+    const char* Tw = lds_t[w];
+    const unsigned lds_w = lds_address(Tw);
+    const typename DT::RowAddr ra = DT::row_addr(li, h);
+    const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E;
 
     bf16x8 k[D / 16], v[D / 16];
@@ -686,63 +866,78 @@ SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
         av[c] = splat16(0.f);
     }
     const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
-    // One tile ahead: the Q and dO tiles and the two row statistics of the tile's 32 queries, one query per lane
-    // (two 4-byte instructions; fetching each lane's 16 values directly would take eight 16-byte ones, as
-    // costly on the vector-memory path as the two tiles).  The statistics reach the accumulator layout
-    // (register r = query acc_row(r, h)) through a small wave-private LDS array.
-    constexpr bool DEEP = D == 32;
-    __shared__ __attribute__((aligned(16))) float lds_stat[BF16_WAVES][2][32];
-    float* St = &lds_stat[w][0][0];
-    struct Pre {
-        u32x4 q[D / 16], go[D / 16];
-        float lse, gneg;
+    constexpr int OPS = 2 * DT::NI + 1;
+    auto tile_id = [&](int i) { return desc[sa.rank + min(i, nu - 1) * sa.step].x; };
+    int Iq = 0;  // query tile the next issue fetches, requested one tile ahead of that issue
+    auto issue = [&](int I, int par) {  // query tile I -> buffer par
+        const unsigned a = lds_w + par * DT::BUF;
+        DT::load(wQ, a, q_voff, I * 32 * ild * 2, q_xstep);
+        DT::load(wG, a + DT::TILE, o_voff, I * 32 * old_ * 2, o_xstep);
+        dma_b32(wS, a + 2 * DT::TILE, l * 4, I * 256);
     };
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int I = desc[sa.rank + min(i, nu - 1) * sa.step].x;
-            ldb_tile<D>(rQ, q_voff, I * 32 * ild * 2, q_step, x.q);
-            ldb_tile<D>(rdO, o_voff, I * 32 * old_ * 2, o_step, x.go);
-            x.lse = ld1(rL, li * 4, I * 128);
-            x.gneg = ld1(rG, li * 4, I * 128);
-        },
-        [&](Pre& c, int) {
-            St[l] = h ? c.gneg : c.lse;  // lanes 0-31: lse of query li, lanes 32-63: -g of query li
-            LT::put_raw(Tq, l, c.q);
-            LT::put_raw(Tg, l, c.go);
-            float lse[16], gn[16];
-            lds_get_rows(St, 0, h, lse);      // lse[r] = St[acc_row(r, h)]
-            lds_get_rows(St + 32, 0, h, gn);  // gn[r]  = St[32 + acc_row(r, h)]
-            bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
-            LT::get_rows(Tq, li, h, qr);
-            LT::get_rows(Tg, li, h, gr);
-            if constexpr (DEEP) {
-                LT::get_tile_t(Tq, tbase, qt);
-                LT::get_tile_t(Tg, tbase, gt);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
-            f32x16 ginit;
+    // d = 64 has no registers for the transposed tiles while the first chains' operands are live: they are read
+    // once the chains are issued, and the buffer is handed to the tile after next after that.
+    constexpr bool DEEP = D == 32;
+    auto compute = [&](int par, int inext) {
+        const char* Tq = Tw + par * DT::BUF;
+        const char* Tg = Tq + DT::TILE;
+        const float* St = reinterpret_cast<const float*>(Tq + 2 * DT::TILE);  // lse2[32], -g[32] of the tile's queries
+        float lse[16], gn[16];
+        lds_get_rows(St, 0, h, lse);      // lse[r] = St[acc_row(r, h)]
+        lds_get_rows(St + 32, 0, h, gn);  // gn[r]  = St[32 + acc_row(r, h)]
+        bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
+        DT::get_rows(Tq, ra, qr);
+        DT::get_rows(Tg, ra, gr);
+        if constexpr (DEEP) {
+            DT::get_tile_t(Tq, ta, qt);
+            DT::get_tile_t(Tg, ta, gt);
+            wait_lgkm0();
+            if (inext >= 0) issue(Iq, par);
+            Iq = tile_id(inext + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
+        f32x16 ginit;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
-            const f32x16 dp = mma_feat_bf16<D>(gr, v, ginit);  // dO_i . v_j - g_i
-            float p[16], ds[16];
+        for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
+        const f32x16 dp = mma_feat_bf16<D>(gr, v, ginit);  // dO_i . v_j - g_i
+        if constexpr (!DEEP) {
+            DT::get_tile_t(Tq, ta, qt);
+            DT::get_tile_t(Tg, ta, gt);
+        }
+        float p[16], ds[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse[r]));
-                ds[r] = p[r] * dp[r];
-            }
-            bf16x8 pb[2], dsb[2];
-            pack16(p, pb);
-            pack16(ds, dsb);
-            if constexpr (!DEEP) {  // d = 64: no registers to hold them across the chains
-                LT::get_tile_t(Tq, tbase, qt);
-                LT::get_tile_t(Tg, tbase, gt);
-            }
-            mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
-            mma_tile_bf16<D>(gt, pb, av);   // dV^T
-        });
+        for (int r = 0; r < 16; ++r) {
+            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse[r]));
+            ds[r] = p[r] * dp[r];
+        }
+        bf16x8 pb[2], dsb[2];
+        pack16(p, pb);
+        pack16(ds, dsb);
+        if constexpr (!DEEP) {
+            wait_lgkm0();
+            if (inext >= 0) issue(Iq, par);
+            Iq = tile_id(inext + 1);
+        }
+        mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
+        mma_tile_bf16<D>(gt, pb, av);   // dV^T
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    settle(k);
+    settle(v);
+    if constexpr (MASK) settle(sinit[0]);
+    if (nu > 0) issue(tile_id(0), 0);
+    if (nu > 1) issue(tile_id(1), 1);
+    if (nu > 2) Iq = tile_id(2);
+    for (int i = 0; i < nu; i += 2) {
+        if (i + 1 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(0, i + 2 < nu ? i + 2 : -1);
+        if (i + 1 >= nu) break;
+        if (i + 2 < nu) wait_vm<OPS>();
+        else wait_vm<0>();
+        compute(1, i + 3 < nu ? i + 3 : -1);
+    }
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
     store_rows_bf16<D>(ak, rdK, gld, J * 32, sa.coop, w, li, h, lds_o, part);

@@ -1740,7 +1740,8 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
                                const Layouts& ly) {
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
-    if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
+    // {lse2, -g} of every strip, 64 floats per strip, from the row pass to the column pass
+    if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L * 2)) return;
     if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
     const dim3 grid_r(pi.n_wg_row * a->NB), grid_c(pi.n_wg_col * a->NB), block(64 * BF16_WAVES);
     const dim3 grid_mr(pi.n_long_row * a->NB * (32 * a->d / 256)), grid_mc(pi.n_long_col * a->NB * (2 * 32 * a->d / 256));
@@ -1759,7 +1760,7 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
                                    ly.H);                                                                             \
         }                                                                                                             \
         if (a->bwd_passes & 2) {                                                                                      \
-            hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM, ST>), grid_c, block, 0, a->hdr.stream, q, k, v, go, Lse,  \
+            hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM, ST>), grid_c, block, 0, a->hdr.stream, q, k, v, go,       \
                                a->ws_rowsum, Mask, dk, dv, pi.d_tcp, pi.d_tcdesc, pi.d_wg_col, pi.n_wg_col, a->L,     \
                                a->NB, a->scale, a->ws_part, pi.slots_col, pi.chunk_col, ly);                          \
             if (pi.n_long_col)                                                                                        \
