@@ -29,6 +29,9 @@ int spion_debug_counter(void* handle, int which);
  *                        (default: strips of at most 16 tiles in a launch of their own, three work-groups to a CU);
  *   SPION_BF16_NO_PAIRS  the bf16 forward takes one strip per wavefront on every pattern (default: two strips per
  *                        wavefront on masks of 64 x 64 blocks and larger).
+ * Read whenever a bf16 handle indexes a pattern (tests):
+ *   SPION_BF16_LANES     number of persistent wavefronts the bf16 kernels are launched with (default: eight per
+ *                        compute unit); a handful makes each one walk many strips of several heads in a row.
  * SPION_QUIET and SPION_ABORT_ON_ERROR (error reporting) are described in spion_hip.h. */
 
 #ifdef __cplusplus

@@ -16,16 +16,15 @@
 //     bf16, is the B operand of the second one register for register.  The A operand (the tile of K, V, Q or
 //     dO seen feature-major) is read from the tile's wave-private LDS copy with the transposing LDS read
 //     of gfx950.
-// Tiles travel global memory -> registers (consecutive addresses across the wavefront, one tile ahead) ->
-// wave-private LDS tile -> operand layouts; same-wave LDS accesses complete in order, so no barrier is involved.
+// Tiles travel global memory -> wave-private LDS buffers (buffer loads with the LDS modifier, two tiles ahead) ->
+// operand layouts; same-wave LDS accesses complete in order, so no barrier is involved.
 // Queries are the lane index of every row-pass accumulator (S^T, dP^T, O^T, dQ^T), so row statistics are
 // lane scalars; keys are the lane index in the column pass.
 //
-// Work-groups have four wavefronts and take one entry of a host-built list: four short strips (one per
-// wavefront, no barriers) or one chunk of a long strip (a global row or column) walked by the four wavefronts
-// together.  A long strip is cut into chunks of about the work of an ordinary work-group, so that it does not
-// outlast the rest of the launch; every chunk leaves fp32 partial results in a workspace slot and a small
-// merge kernel combines the slots of a strip.
+// A launch is a fixed set of persistent one-wavefront work-groups, two per SIMD, each walking a host-built list of
+// items: whole strips, pairs of strips (forward) or chunks of a long strip (a global row or column, cut so that it
+// does not outlast the rest of the launch; every chunk leaves fp32 partial results in a workspace slot and a small
+// merge kernel combines the slots of a strip).
 #pragma once
 #include "tile_kernels.h"
 
@@ -37,11 +36,6 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int BF16_WAVES = 4;
-// OCC wavefronts per SIMD: what the registers of each variant allow without spilling (measured: going from two to
-// three or four changes little, the kernels are bound by the instruction mix of a tile, not by latency).
-#define SPION_BF16_KERNEL(OCC) \
-    __global__ __launch_bounds__(64 * BF16_WAVES) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
 constexpr float BF16_LAZY = 8.f;  // the running row maximum is raised only when a tile exceeds it by 2^8
 
 template <int D>
@@ -51,26 +45,6 @@ __device__ __forceinline__ void ldb_rows(rsrc_t r, int voff, int soff, bf16x8 (&
         x[t] = __builtin_bit_cast(bf16x8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff + 16 * t, 0));
 }
 
-// A 32 x D bf16 tile of a row-major head slice is 64*D consecutive bytes.  Loaded as D/16 instructions in which
-// the 64 lanes read 1 KB of consecutive addresses: 8 cache lines per instruction.  (Reading it directly in the
-// operand layout -- every lane 16 bytes of its own row -- costs one tag lookup per lane and was measured to
-// keep the texture path busy 84 % of the time.)  Lane l, instruction i holds 16-byte piece 64i + l of the tile.
-// With rows ld elements apart (a head that is a view of a wider buffer) the same pieces come from 512 / D rows per
-// instruction: lane offset bf16_tile_voff, `step` = bf16_tile_step bytes from one instruction to the next.
-template <int D>
-__device__ __forceinline__ void ldb_tile(rsrc_t r, int lvoff, int soff, int step, u32x4 (&raw)[D / 16]) {
-#pragma unroll
-    for (int i = 0; i < D / 16; ++i) raw[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lvoff, soff + step * i, 0);
-}
-template <int D>
-__device__ __forceinline__ int bf16_tile_voff(int l, int ld) {
-    constexpr int PPR = D / 8;  // 16-byte pieces per row
-    return ((l / PPR) * ld + (l % PPR) * 8) * 2;
-}
-template <int D>
-__device__ __forceinline__ int bf16_tile_step(int ld) {
-    return (512 / D) * ld * 2;
-}
 // Start (in elements), row stride and size in bytes of head bh: contiguous [NB][L][D] heads (ST = false, compile-time
 // figures) or [B][H][L][D] views given by a layout (strides in elements).
 template <bool ST, int D>
@@ -103,51 +77,6 @@ __device__ __forceinline__ void pack16(const float (&p)[16], bf16x8 (&pb)[2]) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) pb[t][e] = (__bf16)p[8 * t + e];
 }
-
-// Wave-private LDS tile of 32 row-major rows of D bf16, rows RS bytes apart.
-template <int D>
-struct LdsTile {
-    static constexpr int RS = D * 2 + 32;
-    static constexpr int BYTES = 32 * RS;
-    // lane (row li, half h) stores the D/2 features it holds as a head-dimension operand
-    static __device__ __forceinline__ void put_rows(char* T, int li, int h, const bf16x8 (&x)[D / 16]) {
-#pragma unroll
-        for (int t = 0; t < D / 16; ++t) *reinterpret_cast<u32x4*>(T + li * RS + h * D + 16 * t) = __builtin_bit_cast(u32x4, x[t]);
-    }
-    // the tile as loaded by ldb_tile: piece 64i + l is row (64i + l) / (D/8), 16-byte column (64i + l) % (D/8)
-    static __device__ __forceinline__ void put_raw(char* T, int l, const u32x4 (&raw)[D / 16]) {
-        constexpr int CPR = D / 8;
-#pragma unroll
-        for (int i = 0; i < D / 16; ++i)
-            *reinterpret_cast<u32x4*>(T + ((64 * i) / CPR + l / CPR) * RS + (l % CPR) * 16) = raw[i];
-    }
-    // head-dimension operand of lane (row li, half h): features h*D/2 ..
-    static __device__ __forceinline__ void get_rows(const char* T, int li, int h, bf16x8 (&x)[D / 16]) {
-#pragma unroll
-        for (int t = 0; t < D / 16; ++t)
-            x[t] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const u32x4*>(T + li * RS + h * D + 16 * t));
-    }
-    // The transposing read works on groups of 16 lanes: lane j of a group points at 4 consecutive bf16,
-    // and lane 4a+b receives element b of the pieces of lanes a, 4+a, 8+a, 12+a.  With lane j pointing at
-    // row R + j/4, features F + 4(j%4) .., lane 4a+b gets rows R..R+3 of feature F + 4a + b.
-    // lane_base: byte offset of this lane's piece for R = 4h, F = 16*((l/16)%2).
-    static __device__ __forceinline__ int lane_base(int l) {
-        const int h = l >> 5, gm = (l >> 4) & 1, j = l & 15;
-        return (4 * h + (j >> 2)) * RS + (16 * gm + 4 * (j & 3)) * 2;
-    }
-    static __device__ __forceinline__ void get_tile_t(const char* T, int base, bf16x8 (&xt)[D / 32][2]) {
-        typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
-#pragma unroll
-        for (int c = 0; c < D / 32; ++c)
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + base + (16 * t) * RS + c * 64));
-                const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(T + base + (16 * t + 8) * RS + c * 64));
-                xt[c][t] = __builtin_shufflevector(__builtin_bit_cast(bf16x4, lo), __builtin_bit_cast(bf16x4, hi), 0, 1,
-                                                   2, 3, 4, 5, 6, 7);
-            }
-    }
-};
 
 // -------------------------------------------------------------------------------------------------
 // Tiles that go from global memory straight into LDS (buffer loads with the LDS modifier): no registers hold a
@@ -303,39 +232,58 @@ __device__ __forceinline__ float half_swap_sum(float x) {
     return lo + hi;
 }
 
-// Sum the per-wave partial results of a cooperative strip (coop) and store the 32 x D result as bf16 rows.
-// acc[c][r] of lane (li, h): row li, feature 32c + acc_row(r, h).
-// part (chunk of a long strip only): the work-group's sum goes there as fp32, register (c, r) of lane l at
-// [(16c + r)*64 + l], instead of to the tensor.
+// The schedule of a launch (built on the host, see build_bf16_plan): every work-group is one persistent wavefront
+// ("lane") that walks entries lane_ptr[b] .. lane_ptr[b+1]-1 of lane_ent, each {head, item}; an item is
+// {strip, first tile, tiles, kind} with kind >= 0: chunk of a long strip whose partial result goes to workspace slot
+// `kind`; -1: a whole strip; -2 (forward): strips `strip` and `strip + 1` together.
+struct Bf16Sched {
+    const int* items;
+    const int* lane_ptr;
+    const int* lane_ent;
+};
+#define SPION_BF16_LANE(OCC) __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(OCC, OCC)))
+// The index arrays never change while a kernel runs: read through the constant address space, loads with a uniform
+// address are scalar loads wherever they stand (left in the global address space, the compiler turns those that
+// follow a store or an assembly statement into vector loads, whose waits would also wait for the tile loads).
+typedef const __attribute__((address_space(4))) int* const_ints;
+__device__ __forceinline__ const_ints as_constant(const int* p) { return (const_ints) reinterpret_cast<unsigned long long>(p); }
+struct LaneEntry {
+    int x, y;  // head, item
+};
+struct PlanItem {
+    int x, y, z, w;  // strip, first tile, tiles, kind
+};
+__device__ __forceinline__ LaneEntry lane_entry(const_ints ents, int e) { return LaneEntry{ents[2 * e], ents[2 * e + 1]}; }
+__device__ __forceinline__ PlanItem plan_item(const_ints items, int k) {
+    return PlanItem{items[4 * k], items[4 * k + 1], items[4 * k + 2], items[4 * k + 3]};
+}
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+// floats per workspace slot: two 32 x D results (the column pass has dK and dV) and 64 row statistics
 template <int D>
-__device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO, int ld, int row0, bool coop, int w,
-                                                int li, int h, float* lds, float* part = nullptr) {
-    const int l = li + 32 * h;
-    if (coop) {
-        __syncthreads();  // lds is the memory of the wave-private tiles: every wavefront is done with them
-        if (w > 0) {
-#pragma unroll
-            for (int c = 0; c < D / 32; ++c)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) lds[(((w - 1) * (D / 32) + c) * 16 + r) * 64 + l] = acc[c][r];
-        }
-        __syncthreads();
-        if (w > 0) return;
-#pragma unroll
-        for (int ww = 0; ww < BF16_WAVES - 1; ++ww)
-#pragma unroll
-            for (int c = 0; c < D / 32; ++c)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) acc[c][r] += lds[((ww * (D / 32) + c) * 16 + r) * 64 + l];
-        if (part) {
-#pragma unroll
-            for (int c = 0; c < D / 32; ++c)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) part[(16 * c + r) * 64 + l] = acc[c][r];
-            return;
-        }
+constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
+
+// Byte offset of head bh inside a tensor (the tile loads address whole tensors: one resource for all heads)
+template <bool ST, int D>
+__device__ __forceinline__ unsigned bf16_head_bytes(const HeadLayout& y, int H, int bh, int L) {
+    if constexpr (ST) {
+        const int b = bh / H, hh = bh - b * H;
+        return (unsigned)(((size_t)b * y.bstride + (size_t)hh * y.hstride) * 2);
+    } else {
+        return (unsigned)((size_t)bh * L * D * 2);
     }
-    const int voff = (li * ld + 4 * h) * 2;
+}
+
+// A 32 x D result held as acc[c][r] of lane (li, h) = row li, feature 32c + acc_row(r, h), written as bf16 rows
+// through an LDS tile T: every lane writes its 8-byte pieces into the permuted tile image (DmaTile), the tile is
+// read back 1 KB per instruction and stored with the lane offsets of the tile loads -- whole rows per store
+// instruction where every lane storing pieces of its own row would touch 32 cache lines per instruction.
+// soff: byte offset of the strip's first row.
+template <int D>
+__device__ __forceinline__ void stage_store_bf16(const f32x16 (&acc)[D / 32], char* T, rsrc_t r, int lvoff, int soff,
+                                                 int ld, int l) {
+    typedef DmaTile<D> DT;
+    const int li = l & 31, h = l >> 5;
 #pragma unroll
     for (int c = 0; c < D / 32; ++c)
 #pragma unroll
@@ -343,606 +291,640 @@ __device__ __forceinline__ void store_rows_bf16(f32x16 (&acc)[D / 32], rsrc_t rO
             bf16x4 v;
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] = (__bf16)acc[c][4 * g + e];
-            __builtin_amdgcn_raw_buffer_store_b64(__builtin_bit_cast(u32x2, v), rO, voff, row0 * ld * 2 + (32 * c + 8 * g) * 2, 0);
+            *reinterpret_cast<u32x2*>(T + li * DT::ROW + 16 * ((4 * c + g) ^ DT::swz(li)) + 8 * h) = __builtin_bit_cast(u32x2, v);
         }
+#pragma unroll
+    for (int i = 0; i < DT::NI; ++i) {
+        const u32x4 x = *reinterpret_cast<const u32x4*>(T + 1024 * i + 16 * l);
+        store_b128(x, r, lvoff, soff + i * (64 / DT::CPR) * ld * 2);
+    }
+}
+// The same result as fp32 into a workspace slot (chunk of a long strip): register (c, r) of lane l at [(16c + r)*64 + l].
+template <int D>
+__device__ __forceinline__ void store_part(const f32x16 (&acc)[D / 32], float* part, int l) {
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) part[(16 * c + r) * 64 + l] = acc[c][r];
 }
 
-// Work-group entry {a, b, c, d}.  a != b: strips a, b, c, d, one per wavefront (-1: none).  a == b: the four
-// wavefronts walk chunk c of long strip a together (tiles c*chunk .. of the strip, `chunk` a launch parameter) and
-// leave their sum in workspace slot d.
-struct StripAssign {
-    int strip, rank, step, chunk_id, slot;
-    bool coop;
-};
-__device__ __forceinline__ StripAssign strip_of_wave(const int* __restrict__ wg_list, int g, int w) {
-    const int4 e = reinterpret_cast<const int4*>(wg_list)[g];
-    StripAssign s;
-    s.coop = e.x == e.y;
-    s.strip = s.coop ? e.x : (w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w);
-    s.rank = s.coop ? w : 0;
-    s.step = s.coop ? BF16_WAVES : 1;
-    s.chunk_id = s.coop ? e.z : 0;
-    s.slot = s.coop ? e.w : -1;
-    return s;
-}
-// floats per workspace slot: two 32 x D results (the column pass has dK and dV) and 64 row statistics
-template <int D>
-constexpr int bf16_slot_floats() { return 2 * 32 * D + 64; }
+// A lane's loads form one stream across its items.  Every element of the stream is the same three loads -- two
+// 32 x D tiles into the two tile slots of an LDS buffer and 256 bytes into its third slot -- and is either a tile
+// of the item (a K and a V tile and the key penalties; in the column pass a Q and a dO tile and the statistics of
+// the query strip) or, ahead of the item's tiles, the strip's own operands, which reach the registers through LDS
+// like everything else: loads whose lanes each fetch pieces of their own row cost the memory pipeline a cache-line
+// look-up per lane, and, completing in order with the tile loads, would hold the whole stream up.
+// Element number g of the stream lives in buffer g % 2; the loads of element g + 2 are issued as soon as element g
+// has left its buffer -- also when it belongs to the lane's next item, so the stream does not drain at item
+// boundaries.  An item's last element keeps its buffer a little longer: the item's result is staged there
+// (stage_store_bf16).  The kernels keep
+//   g   number of the element being worked on,   gi  elements issued so far (g <= gi <= g + 3),
+//   and the kind and scalar offsets of element gi, looked up one element ahead of its issue.
+// At the start of an element its loads are the oldest outstanding ones and at most one younger batch exists.
+enum { EL_TILE = 0, EL_A = 1, EL_B = 2 };
 
 // -------------------------------------------------------------------------------------------------
-// Forward: one sweep per block row with a lazily raised running maximum.
+// Forward: one sweep per block row with a lazily raised running maximum.  PAIRS: the launch walks the pair plan,
+// whose items of kind -2 give a wavefront strips 2p and 2p+1 (masks of 64 x 64 blocks and larger, where the two
+// hold the same block columns): every K and V tile is fetched and read back as an operand once for the two strips'
+// chains, and the two softmax updates are independent instruction streams.
+// Stream of an item: {Q tile of the strip (twice, or of both strips of a pair)}, then its K / V tiles.
 // -------------------------------------------------------------------------------------------------
-// The LDS space of a forward work-group: the tile buffers of each wavefront (DmaTile; reused for the partial results
-// of a shared strip) and the row statistics the wavefronts of a shared strip exchange.
-template <int D>
-struct Bf16FwdLds {
+template <int D, bool MASK, bool ST, bool PAIRS>
+SPION_BF16_LANE(2) void bf16_fwd_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ tcol,
+    const int* __restrict__ plan_items, const int* __restrict__ lane_ptr, const int* __restrict__ lane_ent, int L,
+    int NB, float scale, float* __restrict__ Part, int n_slots, Layouts ly, unsigned in_bytes, unsigned out_bytes) {
     typedef DmaTile<D> DT;
-    __attribute__((aligned(16))) char t[BF16_WAVES][DT::WAVE];
-    float m[BF16_WAVES][32], z[BF16_WAVES][32];
-};
-
-// One strip (or one chunk of a long strip, shared by the four wavefronts) per wavefront.
-template <int D, bool MASK, bool ST>
-__device__ __forceinline__ void bf16_fwd_strip(
-    Bf16FwdLds<D>& lds, const StripAssign sa, int bh, int w, const __bf16* __restrict__ Q,
-    const __bf16* __restrict__ K, const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O,
-    float* __restrict__ Lse, const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale,
-    float* __restrict__ Part, int n_slots, int chunk, const Layouts& ly) {
-    typedef DmaTile<D> DT;
-    auto& lds_m = lds.m;
-    auto& lds_z = lds.z;
-    float* lds_o = reinterpret_cast<float*>(&lds.t[0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
+    __shared__ __attribute__((aligned(16))) char Tw[DT::WAVE];
     const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int I = sa.strip;
-    const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
-    const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
-    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
-    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    size_t ib, ob, ibytes, obytes;
-    int ild, old_;
-    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
-    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
-    const rsrc_t rQ = make_rsrc(Q + ib, ibytes);
-    const rsrc_t rO = make_rsrc(O + ob, obytes);
-    const u32x4 wK = rsrc_words(K + ib, ibytes), wV = rsrc_words(V + ib, ibytes);
-    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int r_voff = li * ild * 2 + h * D;
+    const int e0 = as_constant(lane_ptr)[blockIdx.x], e1 = as_constant(lane_ptr)[blockIdx.x + 1];
+    if (e0 >= e1) return;
+    const const_ints ents = as_constant(lane_ent), items = as_constant(plan_items), tiles = as_constant(tcol);
+    const int ild = ST ? ly.in.ld : D, old_ = ST ? ly.out.ld : D;
+    const u32x4 wQ = rsrc_words(Q, in_bytes), wK = rsrc_words(K, in_bytes), wV = rsrc_words(V, in_bytes);
+    const u32x4 wM = rsrc_words(MASK ? (const void*)pen : (const void*)K, MASK ? (size_t)NB * L * 4 : in_bytes);
+    const rsrc_t rO = make_rsrc(O, out_bytes);
     const int t_bytes = 32 * ild * 2;
-    const int d_voff = DT::voff(l, ild), d_xstep = DT::extra_step(ild);
-    const char* Tw = lds.t[w];
+    const int vin = DT::voff(l, ild), xin = DT::extra_step(ild), vout = DT::voff(l, old_);
     const unsigned lds_w = lds_address(Tw);
     const typename DT::RowAddr ra = DT::row_addr(li, h);
     const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+    constexpr int E = 1, OPS = 2 * DT::NI + 1;
 
-    bf16x8 q[D / 16];
-    ldb_rows<D>(rQ, r_voff, I * t_bytes, q);
-
-    // Floor of the running maximum (the reference's max(-100, .) / max(0, .), models/block_attn.cu:52): any
-    // value gives the same probabilities; 2^-100 keeps (L - n) * 2^-m finite in fp32 for empty rows.
-    float m = MASK ? 0.f : -100.f, z = 0.f;
-    f32x16 o[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
-
-    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
-    auto tile_id = [&](int i) { return tcol[t0 + sa.rank + min(i, nu - 1) * sa.step]; };
-    auto issue = [&](int J, int par) {  // key tile J -> buffer par
-        const unsigned a = lds_w + par * DT::BUF;
-        DT::load(wK, a, d_voff, J * t_bytes, d_xstep);
-        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, d_xstep);
-        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
-    };
-    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
-    auto compute = [&](int par, int inext) {
-        const char* Tk = Tw + par * DT::BUF;
-        const char* Tv = Tk + DT::TILE;
-        bf16x8 kr[D / 16], vt[D / 32][2];
-        DT::get_rows(Tk, ra, kr);
-        DT::get_tile_t(Tv, ta, vt);
-        f32x16 init = splat16(0.f);
-        if constexpr (MASK) {
-            float pj[16];
-            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
-#pragma unroll
-            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+    LaneEntry en = lane_entry(ents, e0);
+    PlanItem itn = plan_item(items, en.y);
+    int g = 0, gi = 0;
+    int sk = 0, sa = 0, sb = 0, sc = 0, sq_g = -1;  // element sq_g: kind and the offsets of its three loads
+    for (int e = e0; e < e1; ++e) {
+        const int bh = en.x;
+        const PlanItem it = itn;
+        const bool has_next = e + 1 < e1;
+        if (has_next) {
+            en = lane_entry(ents, e + 1);
+            itn = plan_item(items, en.y);
         }
-        wait_lgkm0();  // the tile's operands are in registers: its buffer can take the tile after next
-        if (inext >= 0) issue(Jq, par);
-        Jq = tile_id(inext + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
-        const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
-        if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
-            const float mn = t2 > m + BF16_LAZY ? t2 : m;
-            const float f = __builtin_amdgcn_exp2f(m - mn);
-            z *= f;
+        const int bhn = en.x;
+        const int I = it.x, t0 = it.y, n = it.z;
+        const bool pair = PAIRS && it.w == -2;
+        const int In = itn.x, t0n = itn.y;
+        const bool pairn = PAIRS && itn.w == -2;
+        const int len = E + n, lenn = has_next ? E + itn.z : 0;
+        const int g0 = g;
+        const unsigned hb = bf16_head_bytes<ST, D>(ly.in, ly.H, bh, L), hbn = bf16_head_bytes<ST, D>(ly.in, ly.H, bhn, L);
+        // element k of an item (given by value: selecting between variables captured by reference would pin them to
+        // memory)
+        auto locate_in = [&](int k, int bhX, int IX, int t0X, unsigned hbX, bool pairX) __attribute__((always_inline)) {
+            if (k == 0) {
+                sk = EL_A;
+                sa = uniform((int)(hbX + (unsigned)(IX * t_bytes)));
+                sb = uniform((int)(hbX + (unsigned)((IX + (pairX ? 1 : 0)) * t_bytes)));
+                sc = sa;
+            } else {
+                const int J = tiles[t0X + k - E];
+                sk = EL_TILE;
+                sa = uniform((int)(hbX + (unsigned)(J * t_bytes)));
+                sb = sa;
+                sc = MASK ? uniform((bhX * L + J * 32) * 4) : sa;
+            }
+        };
+        auto locate = [&, bh, bhn, I, In, t0, t0n, hb, hbn, pair, pairn, len, g0](int gg) __attribute__((always_inline)) {
+            const int k = gg - g0;
+            if (k < len) locate_in(k, bh, I, t0, hb, pair);
+            else locate_in(k - len, bhn, In, t0n, hbn, pairn);
+            sq_g = gg;
+        };
+        auto issue = [&]() __attribute__((always_inline)) {  // element gi -> buffer gi % 2, then look the following one up
+            const unsigned a = lds_w + (gi & 1) * DT::BUF;
+            if (sk == EL_TILE) {
+                DT::load(wK, a, vin, sa, xin);
+                DT::load(wV, a + DT::TILE, vin, sb, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, sc);
+            } else {
+                DT::load(wQ, a, vin, sa, xin);
+                DT::load(wQ, a + DT::TILE, vin, sb, xin);
+                dma_b32(wQ, a + 2 * DT::TILE, l * 4, sc);
+            }
+            ++gi;
+            if (gi - g0 < len + lenn) locate(gi);
+        };
+        auto begin = [&]() __attribute__((always_inline)) -> char* {  // wait for element g
+            if (gi - g > 1) wait_vm<OPS>();
+            else wait_vm<0>();
+            return Tw + (g & 1) * DT::BUF;
+        };
+        auto release = [&]() __attribute__((always_inline)) {  // element g has left its buffer
+            wait_lgkm0();
 #pragma unroll
-            for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
-            m = mn;
-        }
-        float p[16];
+            for (int k = 0; k < 2; ++k)
+                if (gi <= g + 2 && sq_g == gi) issue();
+        };
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
-            z += p[r];
+        for (int k = 0; k < 2; ++k)
+            if (gi < g0 + min(2, len)) {
+                if (sq_g != gi) locate(gi);
+                issue();
+            }
+        float* part = it.w >= 0 ? Part + ((size_t)bh * n_slots + it.w) * bf16_slot_floats<D>() : nullptr;
+        const unsigned ho = bf16_head_bytes<ST, D>(ly.out, ly.H, bh, L);
+        // one tile: the operands leave LDS, the buffer goes to the element after next (the item's last tile keeps
+        // it for the result), `math` does the arithmetic
+        auto tile = [&](bool last, auto&& math) __attribute__((always_inline)) {
+            const char* Tk = begin();
+            const char* Tv = Tk + DT::TILE;
+            bf16x8 kr[D / 16], vt[D / 32][2];
+            DT::get_rows(Tk, ra, kr);
+            DT::get_tile_t(Tv, ta, vt);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+                float pj[16];
+                lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+            }
+            if (!last) release();
+            else wait_lgkm0();
+            __builtin_amdgcn_sched_barrier(0);
+            math(kr, vt, init);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) ++g;
+        };
+        // Floor of the running maximum (the reference's max(-100, .) / max(0, .), models/block_attn.cu:52): any
+        // value gives the same probabilities; 2^-100 keeps (L - n) * 2^-m finite in fp32 for empty rows.
+        auto update = [&](const f32x16& s, float& m, float& z, f32x16 (&o)[D / 32], bf16x8 (&pb)[2]) __attribute__((always_inline)) {
+            const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
+            if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
+                const float mn = t2 > m + BF16_LAZY ? t2 : m;
+                const float f = __builtin_amdgcn_exp2f(m - mn);
+                z *= f;
+#pragma unroll
+                for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
+                m = mn;
+            }
+            float p[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
+                z += p[r];
+            }
+            pack16(p, pb);
+        };
+        // rows_all: tiles of the whole strip; T: where the result is staged (a chunk finishes nothing: the merge
+        // kernel does)
+        auto finish = [&](float m, float z, f32x16 (&o)[D / 32], int strip, int rows_all, float* pt, char* T) __attribute__((always_inline)) {
+            z = half_swap_sum(z);
+            if (pt) {  // chunk of a long strip: unnormalised sums relative to m
+                if (h == 0) {
+                    pt[2 * 32 * D + li] = m;
+                    pt[2 * 32 * D + 32 + li] = z;
+                }
+                store_part<D>(o, pt, l);
+                return;
+            }
+            const int off_pattern = L - rows_all * 32;
+            if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);  // models/block_attn.cu:74
+            const float rinv = 1.0f / z;
+#pragma unroll
+            for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
+            if (h == 0) Lse[(size_t)bh * L + strip * 32 + li] = m + __builtin_amdgcn_logf(z);
+            stage_store_bf16<D>(o, T, rO, vout, (int)(ho + (unsigned)(strip * 32 * old_ * 2)), old_, l);
+        };
+        if (pair) {
+            char* Ta = begin();
+            bf16x8 q0[D / 16], q1[D / 16];
+            DT::get_rows(Ta, ra, q0);
+            DT::get_rows(Ta + DT::TILE, ra, q1);
+            if (n > 0) {
+                release();
+                ++g;
+            }
+            float m0 = MASK ? 0.f : -100.f, z0 = 0.f, m1 = m0, z1 = 0.f;
+            f32x16 o0[D / 32], o1[D / 32];
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c) {
+                o0[c] = splat16(0.f);
+                o1[c] = splat16(0.f);
+            }
+            for (int i = 0; i < n; ++i)
+                tile(i + 1 == n, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
+                    const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
+                    const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
+                    bf16x8 pb0[2], pb1[2];
+                    update(s0, m0, z0, o0, pb0);
+                    update(s1, m1, z1, o1, pb1);
+                    mma_tile_bf16<D>(vt, pb0, o0);
+                    mma_tile_bf16<D>(vt, pb1, o1);
+                });
+            char* Tl = Tw + (g & 1) * DT::BUF;  // the item's last element: its buffer stages the results
+            wait_lgkm0();
+            finish(m0, z0, o0, I, n, nullptr, Tl);
+            finish(m1, z1, o1, I + 1, n, nullptr, Tl + DT::TILE);
+        } else {
+            char* Ta = begin();
+            bf16x8 q[D / 16];
+            DT::get_rows(Ta, ra, q);
+            if (n > 0) {
+                release();
+                ++g;
+            }
+            float m = MASK ? 0.f : -100.f, z = 0.f;
+            f32x16 o[D / 32];
+#pragma unroll
+            for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
+            for (int i = 0; i < n; ++i)
+                tile(i + 1 == n, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
+                    const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
+                    bf16x8 pb[2];
+                    update(s, m, z, o, pb);
+                    mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
+                });
+            char* Tl = Tw + (g & 1) * DT::BUF;
+            wait_lgkm0();
+            // the whole strip's tile count decides the off-pattern term; a chunk leaves that to the merge kernel
+            finish(m, z, o, I, n, part, Tl);
         }
-        bf16x8 pb[2];
-        pack16(p, pb);
-        mma_tile_bf16<D>(vt, pb, o);  // O^T: register = feature, lane = query
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    settle(q);
-    if (nu > 0) issue(tile_id(0), 0);
-    if (nu > 1) issue(tile_id(1), 1);
-    if (nu > 2) Jq = tile_id(2);
-    for (int i = 0; i < nu; i += 2) {
-        if (i + 1 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(0, i + 2 < nu ? i + 2 : -1);
-        if (i + 1 >= nu) break;
-        if (i + 2 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(1, i + 3 < nu ? i + 3 : -1);
+        release();
+        ++g;
     }
-    z = half_swap_sum(z);
-    if (sa.coop) {
-        if (h == 0) {
-            lds_m[w][li] = m;
-            lds_z[w][li] = z;
-        }
-        __syncthreads();
-        float M = lds_m[0][li];
-#pragma unroll
-        for (int ww = 1; ww < BF16_WAVES; ++ww) M = fmaxf(M, lds_m[ww][li]);
-        float Z = 0.f;
-#pragma unroll
-        for (int ww = 0; ww < BF16_WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - M);
-        const float f = __builtin_amdgcn_exp2f(m - M);
-#pragma unroll
-        for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
-        m = M;
-        z = Z;
-    }
-    if (part) {  // chunk of a long strip: unnormalised sums relative to m; the merge kernel finishes the rows
-        if (w == 0 && h == 0) {
-            part[2 * 32 * D + li] = m;
-            part[2 * 32 * D + 32 + li] = z;
-        }
-        store_rows_bf16<D>(o, rO, old_, I * 32, true, w, li, h, lds_o, part);
-        return;
-    }
-    const int off_pattern = L - cnt_all * 32;
-    if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);  // models/block_attn.cu:74
-    const float rinv = 1.0f / z;
-#pragma unroll
-    for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
-    if (sa.rank == 0 && h == 0) Lse[(size_t)bh * L + I * 32 + li] = m + __builtin_amdgcn_logf(z);
-    store_rows_bf16<D>(o, rO, old_, I * 32, sa.coop, w, li, h, lds_o);
-}
-
-template <int D, bool MASK, bool ST>
-SPION_BF16_KERNEL(D == 32 ? (MASK ? 3 : 4) : 2) void bf16_fwd_kernel(
-    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
-    __shared__ Bf16FwdLds<D> lds;
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index();
-    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
-    if (sa.strip < 0) return;  // only in entries of independent strips: no barrier is skipped
-    bf16_fwd_strip<D, MASK, ST>(lds, sa, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale, Part, n_slots, chunk, ly);
-}
-
-// -------------------------------------------------------------------------------------------------
-// Forward, two strips per wavefront: for masks of 64 x 64 blocks and larger, strips 2p and 2p+1 hold the same block
-// columns, so one wavefront takes both: every K and V tile is fetched, copied to LDS and read back as an operand
-// once for the two strips' chains, and the two softmax updates are independent instruction streams.  pair_list:
-// four pair indices per work-group (-1: none); pairs whose strips are long enough to be cut into chunks stay with
-// bf16_fwd_kernel.
-// -------------------------------------------------------------------------------------------------
-template <int D, bool MASK>
-__device__ __forceinline__ void bf16_fwd_pair(
-    Bf16FwdLds<D>& lds, int pr, int bh, int w, const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
-    const __bf16* __restrict__ V, const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse,
-    const int* __restrict__ trp, const int* __restrict__ tcol, int L, float scale) {
-    typedef DmaTile<D> DT;
-    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int I = 2 * pr;
-    const int t0 = trp[I], cnt = trp[I + 1] - t0;
-    const size_t hb = (size_t)bh * L * D, hbytes = (size_t)L * D * 2;
-    const rsrc_t rQ = make_rsrc(Q + hb, hbytes);
-    const rsrc_t rO = make_rsrc(O + hb, hbytes);
-    const u32x4 wK = rsrc_words(K + hb, hbytes), wV = rsrc_words(V + hb, hbytes);
-    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int r_voff = li * D * 2 + h * D;
-    const int t_bytes = 32 * D * 2;
-    const int d_voff = DT::voff(l, D);
-    const char* Tw = lds.t[w];
-    const unsigned lds_w = lds_address(Tw);
-    const typename DT::RowAddr ra = DT::row_addr(li, h);
-    const typename DT::TrAddr ta = DT::tr_addr(l);
-    const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
-
-    bf16x8 q0[D / 16], q1[D / 16];
-    ldb_rows<D>(rQ, r_voff, I * t_bytes, q0);
-    ldb_rows<D>(rQ, r_voff, (I + 1) * t_bytes, q1);
-    float m0 = MASK ? 0.f : -100.f, z0 = 0.f, m1 = m0, z1 = 0.f;
-    f32x16 o0[D / 32], o1[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) {
-        o0[c] = splat16(0.f);
-        o1[c] = splat16(0.f);
-    }
-    auto update = [&](const f32x16& s, float& m, float& z, f32x16 (&o)[D / 32], bf16x8 (&pb)[2]) {
-        const float t2 = half_swap_max(max16(s, -3.0e38f)) * c2;
-        if (__builtin_amdgcn_ballot_w64(t2 > m + BF16_LAZY) != 0) {
-            const float mn = t2 > m + BF16_LAZY ? t2 : m;
-            const float f = __builtin_amdgcn_exp2f(m - mn);
-            z *= f;
-#pragma unroll
-            for (int cc = 0; cc < D / 32; ++cc) o[cc] *= f;
-            m = mn;
-        }
-        float p[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -m));
-            z += p[r];
-        }
-        pack16(p, pb);
-    };
-    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
-    auto tile_id = [&](int i) { return tcol[t0 + min(i, cnt - 1)]; };
-    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
-    auto issue = [&](int J, int par) {
-        const unsigned a = lds_w + par * DT::BUF;
-        DT::load(wK, a, d_voff, J * t_bytes, 0);
-        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, 0);
-        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
-    };
-    auto compute = [&](int par, int inext) {
-        const char* Tk = Tw + par * DT::BUF;
-        const char* Tv = Tk + DT::TILE;
-        bf16x8 kr[D / 16], vt[D / 32][2];
-        DT::get_rows(Tk, ra, kr);
-        DT::get_tile_t(Tv, ta, vt);
-        f32x16 init = splat16(0.f);
-        if constexpr (MASK) {
-            float pj[16];
-            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
-        }
-        wait_lgkm0();
-        if (inext >= 0) issue(Jq, par);
-        Jq = tile_id(inext + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
-        const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
-        bf16x8 pb0[2], pb1[2];
-        update(s0, m0, z0, o0, pb0);
-        update(s1, m1, z1, o1, pb1);
-        mma_tile_bf16<D>(vt, pb0, o0);
-        mma_tile_bf16<D>(vt, pb1, o1);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    settle(q0);
-    settle(q1);
-    if (cnt > 0) issue(tile_id(0), 0);
-    if (cnt > 1) issue(tile_id(1), 1);
-    if (cnt > 2) Jq = tile_id(2);
-    for (int i = 0; i < cnt; i += 2) {
-        if (i + 1 < cnt) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(0, i + 2 < cnt ? i + 2 : -1);
-        if (i + 1 >= cnt) break;
-        if (i + 2 < cnt) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(1, i + 3 < cnt ? i + 3 : -1);
-    }
-    const int off_pattern = L - cnt * 32;
-    float* lds_unused = nullptr;
-    auto finish = [&](float m, float z, f32x16 (&o)[D / 32], int strip) {
-        z = half_swap_sum(z);
-        if (off_pattern > 0) z += (float)off_pattern * __builtin_amdgcn_exp2f(-m);
-        const float rinv = 1.0f / z;
-#pragma unroll
-        for (int cc = 0; cc < D / 32; ++cc) o[cc] *= rinv;
-        if (h == 0) Lse[(size_t)bh * L + strip * 32 + li] = m + __builtin_amdgcn_logf(z);
-        store_rows_bf16<D>(o, rO, D, strip * 32, false, w, li, h, lds_unused);
-    };
-    finish(m0, z0, o0, I);
-    finish(m1, z1, o1, I + 1);
-}
-
-// Work-group list of the paired forward: entries {a, a, c, slot} are chunk c of long strip a, shared by the four
-// wavefronts (bf16_fwd_strip; these entries come first), entries {p0, p1, p2, p3} four pairs of strips, one per
-// wavefront (-1: none).  One launch for both kinds: the few work-groups of the long strips would otherwise set the
-// length of a launch of their own (32 us for configuration 5).
-template <int D, bool MASK>
-SPION_BF16_KERNEL(2) void bf16_fwd_pair_kernel(
-    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const float* __restrict__ pen, __bf16* __restrict__ O, float* __restrict__ Lse, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk) {
-    __shared__ Bf16FwdLds<D> lds;
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index();
-    const int4 e = reinterpret_cast<const int4*>(list)[item % n_wg];
-    if (e.x == e.y) {  // uniform over the work-group
-        const StripAssign sa = strip_of_wave(list, item % n_wg, w);
-        bf16_fwd_strip<D, MASK, false>(lds, sa, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale, Part, n_slots, chunk,
-                                       Layouts{});
-        return;
-    }
-    const int pr = w == 0 ? e.x : w == 1 ? e.y : w == 2 ? e.z : e.w;
-    if (pr < 0) return;
-    bf16_fwd_pair<D, MASK>(lds, pr, bh, w, Q, K, V, pen, O, Lse, trp, tcol, L, scale);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, row pass: g_i = dO_i . O_i, P and dP recomputed per tile, dS' = P*(dP - g), dQ += dS'.K_J;
 // the 1/sqrt(d) is applied to the 32 x d result.  Stats receives {lse2, -g} of every strip (64 floats per strip:
 // the 32 lse2 values, then the 32 -g values) for the column pass.
-// K and V tiles go from global memory straight into one of two LDS buffers of the wavefront (DmaTile), two tiles
-// ahead of the one being worked on.
+// Stream of an item: {Q tile, dO tile, lse2 of the strip}, {O tile of the strip}, then its K / V tiles.
 // -------------------------------------------------------------------------------------------------
 template <int D, bool MASK, bool ST>
-SPION_BF16_KERNEL(D == 32 ? 3 : 2) void bf16_bwd_row_kernel(
+SPION_BF16_LANE(2) void bf16_bwd_row_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
     const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
-    const float* __restrict__ pen, float* __restrict__ Stats, __bf16* __restrict__ dQ, const int* __restrict__ trp,
-    const int* __restrict__ tcol, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
+    const float* __restrict__ pen, float* __restrict__ Stats, __bf16* __restrict__ dQ, const int* __restrict__ tcol,
+    const int* __restrict__ plan_items, const int* __restrict__ lane_ptr, const int* __restrict__ lane_ent, int L,
+    int NB, float scale, float* __restrict__ Part, int n_slots, Layouts ly, unsigned in_bytes, unsigned out_bytes,
+    unsigned grad_bytes) {
     typedef DmaTile<D> DT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][DT::WAVE];
-    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
-    if (sa.strip < 0) return;
-    const int I = sa.strip;
-    const int cnt_all = trp[I + 1] - trp[I], tb = sa.chunk_id * chunk;
-    const int t0 = trp[I] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
-    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
-    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    size_t ib, ob, gb, ibytes, obytes, gbytes;
-    int ild, old_, gld;
-    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
-    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
-    bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rQ = make_rsrc(Q + ib, ibytes);
-    const rsrc_t rdO = make_rsrc(dO + ob, obytes), rO = make_rsrc(O + ob, obytes), rdQ = make_rsrc(dQ + gb, gbytes);
-    const u32x4 wK = rsrc_words(K + ib, ibytes), wV = rsrc_words(V + ib, ibytes);
-    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int r_voff = li * ild * 2 + h * D, ro_voff = li * old_ * 2 + h * D;
-    const int t_bytes = 32 * ild * 2;
-    const int d_voff = DT::voff(l, ild), d_xstep = DT::extra_step(ild);
-    const char* Tw = lds_t[w];
+    __shared__ __attribute__((aligned(16))) char Tw[DT::WAVE];
+    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int e0 = as_constant(lane_ptr)[blockIdx.x], e1 = as_constant(lane_ptr)[blockIdx.x + 1];
+    if (e0 >= e1) return;
+    const const_ints ents = as_constant(lane_ent), items = as_constant(plan_items), tiles = as_constant(tcol);
+    const int ild = ST ? ly.in.ld : D, old_ = ST ? ly.out.ld : D, gld = ST ? ly.grad.ld : D;
+    const u32x4 wQ = rsrc_words(Q, in_bytes), wK = rsrc_words(K, in_bytes), wV = rsrc_words(V, in_bytes);
+    const u32x4 wG = rsrc_words(dO, out_bytes), wO = rsrc_words(O, out_bytes);
+    const u32x4 wL = rsrc_words(Lse, (size_t)NB * L * 4);
+    const u32x4 wM = rsrc_words(MASK ? pen : Lse, (size_t)NB * L * 4);
+    const rsrc_t rdQ = make_rsrc(dQ, grad_bytes);
+    const int t_bytes = 32 * ild * 2, o_bytes = 32 * old_ * 2;
+    const int vin = DT::voff(l, ild), xin = DT::extra_step(ild);
+    const int vout = DT::voff(l, old_), xout = DT::extra_step(old_), vgr = DT::voff(l, gld);
     const unsigned lds_w = lds_address(Tw);
     const typename DT::RowAddr ra = DT::row_addr(li, h);
     const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+    constexpr int E = 2, OPS = 2 * DT::NI + 1;
 
-    bf16x8 q[D / 16], go[D / 16];
-    ldb_rows<D>(rQ, r_voff, I * t_bytes, q);
-    ldb_rows<D>(rdO, ro_voff, I * 32 * old_ * 2, go);
-    float g = 0.f;
-    {
-        bf16x8 oo[D / 16];
-        ldb_rows<D>(rO, ro_voff, I * 32 * old_ * 2, oo);
-#pragma unroll
-        for (int t = 0; t < D / 16; ++t)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) g = fmaf((float)go[t][e], (float)oo[t][e], g);
-        g = half_swap_sum(g);
-    }
-    const float lse = Lse[(size_t)bh * L + I * 32 + li];
-    if (sa.rank == 0 && tb == 0) Stats[((size_t)bh * (L / 32) + I) * 64 + l] = h ? -g : lse;
-    const f32x16 gneg = splat16(-g);
-
-    f32x16 acc[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
-    // tile i of this wavefront -> buffer par
-    constexpr int OPS = 2 * DT::NI + (MASK ? 1 : 0);
-    auto tile_id = [&](int i) { return tcol[t0 + sa.rank + min(i, nu - 1) * sa.step]; };
-    auto issue = [&](int J, int par) {
-        const unsigned a = lds_w + par * DT::BUF;
-        DT::load(wK, a, d_voff, J * t_bytes, d_xstep);
-        DT::load(wV, a + DT::TILE, d_voff, J * t_bytes, d_xstep);
-        if constexpr (MASK) dma_b32(wM, a + 2 * DT::TILE, l * 4, J * 128);
-    };
-    int Jq = 0;  // tile the next issue fetches, requested one tile ahead of that issue
-    auto compute = [&](int par, int inext) {
-        const char* Tk = Tw + par * DT::BUF;
-        const char* Tv = Tk + DT::TILE;
-        bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
-        DT::get_rows(Tk, ra, kr);
-        DT::get_rows(Tv, ra, vr);
-        DT::get_tile_t(Tk, ta, kt);
-        f32x16 init = splat16(0.f);
-        if constexpr (MASK) {
-            float pj[16];
-            lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
-#pragma unroll
-            for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+    LaneEntry en = lane_entry(ents, e0);
+    PlanItem itn = plan_item(items, en.y);
+    int g = 0, gi = 0;
+    int sk = 0, sa = 0, sb = 0, sc = 0, sq_g = -1;  // element sq_g: kind and the offsets of its three loads
+    for (int e = e0; e < e1; ++e) {
+        const int bh = en.x;
+        const PlanItem it = itn;
+        const bool has_next = e + 1 < e1;
+        if (has_next) {
+            en = lane_entry(ents, e + 1);
+            itn = plan_item(items, en.y);
         }
-        wait_lgkm0();  // the tile's operands are in registers: its buffer can take the tile after next
-        if (inext >= 0) issue(Jq, par);
-        Jq = tile_id(inext + 1);
-        __builtin_amdgcn_sched_barrier(0);
-        const f32x16 s = mma_feat_bf16<D>(kr, q, init);
-        const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
-        float ds[16];
+        const int bhn = en.x;
+        const int I = it.x, t0 = it.y, n = it.z;
+        const int In = itn.x, t0n = itn.y;
+        const int len = E + n, lenn = has_next ? E + itn.z : 0;
+        const int g0 = g;
+        const unsigned hb = bf16_head_bytes<ST, D>(ly.in, ly.H, bh, L), hbn = bf16_head_bytes<ST, D>(ly.in, ly.H, bhn, L);
+        const unsigned ho = bf16_head_bytes<ST, D>(ly.out, ly.H, bh, L), hon = bf16_head_bytes<ST, D>(ly.out, ly.H, bhn, L);
+        auto locate_in = [&](int k, int bhX, int IX, int t0X, unsigned hbX, unsigned hoX) __attribute__((always_inline)) {
+            const int lsx = (bhX * L + IX * 32) * 4;
+            if (k == 0) {
+                sk = EL_A;
+                sa = uniform((int)(hbX + (unsigned)(IX * t_bytes)));
+                sb = uniform((int)(hoX + (unsigned)(IX * o_bytes)));
+                sc = uniform(lsx);
+            } else if (k == 1) {
+                sk = EL_B;
+                sa = uniform((int)(hoX + (unsigned)(IX * o_bytes)));
+                sb = sa;
+                sc = uniform(lsx);
+            } else {
+                const int J = tiles[t0X + k - E];
+                sk = EL_TILE;
+                sa = uniform((int)(hbX + (unsigned)(J * t_bytes)));
+                sb = sa;
+                sc = uniform(MASK ? (bhX * L + J * 32) * 4 : lsx);
+            }
+        };
+        auto locate = [&, bh, bhn, I, In, t0, t0n, hb, hbn, ho, hon, len, g0](int gg) __attribute__((always_inline)) {
+            const int k = gg - g0;
+            if (k < len) locate_in(k, bh, I, t0, hb, ho);
+            else locate_in(k - len, bhn, In, t0n, hbn, hon);
+            sq_g = gg;
+        };
+        auto issue = [&]() __attribute__((always_inline)) {  // element gi -> buffer gi % 2, then look the following one up
+            const unsigned a = lds_w + (gi & 1) * DT::BUF;
+            if (sk == EL_TILE) {
+                DT::load(wK, a, vin, sa, xin);
+                DT::load(wV, a + DT::TILE, vin, sb, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, sc);
+            } else if (sk == EL_A) {
+                DT::load(wQ, a, vin, sa, xin);
+                DT::load(wG, a + DT::TILE, vout, sb, xout);
+                dma_b32(wL, a + 2 * DT::TILE, l * 4, sc);
+            } else {
+                DT::load(wO, a, vout, sa, xout);
+                DT::load(wO, a + DT::TILE, vout, sb, xout);
+                dma_b32(wL, a + 2 * DT::TILE, l * 4, sc);
+            }
+            ++gi;
+            if (gi - g0 < len + lenn) locate(gi);
+        };
+        auto begin = [&]() __attribute__((always_inline)) -> char* {  // wait for element g
+            if (gi - g > 1) wait_vm<OPS>();
+            else wait_vm<0>();
+            return Tw + (g & 1) * DT::BUF;
+        };
+        auto release = [&]() __attribute__((always_inline)) {  // element g has left its buffer
+            wait_lgkm0();
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
-        bf16x8 dsb[2];
-        pack16(ds, dsb);
-        mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    settle(q);
-    settle(go);
-    settle(lse);
-    if (nu > 0) issue(tile_id(0), 0);
-    if (nu > 1) issue(tile_id(1), 1);
-    if (nu > 2) Jq = tile_id(2);
-    for (int i = 0; i < nu; i += 2) {
-        if (i + 1 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(0, i + 2 < nu ? i + 2 : -1);
-        if (i + 1 >= nu) break;
-        if (i + 2 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(1, i + 3 < nu ? i + 3 : -1);
+            for (int k = 0; k < 2; ++k)
+                if (gi <= g + 2 && sq_g == gi) issue();
+        };
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+            if (gi < g0 + min(2, len)) {
+                if (sq_g != gi) locate(gi);
+                issue();
+            }
+        float* part = it.w >= 0 ? Part + ((size_t)bh * n_slots + it.w) * bf16_slot_floats<D>() : nullptr;
+        // the strip's operands: Q and dO rows and lse2, then O for the row sums g = dO . O
+        bf16x8 q[D / 16], go[D / 16];
+        float lse, gsum = 0.f;
+        {
+            const char* Ta = begin();
+            DT::get_rows(Ta, ra, q);
+            DT::get_rows(Ta + DT::TILE, ra, go);
+            lse = reinterpret_cast<const float*>(Ta + 2 * DT::TILE)[li];
+            release();
+            ++g;
+            const char* Tb = begin();
+            bf16x8 oo[D / 16];
+            DT::get_rows(Tb, ra, oo);
+            if (n > 0) {
+                release();
+                ++g;
+            } else {
+                wait_lgkm0();
+            }
+#pragma unroll
+            for (int t = 0; t < D / 16; ++t)
+#pragma unroll
+                for (int x = 0; x < 8; ++x) gsum = fmaf((float)go[t][x], (float)oo[t][x], gsum);
+            gsum = half_swap_sum(gsum);
+        }
+        Stats[((size_t)bh * (L / 32) + I) * 64 + l] = h ? -gsum : lse;  // every chunk of a strip writes the same values
+        const f32x16 gneg = splat16(-gsum);
+        f32x16 acc[D / 32];
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
+        for (int i = 0; i < n; ++i) {
+            const bool last = i + 1 == n;
+            const char* Tk = begin();
+            const char* Tv = Tk + DT::TILE;
+            bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
+            DT::get_rows(Tk, ra, kr);
+            DT::get_rows(Tv, ra, vr);
+            DT::get_tile_t(Tk, ta, kt);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+                float pj[16];
+                lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+            }
+            if (!last) release();  // the tile's operands are in registers: its buffer can take the element after next
+            else wait_lgkm0();     // (the item's last tile keeps it for the result)
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 s = mma_feat_bf16<D>(kr, q, init);
+            const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse)) * dp[r];
+            bf16x8 dsb[2];
+            pack16(ds, dsb);
+            mma_tile_bf16<D>(kt, dsb, acc);  // dQ^T: register = feature, lane = query
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) ++g;
+        }
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
+        if (part) store_part<D>(acc, part, l);
+        else stage_store_bf16<D>(acc, Tw + (g & 1) * DT::BUF, rdQ, vgr,
+                                 (int)(bf16_head_bytes<ST, D>(ly.grad, ly.H, bh, L) + (unsigned)(I * 32 * gld * 2)), gld, l);
+        release();
+        ++g;
     }
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
-    store_rows_bf16<D>(acc, rdQ, gld, I * 32, sa.coop, w, li, h, lds_o, part);
 }
 
 // -------------------------------------------------------------------------------------------------
 // Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
+// Stats: {lse2, -g} of every strip as the row pass left them (64 floats per strip).
+// Stream of an item: {K tile, V tile, key penalties of the column strip}, then per tile {Q tile, dO tile, statistics
+// of the query strip}.
 // -------------------------------------------------------------------------------------------------
-// Stats: {lse2, -g} of every strip as the row pass left them (64 floats per strip).  The Q and dO tiles and the
-// tile's 64 statistics go from global memory straight into one of two LDS buffers of the wavefront (DmaTile).
 template <int D, bool MASK, bool ST>
-SPION_BF16_KERNEL(2) void bf16_bwd_col_kernel(
+SPION_BF16_LANE(2) void bf16_bwd_col_kernel(
     const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
-    const __bf16* __restrict__ dO, const float* __restrict__ Stats,
-    const float* __restrict__ pen, __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcp,
-    const int* __restrict__ tcdesc, const int* __restrict__ wg_list, int n_wg, int L, int NB, float scale,
-    float* __restrict__ Part, int n_slots, int chunk, Layouts ly) {
+    const __bf16* __restrict__ dO, const float* __restrict__ Stats, const float* __restrict__ pen,
+    __bf16* __restrict__ dK, __bf16* __restrict__ dV, const int* __restrict__ tcdesc,
+    const int* __restrict__ plan_items, const int* __restrict__ lane_ptr, const int* __restrict__ lane_ent, int L, int NB,
+    float scale, float* __restrict__ Part, int n_slots, Layouts ly, unsigned in_bytes, unsigned out_bytes,
+    unsigned grad_bytes) {
     typedef DmaTile<D> DT;
-    __shared__ __attribute__((aligned(16))) char lds_t[BF16_WAVES][DT::WAVE];
-    float* lds_o = reinterpret_cast<float*>(&lds_t[0][0]);  // partial results of a shared strip, after the tiles
-    static_assert((BF16_WAVES - 1) * (D / 32) * 16 * 64 * 4 <= BF16_WAVES * DT::WAVE, "partial results fit");
-    const int item = xcd_remap(blockIdx.x, n_wg * NB);
-    const int bh = item / n_wg;
-    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const StripAssign sa = strip_of_wave(wg_list, item % n_wg, w);
-    if (sa.strip < 0) return;
-    const int J = sa.strip;
-    const int cnt_all = tcp[J + 1] - tcp[J], tb = sa.chunk_id * chunk;
-    const int e0 = tcp[J] + tb, cnt = sa.coop ? min(chunk, cnt_all - tb) : cnt_all;
-    const int nu = cnt > sa.rank ? (cnt - sa.rank + sa.step - 1) / sa.step : 0;
-    float* part = sa.slot >= 0 ? Part + ((size_t)bh * n_slots + sa.slot) * bf16_slot_floats<D>() : nullptr;
-    size_t ib, ob, gb, ibytes, obytes, gbytes;
-    int ild, old_, gld;
-    bf16_head<ST, D>(ly.in, ly.H, bh, L, ib, ild, ibytes);
-    bf16_head<ST, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
-    bf16_head<ST, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rK = make_rsrc(K + ib, ibytes), rV = make_rsrc(V + ib, ibytes);
-    const rsrc_t rdK = make_rsrc(dK + gb, gbytes), rdV = make_rsrc(dV + gb, gbytes);
-    const u32x4 wQ = rsrc_words(Q + ib, ibytes), wG = rsrc_words(dO + ob, obytes);
-    const u32x4 wS = rsrc_words(Stats + (size_t)bh * (L / 32) * 64, (size_t)(L / 32) * 256);
-    const int r_voff = li * ild * 2 + h * D;
-    const int q_voff = DT::voff(l, ild), q_xstep = DT::extra_step(ild);
-    const int o_voff = DT::voff(l, old_), o_xstep = DT::extra_step(old_);
-    const char* Tw = lds_t[w];
+    __shared__ __attribute__((aligned(16))) char Tw[DT::WAVE];
+    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int e0 = as_constant(lane_ptr)[blockIdx.x], e1 = as_constant(lane_ptr)[blockIdx.x + 1];
+    if (e0 >= e1) return;
+    const const_ints ents = as_constant(lane_ent), items = as_constant(plan_items);
+    const const_ints tiles = as_constant(tcdesc);  // four ints per tile of the transposed index, the first its block row
+    const int ild = ST ? ly.in.ld : D, old_ = ST ? ly.out.ld : D, gld = ST ? ly.grad.ld : D;
+    const u32x4 wQ = rsrc_words(Q, in_bytes), wK = rsrc_words(K, in_bytes), wV = rsrc_words(V, in_bytes);
+    const u32x4 wG = rsrc_words(dO, out_bytes);
+    const u32x4 wS = rsrc_words(Stats, (size_t)NB * L * 8);
+    const u32x4 wM = rsrc_words(MASK ? pen : Stats, (size_t)NB * L * 4);
+    const rsrc_t rdK = make_rsrc(dK, grad_bytes), rdV = make_rsrc(dV, grad_bytes);
+    const int t_bytes = 32 * ild * 2, o_bytes = 32 * old_ * 2;
+    const int vin = DT::voff(l, ild), xin = DT::extra_step(ild);
+    const int vout = DT::voff(l, old_), xout = DT::extra_step(old_), vgr = DT::voff(l, gld);
     const unsigned lds_w = lds_address(Tw);
     const typename DT::RowAddr ra = DT::row_addr(li, h);
     const typename DT::TrAddr ta = DT::tr_addr(l);
     const float c2 = scale * LOG2E;
-
-    bf16x8 k[D / 16], v[D / 16];
-    ldb_rows<D>(rK, r_voff, J * 32 * ild * 2, k);
-    ldb_rows<D>(rV, r_voff, J * 32 * ild * 2, v);
-    f32x16 sinit = splat16(0.f);
-    if constexpr (MASK) sinit = splat16(-pen[(size_t)bh * L + J * 32 + li] / scale);
-
-    f32x16 ak[D / 32], av[D / 32];
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) {
-        ak[c] = splat16(0.f);
-        av[c] = splat16(0.f);
-    }
-    const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
-    constexpr int OPS = 2 * DT::NI + 1;
-    auto tile_id = [&](int i) { return desc[sa.rank + min(i, nu - 1) * sa.step].x; };
-    int Iq = 0;  // query tile the next issue fetches, requested one tile ahead of that issue
-    auto issue = [&](int I, int par) {  // query tile I -> buffer par
-        const unsigned a = lds_w + par * DT::BUF;
-        DT::load(wQ, a, q_voff, I * 32 * ild * 2, q_xstep);
-        DT::load(wG, a + DT::TILE, o_voff, I * 32 * old_ * 2, o_xstep);
-        dma_b32(wS, a + 2 * DT::TILE, l * 4, I * 256);
-    };
+    constexpr int E = 1, OPS = 2 * DT::NI + 1;
     // d = 64 has no registers for the transposed tiles while the first chains' operands are live: they are read
-    // once the chains are issued, and the buffer is handed to the tile after next after that.
+    // once the chains are issued, and the buffer is handed on after that.
     constexpr bool DEEP = D == 32;
-    auto compute = [&](int par, int inext) {
-        const char* Tq = Tw + par * DT::BUF;
-        const char* Tg = Tq + DT::TILE;
-        const float* St = reinterpret_cast<const float*>(Tq + 2 * DT::TILE);  // lse2[32], -g[32] of the tile's queries
-        float lse[16], gn[16];
-        lds_get_rows(St, 0, h, lse);      // lse[r] = St[acc_row(r, h)]
-        lds_get_rows(St + 32, 0, h, gn);  // gn[r]  = St[32 + acc_row(r, h)]
-        bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
-        DT::get_rows(Tq, ra, qr);
-        DT::get_rows(Tg, ra, gr);
-        if constexpr (DEEP) {
-            DT::get_tile_t(Tq, ta, qt);
-            DT::get_tile_t(Tg, ta, gt);
+
+    LaneEntry en = lane_entry(ents, e0);
+    PlanItem itn = plan_item(items, en.y);
+    int g = 0, gi = 0;
+    int sk = 0, sa = 0, sb = 0, sc = 0, sq_g = -1;  // element sq_g: kind and the offsets of its three loads
+    for (int e = e0; e < e1; ++e) {
+        const int bh = en.x;
+        const PlanItem it = itn;
+        const bool has_next = e + 1 < e1;
+        if (has_next) {
+            en = lane_entry(ents, e + 1);
+            itn = plan_item(items, en.y);
+        }
+        const int bhn = en.x;
+        const int J = it.x, t0 = it.y, n = it.z;
+        const int Jn = itn.x, t0n = itn.y;
+        const int len = E + n, lenn = has_next ? E + itn.z : 0;
+        const int g0 = g;
+        const unsigned hb = bf16_head_bytes<ST, D>(ly.in, ly.H, bh, L), hbn = bf16_head_bytes<ST, D>(ly.in, ly.H, bhn, L);
+        const unsigned ho = bf16_head_bytes<ST, D>(ly.out, ly.H, bh, L), hon = bf16_head_bytes<ST, D>(ly.out, ly.H, bhn, L);
+        auto locate_in = [&](int k, int bhX, int JX, int t0X, unsigned hbX, unsigned hoX) __attribute__((always_inline)) {
+            if (k == 0) {
+                sk = EL_A;
+                sa = uniform((int)(hbX + (unsigned)(JX * t_bytes)));
+                sb = sa;
+                sc = uniform((bhX * L + JX * 32) * 4);
+            } else {
+                const int I = tiles[4 * (t0X + k - E)];
+                sk = EL_TILE;
+                sa = uniform((int)(hbX + (unsigned)(I * t_bytes)));
+                sb = uniform((int)(hoX + (unsigned)(I * o_bytes)));
+                sc = uniform((bhX * (L / 32) + I) * 256);
+            }
+        };
+        auto locate = [&, bh, bhn, J, Jn, t0, t0n, hb, hbn, ho, hon, len, g0](int gg) __attribute__((always_inline)) {
+            const int k = gg - g0;
+            if (k < len) locate_in(k, bh, J, t0, hb, ho);
+            else locate_in(k - len, bhn, Jn, t0n, hbn, hon);
+            sq_g = gg;
+        };
+        auto issue = [&]() __attribute__((always_inline)) {  // element gi -> buffer gi % 2, then look the following one up
+            const unsigned a = lds_w + (gi & 1) * DT::BUF;
+            if (sk == EL_TILE) {
+                DT::load(wQ, a, vin, sa, xin);
+                DT::load(wG, a + DT::TILE, vout, sb, xout);
+                dma_b32(wS, a + 2 * DT::TILE, l * 4, sc);
+            } else {
+                DT::load(wK, a, vin, sa, xin);
+                DT::load(wV, a + DT::TILE, vin, sb, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, sc);
+            }
+            ++gi;
+            if (gi - g0 < len + lenn) locate(gi);
+        };
+        auto begin = [&]() __attribute__((always_inline)) -> char* {  // wait for element g
+            if (gi - g > 1) wait_vm<OPS>();
+            else wait_vm<0>();
+            return Tw + (g & 1) * DT::BUF;
+        };
+        auto release = [&]() __attribute__((always_inline)) {  // element g has left its buffer
             wait_lgkm0();
-            if (inext >= 0) issue(Iq, par);
-            Iq = tile_id(inext + 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
-        f32x16 ginit;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
-        const f32x16 dp = mma_feat_bf16<D>(gr, v, ginit);  // dO_i . v_j - g_i
-        if constexpr (!DEEP) {
-            DT::get_tile_t(Tq, ta, qt);
-            DT::get_tile_t(Tg, ta, gt);
-        }
-        float p[16], ds[16];
+            for (int k = 0; k < 2; ++k)
+                if (gi <= g + 2 && sq_g == gi) issue();
+        };
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse[r]));
-            ds[r] = p[r] * dp[r];
+        for (int k = 0; k < 2; ++k)
+            if (gi < g0 + min(2, len)) {
+                if (sq_g != gi) locate(gi);
+                issue();
+            }
+        float* part = it.w >= 0 ? Part + ((size_t)bh * n_slots + it.w) * bf16_slot_floats<D>() : nullptr;
+        // the column strip's operands: K and V rows (and the key penalties)
+        bf16x8 k[D / 16], v[D / 16];
+        f32x16 sinit = splat16(0.f);
+        {
+            const char* Ta = begin();
+            DT::get_rows(Ta, ra, k);
+            DT::get_rows(Ta + DT::TILE, ra, v);
+            if constexpr (MASK) sinit = splat16(-reinterpret_cast<const float*>(Ta + 2 * DT::TILE)[li] / scale);
+            if (n > 0) {
+                release();
+                ++g;
+            } else {
+                wait_lgkm0();
+            }
         }
-        bf16x8 pb[2], dsb[2];
-        pack16(p, pb);
-        pack16(ds, dsb);
-        if constexpr (!DEEP) {
-            wait_lgkm0();
-            if (inext >= 0) issue(Iq, par);
-            Iq = tile_id(inext + 1);
+        f32x16 ak[D / 32], av[D / 32];
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) {
+            ak[c] = splat16(0.f);
+            av[c] = splat16(0.f);
         }
-        mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
-        mma_tile_bf16<D>(gt, pb, av);   // dV^T
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    settle(k);
-    settle(v);
-    if constexpr (MASK) settle(sinit[0]);
-    if (nu > 0) issue(tile_id(0), 0);
-    if (nu > 1) issue(tile_id(1), 1);
-    if (nu > 2) Iq = tile_id(2);
-    for (int i = 0; i < nu; i += 2) {
-        if (i + 1 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(0, i + 2 < nu ? i + 2 : -1);
-        if (i + 1 >= nu) break;
-        if (i + 2 < nu) wait_vm<OPS>();
-        else wait_vm<0>();
-        compute(1, i + 3 < nu ? i + 3 : -1);
+        for (int i = 0; i < n; ++i) {
+            const bool last = i + 1 == n;
+            const char* Tq = begin();
+            const char* Tg = Tq + DT::TILE;
+            const float* St = reinterpret_cast<const float*>(Tq + 2 * DT::TILE);  // lse2[32], -g[32] of the tile's queries
+            float lse[16], gn[16];
+            lds_get_rows(St, 0, h, lse);      // lse[r] = St[acc_row(r, h)]
+            lds_get_rows(St + 32, 0, h, gn);  // gn[r]  = St[32 + acc_row(r, h)]
+            bf16x8 qr[D / 16], gr[D / 16], qt[D / 32][2], gt[D / 32][2];
+            DT::get_rows(Tq, ra, qr);
+            DT::get_rows(Tg, ra, gr);
+            if constexpr (DEEP) {
+                DT::get_tile_t(Tq, ta, qt);
+                DT::get_tile_t(Tg, ta, gt);
+                if (!last) release();
+                else wait_lgkm0();
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
+            f32x16 ginit;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ginit[r] = gn[r];
+            const f32x16 dp = mma_feat_bf16<D>(gr, v, ginit);  // dO_i . v_j - g_i
+            if constexpr (!DEEP) {
+                DT::get_tile_t(Tq, ta, qt);
+                DT::get_tile_t(Tg, ta, gt);
+            }
+            float p[16], ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                p[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse[r]));
+                ds[r] = p[r] * dp[r];
+            }
+            bf16x8 pb[2], dsb[2];
+            pack16(p, pb);
+            pack16(ds, dsb);
+            if constexpr (!DEEP) {
+                if (!last) release();
+                else wait_lgkm0();
+            }
+            mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
+            mma_tile_bf16<D>(gt, pb, av);   // dV^T
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) ++g;
+        }
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
+        if (part) {
+            store_part<D>(ak, part, l);
+            store_part<D>(av, part + 32 * D, l);
+        } else {
+            char* Tl = Tw + (g & 1) * DT::BUF;
+            const int so = (int)(bf16_head_bytes<ST, D>(ly.grad, ly.H, bh, L) + (unsigned)(J * 32 * gld * 2));
+            stage_store_bf16<D>(ak, Tl, rdK, vgr, so, gld, l);
+            stage_store_bf16<D>(av, Tl + DT::TILE, rdV, vgr, so, gld, l);
+        }
+        release();
+        ++g;
     }
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
-    store_rows_bf16<D>(ak, rdK, gld, J * 32, sa.coop, w, li, h, lds_o, part);
-    if (sa.coop) __syncthreads();
-    store_rows_bf16<D>(av, rdV, gld, J * 32, sa.coop, w, li, h, lds_o, part ? part + 32 * D : nullptr);
 }
 
 // -------------------------------------------------------------------------------------------------

@@ -21,6 +21,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
+#include <queue>
 #include <vector>
 
 namespace spion {
@@ -390,6 +391,14 @@ __global__ __launch_bounds__(64 * ELEM_WAVES) void elem_bwd_col_kernel(
 // =================================================================================================
 // host side
 // =================================================================================================
+// Device side of a schedule of the bf16 kernels (build_bf16_plan): the lists, the number of persistent wavefronts,
+// the workspace slots of the chunks of long strips and {strip, first slot, chunks, tiles} per long strip.
+struct Bf16Plan {
+    Bf16Sched sched{};
+    const int* d_longs = nullptr;
+    int lanes = 0, slots = 0, n_long = 0;
+};
+
 struct PatternIndex {
     const int* key_off = nullptr;
     const int* key_col = nullptr;
@@ -404,20 +413,13 @@ struct PatternIndex {
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
     // per strip in launch order, {strip, first tile, tiles, P offset}: row pass, forward, column pass
     int *d_rdesc = nullptr, *d_fdesc = nullptr, *d_cdesc = nullptr;
-    int* d_pair_list = nullptr;  // bf16 forward by strip pairs: chunks of long strips, then four pairs per work-group
-    int n_wg_pair = 0;
-    bool bf16_pairs = false;
+    // bf16 family: schedules of persistent wavefronts over block rows, pairs of block rows and block columns
+    Bf16Plan plan_row, plan_pair, plan_col;
     int *d_ccp = nullptr, *d_crow = nullptr, *d_cpos = nullptr;
     // element-sparse pattern whose well-filled 32x32 tiles run on the MFMA units (hybrid_kernels.h)
     bool hybrid = false;
     int hyb_tiles = 0, hyb_nr = 0;
     HybIndex hyb{};
-    // work-group lists of the bf16 kernels (four ints per work-group) over block rows / block columns, and what
-    // their long strips need: chunk length in tiles, workspace slots, {strip, first slot, chunks, tiles} per long strip
-    int *d_wg_row = nullptr, *d_wg_col = nullptr;
-    int n_wg_row = 0, n_wg_col = 0;
-    int chunk_row = 1, chunk_col = 1, slots_row = 0, slots_col = 0, n_long_row = 0, n_long_col = 0;
-    int *d_long_row = nullptr, *d_long_col = nullptr;
     void release() {
         if (d_blob) (void)hipFree(d_blob);
         *this = PatternIndex();
@@ -541,34 +543,106 @@ static int long_strip_threshold(int nstrips, int ntiles) {
     return std::max(4 * avg + 8, 32);
 }
 
-// Work-group list of the bf16 kernels: the chunks of long strips first, each walked by the four wavefronts of a
-// work-group together; the other strips in index order (neighbouring strips of a banded pattern share K/V tiles
-// in the caches), four to a work-group, one per wavefront.  A chunk has about the tiles of an ordinary
-// work-group, so no work-group outlasts the others by much.
-struct WgList {
-    std::vector<int> wg;     // four ints per work-group
-    std::vector<int> longs;  // {strip, first slot, chunks, tiles} per long strip
-    int chunk = 1, slots = 0;
+// Schedule of the bf16 kernels.  A launch is a fixed set of persistent one-wavefront work-groups ("lanes of work");
+// each walks a list of items built here, so that no lane outlasts the others by much and a lane's tile loads run
+// on from one item into the next:
+//   items    {strip, first tile (index into the tile list), tiles, kind} -- kind >= 0: a chunk of a long strip (a global
+//            row or column, cut so that no item is much longer than the average lane's share) that leaves its partial
+//            result in workspace slot `kind`; -1: a whole strip; -2: strips `strip` and `strip + 1`, which hold the
+//            same tiles, walked together (forward only);
+//   lane_ptr / lane_ent  CSR-like: lane s works on entries lane_ptr[s] .. lane_ptr[s+1]-1, each {head, item};
+//   longs    {strip, first slot, chunks, tiles} per long strip, for the merge kernels.
+// Lanes are dealt to the dies in turn (lane s runs on die s % 8, as work-groups are), and a die's lanes share the
+// heads of that die one head after the other (the K/V of a head then stay in the die's L2); within a head the items
+// go longest first to the lane with the least work so far.
+struct Bf16PlanHost {
+    std::vector<int> items, lane_ptr, lane_ent, longs;
+    int slots = 0, lanes = 0;
 };
-static WgList build_wg_list(const std::vector<int>& ptr, int nstrips, int ntiles) {
-    WgList out;
-    const int long_len = long_strip_threshold(nstrips, ntiles);
-    out.chunk = long_len;
-    std::vector<int> rest;
-    for (int i = 0; i < nstrips; ++i) {
+static Bf16PlanHost build_bf16_plan(const std::vector<int>& ptr, int nstrips, bool pairs, int NB, int lanes_wanted) {
+    Bf16PlanHost out;
+    long long ntiles = 0;
+    for (int i = 0; i < nstrips; ++i) ntiles += ptr[i + 1] - ptr[i];
+    const int groups = NB % 8 == 0 ? 8 : 1;  // dies
+    const int lanes = std::max(groups, lanes_wanted / groups * groups);
+    // no item much longer than a lane's share of the launch, nor shorter than a few tiles
+    const long long share = (ntiles * NB + lanes - 1) / lanes;
+    const int avg = nstrips ? (int)((ntiles + nstrips - 1) / nstrips) : 0;
+    const int long_len = (int)std::max<long long>(std::min<long long>(std::max(4 * avg + 8, 32), std::max<long long>(share / 2, 8)), 8);
+    struct It {
+        int strip, t0, n, kind;
+    };
+    std::vector<It> its;
+    const int step = pairs ? 2 : 1;
+    for (int i = 0; i < nstrips; i += step) {
         const int cnt = ptr[i + 1] - ptr[i];
         if (cnt <= long_len) {
-            rest.push_back(i);
+            its.push_back({i, ptr[i], cnt, pairs ? -2 : -1});
             continue;
         }
-        const int chunks = (cnt + out.chunk - 1) / out.chunk;
-        out.longs.insert(out.longs.end(), {i, out.slots, chunks, cnt});
-        for (int c = 0; c < chunks; ++c) out.wg.insert(out.wg.end(), {i, i, c, out.slots + c});
-        out.slots += chunks;
+        for (int k = 0; k < step; ++k) {  // long strips are cut one by one, also where strips are paired
+            const int I = i + k, chunks = (cnt + long_len - 1) / long_len;
+            out.longs.insert(out.longs.end(), {I, out.slots, chunks, cnt});
+            for (int c = 0; c < chunks; ++c) {
+                const int b = (int)((long long)cnt * c / chunks), e = (int)((long long)cnt * (c + 1) / chunks);
+                its.push_back({I, ptr[I] + b, e - b, out.slots + c});
+            }
+            out.slots += chunks;
+        }
     }
-    for (size_t i = 0; i < rest.size(); i += 4)
-        for (size_t w = 0; w < 4; ++w) out.wg.push_back(i + w < rest.size() ? rest[i + w] : -1);
+    std::vector<int> order(its.size());
+    for (size_t i = 0; i < its.size(); ++i) order[i] = (int)i;
+    const int unit = pairs ? 2 : 1;  // a pair does two strips' arithmetic per tile
+    auto weight = [&](const It& x) { return (x.kind == -2 ? unit : 1) * x.n + 2; };
+    std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return weight(its[x]) > weight(its[y]); });
+    for (const It& x : its) out.items.insert(out.items.end(), {x.strip, x.t0, x.n, x.kind});
+    if (out.items.empty()) out.items.assign(4, 0);
+    // deal: per die, head after head, every item to the lane of that die with the least work so far
+    const int per_group = lanes / groups, heads_per_group = NB / groups;
+    std::vector<std::vector<int>> lane_list(lanes);
+    for (int g = 0; g < groups; ++g) {
+        typedef std::pair<long long, int> Load;  // (work so far, lane of this die)
+        std::priority_queue<Load, std::vector<Load>, std::greater<Load>> heap;
+        for (int j = 0; j < per_group; ++j) heap.push({0, j});
+        for (int hh = 0; hh < heads_per_group; ++hh) {
+            const int bh = g * heads_per_group + hh;
+            for (int o : order) {
+                Load top = heap.top();
+                heap.pop();
+                const int lane = top.second * groups + g;
+                lane_list[lane].push_back(bh);
+                lane_list[lane].push_back(o);
+                top.first += weight(its[o]);
+                heap.push(top);
+            }
+        }
+    }
+    out.lane_ptr.assign(1, 0);
+    for (int sidx = 0; sidx < lanes; ++sidx) {
+        out.lane_ent.insert(out.lane_ent.end(), lane_list[sidx].begin(), lane_list[sidx].end());
+        out.lane_ptr.push_back((int)out.lane_ent.size() / 2);
+    }
+    if (out.lane_ent.empty()) out.lane_ent.assign(2, 0);
+    out.lanes = lanes;
     return out;
+}
+
+// Wavefronts a launch of the bf16 kernels keeps resident: two per SIMD on every compute unit of the device.
+// SPION_BF16_LANES (tests; read whenever a pattern is indexed) overrides the number: with a handful of lanes every
+// lane walks many items of several heads even on a small problem.
+static int bf16_lanes() {
+    static int device_lanes = 0;
+    if (!device_lanes) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+            cus <= 0) {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        device_lanes = cus * 8;
+    }
+    if (const char* env = getenv("SPION_BF16_LANES")) return std::min(std::max(1, atoi(env)), 1 << 16);
+    return device_lanes;
 }
 
 // Copy the index to the host once (unless the caller hands over host copies), validate it, detect the tile
@@ -657,8 +731,9 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         while (blob.size() % 4) blob.push_back(0);
         return o;
     };
-    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0, o_wgr = 0, o_wgc = 0;
-    size_t o_lgr = 0, o_lgc = 0, o_rdesc = 0, o_fdesc = 0, o_cdesc = 0, o_plist = 0;
+    size_t o_trp = 0, o_tcol = 0, o_tcp = 0, o_tcdesc = 0, o_ccp = 0, o_crow = 0, o_cpos = 0;
+    size_t o_rdesc = 0, o_fdesc = 0, o_cdesc = 0;
+    size_t o_plan[3][4] = {};
     size_t hyb_off[14] = {};
     if (tiled) {
         const int nt = (int)tcol.size();
@@ -677,7 +752,19 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             }
         }
         for (int J = 0; J < nbr; ++J) mc = std::max(mc, tcp[J + 1] - tcp[J]);
-        const WgList wgr = build_wg_list(trp, nbr, nt), wgc = build_wg_list(tcp, nbr, nt);
+        Bf16PlanHost plan_r, plan_p, plan_c;
+        if (a->is_bf16) {
+            // strips 2k and 2k+1 with the same block columns (masks of 64 x 64 blocks and larger): the forward
+            // gives one wavefront both strips of a pair
+            bool pairs = nbr % 2 == 0 && nt > 0;
+            for (int k = 0; pairs && k < nbr / 2; ++k) {
+                const int a0 = trp[2 * k], a1 = trp[2 * k + 1], n0 = a1 - a0, n1 = trp[2 * k + 2] - a1;
+                pairs = n0 == n1 && std::equal(tcol.begin() + a0, tcol.begin() + a1, tcol.begin() + a1);
+            }
+            plan_r = build_bf16_plan(trp, nbr, false, a->NB, bf16_lanes());
+            plan_c = build_bf16_plan(tcp, nbr, false, a->NB, bf16_lanes());
+            if (pairs) plan_p = build_bf16_plan(trp, nbr, true, a->NB, bf16_lanes());
+        }
         // Behind each pointer array: the order the fp32 kernels walk the strips of a head in.  Strips are
         // bucketed by length class -- rows: more than 2 MAXT tiles of the forward's register budget, more than
         // MAXT, the rest; columns: long ones, the rest -- so that long strips start first,
@@ -732,43 +819,19 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         o_rdesc = append(rdesc);
         o_fdesc = append(fdesc);
         o_cdesc = append(cdesc);
-        {
-            // strips 2k and 2k+1 with the same block columns (masks of 64 x 64 blocks and larger): lists for the bf16
-            // forward that gives one wavefront both strips of a pair -- four short pairs per work-group, and the
-            // work-groups of the chunked long strips on their own
-            bool pairs = nbr % 2 == 0 && nt > 0;
-            for (int k = 0; pairs && k < nbr / 2; ++k) {
-                const int a0 = trp[2 * k], a1 = trp[2 * k + 1], n0 = a1 - a0, n1 = trp[2 * k + 2] - a1;
-                pairs = n0 == n1 && std::equal(tcol.begin() + a0, tcol.begin() + a1, tcol.begin() + a1);
-            }
-            if (pairs) {
-                std::vector<int> plist, longwg;
-                for (int k = 0; k < nbr / 2; ++k)
-                    if (trp[2 * k + 1] - trp[2 * k] <= wgr.chunk) plist.push_back(k);
-                while (plist.size() % 4) plist.push_back(-1);
-                for (size_t g = 0; g + 3 < wgr.wg.size(); g += 4)
-                    if (wgr.wg[g] == wgr.wg[g + 1] && wgr.wg[g] >= 0)
-                        longwg.insert(longwg.end(), wgr.wg.begin() + g, wgr.wg.begin() + g + 4);
-                pi.bf16_pairs = !plist.empty();
-                // one list: the chunks of the long strips first, then the pairs, four to a work-group
-                longwg.insert(longwg.end(), plist.begin(), plist.end());
-                pi.n_wg_pair = (int)longwg.size() / 4;
-                if (longwg.empty()) longwg.push_back(-1);
-                o_plist = append(longwg);
-            }
-        }
-        pi.n_wg_row = (int)wgr.wg.size() / 4;
-        pi.n_wg_col = (int)wgc.wg.size() / 4;
-        pi.chunk_row = wgr.chunk;
-        pi.chunk_col = wgc.chunk;
-        pi.slots_row = wgr.slots;
-        pi.slots_col = wgc.slots;
-        pi.n_long_row = (int)wgr.longs.size() / 4;
-        pi.n_long_col = (int)wgc.longs.size() / 4;
-        o_wgr = append(wgr.wg);
-        o_wgc = append(wgc.wg);
-        o_lgr = append(wgr.longs);
-        o_lgc = append(wgc.longs);
+        auto file_plan = [&](const Bf16PlanHost& ph, Bf16Plan& dst, size_t (&o)[4]) {
+            dst.lanes = ph.lanes;
+            dst.slots = ph.slots;
+            dst.n_long = (int)ph.longs.size() / 4;
+            if (!ph.lanes) return;
+            o[0] = append(ph.items);
+            o[1] = append(ph.lane_ptr);
+            o[2] = append(ph.lane_ent);
+            o[3] = append(ph.longs);
+        };
+        file_plan(plan_r, pi.plan_row, o_plan[0]);
+        file_plan(plan_p, pi.plan_pair, o_plan[1]);
+        file_plan(plan_c, pi.plan_col, o_plan[2]);
         if (tcol.empty()) tcol.push_back(0);
         o_trp = append(trp);
         o_tcol = append(tcol);
@@ -905,13 +968,14 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         pi.d_tcp = pi.d_blob + o_tcp;
         pi.d_tcdesc = pi.d_blob + o_tcdesc;
         pi.d_rdesc = pi.d_blob + o_rdesc;
-        pi.d_pair_list = pi.d_blob + o_plist;
         pi.d_fdesc = pi.d_blob + o_fdesc;
         pi.d_cdesc = pi.d_blob + o_cdesc;
-        pi.d_wg_row = pi.d_blob + o_wgr;
-        pi.d_wg_col = pi.d_blob + o_wgc;
-        pi.d_long_row = pi.d_blob + o_lgr;
-        pi.d_long_col = pi.d_blob + o_lgc;
+        Bf16Plan* plans[3] = {&pi.plan_row, &pi.plan_pair, &pi.plan_col};
+        for (int k = 0; k < 3; ++k)
+            if (plans[k]->lanes) {
+                plans[k]->sched = Bf16Sched{pi.d_blob + o_plan[k][0], pi.d_blob + o_plan[k][1], pi.d_blob + o_plan[k][2]};
+                plans[k]->d_longs = pi.d_blob + o_plan[k][3];
+            }
     } else {
         pi.d_ccp = pi.d_blob + o_ccp;
         pi.d_crow = pi.d_blob + o_crow;
@@ -1697,31 +1761,50 @@ static bool ensure_part_ws(SparseAttn* a, int slots) {
     return ensure_ws_grow(a, &a->ws_part, &a->ws_part_floats, need, "bf16 attention");
 }
 
+// Bytes a tensor of [B][H][L][d] bf16 heads spans from its base pointer (the tile loads address whole tensors with
+// 32-bit offsets); 0 if that is 4 GiB or more.
+static unsigned bf16_extent(const SparseAttn* a, bool strided, const HeadLayout& y, int heads) {
+    unsigned long long e;
+    if (strided) {
+        const int B = a->NB / heads;
+        e = ((unsigned long long)(B - 1) * y.bstride + (unsigned long long)(heads - 1) * y.hstride +
+             (unsigned long long)(a->L - 1) * y.ld + a->d) * 2ull;
+    } else {
+        e = (unsigned long long)a->NB * a->L * a->d * 2ull;
+    }
+    return e >= 0xfffffff0ull ? 0u : (unsigned)e;
+}
+
 template <bool ST>
 static void bf16_forward_impl(SparseAttn* a, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
                               float* Lse, const Layouts& ly) {
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
-    if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
-    const dim3 grid(pi.n_wg_row * a->NB), block(64 * BF16_WAVES), grid_m(pi.n_long_row * a->NB * (32 * a->d / 256));
+    const unsigned in_bytes = bf16_extent(a, ST, ly.in, ly.H), out_bytes = bf16_extent(a, ST, ly.out, ly.H);
+    if (!in_bytes || !out_bytes) {
+        set_error("bf16 attn_forward: the tensors span 4 GiB or more");
+        return;
+    }
+    static const bool no_pairs = getenv("SPION_BF16_NO_PAIRS") != nullptr;
+    const bool by_pairs = !ST && pi.plan_pair.lanes > 0 && !no_pairs;
+    const Bf16Plan& plan = by_pairs ? pi.plan_pair : pi.plan_row;
+    if (!ensure_part_ws(a, std::max(std::max(pi.plan_row.slots, pi.plan_col.slots), pi.plan_pair.slots))) return;
+    const dim3 grid(plan.lanes), block(64), grid_m(plan.n_long * a->NB * (32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
     __bf16* o = static_cast<__bf16*>(Out);
-    static const bool no_pairs = getenv("SPION_BF16_NO_PAIRS") != nullptr;
-    // (with the key mask at d = 64 the pair kernel would spill 56 registers: one strip per wavefront there)
-    const bool by_pairs = !ST && pi.bf16_pairs && !no_pairs && !(a->d == 64 && Mask);
 #define SPION_LAUNCH(DD, MM)                                                                                         \
     do {                                                                                                             \
         if (by_pairs)                                                                                                \
-            hipLaunchKernelGGL((bf16_fwd_pair_kernel<DD, MM>), dim3(pi.n_wg_pair * a->NB), block, 0, a->hdr.stream,  \
-                               q, k, v, Mask, o, Lse, pi.d_trp, pi.d_tcol, pi.d_pair_list, pi.n_wg_pair, a->L,       \
-                               a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row);                             \
+            hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, false, true>), grid, block, 0, a->hdr.stream, q, k, v, Mask, \
+                               o, Lse, pi.d_tcol, plan.sched.items, plan.sched.lane_ptr, plan.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part, plan.slots, ly,     \
+                               in_bytes, out_bytes);                                                                            \
         else                                                                                                         \
-            hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST>), grid, block, 0, a->hdr.stream, q, k, v, Mask, o, Lse,  \
-                               pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L, a->NB, a->scale, a->ws_part,     \
-                               pi.slots_row, pi.chunk_row, ly);                                                      \
-        if (pi.n_long_row)                                                                                           \
+            hipLaunchKernelGGL((bf16_fwd_kernel<DD, MM, ST, false>), grid, block, 0, a->hdr.stream, q, k, v, Mask,   \
+                               o, Lse, pi.d_tcol, plan.sched.items, plan.sched.lane_ptr, plan.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part, plan.slots, ly,     \
+                               in_bytes, out_bytes);                                                                            \
+        if (plan.n_long)                                                                                             \
             hipLaunchKernelGGL((bf16_merge_fwd_kernel<DD, ST>), grid_m, dim3(256), 0, a->hdr.stream, a->ws_part,     \
-                               pi.d_long_row, pi.n_long_row, pi.slots_row, o, Lse, a->L, ly.out, ly.H);              \
+                               plan.d_longs, plan.n_long, plan.slots, o, Lse, a->L, ly.out, ly.H);                   \
     } while (0)
     if (a->d == 32) {
         if (Mask) SPION_LAUNCH(32, true);
@@ -1740,11 +1823,18 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
                                const Layouts& ly) {
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
+    const unsigned in_bytes = bf16_extent(a, ST, ly.in, ly.H), out_bytes = bf16_extent(a, ST, ly.out, ly.H);
+    const unsigned grad_bytes = bf16_extent(a, ST, ly.grad, ly.H);
+    if (!in_bytes || !out_bytes || !grad_bytes) {
+        set_error("bf16 attn_backward: the tensors span 4 GiB or more");
+        return;
+    }
     // {lse2, -g} of every strip, 64 floats per strip, from the row pass to the column pass
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L * 2)) return;
-    if (!ensure_part_ws(a, std::max(pi.slots_row, pi.slots_col))) return;
-    const dim3 grid_r(pi.n_wg_row * a->NB), grid_c(pi.n_wg_col * a->NB), block(64 * BF16_WAVES);
-    const dim3 grid_mr(pi.n_long_row * a->NB * (32 * a->d / 256)), grid_mc(pi.n_long_col * a->NB * (2 * 32 * a->d / 256));
+    if (!ensure_part_ws(a, std::max(std::max(pi.plan_row.slots, pi.plan_col.slots), pi.plan_pair.slots))) return;
+    const Bf16Plan &pr = pi.plan_row, &pc = pi.plan_col;
+    const dim3 grid_r(pr.lanes), grid_c(pc.lanes), block(64);
+    const dim3 grid_mr(pr.n_long * a->NB * (32 * a->d / 256)), grid_mc(pc.n_long * a->NB * (2 * 32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
     const __bf16 *o = static_cast<const __bf16*>(Out), *go = static_cast<const __bf16*>(dO);
     __bf16 *dq = static_cast<__bf16*>(dQ), *dk = static_cast<__bf16*>(dK), *dv = static_cast<__bf16*>(dV);
@@ -1752,20 +1842,19 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
     do {                                                                                                              \
         if (a->bwd_passes & 1) {                                                                                      \
             hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM, ST>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o,    \
-                               Lse, Mask, a->ws_rowsum, dq, pi.d_trp, pi.d_tcol, pi.d_wg_row, pi.n_wg_row, a->L,      \
-                               a->NB, a->scale, a->ws_part, pi.slots_row, pi.chunk_row, ly);                          \
-            if (pi.n_long_row)                                                                                        \
+                               Lse, Mask, a->ws_rowsum, dq, pi.d_tcol, pr.sched.items, pr.sched.lane_ptr, pr.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part,   \
+                               pr.slots, ly, in_bytes, out_bytes, grad_bytes);                                                               \
+            if (pr.n_long)                                                                                            \
                 hipLaunchKernelGGL((bf16_merge_sum_kernel<DD, ST>), grid_mr, dim3(256), 0, a->hdr.stream, a->ws_part, \
-                                   pi.d_long_row, pi.n_long_row, pi.slots_row, dq, (__bf16*)nullptr, a->L, ly.grad,   \
-                                   ly.H);                                                                             \
+                                   pr.d_longs, pr.n_long, pr.slots, dq, (__bf16*)nullptr, a->L, ly.grad, ly.H);       \
         }                                                                                                             \
         if (a->bwd_passes & 2) {                                                                                      \
             hipLaunchKernelGGL((bf16_bwd_col_kernel<DD, MM, ST>), grid_c, block, 0, a->hdr.stream, q, k, v, go,       \
-                               a->ws_rowsum, Mask, dk, dv, pi.d_tcp, pi.d_tcdesc, pi.d_wg_col, pi.n_wg_col, a->L,     \
-                               a->NB, a->scale, a->ws_part, pi.slots_col, pi.chunk_col, ly);                          \
-            if (pi.n_long_col)                                                                                        \
+                               a->ws_rowsum, Mask, dk, dv, pi.d_tcdesc, pc.sched.items, pc.sched.lane_ptr, pc.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part,  \
+                               pc.slots, ly, in_bytes, out_bytes, grad_bytes);                                                    \
+            if (pc.n_long)                                                                                            \
                 hipLaunchKernelGGL((bf16_merge_sum_kernel<DD, ST>), grid_mc, dim3(256), 0, a->hdr.stream, a->ws_part, \
-                                   pi.d_long_col, pi.n_long_col, pi.slots_col, dk, dv, a->L, ly.grad, ly.H);          \
+                                   pc.d_longs, pc.n_long, pc.slots, dk, dv, a->L, ly.grad, ly.H);                     \
         }                                                                                                             \
     } while (0)
     if (a->d == 32) {

@@ -53,10 +53,20 @@ __device__ __forceinline__ float ld1_nt(rsrc_t r, int voff, int soff) {
 __device__ __forceinline__ f32x4 ld4_nt(rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 2));
 }
-__device__ __forceinline__ void st4(rsrc_t r, int voff, int soff, f32x4 v) {
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), r, voff, soff, 0);
+// 128-bit buffer stores.  The hardware reads a store's data registers over several cycles after issue: a VALU write
+// to one of them in the next two issue slots can reach the store (seen on MI355X as single stale 4-byte words, now
+// and then).  The compiler keeps that distance for stores without a register soffset only, so here the two idle
+// slots are part of the instruction sequence.  NT: non-temporal.
+template <bool NT = false, typename X>
+__device__ __forceinline__ void store_b128(X x, rsrc_t r, int voff, int soff) {
+    static_assert(sizeof(X) == 16, "128-bit store");
+    const int so = __builtin_amdgcn_readfirstlane(soff);
+    if (NT)
+        asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen nt\n\ts_nop 1" ::"v"(x), "v"(voff), "s"(r), "s"(so) : "memory");
+    else
+        asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 1" ::"v"(x), "v"(voff), "s"(r), "s"(so) : "memory");
 }
+__device__ __forceinline__ void st4(rsrc_t r, int voff, int soff, f32x4 v) { store_b128(v, r, voff, soff); }
 
 // Operand over the head dimension from a row-major [.][D] head slice: D/2 consecutive floats per lane.
 // voff = ((lane%32)*D + (lane/32)*(D/2))*4 bytes, soff = byte offset of the tile's first row.
@@ -174,10 +184,8 @@ __device__ __forceinline__ void ldr_tile_lin(rsrc_t r, int voff, int soff, int l
 // Non-temporal: the P stream of the forward (written once, far larger than the caches) is kept from displacing
 // the K/V tiles in L2; measured -11 % on the forward kernel, -1.3 % on the whole step.
 __device__ __forceinline__ void str_tile_lin(rsrc_t r, int voff, int soff, int ld, const f32x4 (&raw)[4]) {
-    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, raw[i]), r, voff, soff + 32 * i * ld, 2);
+    for (int i = 0; i < 4; ++i) store_b128<true>(raw[i], r, voff, soff + 32 * i * ld);
 }
 // The same tile access for data a work-group reads back after writing it (partial sums kept in memory): loads are
 // served by the L2 (device-scope policy: the vector L1 is not consulted), stores use the default policy.

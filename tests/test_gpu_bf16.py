@@ -203,6 +203,30 @@ def test_bf16_long_strips_with_key_mask_and_large_logits(d):
     abi.close()
 
 
+@pytest.mark.parametrize("lanes", [3, 8])
+@pytest.mark.parametrize("d,bs,with_mask", [(32, 32, True), (64, 64, False), (64, 32, True)])
+def test_bf16_few_lanes_walk_many_items_each(monkeypatch, lanes, d, bs, with_mask):
+    """With a handful of persistent wavefronts each one walks many strips, chunks and pairs of several heads in a
+    row, so every kind of hand-over inside a wavefront's load stream (item to item, head to head, a staged result
+    followed by the next item's loads, chunk slots of a long strip) is checked against the oracle.  The lane count
+    is read when the pattern is indexed."""
+    L, NB = 1024, 5
+    mat = _mask(L // bs, 0.10, seed=23 + d + bs, global_block=True, empty_row=3)
+    mat[3, 3] = 0
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    monkeypatch.setenv("SPION_BF16_LANES", str(lanes))
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    monkeypatch.delenv("SPION_BF16_LANES")
+    Q, K, V, dO = _bf16_inputs(NB, L, d, seed=6, scale=1.5)
+    pen = None
+    if with_mask:
+        valid = torch.tensor([1024, 700, 1024, 333, 64])
+        pen = (1e6 * (1.0 - (torch.arange(L)[None, :] < valid[:, None]).float())).contiguous().cuda()
+    _run_and_check(abi, Q, K, V, dO, pen, tag=f"bf16 {lanes} lanes d={d} bs={bs}")
+    abi.close()
+
+
 def _bf16_head_views(B, H, L, d, layout, n, seed, fill=None):
     """n bf16 tensors seen as [B, H, L, d]: "proj": each a [B, L, H*d] projection; "fused": slices of one
     [B, L, n, H, d+8] buffer (padded rows)."""
