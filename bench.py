@@ -12,6 +12,10 @@ Prints ONE JSON line.  ``value`` is the effective TFLOP/s of the step (algorithm
 12*n*d*NB divided by the step time); ``roofline`` describes the slowest kernel (its share of the
 algorithmic FLOPs over its own HIP-event time); ``cpu_baseline`` is the dense PyTorch statement of
 the same semantics (the oracle) timed on the host cores over a bounded sample of the batch.
+``window_ms`` holds five further 20-step timings of the same step and their median.  The default run
+adds the other measured workloads as sub-objects of the same line (``config1``, ``config4``,
+``config5``, ``config2``, ``dense_phase``: step time, windows and roofline of each; ``--no-config1``
+and ``--no-extra`` leave them out); their CPU baselines are part of their own ``--workload`` runs.
 """
 from __future__ import annotations
 
@@ -74,6 +78,20 @@ def _timed_steps(step, steps, warmup):
         step()
     torch.cuda.synchronize()
     return 1e3 * (time.perf_counter() - t0) / steps
+
+
+def _windows(step, n_windows=5, per=20):
+    """Five back-to-back windows of 20 steps each, every one between two synchronisations: the ms per step of each
+    window and their median, so that one line shows how much a single timing of this step moves."""
+    out = []
+    for _ in range(n_windows):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(per):
+            step()
+        torch.cuda.synchronize()
+        out.append(1e3 * (time.perf_counter() - t0) / per)
+    return {"windows": [round(x, 4) for x in out], "median": round(float(np.median(out)), 4), "steps_per_window": per}
 
 
 def _profiled_traffic_bytes(kernel):
@@ -193,28 +211,34 @@ def bench_pattern_discovery(args, dev):
 
     spinup_ms = _spin_up(step, args.spinup_ms)
     ms_step = _timed_steps(step, args.steps, args.warmup)
+    window_ms = _windows(step)
     t_evt = _event_ms(step, max(10, args.steps))
     bytes_read = 4.0 * L * L * n_maps
-    t1 = time.perf_counter()
-    reps = 0
-    while time.perf_counter() - t1 < 10.0:
-        for i in range(n_maps):
-            op.generate_mask_conv_ff(maps_cpu[i].numpy(), bs, q, route="torch")
-        reps += 1
-    cpu_ms = 1e3 * (time.perf_counter() - t1) / reps
-    return {
+    cpu = None
+    if not args.no_cpu_baseline:
+        t1 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t1 < 10.0:
+            for i in range(n_maps):
+                op.generate_mask_conv_ff(maps_cpu[i].numpy(), bs, q, route="torch")
+            reps += 1
+        cpu_ms = 1e3 * (time.perf_counter() - t1) / reps
+        cpu = {"value": n_maps / (cpu_ms / 1e3), "unit": "maps/s", "cores": min(os.cpu_count() or 1, torch.get_num_threads()),
+               "kind": "port", "sample": f"the same {n_maps} maps, {reps} repetitions of the PyTorch-CPU route "
+                                         "(F.conv2d, avg_pool2d, quantile) plus the iterative walk"}
+    result = {
         "metric": "pattern discovery (conv filter + block pool + quantile + path walk), maps per second, 1 GPU",
         "value": n_maps / (ms_step / 1e3), "unit": "maps/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "ms_per_step": ms_step, "window_ms": window_ms, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
         "data": "synthetic (seeded softmax(QK^T) maps with a diagonal band boost)",
         "config": {"workload": f"config2: {n_maps} score maps {L}x{L}, 31x31 diagonal filter, {bs}x{bs} pooling, q={q}"},
         "roofline": {"bound": "hbm", "kernel": "conv_pool_cols_kernel + threshold_walk_kernel", "achieved": bytes_read / t_evt / 1e6,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": bytes_read / t_evt / 1e6 / PEAK_HBM_GBS, "traffic": None,
                      "event_ms": t_evt},
-        "cpu_baseline": {"value": n_maps / (cpu_ms / 1e3), "unit": "maps/s", "cores": min(os.cpu_count() or 1, torch.get_num_threads()),
-                         "kind": "port", "sample": f"the same {n_maps} maps, {reps} repetitions of the PyTorch-CPU route "
-                                                   "(F.conv2d, avg_pool2d, quantile) plus the iterative walk"},
     }
+    if cpu:
+        result["cpu_baseline"] = cpu
+    return result
 
 
 def bench_encoder_step(args, dev):
@@ -246,6 +270,7 @@ def bench_encoder_step(args, dev):
 
     spinup_ms = _spin_up(step, args.spinup_ms)
     ms_step = _timed_steps(step, args.steps, args.warmup)
+    window_ms = _windows(step)
 
     # attention share: the two layers' C-ABI kernels, from HIP events around a forward+backward of one layer's
     # attention core at the same shape
@@ -263,7 +288,7 @@ def bench_encoder_step(args, dev):
     return {
         "metric": "2-layer sparse encoder training step (fwd+bwd+AdamW), samples per second, 1 GPU",
         "value": B / (ms_step / 1e3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms_step, "window_ms": window_ms, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (uniform token ids, uniform labels, random-init weights)",
         "config": {"workload": f"config3: 2-layer encoder step, batch {B}, L={L}, d_model 64, FFN 128, H={H}, d_head {d}, "
                                f"block {cfg['block_size']}, discovered block densities {[round(x, 3) for x in density]}"},
@@ -307,6 +332,7 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
 
     spinup_ms = _spin_up(step, args.spinup_ms)
     ms_step = _timed_steps(step, args.steps, args.warmup)
+    window_ms = _windows(step)
 
     core = _lib.core()
     idx = module.csr_cache.get(mat, bs)
@@ -352,7 +378,7 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
     result = {
         "metric": "sparse-attn fwd+bwd effective TFLOP/s (12*n*d*NB algorithmic FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "ms_per_step": ms_step, "window_ms": window_ms, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": f"synthetic (seeded N(0,1)*{in_scale:g} tensors rounded to bf16, seeded block mask)",
         "config": {"workload": f"{shape}{'_bf16' if shape != 'config5' else ''}: bf16 sparse attention fwd+bwd, B={B} H={H} L={L} d={d}, block {bs}, "
                                f"nnz/head={nnz}, block density={round(float(mat_np.mean()), 4)}",
@@ -399,6 +425,7 @@ def bench_dense_phase(args, dev):
 
     spinup_ms = _spin_up(step, args.spinup_ms)
     ms_step = _timed_steps(step, args.steps, args.warmup)
+    window_ms = _windows(step)
     # the same step through the reference's ABI (feature-major operands: four transposes a step)
     module.reads_views = False
     for _ in range(max(3, args.warmup // 4)):
@@ -459,7 +486,7 @@ def bench_dense_phase(args, dev):
     result = {
         "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "ms_per_step": ms_step, "window_ms": window_ms, "spinup_ms": round(spinup_ms, 1), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic (seeded N(0,1) tensors)",
         "config": {"workload": f"dense_phase: softmax attention fwd+bwd with the full probability map, B={B} H={H} L={L} d={d}"},
         "algorithmic": {"gflop": alg_flops / 1e9, "map_gbytes": 4.0 * NB * L * L / 1e9},
@@ -497,6 +524,8 @@ def main():
     ap.add_argument("--workload", default="north_star")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-config1", action="store_true", help="north_star only: leave out the L = 1024 sub-object")
+    ap.add_argument("--no-extra", action="store_true",
+                    help="north_star only: leave out the config4 / config5 / config2 / dense_phase sub-objects")
     ap.add_argument("--spinup-ms", type=float, default=300.0,
                     help="untimed repetitions of the step for this long before the warm-up (clock ramp)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -538,12 +567,26 @@ def main():
         return
 
     result = bench_sparse_layer(args, dev, args.workload, full=True)
-    if args.workload == "north_star" and not args.no_config1:
-        # the metric is quoted at L = 1024 and L = 4096: the L = 1024 point (configuration 1) rides in the same line
-        c1 = bench_sparse_layer(args, dev, "config1", full=False)
-        result["config1"] = {k_: c1[k_] for k_ in ("value", "unit", "ms_per_step", "spinup_ms", "config", "hip_graph",
-                                                    "rowmajor_abi_ms", "kernels_effective_tflops", "roofline",
-                                                    "algorithmic") if k_ in c1}
+    if args.workload == "north_star":
+        # the other measured workloads ride in the same line, each as a sub-object with its own step time, windows and
+        # roofline (CPU baselines only in their own --workload runs, so that the default run stays within minutes)
+        keep = ("metric", "value", "unit", "ms_per_step", "window_ms", "spinup_ms", "dtype", "config", "hip_graph",
+                "rowmajor_abi_ms", "abi_ms", "kernels_effective_tflops", "roofline", "algorithmic")
+        sub = argparse.Namespace(**vars(args))
+        sub.no_cpu_baseline = True
+        extra = []
+        if not args.no_config1:
+            # the metric is quoted at L = 1024 and L = 4096: the L = 1024 point is configuration 1
+            extra.append(("config1", lambda: bench_sparse_layer(sub, dev, "config1", full=False)))
+        if not args.no_extra:
+            extra += [("config4", lambda: bench_sparse_layer(sub, dev, "config4", full=False)),
+                      ("config5", lambda: bench_bf16_scale_up(sub, dev)),
+                      ("config2", lambda: bench_pattern_discovery(sub, dev)),
+                      ("dense_phase", lambda: bench_dense_phase(sub, dev))]
+        for name, run in extra:
+            r = run()
+            result[name] = {k_: r[k_] for k_ in keep if k_ in r}
+            torch.cuda.empty_cache()
     print(json.dumps(result))
 
 
@@ -587,6 +630,7 @@ def bench_sparse_layer(args, dev, workload, full=True):
 
     spinup_ms = _spin_up(step, args.spinup_ms)
     ms_step = _timed_steps(step, args.steps, args.warmup)
+    window_ms = _windows(step)
     path = _lib.core().spion_last_path(handle)
 
     # ---- the same step recorded once as a HIP graph and replayed (what a launch-bound caller would do) ----------
@@ -740,6 +784,7 @@ def bench_sparse_layer(args, dev, workload, full=True):
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_step,
+        "window_ms": window_ms,
         "spinup_ms": round(spinup_ms, 1),
         "higher_is_better": True,
         "scaling": "weak",

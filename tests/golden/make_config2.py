@@ -10,7 +10,11 @@ between the two routes' pooled maps -- so any correct summation order yields the
 A walk makes about ten thousand comparisons per map, so margins above 1e-3 are out of reach: over seeds 0..2999
 the best is 6.3e-4 (seed 2608), the median 2e-5.  The float32 route differs from the float64 one by about 2e-6.
 
+The three runners-up of the scan (the next largest margins) get the same treatment: their masks go to
+config2_more_masks.npy ([3, 2, 32, 32]) and their seeds, margins and route errors to "more" in config2.json.
+
     python tests/golden/make_config2.py [first_seed last_seed]      (default 0 3000: about a quarter of an hour on 8 cores)
+    python tests/golden/make_config2.py more                        (only the runners-up of the scan already on file)
 """
 import json
 import os
@@ -34,12 +38,8 @@ def margins_of(seed):
     return seed, [op.decision_margin(op.pooled_map(maps[i], BS, 31, "fp64"), Q) for i in range(2)]
 
 
-def main():
-    lo, hi = (int(sys.argv[1]), int(sys.argv[2])) if len(sys.argv) == 3 else (0, 3000)
-    with Pool(min(8, os.cpu_count() or 1)) as pool:
-        scan = pool.map(margins_of, range(lo, hi), chunksize=8)
-    scan.sort(key=lambda r: -min(r[1]))
-    seed, margins = scan[0]
+def masks_of(seed, margins):
+    """Masks of one seed's two maps, after checking that both routes agree and the margin dwarfs their difference."""
     maps = workloads.score_maps_config2(2, L, 32, seed=seed).numpy()
     masks, errs = [], []
     for i in range(2):
@@ -51,6 +51,34 @@ def main():
         masks.append(m64)
     if min(margins) <= MIN_FACTOR * max(errs):
         raise SystemExit(f"seed {seed}: margin {min(margins):.3e} is not {MIN_FACTOR:g}x the route error {max(errs):.3e}")
+    return masks, errs
+
+
+def write_more():
+    path = os.path.join(HERE, "config2.json")
+    meta = json.load(open(path))
+    more, stack = [], []
+    for r in meta["runners_up"][:3]:
+        masks, errs = masks_of(r["seed"], r["decision_margin"])
+        stack.append(np.stack(masks))
+        more.append(dict(seed=r["seed"], decision_margin=r["decision_margin"], fp32_route_rel_error=errs,
+                         blocks_set=[int(m.sum()) for m in masks]))
+    np.save(os.path.join(HERE, "config2_more_masks.npy"), np.stack(stack).astype(np.int8))
+    meta["more"] = more
+    json.dump(meta, open(path, "w"), indent=1)
+    print(json.dumps(more, indent=1))
+
+
+def main():
+    if sys.argv[1:] == ["more"]:
+        write_more()
+        return
+    lo, hi = (int(sys.argv[1]), int(sys.argv[2])) if len(sys.argv) == 3 else (0, 3000)
+    with Pool(min(8, os.cpu_count() or 1)) as pool:
+        scan = pool.map(margins_of, range(lo, hi), chunksize=8)
+    scan.sort(key=lambda r: -min(r[1]))
+    seed, margins = scan[0]
+    masks, errs = masks_of(seed, margins)
     np.save(os.path.join(HERE, "config2_masks.npy"), np.stack(masks).astype(np.int8))
     all_min = sorted(min(r[1]) for r in scan)
     meta = dict(seed=seed, quantile=Q, block_size=BS, seq_len=L, decision_margin=margins,
@@ -60,6 +88,7 @@ def main():
                 blocks_set=[int(m.sum()) for m in masks])
     json.dump(meta, open(os.path.join(HERE, "config2.json"), "w"), indent=1)
     print(json.dumps(meta, indent=1))
+    write_more()
 
 
 if __name__ == "__main__":

@@ -21,7 +21,19 @@ REL_TOL_BF16 = 1e-2
 LOG2E = 1.4426950408889634
 
 
-def assert_close_bf16(got, ref, what=""):
+ROW_TOL_BF16 = 2.5e-2
+
+
+def assert_close_bf16(got, ref, what="", extra=None):
+    """Relative L2 error of the tensor within 1e-2, and every element within
+        1e-2 |ref|  +  2.5e-2 rms(ref over the element's own row of d values)  +  1e-2 rms(ref over the tensor).
+    Measured against the oracle on the cases of this file: the tensor's L2 error is 0.22 - 0.26 % (bf16 rounds the
+    result to 2^-9 of the element and P and dS to as much ahead of the second product of each chain), a row's L2
+    error at most 1.2 % of the row, and the largest element error beyond 1e-2 |ref| is 2.1 % of its row's RMS.  Rows
+    differ in scale by more than ten (a global key column collects a term from every query), which is why the
+    tensor's RMS alone does not bound an element's noise (seen: 4 % of it) and its maximum is no bound at all.
+    The last term covers rows that are all but zero.  ``extra`` (same shape) is added to the bound: dQ and dK carry
+    the term that the rounding of O brings in, see ``_oracle``."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
@@ -29,7 +41,10 @@ def assert_close_bf16(got, ref, what=""):
     err = np.abs(got - ref)
     rel_l2 = float(np.sqrt((err * err).sum() / max((ref * ref).sum(), 1e-300)))
     assert rel_l2 <= REL_TOL_BF16, f"{what}: relative L2 error {rel_l2:.3e}"
-    tol = REL_TOL_BF16 * (np.abs(ref) + np.abs(ref).max())
+    row_rms = np.sqrt(np.mean(ref * ref, axis=-1, keepdims=True))
+    tol = REL_TOL_BF16 * np.abs(ref) + ROW_TOL_BF16 * row_rms + REL_TOL_BF16 * np.sqrt(np.mean(ref * ref))
+    if extra is not None:
+        tol = tol + extra
     bad = err > tol
     if bad.any():
         idx = np.unravel_index(np.argmax(err - tol), err.shape)
@@ -107,7 +122,16 @@ def _oracle(Q, K, V, dO, sum_mat, offsets, columns, pen=None):
         np.add.at(z, rows, np.exp(val - big[rows]))
         z += (L - np.asarray(sum_mat)) * np.exp(-big)
         lse[b] = (big + np.log(z)) * LOG2E
-    return dict(O=O, dQ=dQ, dK=dK, dV=dV, lse=lse)
+    # The backward takes g_i = sum_t dO_it O_it from the stored output, which bf16 has rounded by up to 2^-8 of
+    # each element: |delta g_i| <= 2^-8 A_i with A_i = sum_t |dO_it O_it|.  Every dS_ij = P_ij (dP_ij - g_i) of the
+    # row moves by -P_ij delta g_i together, so to first order
+    #     |delta dQ_if| <= scale 2^-8 A_i |sum_j P_ij K_jf|,    |delta dK_jf| <= scale 2^-8 sum_i P_ij A_i |Q_if|.
+    # On rows whose softmax is saturated (dP_ij close to g_i) these terms exceed dQ and dK themselves.
+    scale = float(np.float32(1) / np.sqrt(np.float32(d)))
+    A = np.abs(do * O).sum(-1) * 2.0 ** -8
+    extra_dq = scale * A[:, :, None] * np.abs(osa.csr_spmm(P, k, offsets, columns))
+    extra_dk = scale * osa.csr_spmm_t(P * A[:, rows], np.abs(q), offsets, columns)
+    return dict(O=O, dQ=dQ, dK=dK, dV=dV, lse=lse, extra=dict(dQ=extra_dq, dK=extra_dk))
 
 
 def _run_and_check(abi, Q, K, V, dO, pen=None, tag=""):
@@ -120,7 +144,7 @@ def _run_and_check(abi, Q, K, V, dO, pen=None, tag=""):
     assert np.isfinite(got_lse).all(), f"{tag}: lse not finite"
     assert np.max(np.abs(got_lse - ref["lse"])) < 1e-3, f"{tag}: lse off by {np.max(np.abs(got_lse - ref['lse']))}"
     for name, t in (("O", O), ("dQ", dQ), ("dK", dK), ("dV", dV)):
-        assert_close_bf16(t.float().cpu().numpy(), ref[name], f"{tag} {name}")
+        assert_close_bf16(t.float().cpu().numpy(), ref[name], f"{tag} {name}", extra=ref["extra"].get(name))
 
 
 def _mask(nb, p, seed, global_block=False, empty_row=None, empty_col=None):
@@ -297,7 +321,7 @@ def test_bf16_strided_entry_points(d, layout, glob, with_mask, bs):
         assert (gbufs[0][..., d:] == -7.0).all(), "padding between the heads' rows was written"
     ref = _oracle(Qc, Kc, Vc, dOc, sm, off, col, pen)
     for name, t in (("O", out), ("dQ", dq), ("dK", dk), ("dV", dv)):
-        assert_close_bf16(flat(t).float().cpu().numpy(), ref[name], f"bf16 strided {name}")
+        assert_close_bf16(flat(t).float().cpu().numpy(), ref[name], f"bf16 strided {name}", extra=ref["extra"].get(name))
     # a layout the kernels cannot take is refused
     bad = _lib.HeadLayout(lin.batch_stride, lin.head_stride, lin.row_stride + 4)
     abi.lib.spion_block_bf16_attn_forward_strided(abi.handle, q.data_ptr(), k.data_ptr(), v.data_ptr(), pen_ptr,
@@ -403,7 +427,54 @@ def test_bf16_scale_up_shape_agrees_with_fp32_path():
         assert torch.isfinite(a).all(), name
         rel_l2 = ((a - b).pow(2).sum() / b.pow(2).sum()).sqrt().item()
         assert rel_l2 <= REL_TOL_BF16, f"{name}: relative L2 error {rel_l2:.3e}"
-        excess = ((a - b).abs() - REL_TOL_BF16 * (b.abs() + b.abs().max())).max().item()
+        tol = REL_TOL_BF16 * b.abs() + ROW_TOL_BF16 * b.pow(2).mean(-1, keepdim=True).sqrt() + REL_TOL_BF16 * b.pow(2).mean().sqrt()
+        excess = ((a - b).abs() - tol).max().item()
         assert excess <= 0, f"{name}: exceeds the element tolerance by {excess}"
     abi.close()
     ref.close()
+
+
+def test_bf16_scale_up_shape_matches_oracle_on_bounded_rows():
+    """Config 5 at full size with the inputs of the benchmark (Q, K, V ~ N(0,1)/8, dO ~ N(0,1), rounded to bf16): the
+    kernels run on all of it; the oracle, which cannot, restates a bounded part exactly.  It is given a pattern that
+    keeps, for three heads, the complete rows of a few query strips -- the global block row (cut into chunks and
+    merged), the first band strip, one from the middle, the last -- and of every strip that attends to two chosen key
+    blocks.  O, the row statistic and dQ of those rows depend on nothing else, and neither do dK and dV of the two
+    key blocks, whose contributing rows are all there.  (dK / dV of the global key block need every row; its chunked
+    column strips are covered by the comparison with the fp32 kernels above and, against the oracle, at L = 2048.)"""
+    B, H, L, d, bs = 4, 8, 16384, 64, 64
+    NB, nb = B * H, L // bs
+    mat = workloads.config5_mask()
+    from spion_amd.csr import block_mask_to_csr_host
+    sm, off, col = block_mask_to_csr_host(mat, bs)
+    g = torch.Generator().manual_seed(0)
+    Q, K, V, dO = ((torch.randn(NB, L, d, generator=g) * s).to(torch.bfloat16).cuda() for s in (0.125, 0.125, 0.125, 1.0))
+    abi = BF16ABI(d, L, NB, bs)
+    abi.set_pattern(sm, off, col)
+    O, lse = abi.forward(Q, K, V)
+    dQ, dK, dV = abi.backward(Q, K, V, O, lse, dO)
+    torch.cuda.synchronize()
+
+    heads = [0, 13, 31]
+    key_blocks = [nb // 3, nb - 2]
+    query_blocks = sorted({0, 1, nb // 2, nb - 1} | {int(i) for c in key_blocks for i in np.nonzero(mat[:, c])[0]})
+    assert len(query_blocks) < 40, "the bounded part stays small"
+    rows = np.concatenate([np.arange(i * bs, (i + 1) * bs) for i in query_blocks])
+    sm_r = np.zeros_like(sm)
+    sm_r[rows] = sm[rows]
+    off_r = np.zeros(L + 1, dtype=off.dtype)
+    np.cumsum(sm_r, out=off_r[1:])
+    col_r = np.concatenate([col[off[r]:off[r + 1]] for r in rows]).astype(col.dtype)
+    assert int(off_r[-1]) == col_r.size
+    sel = lambda t: t[heads]
+    ref = _oracle(sel(Q), sel(K), sel(V), sel(dO), sm_r, off_r, col_r)
+    got_lse = sel(lse).cpu().numpy().astype(np.float64)[:, rows]
+    assert np.max(np.abs(got_lse - ref["lse"][:, rows])) < 1e-3
+    for name, t in (("O", O), ("dQ", dQ)):
+        extra = ref["extra"][name][:, rows] if name in ref["extra"] else None
+        assert_close_bf16(sel(t).float().cpu().numpy()[:, rows], ref[name][:, rows], f"config 5 rows {name}", extra=extra)
+    keys = np.concatenate([np.arange(c * bs, (c + 1) * bs) for c in key_blocks])
+    for name, t in (("dK", dK), ("dV", dV)):
+        extra = ref["extra"][name][:, keys] if name in ref["extra"] else None
+        assert_close_bf16(sel(t).float().cpu().numpy()[:, keys], ref[name][:, keys], f"config 5 key blocks {name}", extra=extra)
+    abi.close()
