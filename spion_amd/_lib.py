@@ -43,6 +43,27 @@ def _cdll(name: str) -> ctypes.CDLL:
     return lib
 
 
+def autograd_node():
+    """The compiled autograd node (lib/_spion_node.so, csrc/autograd_node.cpp), or None when SPION_PY_NODE=1 asks for
+    the Python function instead (A/B timing, tests of the Python statement).  Both run the same kernels through the
+    same entry points; a missing build is an error like any other missing library."""
+    if "node" in _cache:
+        return _cache["node"]
+    mod = None
+    if os.environ.get("SPION_PY_NODE", "0") != "1":
+        import importlib.util
+
+        path = lib_path("_spion_node.so")
+        if not os.path.exists(path):
+            raise SpionLibraryError(f"{path} is missing: build the libraries first (python -m spion_amd.build)")
+        core()  # libspion_hip.so first: the node links against it
+        spec = importlib.util.spec_from_file_location("_spion_node", path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+    _cache["node"] = mod
+    return mod
+
+
 def core() -> ctypes.CDLL:
     """libspion_hip.so with argtypes of the entry points that have no reference counterpart."""
     lib = _cdll("libspion_hip.so")

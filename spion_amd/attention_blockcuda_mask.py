@@ -18,5 +18,5 @@ class CUDABlockMaskAttention(_BlockAttentionBase):
         super().__init__(config, attn_cpp, attn_handle)
 
     def forward(self, query, key, value, mask, mat):
-        out, _ = self.attn_func.apply(query, key, value, mask, mat, self)
+        out, _ = self.run(query, key, value, mask, mat)
         return out, 0

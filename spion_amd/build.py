@@ -39,6 +39,26 @@ def _run(cmd, verbose):
         print(out, flush=True)
 
 
+def build_autograd_node(verbose: bool = False) -> str:
+    """csrc/autograd_node.cpp -> lib/_spion_node.so: host code against libtorch and libspion_hip.so (g++, no HIP)."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension
+
+    out = os.path.join(LIB, "_spion_node.so")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-DTORCH_EXTENSION_NAME=_spion_node",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}"]
+    for inc in cpp_extension.include_paths() + [sysconfig.get_paths()["include"]]:
+        cmd += ["-isystem", inc]
+    cmd += [os.path.join(CSRC, "autograd_node.cpp"), "-o", out, f"-L{LIB}", "-lspion_hip", "-Wl,-rpath,$ORIGIN"]
+    for d in cpp_extension.library_paths():
+        cmd += [f"-L{d}", f"-Wl,-rpath,{d}"]
+    cmd += ["-lc10", "-ltorch_cpu", "-ltorch", "-ltorch_python"]
+    _run(cmd, verbose)
+    return out
+
+
 def build_all(verbose: bool = False, jobs: int = 4) -> str:
     os.makedirs(OBJ, exist_ok=True)
 
@@ -56,6 +76,7 @@ def build_all(verbose: bool = False, jobs: int = 4) -> str:
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", f"-DSPION_DROPIN={k}",
               os.path.join(CSRC, "dropin.cpp"), "-o", os.path.join(LIB, name),
               f"-L{LIB}", "-lspion_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed", "-Wl,-z,defs"], verbose)
+    build_autograd_node(verbose)
     return main_lib
 
 
