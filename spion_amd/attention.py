@@ -112,13 +112,10 @@ class Attention(nn.Module):
         self.ff = nn.Linear(self.num_head * self.head_dim, self.dim)
 
     def forward(self, X, mask, mat=None):
-        if X.is_cuda and torch.cuda.is_current_stream_capturing():
-            # Recording the whole layer (torch's GEMMs, concatenations and reductions around the attention core) into
-            # a HIP graph ended in a segmentation fault of the host process inside torch's capture_end on ROCm 7.2 /
-            # PyTorch 2.10; the cause is not established.  The attention core modules themselves replay correctly.
-            raise _lib.SpionLibraryError(
-                "spion_amd.Attention cannot be recorded into a HIP graph as a whole layer; capture the attention "
-                "core (layer.attn / layer.block_attn) and run the projections outside the graph")
+        """Can be recorded into a HIP graph as a whole layer, forward and backward (tests/test_gpu_graph.py), under
+        torch's usual rule for capturing a backward: warm up on a side stream and keep no autograd graph of a step
+        that ran on the default stream alive (its AccumulateGrad nodes belong to the legacy stream, which a capture
+        must not touch; breaking this rule ends in a crash inside capture_end on ROCm, not in an error message)."""
         if self.fused_qkv and X.dtype == torch.float32 and not torch.is_autocast_enabled():
             Q, K, V = _FusedQKV.apply(X, self.W_q.weight, self.W_k.weight, self.W_v.weight, self.W_q.bias,
                                       self.W_k.bias, self.W_v.bias, self.num_head, self.head_dim)

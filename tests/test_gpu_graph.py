@@ -101,11 +101,6 @@ def test_whole_step_graph_replays_match_eager(kind):
     assert np.isfinite(ref_out.float().cpu().numpy()).all()
 
 
-@pytest.mark.skip(reason="recording the whole layer -- torch's own GEMMs, concatenations and reductions around the "
-                         "attention modules -- ended in a segmentation fault of the host process inside "
-                         "torch.cuda.graphs.capture_end on this image; cause not established, so the case stays off "
-                         "the GPU.  The modules' own calls under capture are covered by "
-                         "test_whole_step_graph_replays_match_eager.")
 @pytest.mark.parametrize("sparse", [True, False])
 def test_attention_layer_graph_replays_match_eager(sparse):
     """The whole ``Attention`` layer -- one GEMM for the three projections, heads read in place by the strided entry
@@ -131,11 +126,18 @@ def test_attention_layer_graph_replays_match_eager(sparse):
         y.backward(dY)
         return y
 
-    y = step()
-    ref_y, ref_grads = y.detach().clone(), [t.grad.clone() for t in params]
+    # Every eager step ahead of the capture runs on a side stream and leaves no autograd graph behind.  A step on
+    # the default stream whose output stays referenced keeps its AccumulateGrad nodes alive, and they belong to the
+    # stream they were made on: the captured backward would then have to order the capturing stream against the
+    # legacy default stream, which no capture may touch (torch warns of exactly this: "may ... break CUDA graph
+    # capture if the AccumulateGrad node's stream is the default stream").  An earlier form of this test did that
+    # and ended in a segmentation fault inside capture_end.
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
+        y = step()
+        ref_y, ref_grads = y.detach().clone(), [t.grad.clone() for t in params]
+        del y
         for _ in range(3):
             step()
     torch.cuda.current_stream().wait_stream(side)
