@@ -32,6 +32,12 @@ int spion_debug_counter(void* handle, int which);
  * Read whenever a bf16 handle indexes a pattern (tests):
  *   SPION_BF16_LANES     number of persistent wavefronts the bf16 kernels are launched with (default: eight per
  *                        compute unit); a handful makes each one walk many strips of several heads in a row.
+ * Read once, at the first sparse call:
+ *   SPION_ROCTX=1        roctx ranges around the phases of every sparse call ("spion forward (tile kernels)",
+ *                        "spion backward: row pass (dQ)", "spion backward: column pass (dK, dV)", ...: the host-side
+ *                        intervals in which the phase's kernels are enqueued), as the reference brackets its cuSPARSE
+ *                        steps with nvtx ranges (models/block_attn.cu:163-223); `rocprofv3 --marker-trace` shows
+ *                        them.  The tools library is loaded with dlopen only when the switch is set.
  * SPION_QUIET and SPION_ABORT_ON_ERROR (error reporting) are described in spion_hip.h. */
 
 #ifdef __cplusplus

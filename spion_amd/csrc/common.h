@@ -1,10 +1,12 @@
 // Shared host-side helpers of libspion_hip.so: error slot, HIP status checks, handle header.
 #pragma once
+#include <dlfcn.h>
 #include <hip/hip_runtime.h>
 
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -50,5 +52,40 @@ inline bool check_launch(const char* what) {
     }
     return true;
 }
+
+// Named ranges around the phases of a call (the reference brackets its cuSPARSE steps with nvtxRangePush / Pop,
+// models/block_attn.cu:163-223): with SPION_ROCTX=1 in the environment the ROCm tools library is loaded on first use
+// and every PhaseRange pushes / pops a roctx range, so that a marker trace of a training step attributes host time
+// per phase.  Without the switch (or the library) a PhaseRange does nothing.
+struct RoctxApi {
+    int (*push)(const char*) = nullptr;
+    int (*pop)() = nullptr;
+};
+inline const RoctxApi* roctx_api() {
+    static const RoctxApi api = [] {
+        RoctxApi a;
+        const char* env = std::getenv("SPION_ROCTX");
+        if (!env || env[0] != '1') return a;
+        void* h = dlopen("librocprofiler-sdk-roctx.so", RTLD_NOW | RTLD_GLOBAL);
+        if (!h) h = dlopen("libroctx64.so", RTLD_NOW | RTLD_GLOBAL);
+        if (!h) return a;
+        a.push = reinterpret_cast<int (*)(const char*)>(dlsym(h, "roctxRangePushA"));
+        a.pop = reinterpret_cast<int (*)()>(dlsym(h, "roctxRangePop"));
+        if (!a.push || !a.pop) a = RoctxApi{};
+        return a;
+    }();
+    return api.push ? &api : nullptr;
+}
+struct PhaseRange {
+    const RoctxApi* api;
+    explicit PhaseRange(const char* name) : api(roctx_api()) {
+        if (api) api->push(name);
+    }
+    ~PhaseRange() {
+        if (api) api->pop();
+    }
+    PhaseRange(const PhaseRange&) = delete;
+    PhaseRange& operator=(const PhaseRange&) = delete;
+};
 
 }  // namespace spion

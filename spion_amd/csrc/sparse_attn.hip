@@ -1174,6 +1174,7 @@ static int heads_per_group(const SparseAttn* a) {
 template <int D, bool MASK, bool KROW, bool ST = false>
 static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, const float* V, const float* pen, float* P,
                             float* O, const int* offs, int nnz, const Layouts& ly = Layouts{}) {
+    PhaseRange phase("spion forward (tile kernels)");
     const PatternIndex& pi = a->pat;
     const int nbr = a->L / 32;
     float* ocache = ST ? nullptr : ocache_for_forward(a, P);
@@ -1231,20 +1232,24 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     const float* ocache = Out ? Out : ocache_for_backward(a, P);
 #define SPION_LAUNCH(W)                                                                                             \
     do {                                                                                                            \
-        if ((a->bwd_passes & 1) && ocache)                                                                          \
+        if ((a->bwd_passes & 1) && ocache) {                                                                        \
+            PhaseRange range("spion backward: row pass (dQ)");                                                      \
             hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, K,   \
                                Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB,    \
                                nnz, a->scale, hc, ly);                                                              \
-        else if (a->bwd_passes & 1) {                                                                               \
+        } else if (a->bwd_passes & 1) {                                                                             \
+            PhaseRange range("spion backward: row pass (dQ)");                                                      \
             if constexpr (!ST)                                                                                      \
                 hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream,  \
                                    K, Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr,    \
                                    a->NB, nnz, a->scale, hc, ly);                                                   \
         }                                                                                                           \
-        if (a->bwd_passes & 2)                                                                                      \
+        if (a->bwd_passes & 2) {                                                                                    \
+            PhaseRange range("spion backward: column pass (dK, dV)");                                               \
             hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, \
                                dO, rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
                                hc, ly);                                                                             \
+        }                                                                                                           \
     } while (0)
     if (wv == 1) SPION_LAUNCH(1);
     else if (wv == 2) SPION_LAUNCH(2);
@@ -1257,6 +1262,7 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 template <bool ST>
 static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const float* V, const float* Mask,
                            float* Attn, float* Out, float* ocopy, const int* Offsets, int nnz, const Layouts& ly) {
+    PhaseRange phase("spion forward (hybrid kernels)");
     if (!ensure_ws(&a->ws_stats, (size_t)a->NB * a->L * 2)) return;
     // the remainder's raw logits between the first and the third launch: a compact list of their own (written and
     // read in full lines) rather than their places inside P, where every four-byte store would pull in a line
@@ -1301,6 +1307,7 @@ template <bool ST>
 static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const float* V, const float* P,
                            const float* dO, const float* o, float* dS, float* dQ, float* dK, float* dV, int nnz,
                            const Layouts& ly) {
+    PhaseRange phase("spion backward (hybrid kernels)");
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L)) return;
     a->last_path = 3;
     const int nbr = a->L / 32;
@@ -1341,6 +1348,7 @@ template <int D, bool ST = false>
 static void launch_elem_fwd(SparseAttn* a, const float* Q, const float* Krm, const float* V, const float* pen,
                             float* P, float* O, const int* offs, const int* cols, int nnz,
                             const Layouts& ly = Layouts{}) {
+    PhaseRange phase("spion forward (element kernels)");
     const long long rows = (long long)a->NB * a->L;
     dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
     if (a->has_mask)
@@ -1355,6 +1363,7 @@ template <int D, bool ST = false>
 static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vrm, const float* P,
                             const float* dO, float* dS, float* dQ, float* dK, float* dV, const int* offs,
                             const int* cols, int nnz, const Layouts& ly = Layouts{}) {
+    PhaseRange phase("spion backward (element kernels)");
     const PatternIndex& pi = a->pat;
     const long long rows = (long long)a->NB * a->L;
     dim3 grid((unsigned)((rows + ELEM_WAVES - 1) / ELEM_WAVES));
@@ -1778,6 +1787,7 @@ static unsigned bf16_extent(const SparseAttn* a, bool strided, const HeadLayout&
 template <bool ST>
 static void bf16_forward_impl(SparseAttn* a, const void* Q, const void* K, const void* V, const float* Mask, void* Out,
                               float* Lse, const Layouts& ly) {
+    PhaseRange phase("spion forward (bf16 kernels)");
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
     const unsigned in_bytes = bf16_extent(a, ST, ly.in, ly.H), out_bytes = bf16_extent(a, ST, ly.out, ly.H);
@@ -1821,6 +1831,7 @@ template <bool ST>
 static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, const void* V, const float* Mask,
                                const void* Out, const float* Lse, const void* dO, void* dQ, void* dK, void* dV,
                                const Layouts& ly) {
+    PhaseRange phase("spion backward (bf16 kernels)");
     const PatternIndex& pi = a->pat;
     a->last_path = 1;
     const unsigned in_bytes = bf16_extent(a, ST, ly.in, ly.H), out_bytes = bf16_extent(a, ST, ly.out, ly.H);
