@@ -106,19 +106,36 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
 // wave-private LDS tiles; the map is written non-temporally.
 // RM: Q, V and Out are row-major head slices located by `ly` (heads possibly interleaved in [B][L][H*32] memory,
 // tile_kernels.h) instead of the feature-major [NB][32][L] operands of the reference's ABI; K likewise.
-template <bool MASK, bool RM = false>
-SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
+// MEAN (row-major operands, eight wavefronts with at most four logit tiles each): the launch also accumulates the
+// sum of the maps over the heads.  The grid is nbr x C work-groups instead of nbr x NB: work-group (c, I) walks the
+// heads c, c + C, c + 2C, ... one after the other and adds every probability tile it writes to a register tile of
+// its own, so the sum costs sixteen additions per tile and, once per work-group, the store of its [L][32] slab of
+// Part[c] (key-major like the map).  The mean over batch and heads is then one small reduction of the C partial maps.
+template <bool MASK, bool RM = false, int WAVES = 4, bool MEAN = false>
+SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
-    int L, int nbr, int NB, float scale, Layouts ly) {
-    constexpr int D = 32, KH = 16, WAVES = 4, MAXT = 8;
+    int L, int nbr, int NB, float scale, Layouts ly, float* __restrict__ Part = nullptr, int C = 0) {
+    static_assert(!MEAN || RM, "the mean-emitting forward takes row-major operands");
+    constexpr int D = 32, KH = 16, MAXT = 32 / WAVES;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][2 * 32 * TS];
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
-    const int bh = item / nbr, I = item % nbr;
+    const int item = xcd_remap(blockIdx.x, nbr * (MEAN ? C : NB));
+    const int bh0 = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
-    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w+4, ... of this wavefront
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w + WAVES, ... of this wavefront
+    float* T = lds_t[w];         // map tile on its way to memory
+    float* Tx = T + 32 * TS;     // K tile, later V^T tile
+    f32x16 total[MEAN ? MAXT : 1];
+    if constexpr (MEAN) {
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            total[u] = splat16(0.f);
+        }
+    }
+    int bh = bh0;
+    do {  // one head, or (MEAN) the heads bh0, bh0 + C, ...
     const size_t hb = (size_t)bh * L * D;
     size_t ib, ob, hbytes, obytes;
     int ild, old_;
@@ -127,8 +144,6 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes);
     const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
     const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    float* T = lds_t[w];         // map tile on its way to memory
-    float* Tx = T + 32 * TS;     // K tile, later V^T tile
     const int klin = lin_voff(l, ild), alin = lin_voff(l, L);
     const int vld = RM ? ild : L, vlin = lin_voff(l, vld), VSTEP = RM ? 32 * ild * 4 : 128;
     const float c2 = scale * LOG2E;
@@ -151,14 +166,17 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
     float m = -10.f * LOG2E, z = 0.f;  // models/attn.cu:17
     f32x16 S[MAXT];
     {
-        f32x4 kraw[2][4];
-        if (nu > 0) ldr_tile_lin(rK, klin, w * 32 * ild * 4, ild, kraw[0]);
+        // PRE: the next tile is requested while one is worked on (the mean-emitting form has no registers for that)
+        constexpr int PRE = MEAN ? 0 : 1;
+        f32x4 kraw[1 + PRE][4];
+        if (PRE && nu > 0) ldr_tile_lin(rK, klin, w * 32 * ild * 4, ild, kraw[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int J = w + u * WAVES;
-                if (u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * ild * 4, ild, kraw[(u + 1) & 1]);
-                lds_put_lin(Tx, l, kraw[u & 1]);
+                if (PRE && u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * ild * 4, ild, kraw[(u + 1) & PRE]);
+                if (!PRE) ldr_tile_lin(rK, klin, J * 32 * ild * 4, ild, kraw[0]);
+                lds_put_lin(Tx, l, kraw[u & PRE]);
                 float kf[KH];
                 lds_get_feat32(Tx, li, h, kf);
                 __builtin_amdgcn_sched_barrier(0);
@@ -200,17 +218,23 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
 
     f32x16 o[1] = {splat16(0.f)};  // O^T: register = feature, lane = query
     {
-        f32x4 vraw[2][4];
-        if (nu > 0) ldr_tile_lin(rV, vlin, w * VSTEP, vld, vraw[0]);
+        constexpr int PRE = MEAN ? 0 : 1;  // see above
+        f32x4 vraw[1 + PRE][4];
+        if (PRE && nu > 0) ldr_tile_lin(rV, vlin, w * VSTEP, vld, vraw[0]);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int J = w + u * WAVES;
-                if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * VSTEP, vld, vraw[(u + 1) & 1]);
-                lds_put_lin(Tx, l, vraw[u & 1]);
+                if (PRE && u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * VSTEP, vld, vraw[(u + 1) & PRE]);
+                if (!PRE) ldr_tile_lin(rV, vlin, J * VSTEP, vld, vraw[0]);
+                lds_put_lin(Tx, l, vraw[u & PRE]);
                 float p[16], vb[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                if constexpr (MEAN) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) total[u][r] += p[r];
+                }
                 lds_put_cols(T, li, h, p);        // T[key][query]: the map is stored key-major
                 if constexpr (RM) lds_get_cols(Tx, li, h, vb);  // vb[s] = V[key acc_row(s, h)][feature li]
                 else lds_get_rows(Tx, li, h, vb);
@@ -230,6 +254,25 @@ SPION_TILE_KERNEL(4) void dense_fwd_reg_kernel(
         if (OutCopy) {
             __syncthreads();
             reduce_store<D, WAVES, true>(o, OutCopy + hb, I * 32, w, li, h, lds, L);
+        }
+    }
+    if constexpr (MEAN) __syncthreads();  // the shared arrays are free for the next head
+    bh += MEAN ? C : NB;
+    } while (MEAN && bh < NB);
+    if constexpr (MEAN) {
+        const rsrc_t rS = make_rsrc(Part + (size_t)bh0 * L * L, (size_t)L * L * 4);
+        const int alin = lin_voff(l, L);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                float p[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = total[u][r];
+                lds_put_cols(T, li, h, p);
+                f32x4 pl[4];
+                lds_get_lin(T, l, pl);
+                str_tile_lin_cached(rS, alin, ((w + u * WAVES) * 32 * L + I * 32) * 4, L, pl);
+            }
         }
     }
 }
@@ -919,10 +962,22 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
     const dim3 grid(nbr * a->NB), block4(64 * 4);
     a->out_key = nullptr;  // no kept copy: the strided backward is handed Out
     if (Mean) {
-        // C partial maps: the smallest divisor of NB that gives the launch two work-groups per CU
+        // C partial maps: the smallest divisor of NB that fills the device -- one eight-wavefront work-group per CU
+        // for the register-resident form (measured at B=256, H=2, L=1024: 0.95 ms with 256 work-groups, 1.05 with
+        // 512, 1.22 with 1024: fewer, longer work-groups store fewer partial maps), two four-wavefront ones otherwise
+        static int cus = 0;
+        if (!cus) {
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess ||
+                hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+                (void)hipGetLastError();
+                cus = 256;
+            }
+        }
+        const long long want = nbr <= 32 ? cus : 2LL * cus;
         int C = a->NB;
         for (int c = 1; c <= a->NB; ++c)
-            if (a->NB % c == 0 && (long long)c * nbr >= 512) {
+            if (a->NB % c == 0 && (long long)c * nbr >= want) {
                 C = c;
                 break;
             }
@@ -944,8 +999,16 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
 #define SPION_LAUNCH(KERNEL, MM)                                                                                     \
     hipLaunchKernelGGL((KERNEL<MM, true, true>), grid_m, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out, nullptr, \
                        a->L, nbr, a->NB, a->scale, ly, a->ws_mean, C)
-        // the two-sweep kernel for every length: the register-resident one has no registers left for the partial sums
-        if (a->has_mask) SPION_LAUNCH(dense_fwd_sweep32_kernel, true);
+        if (nbr <= 32) {
+            // register-resident logits on eight wavefronts, the partial sums in registers as well
+            const dim3 block8(64 * 8);
+            if (a->has_mask)
+                hipLaunchKernelGGL((dense_fwd_reg_kernel<true, true, 8, true>), grid_m, block8, 0, a->hdr.stream, Q, K, V,
+                                   Mask, Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly, a->ws_mean, C);
+            else
+                hipLaunchKernelGGL((dense_fwd_reg_kernel<false, true, 8, true>), grid_m, block8, 0, a->hdr.stream, Q, K, V,
+                                   Mask, Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly, a->ws_mean, C);
+        } else if (a->has_mask) SPION_LAUNCH(dense_fwd_sweep32_kernel, true);
         else SPION_LAUNCH(dense_fwd_sweep32_kernel, false);
 #undef SPION_LAUNCH
         if (!check_launch("dense_fwd kernels")) return;

@@ -55,16 +55,16 @@ __device__ __forceinline__ f32x4 ld4_nt(rsrc_t r, int voff, int soff) {
 }
 // 128-bit buffer stores.  The hardware reads a store's data registers over several cycles after issue: a VALU write
 // to one of them in the next two issue slots can reach the store (seen on MI355X as single stale 4-byte words, now
-// and then).  The compiler keeps that distance for stores without a register soffset only, so here the two idle
-// slots are part of the instruction sequence.  NT: non-temporal.
+// and then).  The compiler keeps that distance, but only for stores whose soffset is not a register (with a register
+// there it relies on an extra issue cycle that covers one of the two slots).  So the scalar part of the address is
+// added to the lane offset and the soffset field stays zero: every hazard of the instruction is then the compiler's
+// to handle, which inline assembly would hide from it (the wait states between a VALU write of a scalar register
+// and a memory instruction that reads it, for one).  NT: non-temporal.
 template <bool NT = false, typename X>
 __device__ __forceinline__ void store_b128(X x, rsrc_t r, int voff, int soff) {
     static_assert(sizeof(X) == 16, "128-bit store");
-    const int so = __builtin_amdgcn_readfirstlane(soff);
-    if (NT)
-        asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen nt\n\ts_nop 1" ::"v"(x), "v"(voff), "s"(r), "s"(so) : "memory");
-    else
-        asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 1" ::"v"(x), "v"(voff), "s"(r), "s"(so) : "memory");
+    typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, x), r, voff + soff, 0, NT ? 2 : 0);
 }
 __device__ __forceinline__ void st4(rsrc_t r, int voff, int soff, f32x4 v) { store_b128(v, r, voff, soff); }
 
