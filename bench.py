@@ -455,7 +455,13 @@ def bench_dense_phase(args, dev):
         handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), attn.data_ptr(), out_r.data_ptr(), dOr.data_ptr(),
         gq.data_ptr(), gk.data_ptr(), gv.data_ptr(), H, A, A, A), max(10, args.steps // 4))
     _lib.check_error("dense backward (row-major)")
-    del Qr, Kr, Vr, dOr, out_r, gq, gk, gv
+    # the same forward leaving the mean of all maps as well (what pattern discovery reads)
+    mean_map = torch.empty(L, L, device=dev)
+    t_fwd_mean = _event_ms(lambda: core.spion_dense_forward_strided_mean(
+        handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), None, attn.data_ptr(), out_r.data_ptr(),
+        mean_map.data_ptr(), H, A, A), max(10, args.steps // 4))
+    _lib.check_error("dense forward with mean (row-major)")
+    del Qr, Kr, Vr, dOr, out_r, gq, gk, gv, mean_map
 
     # forward kernel alone at the C ABI (operands in the layouts it takes: Qt, Vt feature-major)
     Qt = _lib.transpose_last2(q.detach().reshape(NB, L, d))
@@ -481,6 +487,7 @@ def bench_dense_phase(args, dev):
     roof["kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd_rm, 4),
                          "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd_rm, 4)}
     roof["backward_frac"] = alg_flops * 2.0 / 3.0 / t_bwd_rm / 1e9 / PEAK_FP32_MFMA_TFLOPS
+    roof["forward_with_mean_ms"] = round(t_fwd_mean, 4)  # spion_dense_forward_strided_mean: maps + their mean
     roof["reference_abi_kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd, 4),
                                        "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd, 4)}
     result = {
