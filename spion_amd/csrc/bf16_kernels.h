@@ -419,7 +419,10 @@ SPION_BF16_LANE(2) void bf16_fwd_kernel(
             wait_lgkm0();
 #pragma unroll
             for (int k = 0; k < 2; ++k)
-                if (gi <= g + 2 && sq_g == gi) issue();
+                if (gi <= g + 2 && gi - g0 < len + lenn) {
+                    if (sq_g != gi) locate(gi);  // the tile loop's short cut issues without looking up
+                    issue();
+                }
         };
 #pragma unroll
         for (int k = 0; k < 2; ++k)
@@ -431,8 +434,21 @@ SPION_BF16_LANE(2) void bf16_fwd_kernel(
         const unsigned ho = bf16_head_bytes<ST, D>(ly.out, ly.H, bh, L);
         // one tile: the operands leave LDS, the buffer goes to the element after next (the item's last tile keeps
         // it for the result), `math` does the arithmetic
-        auto tile = [&](bool last, auto&& math) __attribute__((always_inline)) {
-            const char* Tk = begin();
+        // Short cut for all but an item's last two tiles: the element after next is tile i + 2 of the same item, so
+        // its loads need one index look-up and none of the general stream's case distinctions (which cost more
+        // scalar instructions and branches per tile than the tile's arithmetic has MFMAs).
+        auto tile = [&](int i, auto&& math) __attribute__((always_inline)) {
+            const bool last = i + 1 == n;
+            const bool quick = i + 2 < n && gi == g + 2;
+            int J2 = 0;
+            if (quick) J2 = tiles[t0 + i + 2];
+            const char* Tk;
+            if (quick) {
+                wait_vm<OPS>();
+                Tk = Tw + (g & 1) * DT::BUF;
+            } else {
+                Tk = begin();
+            }
             const char* Tv = Tk + DT::TILE;
             bf16x8 kr[D / 16], vt[D / 32][2];
             DT::get_rows(Tk, ra, kr);
@@ -444,8 +460,19 @@ SPION_BF16_LANE(2) void bf16_fwd_kernel(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
             }
-            if (!last) release();
-            else wait_lgkm0();
+            if (quick) {
+                wait_lgkm0();
+                const unsigned a = lds_w + (g & 1) * DT::BUF;  // element g + 2 takes the buffer of element g
+                const int s2 = uniform((int)(hb + (unsigned)(J2 * t_bytes)));
+                DT::load(wK, a, vin, s2, xin);
+                DT::load(wV, a + DT::TILE, vin, s2, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, MASK ? uniform((bh * L + J2 * 32) * 4) : s2);
+                ++gi;
+            } else if (!last) {
+                release();
+            } else {
+                wait_lgkm0();
+            }
             __builtin_amdgcn_sched_barrier(0);
             math(kr, vt, init);
             __builtin_amdgcn_sched_barrier(0);
@@ -508,7 +535,7 @@ SPION_BF16_LANE(2) void bf16_fwd_kernel(
                 o1[c] = splat16(0.f);
             }
             for (int i = 0; i < n; ++i)
-                tile(i + 1 == n, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
+                tile(i, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
                     const f32x16 s0 = mma_feat_bf16<D>(kr, q0, init);
                     const f32x16 s1 = mma_feat_bf16<D>(kr, q1, init);
                     bf16x8 pb0[2], pb1[2];
@@ -534,7 +561,7 @@ SPION_BF16_LANE(2) void bf16_fwd_kernel(
 #pragma unroll
             for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
             for (int i = 0; i < n; ++i)
-                tile(i + 1 == n, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
+                tile(i, [&](const bf16x8 (&kr)[D / 16], const bf16x8 (&vt)[D / 32][2], const f32x16& init) __attribute__((always_inline)) {
                     const f32x16 s = mma_feat_bf16<D>(kr, q, init);  // S^T: register = key, lane = query
                     bf16x8 pb[2];
                     update(s, m, z, o, pb);
@@ -657,7 +684,10 @@ SPION_BF16_LANE(2) void bf16_bwd_row_kernel(
             wait_lgkm0();
 #pragma unroll
             for (int k = 0; k < 2; ++k)
-                if (gi <= g + 2 && sq_g == gi) issue();
+                if (gi <= g + 2 && gi - g0 < len + lenn) {
+                    if (sq_g != gi) locate(gi);  // the tile loop's short cut issues without looking up
+                    issue();
+                }
         };
 #pragma unroll
         for (int k = 0; k < 2; ++k)
@@ -696,9 +726,20 @@ SPION_BF16_LANE(2) void bf16_bwd_row_kernel(
         f32x16 acc[D / 32];
 #pragma unroll
         for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
+        const int ls_item = (bh * L + I * 32) * 4;
         for (int i = 0; i < n; ++i) {
             const bool last = i + 1 == n;
-            const char* Tk = begin();
+            // all but the item's last two tiles: the element after next is tile i + 2 of this item (see the forward)
+            const bool quick = i + 2 < n && gi == g + 2;
+            int J2 = 0;
+            if (quick) J2 = tiles[t0 + i + 2];
+            const char* Tk;
+            if (quick) {
+                wait_vm<OPS>();
+                Tk = Tw + (g & 1) * DT::BUF;
+            } else {
+                Tk = begin();
+            }
             const char* Tv = Tk + DT::TILE;
             bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
             DT::get_rows(Tk, ra, kr);
@@ -711,8 +752,19 @@ SPION_BF16_LANE(2) void bf16_bwd_row_kernel(
 #pragma unroll
                 for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
             }
-            if (!last) release();  // the tile's operands are in registers: its buffer can take the element after next
-            else wait_lgkm0();     // (the item's last tile keeps it for the result)
+            if (quick) {
+                wait_lgkm0();
+                const unsigned a = lds_w + (g & 1) * DT::BUF;
+                const int s2 = uniform((int)(hb + (unsigned)(J2 * t_bytes)));
+                DT::load(wK, a, vin, s2, xin);
+                DT::load(wV, a + DT::TILE, vin, s2, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, uniform(MASK ? (bh * L + J2 * 32) * 4 : ls_item));
+                ++gi;
+            } else if (!last) {
+                release();  // the tile's operands are in registers: its buffer can take the element after next
+            } else {
+                wait_lgkm0();  // (the item's last tile keeps it for the result)
+            }
             __builtin_amdgcn_sched_barrier(0);
             const f32x16 s = mma_feat_bf16<D>(kr, q, init);
             const f32x16 dp = mma_feat_bf16<D>(vr, go, gneg);  // dO_i . v_j - g_i
@@ -836,7 +888,10 @@ SPION_BF16_LANE(2) void bf16_bwd_col_kernel(
             wait_lgkm0();
 #pragma unroll
             for (int k = 0; k < 2; ++k)
-                if (gi <= g + 2 && sq_g == gi) issue();
+                if (gi <= g + 2 && gi - g0 < len + lenn) {
+                    if (sq_g != gi) locate(gi);  // the tile loop's short cut issues without looking up
+                    issue();
+                }
         };
 #pragma unroll
         for (int k = 0; k < 2; ++k)
@@ -866,9 +921,26 @@ SPION_BF16_LANE(2) void bf16_bwd_col_kernel(
             ak[c] = splat16(0.f);
             av[c] = splat16(0.f);
         }
+        // all but the item's last two tiles: the element after next is tile i + 2 of this item (see the forward)
+        auto quick_issue = [&](int I2) __attribute__((always_inline)) {
+            const unsigned a = lds_w + (g & 1) * DT::BUF;
+            DT::load(wQ, a, vin, uniform((int)(hb + (unsigned)(I2 * t_bytes))), xin);
+            DT::load(wG, a + DT::TILE, vout, uniform((int)(ho + (unsigned)(I2 * o_bytes))), xout);
+            dma_b32(wS, a + 2 * DT::TILE, l * 4, uniform((bh * (L / 32) + I2) * 256));
+            ++gi;
+        };
         for (int i = 0; i < n; ++i) {
             const bool last = i + 1 == n;
-            const char* Tq = begin();
+            const bool quick = i + 2 < n && gi == g + 2;
+            int I2 = 0;
+            if (quick) I2 = tiles[4 * (t0 + i + 2)];
+            const char* Tq;
+            if (quick) {
+                wait_vm<OPS>();
+                Tq = Tw + (g & 1) * DT::BUF;
+            } else {
+                Tq = begin();
+            }
             const char* Tg = Tq + DT::TILE;
             const float* St = reinterpret_cast<const float*>(Tq + 2 * DT::TILE);  // lse2[32], -g[32] of the tile's queries
             float lse[16], gn[16];
@@ -880,8 +952,14 @@ SPION_BF16_LANE(2) void bf16_bwd_col_kernel(
             if constexpr (DEEP) {
                 DT::get_tile_t(Tq, ta, qt);
                 DT::get_tile_t(Tg, ta, gt);
-                if (!last) release();
-                else wait_lgkm0();
+                if (quick) {
+                    wait_lgkm0();
+                    quick_issue(I2);
+                } else if (!last) {
+                    release();
+                } else {
+                    wait_lgkm0();
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
             const f32x16 s = mma_feat_bf16<D>(qr, k, sinit);  // S: register = query, lane = key
@@ -903,8 +981,14 @@ SPION_BF16_LANE(2) void bf16_bwd_col_kernel(
             pack16(p, pb);
             pack16(ds, dsb);
             if constexpr (!DEEP) {
-                if (!last) release();
-                else wait_lgkm0();
+                if (quick) {
+                    wait_lgkm0();
+                    quick_issue(I2);
+                } else if (!last) {
+                    release();
+                } else {
+                    wait_lgkm0();
+                }
             }
             mma_tile_bf16<D>(qt, dsb, ak);  // dK^T: register = feature, lane = key
             mma_tile_bf16<D>(gt, pb, av);   // dV^T
