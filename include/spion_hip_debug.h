@@ -27,8 +27,9 @@ int spion_debug_counter(void* handle, int which);
 /* Environment switches read once per process, for A/B measurements only (results are the same either way):
  *   SPION_NO_FWD_SPLIT   the fp32 tile forward runs all strips in one launch, eight logit tiles per wavefront
  *                        (default: strips of at most 16 tiles in a launch of their own, three work-groups to a CU);
- *   SPION_BF16_NO_PAIRS  the bf16 forward takes one strip per wavefront on every pattern (default: two strips per
- *                        wavefront on masks of 64 x 64 blocks and larger).
+ *   SPION_BF16_NO_PAIRS  the bf16 forward and row pass take one strip per wavefront on every pattern (default: two
+ *                        strips per wavefront on masks of 64 x 64 blocks and larger, contiguous heads);
+ *   SPION_BF16_ROW_PAIRS=0  the same for the row pass alone.
  * Read whenever a bf16 handle indexes a pattern (tests):
  *   SPION_BF16_LANES     number of persistent wavefronts the bf16 kernels are launched with (default: eight per
  *                        compute unit); a handful makes each one walk many strips of several heads in a row.

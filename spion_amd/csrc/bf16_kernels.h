@@ -788,6 +788,260 @@ SPION_BF16_LANE(2) void bf16_bwd_row_kernel(
 }
 
 // -------------------------------------------------------------------------------------------------
+// Backward, row pass with two strips per wavefront (masks of 64 x 64 blocks and larger, contiguous heads): the
+// launch walks the pair plan, whose items of kind -2 give a wavefront strips 2p and 2p+1.  Every K and V tile is
+// fetched and read back as an operand once for the two strips' chains, which run one after the other on the same
+// operand registers.  Other items of the plan (chunks of long strips) are single strips and take the first half of
+// the same code.
+// Stream of an item: {Q tiles of the two strips, lse2 of both}, {dO tiles}, {O tiles}, then its K / V tiles.
+// -------------------------------------------------------------------------------------------------
+template <int D, bool MASK>
+SPION_BF16_LANE(2) void bf16_bwd_row_pair_kernel(
+    const __bf16* __restrict__ Q, const __bf16* __restrict__ K, const __bf16* __restrict__ V,
+    const __bf16* __restrict__ dO, const __bf16* __restrict__ O, const float* __restrict__ Lse,
+    const float* __restrict__ pen, float* __restrict__ Stats, __bf16* __restrict__ dQ, const int* __restrict__ tcol,
+    const int* __restrict__ plan_items, const int* __restrict__ lane_ptr, const int* __restrict__ lane_ent, int L,
+    int NB, float scale, float* __restrict__ Part, int n_slots, Layouts ly, unsigned in_bytes, unsigned out_bytes,
+    unsigned grad_bytes) {
+    constexpr bool ST = false;
+    constexpr int EL_C = 3;
+    typedef DmaTile<D> DT;
+    __shared__ __attribute__((aligned(16))) char Tw[DT::WAVE];
+    const int l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int e0 = as_constant(lane_ptr)[blockIdx.x], e1 = as_constant(lane_ptr)[blockIdx.x + 1];
+    if (e0 >= e1) return;
+    const const_ints ents = as_constant(lane_ent), items = as_constant(plan_items), tiles = as_constant(tcol);
+    const int ild = ST ? ly.in.ld : D, old_ = ST ? ly.out.ld : D, gld = ST ? ly.grad.ld : D;
+    const u32x4 wQ = rsrc_words(Q, in_bytes), wK = rsrc_words(K, in_bytes), wV = rsrc_words(V, in_bytes);
+    const u32x4 wG = rsrc_words(dO, out_bytes), wO = rsrc_words(O, out_bytes);
+    const u32x4 wL = rsrc_words(Lse, (size_t)NB * L * 4);
+    const u32x4 wM = rsrc_words(MASK ? pen : Lse, (size_t)NB * L * 4);
+    const rsrc_t rdQ = make_rsrc(dQ, grad_bytes);
+    const int t_bytes = 32 * ild * 2, o_bytes = 32 * old_ * 2;
+    const int vin = DT::voff(l, ild), xin = DT::extra_step(ild);
+    const int vout = DT::voff(l, old_), xout = DT::extra_step(old_), vgr = DT::voff(l, gld);
+    const unsigned lds_w = lds_address(Tw);
+    const typename DT::RowAddr ra = DT::row_addr(li, h);
+    const typename DT::TrAddr ta = DT::tr_addr(l);
+    const float c2 = scale * LOG2E, pen_mul = -1.0f / scale;
+    constexpr int E = 3, OPS = 2 * DT::NI + 1;
+
+    LaneEntry en = lane_entry(ents, e0);
+    PlanItem itn = plan_item(items, en.y);
+    int g = 0, gi = 0;
+    int sk = 0, sa = 0, sb = 0, sc = 0, sq_g = -1;  // element sq_g: kind and the offsets of its three loads
+    for (int e = e0; e < e1; ++e) {
+        const int bh = en.x;
+        const PlanItem it = itn;
+        const bool has_next = e + 1 < e1;
+        if (has_next) {
+            en = lane_entry(ents, e + 1);
+            itn = plan_item(items, en.y);
+        }
+        const int bhn = en.x;
+        const int I = it.x, t0 = it.y, n = it.z;
+        const bool pair = it.w == -2;
+        const int In = itn.x, t0n = itn.y;
+        const bool pairn = itn.w == -2;
+        const int len = E + n, lenn = has_next ? E + itn.z : 0;
+        const int g0 = g;
+        const unsigned hb = bf16_head_bytes<ST, D>(ly.in, ly.H, bh, L), hbn = bf16_head_bytes<ST, D>(ly.in, ly.H, bhn, L);
+        const unsigned ho = bf16_head_bytes<ST, D>(ly.out, ly.H, bh, L), hon = bf16_head_bytes<ST, D>(ly.out, ly.H, bhn, L);
+        auto locate_in = [&](int k, int bhX, int IX, int t0X, unsigned hbX, unsigned hoX, bool pairX) __attribute__((always_inline)) {
+            const int lsx = (bhX * L + IX * 32) * 4;
+            const int Ib = IX + (pairX ? 1 : 0);
+            if (k < E) {
+                sk = k == 0 ? EL_A : k == 1 ? EL_B : EL_C;
+                const unsigned base = k == 0 ? hbX : hoX;
+                const int step = k == 0 ? t_bytes : o_bytes;
+                sa = uniform((int)(base + (unsigned)(IX * step)));
+                sb = uniform((int)(base + (unsigned)(Ib * step)));
+                sc = uniform(lsx);
+            } else {
+                const int J = tiles[t0X + k - E];
+                sk = EL_TILE;
+                sa = uniform((int)(hbX + (unsigned)(J * t_bytes)));
+                sb = sa;
+                sc = uniform(MASK ? (bhX * L + J * 32) * 4 : lsx);
+            }
+        };
+        auto locate = [&, bh, bhn, I, In, t0, t0n, hb, hbn, ho, hon, len, g0, pair, pairn](int gg) __attribute__((always_inline)) {
+            const int k = gg - g0;
+            if (k < len) locate_in(k, bh, I, t0, hb, ho, pair);
+            else locate_in(k - len, bhn, In, t0n, hbn, hon, pairn);
+            sq_g = gg;
+        };
+        auto issue = [&]() __attribute__((always_inline)) {  // element gi -> buffer gi % 2, then look the following one up
+            const unsigned a = lds_w + (gi & 1) * DT::BUF;
+            if (sk == EL_TILE) {
+                DT::load(wK, a, vin, sa, xin);
+                DT::load(wV, a + DT::TILE, vin, sb, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, sc);
+            } else if (sk == EL_A) {
+                DT::load(wQ, a, vin, sa, xin);
+                DT::load(wQ, a + DT::TILE, vin, sb, xin);
+                dma_b32(wL, a + 2 * DT::TILE, l * 4, sc);
+            } else if (sk == EL_B) {
+                DT::load(wG, a, vout, sa, xout);
+                DT::load(wG, a + DT::TILE, vout, sb, xout);
+                dma_b32(wL, a + 2 * DT::TILE, l * 4, sc);
+            } else {
+                DT::load(wO, a, vout, sa, xout);
+                DT::load(wO, a + DT::TILE, vout, sb, xout);
+                dma_b32(wL, a + 2 * DT::TILE, l * 4, sc);
+            }
+            ++gi;
+            if (gi - g0 < len + lenn) locate(gi);
+        };
+        auto begin = [&]() __attribute__((always_inline)) -> char* {  // wait for element g
+            if (gi - g > 1) wait_vm<OPS>();
+            else wait_vm<0>();
+            return Tw + (g & 1) * DT::BUF;
+        };
+        auto release = [&]() __attribute__((always_inline)) {  // element g has left its buffer
+            wait_lgkm0();
+#pragma unroll
+            for (int k = 0; k < 2; ++k)
+                if (gi <= g + 2 && gi - g0 < len + lenn) {
+                    if (sq_g != gi) locate(gi);  // the tile loop's short cut issues without looking up
+                    issue();
+                }
+        };
+#pragma unroll
+        for (int k = 0; k < 2; ++k)
+            if (gi < g0 + min(2, len)) {
+                if (sq_g != gi) locate(gi);
+                issue();
+            }
+        float* part = it.w >= 0 ? Part + ((size_t)bh * n_slots + it.w) * bf16_slot_floats<D>() : nullptr;
+        // the strips' operands: Q rows and lse2, dO rows, then O for the row sums g = dO . O
+        bf16x8 qa[D / 16], qb[D / 16], ga[D / 16], gb[D / 16];
+        float lse_a, lse_b, gsum_a = 0.f, gsum_b = 0.f;
+        {
+            const char* Ta = begin();
+            DT::get_rows(Ta, ra, qa);
+            DT::get_rows(Ta + DT::TILE, ra, qb);
+            lse_a = reinterpret_cast<const float*>(Ta + 2 * DT::TILE)[li];
+            lse_b = reinterpret_cast<const float*>(Ta + 2 * DT::TILE)[32 + li];
+            release();
+            ++g;
+            const char* Tb = begin();
+            DT::get_rows(Tb, ra, ga);
+            DT::get_rows(Tb + DT::TILE, ra, gb);
+            release();
+            ++g;
+            const char* Tc = begin();
+            bf16x8 oa[D / 16], ob[D / 16];
+            DT::get_rows(Tc, ra, oa);
+            DT::get_rows(Tc + DT::TILE, ra, ob);
+            if (n > 0) {
+                release();
+                ++g;
+            } else {
+                wait_lgkm0();
+            }
+#pragma unroll
+            for (int t = 0; t < D / 16; ++t)
+#pragma unroll
+                for (int x = 0; x < 8; ++x) {
+                    gsum_a = fmaf((float)ga[t][x], (float)oa[t][x], gsum_a);
+                    gsum_b = fmaf((float)gb[t][x], (float)ob[t][x], gsum_b);
+                }
+            gsum_a = half_swap_sum(gsum_a);
+            gsum_b = half_swap_sum(gsum_b);
+        }
+        // every chunk of a strip writes the same values
+        Stats[((size_t)bh * (L / 32) + I) * 64 + l] = h ? -gsum_a : lse_a;
+        if (pair) Stats[((size_t)bh * (L / 32) + I + 1) * 64 + l] = h ? -gsum_b : lse_b;
+        const f32x16 gneg_a = splat16(-gsum_a), gneg_b = splat16(-gsum_b);
+        f32x16 acc_a[D / 32], acc_b[D / 32];
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) {
+            acc_a[c] = splat16(0.f);
+            acc_b[c] = splat16(0.f);
+        }
+        const int ls_item = (bh * L + I * 32) * 4;
+        for (int i = 0; i < n; ++i) {
+            const bool last = i + 1 == n;
+            // all but the item's last two tiles: the element after next is tile i + 2 of this item (see the forward)
+            const bool quick = i + 2 < n && gi == g + 2;
+            int J2 = 0;
+            if (quick) J2 = tiles[t0 + i + 2];
+            const char* Tk;
+            if (quick) {
+                wait_vm<OPS>();
+                Tk = Tw + (g & 1) * DT::BUF;
+            } else {
+                Tk = begin();
+            }
+            const char* Tv = Tk + DT::TILE;
+            bf16x8 kr[D / 16], vr[D / 16], kt[D / 32][2];
+            DT::get_rows(Tk, ra, kr);
+            DT::get_rows(Tv, ra, vr);
+            DT::get_tile_t(Tk, ta, kt);
+            f32x16 init = splat16(0.f);
+            if constexpr (MASK) {
+                float pj[16];
+                lds_get_rows(reinterpret_cast<const float*>(Tk + 2 * DT::TILE), 0, h, pj);  // pj[r] = pen[acc_row(r, h)]
+#pragma unroll
+                for (int r = 0; r < 16; ++r) init[r] = pj[r] * pen_mul;
+            }
+            if (quick) {
+                wait_lgkm0();
+                const unsigned a = lds_w + (g & 1) * DT::BUF;
+                const int s2 = uniform((int)(hb + (unsigned)(J2 * t_bytes)));
+                DT::load(wK, a, vin, s2, xin);
+                DT::load(wV, a + DT::TILE, vin, s2, xin);
+                dma_b32(wM, a + 2 * DT::TILE, l * 4, uniform(MASK ? (bh * L + J2 * 32) * 4 : ls_item));
+                ++gi;
+            } else if (!last) {
+                release();  // the tile's operands are in registers: its buffer can take the element after next
+            } else {
+                wait_lgkm0();  // (the item's last tile keeps it for the result)
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            {
+                const f32x16 s = mma_feat_bf16<D>(kr, qa, init);
+                const f32x16 dp = mma_feat_bf16<D>(vr, ga, gneg_a);  // dO_i . v_j - g_i
+                float ds[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse_a)) * dp[r];
+                bf16x8 dsb[2];
+                pack16(ds, dsb);
+                mma_tile_bf16<D>(kt, dsb, acc_a);  // dQ^T: register = feature, lane = query
+            }
+            if (pair) {
+                const f32x16 s = mma_feat_bf16<D>(kr, qb, init);
+                const f32x16 dp = mma_feat_bf16<D>(vr, gb, gneg_b);
+                float ds[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ds[r] = __builtin_amdgcn_exp2f(fmaf(s[r], c2, -lse_b)) * dp[r];
+                bf16x8 dsb[2];
+                pack16(ds, dsb);
+                mma_tile_bf16<D>(kt, dsb, acc_b);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (!last) ++g;
+        }
+#pragma unroll
+        for (int c = 0; c < D / 32; ++c) {
+            acc_a[c] *= scale;
+            acc_b[c] *= scale;
+        }
+        if (part) {
+            store_part<D>(acc_a, part, l);
+        } else {
+            char* Tl = Tw + (g & 1) * DT::BUF;
+            const int so = (int)(bf16_head_bytes<ST, D>(ly.grad, ly.H, bh, L) + (unsigned)(I * 32 * gld * 2));
+            stage_store_bf16<D>(acc_a, Tl, rdQ, vgr, so, gld, l);
+            if (pair) stage_store_bf16<D>(acc_b, Tl + DT::TILE, rdQ, vgr, so + 32 * gld * 2, gld, l);
+        }
+        release();
+        ++g;
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
 // Backward, column pass over the transposed tile index: dK_J = sum_I dS_IJ^T Q_I, dV_J = sum_I P_IJ^T dO_I.
 // Stats: {lse2, -g} of every strip as the row pass left them (64 floats per strip).
 // Stream of an item: {K tile, V tile, key penalties of the column strip}, then per tile {Q tile, dO tile, statistics

@@ -1843,7 +1843,11 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
     // {lse2, -g} of every strip, 64 floats per strip, from the row pass to the column pass
     if (!ensure_ws(&a->ws_rowsum, (size_t)a->NB * a->L * 2)) return;
     if (!ensure_part_ws(a, std::max(std::max(pi.plan_row.slots, pi.plan_col.slots), pi.plan_pair.slots))) return;
-    const Bf16Plan &pr = pi.plan_row, &pc = pi.plan_col;
+    // row pass: two strips per wavefront where the pattern has the pairs (SPION_BF16_ROW_PAIRS=0 keeps one strip)
+    static const bool no_pairs = getenv("SPION_BF16_NO_PAIRS") != nullptr ||
+                                 (getenv("SPION_BF16_ROW_PAIRS") && getenv("SPION_BF16_ROW_PAIRS")[0] == '0');
+    const bool by_pairs = !ST && pi.plan_pair.lanes > 0 && !no_pairs;
+    const Bf16Plan &pr = by_pairs ? pi.plan_pair : pi.plan_row, &pc = pi.plan_col;
     const dim3 grid_r(pr.lanes), grid_c(pc.lanes), block(64);
     const dim3 grid_mr(pr.n_long * a->NB * (32 * a->d / 256)), grid_mc(pc.n_long * a->NB * (2 * 32 * a->d / 256));
     const __bf16 *q = static_cast<const __bf16*>(Q), *k = static_cast<const __bf16*>(K), *v = static_cast<const __bf16*>(V);
@@ -1852,6 +1856,12 @@ static void bf16_backward_impl(SparseAttn* a, const void* Q, const void* K, cons
 #define SPION_LAUNCH(DD, MM)                                                                                          \
     do {                                                                                                              \
         if (a->bwd_passes & 1) {                                                                                      \
+            if (by_pairs)                                                                                             \
+                hipLaunchKernelGGL((bf16_bwd_row_pair_kernel<DD, MM>), grid_r, block, 0, a->hdr.stream, q, k, v, go, \
+                                   o, Lse, Mask, a->ws_rowsum, dq, pi.d_tcol, pr.sched.items, pr.sched.lane_ptr,      \
+                                   pr.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part, pr.slots, ly, in_bytes,      \
+                                   out_bytes, grad_bytes);                                                            \
+            else                                                                                                      \
             hipLaunchKernelGGL((bf16_bwd_row_kernel<DD, MM, ST>), grid_r, block, 0, a->hdr.stream, q, k, v, go, o,    \
                                Lse, Mask, a->ws_rowsum, dq, pi.d_tcol, pr.sched.items, pr.sched.lane_ptr, pr.sched.lane_ent, a->L, a->NB, a->scale, a->ws_part,   \
                                pr.slots, ly, in_bytes, out_bytes, grad_bytes);                                                               \
