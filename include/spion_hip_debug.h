@@ -24,6 +24,19 @@ void spion_set_backward_passes(void* handle, int mask);
  * graph recorded before the growth still points at them).  -1 otherwise. */
 int spion_debug_counter(void* handle, int which);
 
+/* The schedule the bf16 kernels would walk for a tile list (host only: needs no device).  tile_ptr[nstrips + 1]: first
+ * tile of every 32-row (or 32-column) strip; pairs != 0: strips 2p and 2p+1 hold the same tiles and are walked
+ * together; lanes: persistent wavefronts asked for.  Returns the number of lanes the schedule uses (-1 on bad
+ * arguments) and fills, where the arrays are large enough (cap_* in ints):
+ *   items     {strip, first tile, tiles, kind} per item -- kind >= 0: chunk of a long strip, its workspace slot;
+ *             -1: whole strip; -2: the pair (strip, strip + 1);
+ *   lane_ptr  [lanes + 1], lane_ent {head, item} per entry: lane s walks entries lane_ptr[s] .. lane_ptr[s+1]-1;
+ *   longs     {strip, first slot, chunks, tiles} per long strip;
+ *   counts    {ints in items, ints in lane_ent, ints in longs, workspace slots}. */
+int spion_debug_bf16_plan(const int* tile_ptr, int nstrips, int pairs, int num_batches, int lanes, int* items,
+                          int cap_items, int* lane_ptr, int cap_ptr, int* lane_ent, int cap_ent, int* longs,
+                          int cap_longs, int* counts);
+
 /* Environment switches read once per process, for A/B measurements only (results are the same either way):
  *   SPION_NO_FWD_SPLIT   the fp32 tile forward runs all strips in one launch, eight logit tiles per wavefront
  *                        (default: strips of at most 16 tiles in a launch of their own, three work-groups to a CU);

@@ -70,6 +70,7 @@ int sparse_last_path(void*);
 void sparse_force_element(void*, int);
 void sparse_set_bwd_passes(void*, int);
 int sparse_debug_counter(void*, int);
+int sparse_debug_bf16_plan(const int*, int, int, int, int, int*, int, int*, int, int*, int, int*, int, int*);
 void sparse_use_ocache(void*, int);
 void* sparse_bf16_init(int, int, int, int);
 void sparse_bf16_forward(void*, const void*, const void*, const void*, const float*, void*, float*, const int*,
@@ -278,6 +279,12 @@ int spion_last_path(void* h) { return sparse_last_path(h); }
 void spion_force_element_path(void* h, int on) { sparse_force_element(h, on); }
 void spion_set_backward_passes(void* h, int mask) { sparse_set_bwd_passes(h, mask); }
 int spion_debug_counter(void* h, int which) { return sparse_debug_counter(h, which); }
+int spion_debug_bf16_plan(const int* tile_ptr, int nstrips, int pairs, int num_batches, int lanes, int* items,
+                          int cap_items, int* lane_ptr, int cap_ptr, int* lane_ent, int cap_ent, int* longs,
+                          int cap_longs, int* counts) {
+    return sparse_debug_bf16_plan(tile_ptr, nstrips, pairs, num_batches, lanes, items, cap_items, lane_ptr, cap_ptr,
+                                  lane_ent, cap_ent, longs, cap_longs, counts);
+}
 void spion_use_output_cache(void* h, int on) { sparse_use_ocache(h, on); }
 void spion_attn_backward_with_out(void* h, const float* Q, const float* K, const float* Vt, const float* P,
                                   const float* Out, const float* dO, float* dP, float* dS, float* dQ, float* dK,

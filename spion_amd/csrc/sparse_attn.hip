@@ -2055,6 +2055,31 @@ int sparse_last_path(void* h) {
     SparseAttn* a = as_sparse(h, "spion_last_path");
     return a ? a->last_path : 0;
 }
+// The schedule build_bf16_plan makes for a tile list, copied out for inspection (host only: nothing is launched or
+// allocated on a device).  Returns the number of lanes; counts = {ints in items, ints in lane_ent, ints in longs,
+// workspace slots}.  Arrays that are null or too small (cap_* in ints) are left alone.
+int sparse_debug_bf16_plan(const int* ptr, int nstrips, int pairs, int NB, int lanes_wanted, int* items, int cap_items,
+                           int* lane_ptr, int cap_ptr, int* lane_ent, int cap_ent, int* longs, int cap_longs,
+                           int* counts) {
+    if (!ptr || nstrips < 0 || NB <= 0 || lanes_wanted <= 0) return -1;
+    const std::vector<int> p(ptr, ptr + nstrips + 1);
+    const Bf16PlanHost plan = build_bf16_plan(p, nstrips, pairs != 0, NB, lanes_wanted);
+    auto copy = [](const std::vector<int>& v, int* out, int cap) {
+        if (out && (size_t)cap >= v.size()) std::copy(v.begin(), v.end(), out);
+    };
+    copy(plan.items, items, cap_items);
+    copy(plan.lane_ptr, lane_ptr, cap_ptr);
+    copy(plan.lane_ent, lane_ent, cap_ent);
+    copy(plan.longs, longs, cap_longs);
+    if (counts) {
+        counts[0] = (int)plan.items.size();
+        counts[1] = (int)plan.lane_ent.size();
+        counts[2] = (int)plan.longs.size();
+        counts[3] = plan.slots;
+    }
+    return plan.lanes;
+}
+
 int sparse_debug_counter(void* h, int which) {
     SparseAttn* a = as_sparse(h, "spion_debug_counter");
     if (!a) return -1;
