@@ -14,6 +14,18 @@ namespace spion {
 
 typedef float gather_f32x4 __attribute__((ext_vector_type(4)));
 
+// The rows are fetched with buffer loads: a 32-bit byte offset per lane (row * ld + piece, two VALU instructions)
+// instead of a 64-bit address (five), which matters in kernels whose bound is VALU issue.  X: first row of the head
+// (wave-uniform); the rows of a head span less than 2 GiB.
+typedef __amdgpu_buffer_rsrc_t gather_rsrc_t;
+typedef unsigned gather_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ gather_rsrc_t gather_rsrc(const float* X) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(X), 0, 0x7ffffffc, 0x00020000);
+}
+__device__ __forceinline__ gather_f32x4 gather_load16(gather_rsrc_t r, int row, int ld, int piece) {
+    return __builtin_bit_cast(gather_f32x4, __builtin_amdgcn_raw_buffer_load_b128(r, (row * ld + 4 * piece) * 4, 0, 0));
+}
+
 template <int LPR>
 __device__ __forceinline__ int gather_entry_of_lane(int lane) {
     constexpr int G = 64 / LPR;
@@ -43,11 +55,12 @@ __device__ __forceinline__ float gather_dot(const gather_f32x4 a4, const float* 
                                             int nk, int lane) {
     constexpr int G = 64 / LPR;
     const int base = lane & ~(LPR - 1), cl = lane & (LPR - 1);
+    const gather_rsrc_t rx = gather_rsrc(X);
     gather_f32x4 x[LPR];
 #pragma unroll
     for (int j = 0; j < LPR; ++j) {
         const int rr = __shfl(row_l, base + j, 64);
-        if (j * G < nk) x[j] = reinterpret_cast<const gather_f32x4*>(X + (size_t)rr * ld)[cl];
+        if (j * G < nk) x[j] = gather_load16(rx, rr, ld, cl);
     }
     float r = 0.f;
 #pragma unroll
@@ -74,13 +87,14 @@ struct GatherRowAcc {
                                           int lane) {
         constexpr int G = 64 / LPR;
         const int base = lane & ~(LPR - 1), cl = lane & (LPR - 1);
+        const gather_rsrc_t rx = gather_rsrc(X);
         float w[LPR];
         gather_f32x4 x[LPR];
 #pragma unroll
         for (int j = 0; j < LPR; ++j) {
             w[j] = __shfl(w_l, base + j, 64);
             const int rr = __shfl(row_l, base + j, 64);
-            if (j * G < nk) x[j] = reinterpret_cast<const gather_f32x4*>(X + (size_t)rr * ld)[cl];
+            if (j * G < nk) x[j] = gather_load16(rx, rr, ld, cl);
         }
 #pragma unroll
         for (int j = 0; j < LPR; ++j)
