@@ -33,7 +33,6 @@ namespace spion {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr float BF16_LAZY = 8.f;  // the running row maximum is raised only when a tile exceeds it by 2^8
@@ -91,28 +90,6 @@ __device__ __forceinline__ void pack16(const float (&p)[16], bf16x8 (&pb)[2]) {
 // return in order, and the compiler's own counts can only wait longer than needed) and order them against their
 // LDS reads with wait_lgkm0; both carry a memory clobber, so no LDS access moves across them.
 // -------------------------------------------------------------------------------------------------
-__device__ __forceinline__ u32x4 rsrc_words(const void* p, size_t bytes) {
-    const unsigned long long a = reinterpret_cast<unsigned long long>(p);
-    u32x4 r;
-    r.x = (unsigned)a;
-    r.y = (unsigned)(a >> 32);  // stride 0, no swizzle
-    r.z = bytes > 0xfffffff0ull ? 0xfffffff0u : (unsigned)bytes;
-    r.w = 0x00020000u;
-    // wave-uniform by construction; keep it in scalar registers
-    r.x = __builtin_amdgcn_readfirstlane(r.x);
-    r.y = __builtin_amdgcn_readfirstlane(r.y);
-    r.z = __builtin_amdgcn_readfirstlane(r.z);
-    return r;
-}
-__device__ __forceinline__ unsigned lds_address(const void* p) {
-    typedef __attribute__((address_space(3))) const char* lds_ptr;
-    return __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<unsigned long long>((lds_ptr)p));
-}
-template <int N>
-__device__ __forceinline__ void wait_vm() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // An empty use of operand registers.  The compiler waits for the loads that fill them before this point -- else it
 // puts that wait at their first use inside the tile loop, as vmcnt(0), where it would also wait, on every
 // iteration, for the tile loads just issued (which it does not know of).
@@ -121,14 +98,6 @@ __device__ __forceinline__ void settle(const bf16x8 (&x)[N]) {
 #pragma unroll
     for (int t = 0; t < N; ++t) asm volatile("" ::"v"(x[t]));
 }
-__device__ __forceinline__ void settle(float x) { asm volatile("" ::"v"(x)); }
-// 64 floats (lane l: 4 bytes at voff) to 256 bytes of LDS
-__device__ __forceinline__ void dma_b32(u32x4 r, unsigned lds, int voff, int soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds), "v"(voff), "s"(r),
-                 "s"(soff)
-                 : "memory");
-}
-
 template <int D>
 struct DmaTile {
     static constexpr int ROW = D * 2;     // bytes per LDS row

@@ -1190,6 +1190,14 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     // forward 0.1756 -> 0.1721 ms; six wavefronts of four tiles for the long strips instead: 44 against 36 us)
     static const bool no_split = getenv("SPION_NO_FWD_SPLIT") != nullptr;
     if constexpr (D == 32) {
+        // longest strip of 17 to 24 tiles: six logit tiles per wavefront still fit three work-groups to a CU (161
+        // registers), so one launch takes every strip (north star: forward 0.171 -> 0.166 ms against the split)
+        if (wv == 4 && pi.max_row_tiles <= 24 && pi.max_row_tiles > 16) {
+            hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 6, KROW, ST>), dim3(nbr * a->NB), dim3(256), 0, a->hdr.stream,
+                               Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, 0, nbr,
+                               hc, ly);
+            return;
+        }
         if (wv == 4 && !no_split && pi.max_row_tiles <= 4 * MAXT && pi.n_fwd_long < nbr && pi.max_row_tiles > 16) {
             const int nl = pi.n_fwd_long;
             if (nl > 0)

@@ -14,10 +14,12 @@
 //     pieces per instruction), is read and written with one full 128-byte row per half-wave instead and
 //     transposed through a wave-private LDS tile; LDS instructions do not compete with the MFMAs either;
 //   * software-pipeline each wavefront's tile list (operands of the next tile are requested before the
-//     current MFMA chain starts).  Loads are never issued under a branch between a load and its use: the
+//     current MFMA chain starts).  d = 32: the tiles go from global memory straight into wave-private LDS
+//     (DmaTileF32 below), so nothing but LDS holds a tile in flight.  d = 64 loads into registers
+//     (tile_pipeline): there loads are never issued under a branch between a load and its use -- the
 //     compiler's s_waitcnt insertion merges conditional paths conservatively and would otherwise wait for
-//     the loads just issued.  When there is no next tile the current one is simply requested again.
-//     A wavefront's tiles are processed in pairs inside the loop (two register sets, no copies) and an odd
+//     the loads just issued; when there is no next tile the current one is simply requested again, and a
+//     wavefront's tiles are processed in pairs inside the loop (two register sets, no copies) with an odd
 //     last tile after it: a prefetch whose only consumer sits in a conditional block would be sunk into
 //     that block by the compiler, next to its use.
 #pragma once
@@ -212,6 +214,147 @@ __device__ __forceinline__ void lds_get_featcols32(const float* T, int li, int h
     for (int s = 0; s < 16; ++s) x[s] = T[(16 * h + s) * TS + li];
 }
 
+// -------------------------------------------------------------------------------------------------
+// 32 x 32 fp32 tiles that go from global memory straight into LDS (buffer loads with the LDS modifier): no
+// registers hold a tile in flight, no ds_write is spent on it, and the path delivers about twice the bytes per
+// clock of loads into registers.  One instruction moves 64 x 16 bytes to 1 KB of consecutive LDS addresses starting
+// at M0 (+ the instruction's immediate offset, which is added to the global address as well): eight 128-byte tile
+// rows.  Which 16-byte piece of a row a lane fetches is free, so the LDS image is unpadded rows with the pieces of
+// row r permuted: piece c lies at position c ^ (r % 8).  Every read the kernels make of such a tile is then free of
+// bank conflicts: a lane's own row in 16-byte pieces (eight consecutive rows of one piece land in eight different
+// positions) and one column of a given row across a half-wave (the 32 floats of a row, in some order).
+// The loads are inline assembly: the compiler neither counts them in its s_waitcnt bookkeeping nor knows that they
+// write LDS.  The kernels wait for them with wait_vm<N> (N = loads issued after the ones waited for; loads return
+// in order, and the compiler's own counts can then only wait longer than needed) and finish their LDS reads with
+// wait_lgkm0 before a tile's space is requested again; both carry a memory clobber, so no LDS access moves across.
+// Scalar operands of the assembly come from scalar loads and SALU arithmetic only (a scalar register written by a
+// vector instruction needs wait states before a memory instruction reads it, which the compiler cannot add here).
+// -------------------------------------------------------------------------------------------------
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ u32x4 rsrc_words(const void* p, size_t bytes) {
+    const unsigned long long a = reinterpret_cast<unsigned long long>(p);
+    u32x4 r;
+    r.x = (unsigned)a;
+    r.y = (unsigned)(a >> 32);  // stride 0, no swizzle
+    r.z = bytes > 0xfffffff0ull ? 0xfffffff0u : (unsigned)bytes;
+    r.w = 0x00020000u;
+    // wave-uniform by construction; keep it in scalar registers
+    r.x = __builtin_amdgcn_readfirstlane(r.x);
+    r.y = __builtin_amdgcn_readfirstlane(r.y);
+    r.z = __builtin_amdgcn_readfirstlane(r.z);
+    return r;
+}
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    typedef __attribute__((address_space(3))) const char* lds_ptr;
+    return __builtin_amdgcn_readfirstlane((unsigned)reinterpret_cast<unsigned long long>((lds_ptr)p));
+}
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// n = 0, 4, 8 or 12 operations may stay outstanding
+__device__ __forceinline__ void wait_vm_upto(int n) {
+    if (n >= 12) wait_vm<12>();
+    else if (n >= 8) wait_vm<8>();
+    else if (n >= 4) wait_vm<4>();
+    else wait_vm<0>();
+}
+__device__ __forceinline__ void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// An empty use of registers.  The compiler waits for the loads that fill them before this point -- else it puts that
+// wait at their first use inside a tile loop, as vmcnt(0), where it would also wait, on every iteration, for the
+// tile loads just issued (which it does not know of).
+__device__ __forceinline__ void settle(float x) { asm volatile("" ::"v"(x)); }
+template <int N>
+__device__ __forceinline__ void settle(const float (&x)[N]) {
+#pragma unroll
+    for (int t = 0; t < N; ++t) asm volatile("" ::"v"(x[t]));
+}
+// 64 floats (lane l: 4 bytes at voff) to 256 bytes of LDS
+__device__ __forceinline__ void dma_b32(u32x4 r, unsigned lds, int voff, int soff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds), "v"(voff), "s"(r),
+                 "s"(soff)
+                 : "memory");
+}
+struct DmaTileF32 {
+    static constexpr int TILE = 4096;  // bytes
+    // Lane offset (bytes) into an array whose rows are `ld` floats apart: lane l fills position l % 8 of row l / 8
+    // (+ 8 rows per instruction) with the piece that belongs there.
+    __device__ static __forceinline__ int voff(int l, int ld) { return ((l >> 3) * ld + 4 * ((l & 7) ^ (l >> 3))) * 4; }
+    // what the scalar offset advances by from one instruction to the next, beyond the 1024 its immediate adds
+    __device__ static __forceinline__ int extra_step(int ld) { return 32 * ld - 1024; }
+    template <bool NT = false>
+    __device__ static __forceinline__ void load(u32x4 r, unsigned lds, int lvoff, int soff, int xstep) {
+        if constexpr (NT)
+            asm volatile(
+                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "buffer_load_dwordx4 %1, %2, %3 offen nt lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 nt lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 nt lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %6 offen offset:3072 nt lds" ::"s"(lds),
+                "v"(lvoff), "s"(r), "s"(soff), "s"(soff + xstep), "s"(soff + 2 * xstep), "s"(soff + 3 * xstep)
+                : "memory");
+        else
+            asm volatile(
+                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 lds\n\t"
+                "buffer_load_dwordx4 %1, %2, %6 offen offset:3072 lds" ::"s"(lds),
+                "v"(lvoff), "s"(r), "s"(soff), "s"(soff + xstep), "s"(soff + 2 * xstep), "s"(soff + 3 * xstep)
+                : "memory");
+    }
+    // Lane (li, h)'s pieces of its own row li: piece p0 + pstep*g, g = 0..3 (four 16-byte reads).
+    struct Own {
+        const char* a[4];
+    };
+    __device__ static __forceinline__ Own own_addr(const char* T, int li, int p0, int pstep) {
+        Own x;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) x.a[g] = T + li * 128 + 16 * ((p0 + pstep * g) ^ (li & 7));
+        return x;
+    }
+    // (`off`: byte distance of the tile from the one the addresses were made for)
+    __device__ static __forceinline__ void get(const Own& o, float (&x)[16], int off = 0) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(o.a[g] + off);
+            x[4 * g + 0] = v.x;
+            x[4 * g + 1] = v.y;
+            x[4 * g + 2] = v.z;
+            x[4 * g + 3] = v.w;
+        }
+    }
+    // Column li of the rows acc_row(q, h) = 8(q/4) + 4h + q%4, q = 0..15 (the tile in col-owner layout): one
+    // address per q%4, the q/4 step is an immediate (rows 8 apart share their permutation).
+    struct Cols {
+        const char* a[4];
+    };
+    __device__ static __forceinline__ Cols cols_addr(const char* T, int li, int h) {
+        Cols x;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) x.a[b] = T + (4 * h + b) * 128 + 16 * ((li >> 2) ^ (4 * h + b)) + 4 * (li & 3);
+        return x;
+    }
+    __device__ static __forceinline__ void get(const Cols& c, float (&x)[16], int off = 0) {
+#pragma unroll
+        for (int q = 0; q < 16; ++q) x[q] = *reinterpret_cast<const float*>(c.a[q & 3] + 1024 * (q >> 2) + off);
+    }
+    // Column li of the rows 16h + s, s = 0..15 (operand over 32 features from a feature-major tile).
+    struct FeatCols {
+        const char* a[8];
+    };
+    __device__ static __forceinline__ FeatCols featcols_addr(const char* T, int li, int h) {
+        FeatCols x;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) x.a[j] = T + (16 * h + j) * 128 + 16 * ((li >> 2) ^ j) + 4 * (li & 3);
+        return x;
+    }
+    __device__ static __forceinline__ void get(const FeatCols& c, float (&x)[16], int off = 0) {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[s] = *reinterpret_cast<const float*>(c.a[s & 7] + 1024 * (s >> 3) + off);
+    }
+};
+
 // acc = init + A.B over the head dimension (chain of D/2 MFMA).
 template <int D>
 __device__ __forceinline__ f32x16 mma_feat_init(const float (&a)[D / 2], const float (&b)[D / 2], f32x16 init) {
@@ -344,10 +487,10 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // reference's ABI asks for) instead of feature-major [NB][D][L].  For d = 64 every lane then reads 128 bytes of
 // its own row (one cache line per lane), which is slower than the feature-major form: the row-major entry points
 // for contiguous heads therefore still transpose once; only the strided entry points use it.
-// MAXT == 4 at d = 32 (at most four logit tiles per wavefront) fits three wavefronts per SIMD: the buffer of the
+// MAXT <= 6 at d = 32 (at most six logit tiles per wavefront) fits three wavefronts per SIMD: the buffer of the
 // final reduction then shares the space of the wave-private tiles (a barrier in between).
 template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(D == 32 && MAXT == 4 ? 3 : 2, D == 32 && MAXT == 4 ? 3 : 2)))
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(D == 32 && MAXT > 0 && MAXT <= 6 ? 3 : 2, D == 32 && MAXT > 0 && MAXT <= 6 ? 3 : 2)))
 void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
@@ -355,11 +498,14 @@ void tile_fwd_kernel(
     int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
     static_assert(!ST || KROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
-    constexpr bool SHARE = D == 32 && MAXT == 4 && WAVES > 1;  // reduction buffer inside the tile space
+    constexpr bool SHARE = D == 32 && MAXT > 0 && MAXT <= 6 && WAVES > 1;  // reduction buffer inside the tile space
     __shared__ float lds_own[!SHARE && WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 && MAXT > 0 ? 2 : 1) * 32 * TS];
-    static_assert(!SHARE || WAVES * 2 * 32 * TS >= WAVES * 16 * 64, "the reduction fits in the tile space");
+    // per wavefront: one padded tile (layout changes of P) and, d = 32 with the logits in registers, two 4 KB
+    // tiles filled straight from global memory
+    constexpr int TW = 32 * TS + (D == 32 && MAXT > 0 ? 2 * 1024 + (MASK ? 128 : 0) : 0);
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][TW];
+    static_assert(!SHARE || WAVES * TW >= WAVES * 16 * 64, "the reduction fits in the tile space");
     float* lds = SHARE ? &lds_t[0][0] : lds_own;
     // this launch covers strips s0 .. s0+ns-1 of the longest-first order of every head
     const int item = xcd_remap(blockIdx.x, ns * NB);
@@ -428,24 +574,57 @@ void tile_fwd_kernel(
         // in wave-private LDS tiles: a quarter of the vector-memory instructions, which keeps the wavefront
         // clear of the 63 outstanding instructions it may have (loads and stores share that counter).
         constexpr bool LIN = D == 32;
-        float* Tx = T + 32 * TS;  // K^T tile, later V tile (LIN only)
+        // d = 32: K^T and V tiles go straight into two wave-private LDS tiles, alternately (tile u + 1 is requested
+        // before the chain of tile u starts); P tiles leave as four 16-byte instructions after a layout change
+        // in the padded tile.  Loads into LDS and the P stores share one in-order counter (wait_vm).
+        const char* Tb = reinterpret_cast<const char*>(T + 32 * TS);
+        const unsigned lb = LIN ? lds_address(Tb) : 0;
         // a K tile is 32 features x 32 keys with rows L floats apart, or (KROW) 32 keys x 32 features, contiguous
         const int KSTEP = KROW ? 32 * ild * 4 : 128;
         const int kld = KROW ? ild : L;
-        const int klin = lin_voff(l, kld), vlin = lin_voff(l, ild), plin = lin_voff(l, rn);
+        const int plin = lin_voff(l, rn);
         if constexpr (LIN) {
-            f32x4 kraw[2][4];
-            if (nu > 0) ldr_tile_lin(rK, klin, Js[0] * KSTEP, kld, kraw[0]);
+            const u32x4 wK = rsrc_words(Kt + ib, hbytes);
+            const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+            const int kl = DmaTileF32::voff(l, kld), kx = DmaTileF32::extra_step(kld);
+            const auto a_k0 = [&] {
+                if constexpr (KROW) return DmaTileF32::own_addr(Tb, li, 4 * h, 1);
+                else return DmaTileF32::featcols_addr(Tb, li, h);
+            }();
+            // the key penalties of a tile travel with it (64 floats, of which the first 32 are the tile's)
+            const char* Tm = Tb + 2 * DmaTileF32::TILE + 16 * h;
+            constexpr int KOPS = MASK ? 5 : 4;
+            auto issue_k = [&](int u) {
+                DmaTileF32::load(wK, lb + (u & 1) * DmaTileF32::TILE, kl, Js[u] * KSTEP, kx);
+                if constexpr (MASK) dma_b32(wM, lb + 2 * DmaTileF32::TILE + (u & 1) * 256, l * 4, Js[u] * 128);
+            };
+            asm volatile("s_nop 4");  // the resource words come out of vector instructions
+            if (nu > 0) issue_k(0);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
-                    if (u + 1 < MAXT) ldr_tile_lin(rK, klin, Js[u + 1 < MAXT ? u + 1 : u] * KSTEP, kld, kraw[(u + 1) & 1]);
-                    lds_put_lin(Tx, l, kraw[u & 1]);
+                    if (u + 1 < MAXT && u + 1 < nu) {
+                        issue_k(u + 1 < MAXT ? u + 1 : u);
+                        wait_vm<KOPS>();
+                    } else {
+                        wait_vm<0>();
+                    }
                     float kf[KH];
-                    if constexpr (KROW) lds_get_feat32(Tx, li, h, kf);
-                    else lds_get_featcols32(Tx, li, h, kf);
+                    DmaTileF32::get(a_k0, kf, (u & 1) * DmaTileF32::TILE);
+                    f32x16 init = splat16(0.f);
+                    if constexpr (MASK) {  // minus the key penalties, in the log2 domain
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const f32x4 v = *reinterpret_cast<const f32x4*>(Tm + (u & 1) * 256 + 32 * g);
+                            init[4 * g + 0] = -LOG2E * v.x;
+                            init[4 * g + 1] = -LOG2E * v.y;
+                            init[4 * g + 2] = -LOG2E * v.z;
+                            init[4 * g + 3] = -LOG2E * v.w;
+                        }
+                    }
+                    wait_lgkm0();  // the tile's space is requested again one iteration on
                     __builtin_amdgcn_sched_barrier(0);
-                    S[u] = mma_feat_init<D>(kf, q, chain_init(Js[u]));
+                    S[u] = mma_feat_init<D>(kf, q, init);
                     m = max16(S[u], m);
                 }
             }
@@ -498,21 +677,33 @@ void tile_fwd_kernel(
         const float rinv = __builtin_amdgcn_exp2f(m_own - m) * (1.0f / z);
 
         if constexpr (LIN) {
-            f32x4 vraw[2][4];
-            if (nu > 0) ldr_tile_lin(rV, vlin, Js[0] * 32 * ild * 4, ild, vraw[0]);
+            // V tiles the same way: request u + 2 goes out when tile u has been read.  What was issued after the
+            // loads of tile u when its turn comes: the loads of tile u + 1 (if any), and the P stores of the one
+            // or two tiles before it.
+            const u32x4 wV = rsrc_words(V + ib, hbytes);
+            const int vl = DmaTileF32::voff(l, ild), vx = DmaTileF32::extra_step(ild);
+            const auto a_v0 = DmaTileF32::cols_addr(Tb, li, h);
+            auto issue_v = [&](int u) {
+                DmaTileF32::load(wV, lb + (u & 1) * DmaTileF32::TILE, vl, Js[u] * 32 * ild * 4, vx);
+            };
+            asm volatile("s_nop 4");
+            if (nu > 0) issue_v(0);
+            if (MAXT > 1 && nu > 1) issue_v(1 < MAXT ? 1 : 0);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
                     const int t = w + u * WAVES;
-                    if (u + 1 < MAXT) ldr_tile_lin(rV, vlin, Js[u + 1 < MAXT ? u + 1 : u] * 32 * ild * 4, ild, vraw[(u + 1) & 1]);
-                    lds_put_lin(Tx, l, vraw[u & 1]);
+                    const int stores = u == 0 ? 0 : u == 1 ? 4 : 8;  // P stores issued after V tile u was requested
+                    wait_vm_upto(stores + (u + 1 < MAXT && u + 1 < nu ? 4 : 0));
                     float p[16], vb[1][16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
                     lds_put_rows(T, li, h, p);
-                    lds_get_cols(Tx, li, h, vb[0]);
+                    DmaTileF32::get(a_v0, vb[0], (u & 1) * DmaTileF32::TILE);
                     f32x4 pl[4];
                     lds_get_lin(T, l, pl);
+                    wait_lgkm0();
+                    if (u + 2 < MAXT && u + 2 < nu) issue_v(u + 2 < MAXT ? u + 2 : u);
                     __builtin_amdgcn_sched_barrier(0);
                     mma_b<D>(p, vb, o);
                     str_tile_lin(rP, plin, p_base + t * 128, rn, pl);
@@ -615,7 +806,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_g[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][(D == 32 ? 3 : 1) * 32 * TS];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][D == 32 ? 3 * 1024 : 32 * TS];
     // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     int bh, pos;
@@ -692,46 +883,52 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] = splat16(0.f);
     if constexpr (D == 32) {
-        // One tile ahead: the V^T tile, the P tile and the K tile, each fetched linearly (12 instructions a
-        // tile instead of 48) and turned into operands through wave-private LDS copies.
-        struct Pre {
-            f32x4 vt[4], pv[4], kb[4];
-        };
-        float* Tv = T;
-        float* Tp = T + 32 * TS;
-        float* Tk = T + 64 * TS;
+        // The V^T, P and K tiles of a tile go straight into wave-private LDS (twelve instructions, no registers in
+        // flight); the operands of tile i are read out of LDS into registers, then the same space is requested for
+        // tile i + 1, whose loads have the two chains of tile i to arrive.
+        const char* Tv = reinterpret_cast<const char*>(T);
+        const char* Tp = Tv + DmaTileF32::TILE;
+        const char* Tk = Tv + 2 * DmaTileF32::TILE;
+        const unsigned lv = lds_address(Tv), lp = lv + DmaTileF32::TILE, lk = lv + 2 * DmaTileF32::TILE;
+        const u32x4 wV = rsrc_words(Vt + ib, hbytes), wK = rsrc_words(K + ib, hbytes);
+        const u32x4 wP = rsrc_words(P + (size_t)bh * nnz, (size_t)nnz * 4);
         const int VSTEP = VROW ? 32 * ild * 4 : 128;
         const int vld = VROW ? ild : L;
-        const int vl = lin_voff(l, vld), pl = lin_voff(l, rn), kl = lin_voff(l, ild);
-        Pre xa, xb;
-        tile_pipeline(
-            nu, xa, xb,
-            [&](Pre& x, int i) {
-                const int t = w + min(i, nu - 1) * WAVES;
-                const int J = tcol[t0 + t];
-                ldr_tile_lin(rV, vl, J * VSTEP, vld, x.vt);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) x.pv[i] = ld4_nt(rP, pl, p_base + t * 128 + 32 * i * rn);
-                ldr_tile_lin(rK, kl, J * 32 * ild * 4, ild, x.kb);
-            },
-            [&](Pre& c, int) {
-                lds_put_lin(Tv, l, c.vt);
-                lds_put_lin(Tp, l, c.pv);
-                lds_put_lin(Tk, l, c.kb);
-                // every LDS read is issued before the first chain starts (left to itself the compiler sinks
-                // each read next to the MFMA that uses it and waits for it there)
+        const int vl = DmaTileF32::voff(l, vld), pl = DmaTileF32::voff(l, rn), kl = DmaTileF32::voff(l, ild);
+        const int vx = DmaTileF32::extra_step(vld), px = DmaTileF32::extra_step(rn), kx = DmaTileF32::extra_step(ild);
+        const auto a_v = [&] {
+            if constexpr (VROW) return DmaTileF32::own_addr(Tv, li, 4 * h, 1);
+            else return DmaTileF32::featcols_addr(Tv, li, h);
+        }();
+        const auto a_p = DmaTileF32::own_addr(Tp, li, h, 2);
+        const auto a_k = DmaTileF32::cols_addr(Tk, li, h);
+        auto issue = [&](int t, int J) {
+            DmaTileF32::load(wV, lv, vl, J * VSTEP, vx);
+            DmaTileF32::load<true>(wP, lp, pl, p_base + t * 128, px);
+            DmaTileF32::load(wK, lk, kl, J * 32 * ild * 4, kx);
+        };
+        if (nu > 0) {
+            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+            issue(w, tcol[t0 + w]);
+            int Jn = tcol[t0 + w + (nu > 1 ? WAVES : 0)];
+            for (int i = 0; i < nu; ++i) {
+                const int Jnn = tcol[t0 + w + min(i + 2, nu - 1) * WAVES];  // index of the tile after the next
+                wait_vm<0>();
                 float vt[16], pr[16], kb[1][16];
-                if constexpr (VROW) lds_get_feat32(Tv, li, h, vt);
-                else lds_get_featcols32(Tv, li, h, vt);
-                lds_get_rows(Tp, li, h, pr);
-                lds_get_cols(Tk, li, h, kb[0]);
+                DmaTileF32::get(a_v, vt);
+                DmaTileF32::get(a_p, pr);
+                DmaTileF32::get(a_k, kb[0]);
+                wait_lgkm0();
+                if (i + 1 < nu) issue(w + (i + 1) * WAVES, Jn);
+                Jn = Jnn;
                 __builtin_amdgcn_sched_barrier(0);
                 f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
                 mma_b<D>(ds, kb, acc);
-            });
+            }
+        }
     } else {
         // One tile ahead: V^T operand, P tile and (d = 32) the K operand of the second product; for d = 64
         // that operand would not fit in registers and is requested when the tile's first chain starts.
@@ -788,7 +985,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     static_assert(!ST || VROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
     __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][D == 32 ? 3 * 1024 + 64 : 4];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     int bh, pos;
     item_to_head_strip(item, nbr, hc, bh, pos);
@@ -818,67 +1015,106 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     }
     // Per tile of the transposed index: {block row I, offset of the tile in this head's P, row stride}.
     const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
-    // One tile ahead: P tile, -g and, for d = 32, the Q and dO operands of the second products; the dO tile
-    // is then loaded once (one full row per half-wave) and its other layout, the A operand of the dP chain,
-    // comes out of a wave-private LDS transpose.  For d = 64 the operands of the second products would not
-    // fit in registers: they are requested when the tile's first chain starts and the dO rows separately.
-    constexpr bool DEEP = D == 32;
-    float* T = lds_t[w];
-    struct Pre {
-        float go[DEEP ? 1 : KH];
-        float p[16];
-        float gneg[16];
-        float qb[DEEP ? D / 32 : 1][16];
-        float ob[DEEP ? D / 32 : 1][16];
-        int I;
-    };
     const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int4 d = desc[w + min(i, nu - 1) * WAVES];
+    float* T = lds_t[w];
+    if constexpr (D == 32) {
+        // The P, Q and dO tiles and the 32 values of -g go straight into wave-private LDS (thirteen instructions, no
+        // registers in flight); the operands of tile i are read out of LDS into registers -- the dO tile in both
+        // of its roles -- then the same space is requested for tile i + 1, whose loads have the three chains of
+        // tile i to arrive.
+        const char* Tp = reinterpret_cast<const char*>(T);
+        const char* Tq = Tp + DmaTileF32::TILE;
+        const char* To = Tp + 2 * DmaTileF32::TILE;
+        const char* Tg = Tp + 3 * DmaTileF32::TILE;
+        const unsigned lp = lds_address(Tp), lq = lp + DmaTileF32::TILE, lo = lp + 2 * DmaTileF32::TILE,
+                       lg = lp + 3 * DmaTileF32::TILE;
+        const u32x4 wQ = rsrc_words(Q + ib, hbytes), wO = rsrc_words(dO + ob, obytes);
+        const u32x4 wP = rsrc_words(P + (size_t)bh * nnz, (size_t)nnz * 4), wG = rsrc_words(G + (size_t)bh * L, (size_t)L * 4);
+        const int ql = DmaTileF32::voff(l, ild), ol = DmaTileF32::voff(l, old_);
+        const int qx = DmaTileF32::extra_step(ild), ox = DmaTileF32::extra_step(old_);
+        const int pl0 = 16 * ((l & 7) ^ (l >> 3)), pl1 = (l >> 3) * 4;  // lane offset into a P tile: pl0 + pl1 * row stride
+        const auto a_p = DmaTileF32::cols_addr(Tp, li, h), a_q = DmaTileF32::cols_addr(Tq, li, h),
+                   a_o = DmaTileF32::cols_addr(To, li, h);
+        const auto a_go = DmaTileF32::own_addr(To, li, 4 * h, 1);
+        const char* a_g = Tg + 16 * h;
+        auto issue = [&](const int4 d) {
             const int I = d.x, rn = d.z;
-            x.I = I;
-            if constexpr (!DEEP) ldr_rows<D>(rdO, ro_voff, I * 32 * old_ * 4, x.go);
-            const int pv = (4 * h * rn + li) * 4;
+            DmaTileF32::load<true>(wP, lp, pl0 + pl1 * rn, d.y * 4, DmaTileF32::extra_step(rn));
+            DmaTileF32::load(wQ, lq, ql, I * 32 * ild * 4, qx);
+            DmaTileF32::load(wO, lo, ol, I * 32 * old_ * 4, ox);
+            dma_b32(wG, lg, l * 4, I * 128);
+        };
+        settle(vt);
+        if (nu > 0) {
+            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+            issue(desc[w]);
+            int4 dn = desc[w + (nu > 1 ? WAVES : 0)];
+            for (int i = 0; i < nu; ++i) {
+                const int4 dnn = desc[w + min(i + 2, nu - 1) * WAVES];  // descriptor of the tile after the next
+                wait_vm<0>();
+                float pc[16], qb[1][16], ob[1][16], go[KH];
+                f32x16 init;
+                DmaTileF32::get(a_o, ob[0]);
+                DmaTileF32::get(a_go, go);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) x.p[r] = ld1_nt(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
-            ldr_4x4(rG, 16 * h, I * 128, x.gneg);
-            if constexpr (DEEP) {
-                ldr_tile_b<D>(rQ, b_voff, I * 32 * ild * 4, x.qb, ild);
-                ldr_tile_b<D>(rdO, bo_voff, I * 32 * old_ * 4, x.ob, old_);
+                for (int g = 0; g < 4; ++g) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(a_g + 32 * g);
+                    init[4 * g + 0] = v.x;
+                    init[4 * g + 1] = v.y;
+                    init[4 * g + 2] = v.z;
+                    init[4 * g + 3] = v.w;
+                }
+                DmaTileF32::get(a_p, pc);
+                DmaTileF32::get(a_q, qb[0]);
+                wait_lgkm0();
+                if (i + 1 < nu) issue(dn);
+                dn = dnn;
+                __builtin_amdgcn_sched_barrier(0);
+                f32x16 dp = mma_feat_init<D>(go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+                float ds[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pc[r];
+                mma_b<D>(ds, qb, ak);
+                mma_b<D>(pc, ob, av);
             }
-        },
-        [&](Pre& c, int) {
-            float qb2[D / 32][16], ob2[D / 32][16];
-            if constexpr (!DEEP) {
+        }
+    } else {
+        // One tile ahead: the dO rows, the P tile and -g; the operands of the second products would not fit in
+        // registers beside them and are requested when the tile's first chain starts.
+        struct Pre {
+            float go[KH];
+            float p[16];
+            float gneg[16];
+            int I;
+        };
+        Pre xa, xb;
+        tile_pipeline(
+            nu, xa, xb,
+            [&](Pre& x, int i) {
+                const int4 d = desc[w + min(i, nu - 1) * WAVES];
+                const int I = d.x, rn = d.z;
+                x.I = I;
+                ldr_rows<D>(rdO, ro_voff, I * 32 * old_ * 4, x.go);
+                const int pv = (4 * h * rn + li) * 4;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) x.p[r] = ld1_nt(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
+                ldr_4x4(rG, 16 * h, I * 128, x.gneg);
+            },
+            [&](Pre& c, int) {
+                float qb2[D / 32][16], ob2[D / 32][16];
                 ldr_tile_b<D>(rQ, b_voff, c.I * 32 * ild * 4, qb2, ild);
                 ldr_tile_b<D>(rdO, bo_voff, c.I * 32 * old_ * 4, ob2, old_);
-            }
-            f32x16 init;
+                f32x16 init;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
-            f32x16 dp;  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
-            if constexpr (DEEP) {
-                float go[KH];
-                lds_put_cols(T, li, h, c.ob[0]);
-                lds_get_feat32(T, li, h, go);
-                dp = mma_feat_init<D>(go, vt, init);
-            } else {
-                dp = mma_feat_init<D>(c.go, vt, init);
-            }
-            float ds[16];
+                for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
+                f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+                float ds[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
-            if constexpr (DEEP) {
-                mma_b<D>(ds, c.qb, ak);
-                mma_b<D>(c.p, c.ob, av);
-            } else {
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
                 mma_b<D>(ds, qb2, ak);
                 mma_b<D>(c.p, ob2, av);
-            }
-        });
+            });
+    }
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
     reduce_store<D, WAVES>(ak, dK + gb, J * 32, w, li, h, lds, gld);
