@@ -102,8 +102,8 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
 // Forward for d = 32 and L <= 1024 (at most 32 key tiles per query strip): the register-resident scheme of the
 // sparse forward (tile_kernels.h) on the dense layouts.  Each of the four wavefronts keeps the logit tiles of its
 // share of the strip (at most 8) in registers, so a tile costs one QK^T chain and one PV chain instead of the
-// two-sweep kernel's three; K, V^T and map tiles move as four 16-byte instructions each and change layout in
-// wave-private LDS tiles; the map is written non-temporally.
+// two-sweep kernel's three; K and V tiles go from global memory straight into wave-private LDS tiles, map tiles
+// change layout in a padded LDS tile and leave as four 16-byte instructions, non-temporally.
 // RM: Q, V and Out are row-major head slices located by `ly` (heads possibly interleaved in [B][L][H*32] memory,
 // tile_kernels.h) instead of the feature-major [NB][32][L] operands of the reference's ABI; K likewise.
 // MEAN (row-major operands, eight wavefronts with at most four logit tiles each): the launch also accumulates the
@@ -120,13 +120,16 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     constexpr int D = 32, KH = 16, MAXT = 32 / WAVES;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][2 * 32 * TS];
+    // per wavefront: one padded tile (the map tile on its way to memory), two 4 KB tiles filled straight from global
+    // memory and the key penalties that travel with them
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS + 2 * 1024 + (MASK ? 128 : 0)];
     const int item = xcd_remap(blockIdx.x, nbr * (MEAN ? C : NB));
     const int bh0 = item / nbr, I = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w + WAVES, ... of this wavefront
-    float* T = lds_t[w];         // map tile on its way to memory
-    float* Tx = T + 32 * TS;     // K tile, later V^T tile
+    float* T = lds_t[w];  // map tile on its way to memory
+    const char* Tb = reinterpret_cast<const char*>(T + 32 * TS);  // K tiles, later V tiles, alternately in two places
+    const unsigned lb = lds_address(Tb);
     f32x16 total[MEAN ? MAXT : 1];
     if constexpr (MEAN) {
 #pragma unroll
@@ -141,11 +144,14 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     int ild, old_;
     head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
     head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
-    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rK = make_rsrc(K + ib, hbytes), rV = make_rsrc(Vt + ib, hbytes);
+    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes);
     const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
-    const rsrc_t rM = make_rsrc(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
-    const int klin = lin_voff(l, ild), alin = lin_voff(l, L);
-    const int vld = RM ? ild : L, vlin = lin_voff(l, vld), VSTEP = RM ? 32 * ild * 4 : 128;
+    const u32x4 wK = rsrc_words(K + ib, hbytes), wV = rsrc_words(Vt + ib, hbytes);
+    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int alin = lin_voff(l, L);
+    const int vld = RM ? ild : L, VSTEP = RM ? 32 * ild * 4 : 128;
+    const int kl = DmaTileF32::voff(l, ild), kx = DmaTileF32::extra_step(ild);
+    const int vl = DmaTileF32::voff(l, vld), vx = DmaTileF32::extra_step(vld);
     const float c2 = scale * LOG2E;
 
     float q[KH];
@@ -153,34 +159,47 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     else ldr_cols<D>(rQ, L, (h * KH * L + li) * 4, I * 128, q);
 #pragma unroll
     for (int s = 0; s < KH; ++s) q[s] *= c2;
-    auto chain_init = [&](int J) -> f32x16 {  // minus the key penalties of the tile, log2 domain
-        if (!MASK) return splat16(0.f);
-        float pj[16];
-        ldr_4x4(rM, 16 * h, J * 128, pj);
-        f32x16 v;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) v[r] = -LOG2E * pj[r];
-        return v;
-    };
 
     float m = -10.f * LOG2E, z = 0.f;  // models/attn.cu:17
     f32x16 S[MAXT];
     {
-        // PRE: the next tile is requested while one is worked on (the mean-emitting form has no registers for that)
-        constexpr int PRE = MEAN ? 0 : 1;
-        f32x4 kraw[1 + PRE][4];
-        if (PRE && nu > 0) ldr_tile_lin(rK, klin, w * 32 * ild * 4, ild, kraw[0]);
+        // K tile u + 1 (and its key penalties) is requested before the chain of tile u starts; loads into LDS and
+        // the map's stores share one in-order counter (wait_vm)
+        const auto a_k = DmaTileF32::own_addr(Tb, li, 4 * h, 1);  // K[key li][feature 16h + s]
+        const char* Tm = Tb + 2 * DmaTileF32::TILE + 16 * h;
+        constexpr int KOPS = MASK ? 5 : 4;
+        auto issue_k = [&](int u) {
+            const int J = w + u * WAVES;
+            DmaTileF32::load(wK, lb + (u & 1) * DmaTileF32::TILE, kl, J * 32 * ild * 4, kx);
+            if constexpr (MASK) dma_b32(wM, lb + 2 * DmaTileF32::TILE + (u & 1) * 256, l * 4, J * 128);
+        };
+        asm volatile("s_nop 4");  // the resource words come out of vector instructions
+        if (nu > 0) issue_k(0);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
-                const int J = w + u * WAVES;
-                if (PRE && u + 1 < MAXT) ldr_tile_lin(rK, klin, min(J + WAVES, nbr - 1) * 32 * ild * 4, ild, kraw[(u + 1) & PRE]);
-                if (!PRE) ldr_tile_lin(rK, klin, J * 32 * ild * 4, ild, kraw[0]);
-                lds_put_lin(Tx, l, kraw[u & PRE]);
+                if (u + 1 < MAXT && u + 1 < nu) {
+                    issue_k(u + 1);
+                    wait_vm<KOPS>();
+                } else {
+                    wait_vm<0>();
+                }
                 float kf[KH];
-                lds_get_feat32(Tx, li, h, kf);
+                DmaTileF32::get(a_k, kf, (u & 1) * DmaTileF32::TILE);
+                f32x16 init = splat16(0.f);
+                if constexpr (MASK) {  // minus the key penalties of the tile, log2 domain
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 x = *reinterpret_cast<const f32x4*>(Tm + (u & 1) * 256 + 32 * g);
+                        init[4 * g + 0] = -LOG2E * x.x;
+                        init[4 * g + 1] = -LOG2E * x.y;
+                        init[4 * g + 2] = -LOG2E * x.z;
+                        init[4 * g + 3] = -LOG2E * x.w;
+                    }
+                }
+                wait_lgkm0();  // the tile's space is requested again one iteration on
                 __builtin_amdgcn_sched_barrier(0);
-                S[u] = mma_feat_init<D>(kf, q, chain_init(J));  // S^T: register = key, lane = query
+                S[u] = mma_feat_init<D>(kf, q, init);  // S^T: register = key, lane = query
                 m = max16(S[u], m);
             }
         }
@@ -218,16 +237,24 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
 
     f32x16 o[1] = {splat16(0.f)};  // O^T: register = feature, lane = query
     {
-        constexpr int PRE = MEAN ? 0 : 1;  // see above
-        f32x4 vraw[1 + PRE][4];
-        if (PRE && nu > 0) ldr_tile_lin(rV, vlin, w * VSTEP, vld, vraw[0]);
+        // V tiles the same way, two ahead: request u + 2 goes out when tile u has been read.  What was issued after
+        // the loads of tile u when its turn comes: the loads of tile u + 1 (if any) and the map stores of the one or
+        // two tiles before it.
+        const auto a_v = [&] {
+            if constexpr (RM) return DmaTileF32::cols_addr(Tb, li, h);  // vb[s] = V[key acc_row(s, h)][feature li]
+            else return DmaTileF32::own_addr(Tb, li, h, 2);
+        }();
+        auto issue_v = [&](int u) {
+            DmaTileF32::load(wV, lb + (u & 1) * DmaTileF32::TILE, vl, (w + u * WAVES) * VSTEP, vx);
+        };
+        if (nu > 0) issue_v(0);
+        if (MAXT > 1 && nu > 1) issue_v(1);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
             if (u < nu) {
                 const int J = w + u * WAVES;
-                if (PRE && u + 1 < MAXT) ldr_tile_lin(rV, vlin, min(J + WAVES, nbr - 1) * VSTEP, vld, vraw[(u + 1) & PRE]);
-                if (!PRE) ldr_tile_lin(rV, vlin, J * VSTEP, vld, vraw[0]);
-                lds_put_lin(Tx, l, vraw[u & PRE]);
+                const int stores = u == 0 ? 0 : u == 1 ? 4 : 8;  // map stores issued after V tile u was requested
+                wait_vm_upto(stores + (u + 1 < MAXT && u + 1 < nu ? 4 : 0));
                 float p[16], vb[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
@@ -235,11 +262,12 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
 #pragma unroll
                     for (int r = 0; r < 16; ++r) total[u][r] += p[r];
                 }
-                lds_put_cols(T, li, h, p);        // T[key][query]: the map is stored key-major
-                if constexpr (RM) lds_get_cols(Tx, li, h, vb);  // vb[s] = V[key acc_row(s, h)][feature li]
-                else lds_get_rows(Tx, li, h, vb);
+                lds_put_cols(T, li, h, p);  // T[key][query]: the map is stored key-major
+                DmaTileF32::get(a_v, vb, (u & 1) * DmaTileF32::TILE);
                 f32x4 pl[4];
                 lds_get_lin(T, l, pl);
+                wait_lgkm0();
+                if (u + 2 < MAXT && u + 2 < nu) issue_v(u + 2);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int s = 0; s < 16; ++s) o[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[s], p[s], o[0], 0, 0, 0);
@@ -576,8 +604,8 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_bwd_col_kernel(
 }
 
 // Backward passes for d = 32 with the kept copy of Out: the schedule of the sparse tile kernels (tile_kernels.h)
-// on the dense layouts.  Every operand tile -- V, K^T, Q^T, dO^T and the key-major map tile -- is fetched as four
-// 16-byte instructions one tile ahead and turned into MFMA operands through wave-private LDS copies; -g enters as
+// on the dense layouts.  Every operand tile -- V, K^T, Q^T, dO^T and the key-major map tile -- goes from global
+// memory straight into a wave-private LDS tile, one tile ahead, and is read from there as MFMA operands; -g enters as
 // the initial accumulator of the dP chain; the 1/sqrt(d) is applied to the 32 x d results.
 // RM: K, dO, Out (OutCopy) and dQ are row-major head slices located by `ly`, V as well.
 template <int WAVES, bool RM = false>
@@ -587,7 +615,7 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     float* __restrict__ dQ, int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ float lds[WAVES * 16 * 64];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 1024];
     // last head first: the tail of the map is what the memory-side cache still holds after the forward
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = NB - 1 - item / nbr, I = item % nbr;
@@ -599,11 +627,10 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
     head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
     head_slice<RM, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rK = make_rsrc(Kt + ib, hbytes), rV = make_rsrc(V + ib, hbytes), rdO = make_rsrc(dOt + ob, obytes);
-    const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
-    float* Tv = lds_t[w];
-    float* Tp = Tv + 32 * TS;
-    float* Tk = Tv + 64 * TS;
+    const rsrc_t rdO = make_rsrc(dOt + ob, obytes);
+    const char* Tv = reinterpret_cast<const char*>(lds_t[w]);
+    const char* Tp = Tv + DmaTileF32::TILE;
+    const char* Tk = Tv + 2 * DmaTileF32::TILE;
 
     float go[KH], oo[KH];
     if constexpr (RM) {
@@ -621,30 +648,36 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
     const f32x16 gneg = splat16(-g);
 
     f32x16 acc = splat16(0.f);  // dQ^T: register = feature, lane = query
-    struct Pre {
-        f32x4 v[4], p[4], k[4];
+    // The V, map and K tiles go straight into wave-private LDS; the operands of tile i are read out into registers,
+    // then the same space is requested for tile i + 1, whose loads have the two chains of tile i to arrive.
+    const unsigned lv = lds_address(Tv), lp = lv + DmaTileF32::TILE, lk = lv + 2 * DmaTileF32::TILE;
+    const u32x4 wV = rsrc_words(V + ib, hbytes), wK = rsrc_words(Kt + ib, hbytes);
+    const u32x4 wP = rsrc_words(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const int kld = RM ? ild : L, KSTEP = RM ? 32 * ild * 4 : 128;
+    const int vl = DmaTileF32::voff(l, ild), pl = DmaTileF32::voff(l, L), kl = DmaTileF32::voff(l, kld);
+    const int vx = DmaTileF32::extra_step(ild), px = DmaTileF32::extra_step(L), kx = DmaTileF32::extra_step(kld);
+    const auto a_v = DmaTileF32::own_addr(Tv, li, 4 * h, 1);  // V[key li][feature 16h + s]
+    const auto a_p = DmaTileF32::cols_addr(Tp, li, h);        // P[query li][key acc_row(r, h)]
+    const auto a_k = [&] {
+        if constexpr (RM) return DmaTileF32::cols_addr(Tk, li, h);  // K^T[feature li][key acc_row(s, h)]
+        else return DmaTileF32::own_addr(Tk, li, h, 2);
+    }();
+    auto issue = [&](int J) {
+        DmaTileF32::load(wV, lv, vl, J * 32 * ild * 4, vx);
+        DmaTileF32::load<true>(wP, lp, pl, (J * 32 * L + I * 32) * 4, px);
+        DmaTileF32::load(wK, lk, kl, J * KSTEP, kx);
     };
-    const int vl = lin_voff(l, ild), ll = lin_voff(l, L);
-    const int kld = RM ? ild : L, kl = lin_voff(l, kld), KSTEP = RM ? 32 * ild * 4 : 128;
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int J = w + min(i, nu - 1) * WAVES;
-            ldr_tile_lin(rV, vl, J * 32 * ild * 4, ild, x.v);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
-            ldr_tile_lin(rK, kl, J * KSTEP, kld, x.k);
-        },
-        [&](Pre& c, int) {
-            lds_put_lin(Tv, l, c.v);
-            lds_put_lin(Tp, l, c.p);
-            lds_put_lin(Tk, l, c.k);
+    if (nu > 0) {
+        asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+        issue(w);
+        for (int i = 0; i < nu; ++i) {
+            wait_vm<0>();
             float vt[16], pr[16], kb[16];
-            lds_get_feat32(Tv, li, h, vt);  // V[key li][feature 16h + s]
-            lds_get_cols(Tp, li, h, pr);    // P[query li][key acc_row(r, h)]
-            if constexpr (RM) lds_get_cols(Tk, li, h, kb);  // K^T[feature li][key acc_row(s, h)]
-            else lds_get_rows(Tk, li, h, kb);
+            DmaTileF32::get(a_v, vt);
+            DmaTileF32::get(a_p, pr);
+            DmaTileF32::get(a_k, kb);
+            wait_lgkm0();
+            if (i + 1 < nu) issue(w + (i + 1) * WAVES);
             __builtin_amdgcn_sched_barrier(0);
             f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // register = key, lane = query: dO_i . v_j - g_i
             float ds[16];
@@ -652,7 +685,8 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
             for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
 #pragma unroll
             for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(kb[s], ds[s], acc, 0, 0, 0);
-        });
+        }
+    }
     f32x16 out[1] = {acc * scale};
     if constexpr (RM) reduce_store_rows<WAVES>(out[0], dQ + gb, I * 32, w, li, h, lds, gld);
     else reduce_store<D, WAVES, true>(out, dQ + hb, I * 32, w, li, h, lds, L);
@@ -665,7 +699,7 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     int L, int nbr, int NB, float scale, Layouts ly) {
     constexpr int D = 32, KH = 16;
     __shared__ float lds[WAVES * 16 * 64];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 32 * TS + 32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][3 * 1024 + 64];
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     const int bh = item / nbr, J = item % nbr;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
@@ -676,57 +710,69 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     head_slice<RM, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
     head_slice<RM, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
     head_slice<RM, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
-    const rsrc_t rQ = make_rsrc(Qt + ib, hbytes), rV = make_rsrc(V + ib, hbytes), rdO = make_rsrc(dOt + ob, obytes);
-    const rsrc_t rP = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
-    const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
-    float* To = lds_t[w];
-    float* Tp = To + 32 * TS;
-    float* Tq = To + 64 * TS;
-    float* Tg = To + 96 * TS;
+    const rsrc_t rV = make_rsrc(V + ib, hbytes);
+    const char* To = reinterpret_cast<const char*>(lds_t[w]);
+    const char* Tp = To + DmaTileF32::TILE;
+    const char* Tq = To + 2 * DmaTileF32::TILE;
+    const char* Tg = To + 3 * DmaTileF32::TILE;
 
     float v[KH];
     ldr_rows<D>(rV, (li * ild + h * KH) * 4, J * 32 * ild * 4, v);
 
     f32x16 ak = splat16(0.f), av = splat16(0.f);  // dK^T, dV^T: register = feature, lane = key
-    struct Pre {
-        f32x4 o[4], p[4], q[4];
-        float gneg;  // of query li; spread over the registers of dP through LDS
+    // The dO, map and Q tiles and the 32 values of -g go straight into wave-private LDS; the operands of tile i are
+    // read out into registers (the dO tile in both of its roles), then the same space is requested for tile i + 1.
+    const unsigned lo = lds_address(To), lp = lo + DmaTileF32::TILE, lq = lo + 2 * DmaTileF32::TILE,
+                   lg = lo + 3 * DmaTileF32::TILE;
+    const u32x4 wO = rsrc_words(dOt + ob, obytes), wQ = rsrc_words(Qt + ib, hbytes);
+    const u32x4 wP = rsrc_words(Attn + (size_t)bh * L * L, (size_t)L * L * 4), wG = rsrc_words(G + (size_t)bh * L, (size_t)L * 4);
+    const int qld = RM ? ild : L, QSTEP = RM ? 32 * ild * 4 : 128;
+    const int dld = RM ? old_ : L, DSTEP = RM ? 32 * old_ * 4 : 128;
+    const int dl = DmaTileF32::voff(l, dld), pl = DmaTileF32::voff(l, L), ql = DmaTileF32::voff(l, qld);
+    const int dx = DmaTileF32::extra_step(dld), px = DmaTileF32::extra_step(L), qx = DmaTileF32::extra_step(qld);
+    const auto a_p = DmaTileF32::own_addr(Tp, li, h, 2);  // P[query acc_row(r, h)][key li]
+    const char* a_g = Tg + 16 * h;                        // -g[query acc_row(r, h)]
+    const auto a_go = [&] {
+        if constexpr (RM) return DmaTileF32::own_addr(To, li, 4 * h, 1);  // dO[query li][feature 16h + s]
+        else return DmaTileF32::featcols_addr(To, li, h);
+    }();
+    const auto a_qb = [&] {
+        if constexpr (RM) return DmaTileF32::cols_addr(Tq, li, h);  // Q^T[feature li][query acc_row(s, h)]
+        else return DmaTileF32::own_addr(Tq, li, h, 2);
+    }();
+    const auto a_ob = [&] {
+        if constexpr (RM) return DmaTileF32::cols_addr(To, li, h);  // dO^T[feature li][query acc_row(s, h)]
+        else return DmaTileF32::own_addr(To, li, h, 2);
+    }();
+    auto issue = [&](int I) {
+        DmaTileF32::load(wO, lo, dl, I * DSTEP, dx);
+        DmaTileF32::load<true>(wP, lp, pl, (J * 32 * L + I * 32) * 4, px);
+        DmaTileF32::load(wQ, lq, ql, I * QSTEP, qx);
+        dma_b32(wG, lg, l * 4, I * 128);
     };
-    const int ll = lin_voff(l, L);
-    const int qld = RM ? ild : L, ql = lin_voff(l, qld), QSTEP = RM ? 32 * ild * 4 : 128;
-    const int dld = RM ? old_ : L, dl = lin_voff(l, dld), DSTEP = RM ? 32 * old_ * 4 : 128;
-    Pre xa, xb;
-    tile_pipeline(
-        nu, xa, xb,
-        [&](Pre& x, int i) {
-            const int I = w + min(i, nu - 1) * WAVES;
-            ldr_tile_lin(rdO, dl, I * DSTEP, dld, x.o);
-#pragma unroll
-            for (int c = 0; c < 4; ++c) x.p[c] = ld4_nt(rP, ll, (J * 32 * L + I * 32) * 4 + 32 * c * L);
-            ldr_tile_lin(rQ, ql, I * QSTEP, qld, x.q);
-            x.gneg = ld1(rG, li * 4, I * 128);
-        },
-        [&](Pre& c, int) {
-            lds_put_lin(To, l, c.o);
-            lds_put_lin(Tp, l, c.p);
-            lds_put_lin(Tq, l, c.q);
-            Tg[li] = c.gneg;
-            float go[16], ob[16], p[16], qb[16], gn[16];
-            lds_get_rows(Tg, 0, h, gn);         // -g[query acc_row(r, h)]
-            lds_get_rows(Tp, li, h, p);         // P[query acc_row(r, h)][key li]
-            if constexpr (RM) {
-                lds_get_feat32(To, li, h, go);  // dO[query li][feature 16h + s]
-                lds_get_cols(Tq, li, h, qb);    // Q^T[feature li][query acc_row(s, h)]
-                lds_get_cols(To, li, h, ob);    // dO^T[feature li][query acc_row(s, h)]
-            } else {
-                lds_get_featcols32(To, li, h, go);
-                lds_get_rows(Tq, li, h, qb);
-                lds_get_rows(To, li, h, ob);
-            }
-            __builtin_amdgcn_sched_barrier(0);
+    settle(v);
+    if (nu > 0) {
+        asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+        issue(w);
+        for (int i = 0; i < nu; ++i) {
+            wait_vm<0>();
+            float go[16], ob[16], p[16], qb[16];
             f32x16 init;
+            DmaTileF32::get(a_go, go);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) init[r] = gn[r];
+            for (int g = 0; g < 4; ++g) {
+                const f32x4 x = *reinterpret_cast<const f32x4*>(a_g + 32 * g);
+                init[4 * g + 0] = x.x;
+                init[4 * g + 1] = x.y;
+                init[4 * g + 2] = x.z;
+                init[4 * g + 3] = x.w;
+            }
+            DmaTileF32::get(a_p, p);
+            DmaTileF32::get(a_qb, qb);
+            DmaTileF32::get(a_ob, ob);
+            wait_lgkm0();
+            if (i + 1 < nu) issue(w + (i + 1) * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
             f32x16 dp = mma_feat_init<D>(go, v, init);  // register = query, lane = key
             float ds[16];
 #pragma unroll
@@ -735,7 +781,8 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
             for (int s = 0; s < 16; ++s) ak = __builtin_amdgcn_mfma_f32_32x32x2f32(qb[s], ds[s], ak, 0, 0, 0);
 #pragma unroll
             for (int s = 0; s < 16; ++s) av = __builtin_amdgcn_mfma_f32_32x32x2f32(ob[s], p[s], av, 0, 0, 0);
-        });
+        }
+    }
     f32x16 out[1] = {ak * scale};
     if constexpr (RM) {
         reduce_store_rows<WAVES>(out[0], dK + gb, J * 32, w, li, h, lds, gld);
