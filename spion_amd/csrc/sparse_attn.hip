@@ -408,6 +408,7 @@ struct PatternIndex {
     int ntiles = 0;
     int max_row_tiles = 0, max_col_tiles = 0;
     int n_fwd_long = 0;  // strips of more than 16 tiles: the first entries of the forward's strip order
+    int n_fwd_long24 = 0;  // strips of more than 24 tiles
     int* d_blob = nullptr;  // one allocation holding every array below
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
@@ -816,6 +817,8 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
         }
         for (int p = 0; p < nbr; ++p)
             if (fdesc[4 * p + 2] > 16) pi.n_fwd_long++;
+        for (int p = 0; p < nbr; ++p)
+            if (fdesc[4 * p + 2] > 24) pi.n_fwd_long24++;
         o_rdesc = append(rdesc);
         o_fdesc = append(fdesc);
         o_cdesc = append(cdesc);
@@ -1207,6 +1210,16 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
             hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 4, KROW, ST>), dim3((nbr - nl) * a->NB), dim3(256), 0,
                                a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz,
                                a->scale, nl, nbr - nl, hc, ly);
+            return;
+        }
+    }
+    if constexpr (D == 64) {
+        // most strips of at most 24 tiles, a few longer ones: six logit tiles per wavefront, and the long strips take
+        // the two sweeps inside the same launch
+        if (wv == 4 && pi.max_row_tiles > 4 * MAXT && pi.n_fwd_long24 * 4 < nbr) {
+            hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 6, KROW, ST>), dim3(nbr * a->NB), dim3(256), 0, a->hdr.stream,
+                               Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, 0, nbr,
+                               hc, ly);
             return;
         }
     }

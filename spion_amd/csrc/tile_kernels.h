@@ -564,7 +564,72 @@ void tile_fwd_kernel(
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) o[c] = splat16(0.f);
 
+    auto two_sweeps = [&]() {
+        // ---- sweep 1: online row maximum and denominator -------------------------------------------
+        const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
+        struct PreK {
+            float k[KH];
+            float pj[16];  // key penalties of the tile (MASK only)
+        };
+        auto fetch_k = [&](PreK& x, int i) {
+            const int J = tcol[t0 + w + min(i, nu - 1) * WAVES];
+            load_kf(J, x.k);
+            if constexpr (MASK) ldr_4x4(rM, m_voff, J * 128, x.pj);
+        };
+        auto init_of = [&](const PreK& x, float shift) -> f32x16 {
+            f32x16 v;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                if constexpr (MASK) v[r] = -LOG2E * x.pj[r] - shift;
+                else v[r] = -shift;
+            }
+            return v;
+        };
+        {
+            PreK ka, kb;
+            tile_pipeline(nu, ka, kb, fetch_k, [&](PreK& c, int) {
+                f32x16 s = mma_feat_init<D>(c.k, q, init_of(c, 0.f));
+                const float tm = max16(s, m);
+                float zz = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) zz += __builtin_amdgcn_exp2f(s[r] - tm);
+                z = z * __builtin_amdgcn_exp2f(m - tm) + zz;
+                m = tm;
+            });
+        }
+        merge_max_sum<WAVES>(m, z, w, h, li, lds_m, lds_z);
+        z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
+        const float rinv = 1.0f / z;
+        // ---- sweep 2: logits again (minus the row maximum, folded into the chain), P, O ------------
+        {
+            struct PreKV {
+                PreK k;
+                float vb[D / 32][16];
+            };
+            PreKV xa, xb;
+            tile_pipeline(
+                nu, xa, xb,
+                [&](PreKV& x, int i) {
+                    fetch_k(x.k, i);
+                    ldr_tile_b<D>(rV, b_voff, tcol[t0 + w + min(i, nu - 1) * WAVES] * 32 * ild * 4, x.vb, ild);
+                },
+                [&](PreKV& c, int i) {
+                    f32x16 s = mma_feat_init<D>(c.k.k, q, init_of(c.k, m));
+                    float p[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
+                    store_p(p, w + i * WAVES);
+                    mma_b<D>(p, c.vb, o);
+                });
+        }
+    };
+    // d = 64: a strip too long for the registers of its wavefronts takes the two sweeps inside the same launch (one
+    // launch then serves patterns whose few long strips -- global rows -- would force the sweeps on all)
+    constexpr bool FALLBACK = D == 64 && MAXT > 0;
     if constexpr (MAXT > 0) {
+      if (FALLBACK && cnt > MAXT * WAVES) {
+        two_sweeps();
+      } else {
         const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
         f32x16 S[MAXT];
         int Js[MAXT];  // tile ids of this wavefront, fetched up front (scalar loads, one wait)
@@ -725,64 +790,9 @@ void tile_fwd_kernel(
                 }
             }
         }
+      }
     } else {
-        // ---- sweep 1: online row maximum and denominator -------------------------------------------
-        const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
-        struct PreK {
-            float k[KH];
-            float pj[16];  // key penalties of the tile (MASK only)
-        };
-        auto fetch_k = [&](PreK& x, int i) {
-            const int J = tcol[t0 + w + min(i, nu - 1) * WAVES];
-            load_kf(J, x.k);
-            if constexpr (MASK) ldr_4x4(rM, m_voff, J * 128, x.pj);
-        };
-        auto init_of = [&](const PreK& x, float shift) -> f32x16 {
-            f32x16 v;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                if constexpr (MASK) v[r] = -LOG2E * x.pj[r] - shift;
-                else v[r] = -shift;
-            }
-            return v;
-        };
-        {
-            PreK ka, kb;
-            tile_pipeline(nu, ka, kb, fetch_k, [&](PreK& c, int) {
-                f32x16 s = mma_feat_init<D>(c.k, q, init_of(c, 0.f));
-                const float tm = max16(s, m);
-                float zz = 0.f;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) zz += __builtin_amdgcn_exp2f(s[r] - tm);
-                z = z * __builtin_amdgcn_exp2f(m - tm) + zz;
-                m = tm;
-            });
-        }
-        merge_max_sum<WAVES>(m, z, w, h, li, lds_m, lds_z);
-        z += (float)(L - rn) * __builtin_amdgcn_exp2f(-m);
-        const float rinv = 1.0f / z;
-        // ---- sweep 2: logits again (minus the row maximum, folded into the chain), P, O ------------
-        {
-            struct PreKV {
-                PreK k;
-                float vb[D / 32][16];
-            };
-            PreKV xa, xb;
-            tile_pipeline(
-                nu, xa, xb,
-                [&](PreKV& x, int i) {
-                    fetch_k(x.k, i);
-                    ldr_tile_b<D>(rV, b_voff, tcol[t0 + w + min(i, nu - 1) * WAVES] * 32 * ild * 4, x.vb, ild);
-                },
-                [&](PreKV& c, int i) {
-                    f32x16 s = mma_feat_init<D>(c.k.k, q, init_of(c.k, m));
-                    float p[16];
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) p[r] = __builtin_amdgcn_exp2f(s[r]) * rinv;
-                    store_p(p, w + i * WAVES);
-                    mma_b<D>(p, c.vb, o);
-                });
-        }
+        two_sweeps();
     }
     if constexpr (SHARE) __syncthreads();  // every wavefront is done with its tiles
     if (!ST && Ocache) reduce_store2<D, WAVES>(o, O + hb, Ocache + hb, I * 32, w, li, h, lds);

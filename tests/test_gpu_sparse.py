@@ -134,6 +134,31 @@ def test_tile_path_global_row_and_column(L, d, with_mask):
     abi.close()
 
 
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_tile_path_d64_mixed_strip_lengths_in_one_forward_launch(with_mask):
+    """Head dimension 64, four wavefronts per strip, most strips of 12 to 23 tiles and one global block row of 64: the
+    forward keeps six logit tiles per wavefront in registers and the global row takes the two sweeps inside the same
+    launch (models/block_attn.cu:33-130 makes no such distinction; the results must not show it)."""
+    L, d, bs, B, H = 2048, 64, 32, 1, 2
+    NB, nb = B * H, L // bs
+    mat = workloads.band_random_block_mask(nb, 8, extra_frac=0.05, seed=9)
+    mat[0, :] = 1
+    rows = mat.sum(1)
+    assert rows.max() == nb and np.sort(rows)[-2] <= 24 and np.median(rows) > 16
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=with_mask)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=21, scale=1.2)
+    pen = None
+    if with_mask:
+        key_mask = np.ones((B, L), np.float32)
+        key_mask[0, L - 200:] = 0
+        pen = torch.from_numpy(osa.key_penalty_from_mask(key_mask, H)).cuda()
+    run_and_check(abi, Q, K, V, dO, penalty=pen, tag=f"d=64 mixed strip lengths mask={with_mask}")
+    assert abi.last_path() == 1
+    abi.close()
+
+
 def test_row_sum_invariant_large_logits_and_guard():
     # logits of +-30: exp range exercised; every row still obeys sum P = 1 - (L-n) e^{-m} / Z
     L, bs, d, NB = 128, 32, 32, 2
