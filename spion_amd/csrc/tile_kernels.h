@@ -324,6 +324,26 @@ struct DmaTileF32 {
             x[4 * g + 3] = v.w;
         }
     }
+    // All eight pieces of the lane's own row li (32 floats).
+    struct Own8 {
+        const char* a[8];
+    };
+    __device__ static __forceinline__ Own8 own8_addr(const char* T, int li) {
+        Own8 x;
+#pragma unroll
+        for (int g = 0; g < 8; ++g) x.a[g] = T + li * 128 + 16 * (g ^ (li & 7));
+        return x;
+    }
+    __device__ static __forceinline__ void get32(const Own8& o, float (&x)[32]) {
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(o.a[g]);
+            x[4 * g + 0] = v.x;
+            x[4 * g + 1] = v.y;
+            x[4 * g + 2] = v.z;
+            x[4 * g + 3] = v.w;
+        }
+    }
     // Column li of the rows acc_row(q, h) = 8(q/4) + 4h + q%4, q = 0..15 (the tile in col-owner layout): one
     // address per q%4, the q/4 step is an immediate (rows 8 apart share their permutation).
     struct Cols {
@@ -348,6 +368,11 @@ struct DmaTileF32 {
 #pragma unroll
         for (int j = 0; j < 8; ++j) x.a[j] = T + (16 * h + j) * 128 + 16 * ((li >> 2) ^ j) + 4 * (li & 3);
         return x;
+    }
+    // column li of all 32 rows (addresses made with h = 0)
+    __device__ static __forceinline__ void get32(const FeatCols& c, float (&x)[32]) {
+#pragma unroll
+        for (int s = 0; s < 32; ++s) x[s] = *reinterpret_cast<const float*>(c.a[s & 7] + 1024 * (s >> 3));
     }
     __device__ static __forceinline__ void get(const FeatCols& c, float (&x)[16], int off = 0) {
 #pragma unroll
@@ -814,9 +839,18 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
     static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, Out given");
     constexpr int KH = D / 2;
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    __shared__ float lds_g[WAVES][32];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][D == 32 ? 3 * 1024 : 32 * TS];
+    // LDS of a wavefront: the V, P and K tiles of one pattern tile, 4 KB per 32 features.  d = 64 needs 20 KB, which
+    // eight wavefronts per CU fill to the last byte: the buffer of the final reduction and the partial row sums
+    // of the first sweep then lie inside that space (CARVE), each separated from the tiles by a barrier.
+    constexpr bool CARVE = D == 64;
+    constexpr int WB = (1 + 2 * (D / 32)) * DmaTileF32::TILE;
+    constexpr int RED = WAVES > 1 ? WAVES * (D / 32) * 16 * 64 * 4 : 0;
+    static_assert(!CARVE || RED <= WAVES * WB, "the reduction fits in the tile space");
+    __shared__ __attribute__((aligned(16))) char smem[CARVE ? WAVES * WB : WAVES * WB + RED + WAVES * 128];
+    float* lds = reinterpret_cast<float*>(CARVE ? smem : smem + WAVES * WB);
+    auto lds_g = [&](int ww) {
+        return reinterpret_cast<float*>(CARVE ? smem + ww * WB + WB - 128 : smem + WAVES * WB + RED + ww * 128);
+    };
     // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     int bh, pos;
@@ -839,7 +873,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const int col_voff = (h * KH * L + li) * 4;
     const int b_voff = (4 * h * ild + li) * 4;
     const int r_voff = (li * ild + h * KH) * 4, ro_voff = (li * old_ + h * KH) * 4;
-    float* T = lds_t[w];
+    float* T = reinterpret_cast<float*>(smem + w * WB);
     // P tile as loaded (col owner) -> row-owner layout, the one dP^T comes in
     auto p_rows = [&](const float (&pc)[16], float (&pr)[16]) {
         lds_put_cols(T, li, h, pc);
@@ -879,11 +913,12 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             });
         g += __shfl_xor(g, 32, 64);
         if (WAVES > 1) {
-            if (h == 0) lds_g[w][li] = g;
+            if (h == 0) lds_g(w)[li] = g;
             __syncthreads();
             g = 0.f;
 #pragma unroll
-            for (int ww = 0; ww < WAVES; ++ww) g += lds_g[ww][li];
+            for (int ww = 0; ww < WAVES; ++ww) g += lds_g(ww)[li];
+            if constexpr (CARVE) __syncthreads();  // the partial sums lie where tiles are about to land
         }
     }
     if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;
@@ -940,41 +975,59 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             }
         }
     } else {
-        // One tile ahead: V^T operand, P tile and (d = 32) the K operand of the second product; for d = 64
-        // that operand would not fit in registers and is requested when the tile's first chain starts.
-        constexpr bool DEEP = D == 32;
-        struct Pre {
-            float vt[KH];
-            float pv[16];
-            float kb[DEEP ? D / 32 : 1][16];
-            int J;
+        // d = 64, the same schedule: the V and K tiles are two 4 KB tiles each (features 0..31 and 32..63), the P
+        // tile one; twenty instructions a tile.
+        static_assert(D == 64, "head dimension 32 or 64");
+        const char* Tv = reinterpret_cast<const char*>(T);
+        const char* Tk = Tv + 2 * DmaTileF32::TILE;
+        const char* Tp = Tv + 4 * DmaTileF32::TILE;
+        const unsigned lv = lds_address(Tv), lk = lv + 2 * DmaTileF32::TILE, lp = lv + 4 * DmaTileF32::TILE;
+        const u32x4 wV = rsrc_words(Vt + ib, hbytes), wK = rsrc_words(K + ib, hbytes);
+        const u32x4 wP = rsrc_words(P + (size_t)bh * nnz, (size_t)nnz * 4);
+        // V: feature-major, the halves are 32 rows of L floats apart; row-major, 32 floats apart inside a row
+        const int VSTEP = VROW ? 32 * ild * 4 : 128, VHALF = VROW ? 128 : 32 * L * 4;
+        const int vld = VROW ? ild : L;
+        const int vl = DmaTileF32::voff(l, vld), pl = DmaTileF32::voff(l, rn), kl = DmaTileF32::voff(l, ild);
+        const int vx = DmaTileF32::extra_step(vld), px = DmaTileF32::extra_step(rn), kx = DmaTileF32::extra_step(ild);
+        // operand of the first chain: features 32h .. 32h+31 of key li, i.e. the half-wave's own V tile
+        const auto a_v = [&] {
+            if constexpr (VROW) return DmaTileF32::own8_addr(Tv + h * DmaTileF32::TILE, li);
+            else return DmaTileF32::featcols_addr(Tv + h * DmaTileF32::TILE, li, 0);
+        }();
+        const auto a_p = DmaTileF32::own_addr(Tp, li, h, 2);
+        const auto a_k = DmaTileF32::cols_addr(Tk, li, h);
+        auto issue = [&](int t, int J) {
+            DmaTileF32::load(wV, lv, vl, J * VSTEP, vx);
+            DmaTileF32::load(wV, lv + DmaTileF32::TILE, vl, J * VSTEP + VHALF, vx);
+            DmaTileF32::load<true>(wP, lp, pl, p_base + t * 128, px);
+            DmaTileF32::load(wK, lk, kl, J * 32 * ild * 4, kx);
+            DmaTileF32::load(wK, lk + DmaTileF32::TILE, kl, J * 32 * ild * 4 + 128, kx);
         };
-        Pre xa, xb;  // a third register set (two tiles of lead) was measured and brings nothing
-        tile_pipeline(
-            nu, xa, xb,
-            [&](Pre& x, int i) {
-                const int t = w + min(i, nu - 1) * WAVES;
-                x.J = tcol[t0 + t];
-                if constexpr (VROW) ldr_rows<D>(rV, r_voff, x.J * 32 * ild * 4, x.vt);
-                else ldr_cols<D>(rV, L, col_voff, x.J * 128, x.vt);
-                // the P tile straight in the layout dP^T comes in (every lane pieces of its own row): measured
-                // twice as fast here as full rows plus an LDS transpose, which costs this path its registers
-                // (not non-temporal: a lane reads its 128-byte row in four instructions)
-                ldr_4x4(rP, (li * rn + 4 * h) * 4, p_base + t * 128, x.pv);
-                if constexpr (DEEP) ldr_tile_b<D>(rK, b_voff, x.J * 32 * ild * 4, x.kb, ild);
-            },
-            [&](Pre& c, int) {
-                float kb2[D / 32][16];
-                if constexpr (!DEEP) ldr_tile_b<D>(rK, b_voff, c.J * 32 * ild * 4, kb2, ild);
-                const float (&pr)[16] = c.pv;
-                f32x16 dp = mma_feat_init<D>(c.vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
+        if (nu > 0) {
+            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+            issue(w, tcol[t0 + w]);
+            int Jn = tcol[t0 + w + (nu > 1 ? WAVES : 0)];
+            for (int i = 0; i < nu; ++i) {
+                const int Jnn = tcol[t0 + w + min(i + 2, nu - 1) * WAVES];  // index of the tile after the next
+                wait_vm<0>();
+                float vt[KH], pr[16], kb[2][16];
+                DmaTileF32::get32(a_v, vt);
+                DmaTileF32::get(a_p, pr);
+                DmaTileF32::get(a_k, kb[0]);
+                DmaTileF32::get(a_k, kb[1], DmaTileF32::TILE);
+                wait_lgkm0();
+                if (i + 1 < nu) issue(w + (i + 1) * WAVES, Jn);
+                Jn = Jnn;
+                __builtin_amdgcn_sched_barrier(0);
+                f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // dp[r] = dO_i . v_j - g_i
                 float ds[16];
 #pragma unroll
                 for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
-                if constexpr (DEEP) mma_b<D>(ds, c.kb, acc);
-                else mma_b<D>(ds, kb2, acc);
-            });
+                mma_b<D>(ds, kb, acc);
+            }
+        }
     }
+    if constexpr (CARVE && WAVES > 1) __syncthreads();  // every wavefront is done with its tiles
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) acc[c] *= scale;
     reduce_store<D, WAVES>(acc, dQ + gb, I * 32, w, li, h, lds, gld);
