@@ -1047,8 +1047,15 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     int hc, Layouts ly) {
     static_assert(!ST || VROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
-    __shared__ float lds[WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
-    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][D == 32 ? 3 * 1024 + 64 : 4];
+    // LDS of a wavefront: d = 32, the P, Q and dO tiles and 64 floats of -g; d = 64, the P tile and two tiles each for
+    // Q and dO, 20 KB, which eight wavefronts per CU fill to the last byte: -g then travels in a register, and the
+    // buffer of the final reductions lies inside the tile space (CARVE), a barrier in between.
+    constexpr bool CARVE = D == 64;
+    constexpr int WB = D == 32 ? 3 * DmaTileF32::TILE + 256 : 5 * DmaTileF32::TILE;
+    constexpr int RED = WAVES > 1 ? WAVES * (D / 32) * 16 * 64 * 4 : 0;
+    static_assert(!CARVE || RED <= WAVES * WB, "the reduction fits in the tile space");
+    __shared__ __attribute__((aligned(16))) char smem[CARVE ? WAVES * WB : WAVES * WB + (RED ? RED : 4)];
+    float* lds = reinterpret_cast<float*>(CARVE ? smem : smem + WAVES * WB);
     const int item = xcd_remap(blockIdx.x, nbr * NB);
     int bh, pos;
     item_to_head_strip(item, nbr, hc, bh, pos);
@@ -1079,7 +1086,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     // Per tile of the transposed index: {block row I, offset of the tile in this head's P, row stride}.
     const int4* __restrict__ desc = reinterpret_cast<const int4*>(tcdesc) + e0;
     const int nu = cnt > w ? (cnt - w + WAVES - 1) / WAVES : 0;  // tiles of this wavefront
-    float* T = lds_t[w];
+    float* T = reinterpret_cast<float*>(smem + w * WB);
     if constexpr (D == 32) {
         // The P, Q and dO tiles and the 32 values of -g go straight into wave-private LDS (thirteen instructions, no
         // registers in flight); the operands of tile i are read out of LDS into registers -- the dO tile in both
@@ -1142,42 +1149,69 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
             }
         }
     } else {
-        // One tile ahead: the dO rows, the P tile and -g; the operands of the second products would not fit in
-        // registers beside them and are requested when the tile's first chain starts.
-        struct Pre {
-            float go[KH];
-            float p[16];
-            float gneg[16];
-            int I;
+        // d = 64, the same schedule: the Q and dO tiles are two 4 KB tiles each (features 0..31 and 32..63), the P
+        // tile one; twenty instructions a tile.  No room is left for -g: each lane loads the value of query row
+        // lane % 32 of the next tile with an ordinary load (the compiler's wait for it falls where everything in
+        // flight is waited for anyway, see settle), and one extra MFMA step -- A = that value in the lower half-wave,
+        // zero in the upper, B = 1 -- spreads it over the accumulator the dP chain starts from.
+        static_assert(D == 64, "head dimension 32 or 64");
+        const char* Tp = reinterpret_cast<const char*>(T);
+        const char* Tq = Tp + DmaTileF32::TILE;
+        const char* To = Tp + 3 * DmaTileF32::TILE;
+        const unsigned lp = lds_address(Tp), lq = lp + DmaTileF32::TILE, lo = lp + 3 * DmaTileF32::TILE;
+        const u32x4 wQ = rsrc_words(Q + ib, hbytes), wO = rsrc_words(dO + ob, obytes);
+        const u32x4 wP = rsrc_words(P + (size_t)bh * nnz, (size_t)nnz * 4);
+        const int ql = DmaTileF32::voff(l, ild), ol = DmaTileF32::voff(l, old_);
+        const int qx = DmaTileF32::extra_step(ild), ox = DmaTileF32::extra_step(old_);
+        const int pl0 = 16 * ((l & 7) ^ (l >> 3)), pl1 = (l >> 3) * 4;  // lane offset into a P tile: pl0 + pl1 * row stride
+        const auto a_p = DmaTileF32::cols_addr(Tp, li, h), a_q = DmaTileF32::cols_addr(Tq, li, h),
+                   a_o = DmaTileF32::cols_addr(To, li, h);
+        const auto a_go = DmaTileF32::own8_addr(To + h * DmaTileF32::TILE, li);  // dO[query li][feature 32h + s]
+        auto issue = [&](const int4 d) {
+            const int I = d.x, rn = d.z;
+            DmaTileF32::load<true>(wP, lp, pl0 + pl1 * rn, d.y * 4, DmaTileF32::extra_step(rn));
+            DmaTileF32::load(wQ, lq, ql, I * 32 * ild * 4, qx);
+            DmaTileF32::load(wQ, lq + DmaTileF32::TILE, ql, I * 32 * ild * 4 + 128, qx);
+            DmaTileF32::load(wO, lo, ol, I * 32 * old_ * 4, ox);
+            DmaTileF32::load(wO, lo + DmaTileF32::TILE, ol, I * 32 * old_ * 4 + 128, ox);
         };
-        Pre xa, xb;
-        tile_pipeline(
-            nu, xa, xb,
-            [&](Pre& x, int i) {
-                const int4 d = desc[w + min(i, nu - 1) * WAVES];
-                const int I = d.x, rn = d.z;
-                x.I = I;
-                ldr_rows<D>(rdO, ro_voff, I * 32 * old_ * 4, x.go);
-                const int pv = (4 * h * rn + li) * 4;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) x.p[r] = ld1_nt(rP, pv, (d.y + (8 * (r >> 2) + (r & 3)) * rn) * 4);
-                ldr_4x4(rG, 16 * h, I * 128, x.gneg);
-            },
-            [&](Pre& c, int) {
-                float qb2[D / 32][16], ob2[D / 32][16];
-                ldr_tile_b<D>(rQ, b_voff, c.I * 32 * ild * 4, qb2, ild);
-                ldr_tile_b<D>(rdO, bo_voff, c.I * 32 * old_ * 4, ob2, old_);
-                f32x16 init;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) init[r] = c.gneg[r];
-                f32x16 dp = mma_feat_init<D>(c.go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
+        settle(vt);
+        if (nu > 0) {
+            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
+            int4 dn = desc[w];
+            issue(dn);
+            float gl = ld1(rG, li * 4, dn.x * 128);
+            dn = desc[w + (nu > 1 ? WAVES : 0)];
+            for (int i = 0; i < nu; ++i) {
+                const int4 dnn = desc[w + min(i + 2, nu - 1) * WAVES];  // descriptor of the tile after the next
+                wait_vm<0>();
+                settle(gl);
+                const float ga = h == 0 ? gl : 0.f;
+                float pc[16], qb[2][16], ob[2][16], go[KH];
+                DmaTileF32::get32(a_go, go);
+                DmaTileF32::get(a_p, pc);
+                DmaTileF32::get(a_q, qb[0]);
+                DmaTileF32::get(a_q, qb[1], DmaTileF32::TILE);
+                DmaTileF32::get(a_o, ob[0]);
+                DmaTileF32::get(a_o, ob[1], DmaTileF32::TILE);
+                wait_lgkm0();
+                if (i + 1 < nu) {
+                    issue(dn);
+                    gl = ld1(rG, li * 4, dn.x * 128);
+                }
+                dn = dnn;
+                __builtin_amdgcn_sched_barrier(0);
+                const f32x16 init = __builtin_amdgcn_mfma_f32_32x32x2f32(ga, 1.0f, splat16(0.f), 0, 0, 0);  // -g_i in every column
+                f32x16 dp = mma_feat_init<D>(go, vt, init);  // dO_i . v_j - g_i, i = I*32+acc_row(r,h), j = J*32+li
                 float ds[16];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * c.p[r];
-                mma_b<D>(ds, qb2, ak);
-                mma_b<D>(c.p, ob2, av);
-            });
+                for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pc[r];
+                mma_b<D>(ds, qb, ak);
+                mma_b<D>(pc, ob, av);
+            }
+        }
     }
+    if constexpr (CARVE && WAVES > 1) __syncthreads();  // every wavefront is done with its tiles
 #pragma unroll
     for (int c = 0; c < D / 32; ++c) ak[c] *= scale;
     reduce_store<D, WAVES>(ak, dK + gb, J * 32, w, li, h, lds, gld);
