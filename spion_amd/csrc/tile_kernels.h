@@ -660,9 +660,6 @@ void tile_fwd_kernel(
         int Js[MAXT];  // tile ids of this wavefront, fetched up front (scalar loads, one wait)
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) Js[u] = u < nu ? tcol[t0 + w + u * WAVES] : 0;
-        // d = 32: K^T, V and P tiles move as four 16-byte instructions each (linear layout) and change layout
-        // in wave-private LDS tiles: a quarter of the vector-memory instructions, which keeps the wavefront
-        // clear of the 63 outstanding instructions it may have (loads and stores share that counter).
         constexpr bool LIN = D == 32;
         // d = 32: K^T and V tiles go straight into two wave-private LDS tiles, alternately (tile u + 1 is requested
         // before the chain of tile u starts); P tiles leave as four 16-byte instructions after a layout change
