@@ -119,7 +119,7 @@ struct DmaTile {
     __device__ static __forceinline__ void load(u32x4 r, unsigned lds, int lvoff, int soff, int xstep) {
         if constexpr (D == 64)
             asm volatile(
-                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "s_mov_b32 m0, %0\n\ts_nop 3\n\t"
                 "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 lds\n\t"
@@ -128,7 +128,7 @@ struct DmaTile {
                 : "memory");
         else
             asm volatile(
-                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "s_mov_b32 m0, %0\n\ts_nop 3\n\t"
                 "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds" ::"s"(lds),
                 "v"(lvoff), "s"(r), "s"(soff), "s"(soff + xstep)

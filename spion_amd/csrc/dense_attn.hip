@@ -173,7 +173,6 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
             DmaTileF32::load(wK, lb + (u & 1) * DmaTileF32::TILE, kl, J * 32 * ild * 4, kx);
             if constexpr (MASK) dma_b32(wM, lb + 2 * DmaTileF32::TILE + (u & 1) * 256, l * 4, J * 128);
         };
-        asm volatile("s_nop 4");  // the resource words come out of vector instructions
         if (nu > 0) issue_k(0);
 #pragma unroll
         for (int u = 0; u < MAXT; ++u) {
@@ -668,7 +667,6 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_row32_kernel(
         DmaTileF32::load(wK, lk, kl, J * KSTEP, kx);
     };
     if (nu > 0) {
-        asm volatile("s_nop 4");  // the resource words above come out of vector instructions
         issue(w);
         for (int i = 0; i < nu; ++i) {
             wait_vm<0>();
@@ -752,7 +750,6 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     };
     settle(v);
     if (nu > 0) {
-        asm volatile("s_nop 4");  // the resource words above come out of vector instructions
         issue(w);
         for (int i = 0; i < nu; ++i) {
             wait_vm<0>();

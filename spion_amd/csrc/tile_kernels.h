@@ -227,8 +227,9 @@ __device__ __forceinline__ void lds_get_featcols32(const float* T, int li, int h
 // write LDS.  The kernels wait for them with wait_vm<N> (N = loads issued after the ones waited for; loads return
 // in order, and the compiler's own counts can then only wait longer than needed) and finish their LDS reads with
 // wait_lgkm0 before a tile's space is requested again; both carry a memory clobber, so no LDS access moves across.
-// Scalar operands of the assembly come from scalar loads and SALU arithmetic only (a scalar register written by a
-// vector instruction needs wait states before a memory instruction reads it, which the compiler cannot add here).
+// Every block of loads starts with five wait states (s_mov to M0, s_nop 3): a scalar register written by a vector
+// instruction -- v_readfirstlane, or v_readlane when the compiler restores a spilled scalar -- needs that distance
+// before a memory instruction reads it, and the compiler, which adds it elsewhere, does not look inside assembly.
 // -------------------------------------------------------------------------------------------------
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ u32x4 rsrc_words(const void* p, size_t bytes) {
@@ -271,7 +272,7 @@ __device__ __forceinline__ void settle(const float (&x)[N]) {
 }
 // 64 floats (lane l: 4 bytes at voff) to 256 bytes of LDS
 __device__ __forceinline__ void dma_b32(u32x4 r, unsigned lds, int voff, int soff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds), "v"(voff), "s"(r),
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dword %1, %2, %3 offen lds" ::"s"(lds), "v"(voff), "s"(r),
                  "s"(soff)
                  : "memory");
 }
@@ -286,7 +287,7 @@ struct DmaTileF32 {
     __device__ static __forceinline__ void load(u32x4 r, unsigned lds, int lvoff, int soff, int xstep) {
         if constexpr (NT)
             asm volatile(
-                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "s_mov_b32 m0, %0\n\ts_nop 3\n\t"
                 "buffer_load_dwordx4 %1, %2, %3 offen nt lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 nt lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 nt lds\n\t"
@@ -295,7 +296,7 @@ struct DmaTileF32 {
                 : "memory");
         else
             asm volatile(
-                "s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                "s_mov_b32 m0, %0\n\ts_nop 3\n\t"
                 "buffer_load_dwordx4 %1, %2, %3 offen lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %4 offen offset:1024 lds\n\t"
                 "buffer_load_dwordx4 %1, %2, %5 offen offset:2048 lds\n\t"
@@ -685,7 +686,6 @@ void tile_fwd_kernel(
                 DmaTileF32::load(wK, lb + (u & 1) * DmaTileF32::TILE, kl, Js[u] * KSTEP, kx);
                 if constexpr (MASK) dma_b32(wM, lb + 2 * DmaTileF32::TILE + (u & 1) * 256, l * 4, Js[u] * 128);
             };
-            asm volatile("s_nop 4");  // the resource words come out of vector instructions
             if (nu > 0) issue_k(0);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
@@ -773,7 +773,6 @@ void tile_fwd_kernel(
             auto issue_v = [&](int u) {
                 DmaTileF32::load(wV, lb + (u & 1) * DmaTileF32::TILE, vl, Js[u] * 32 * ild * 4, vx);
             };
-            asm volatile("s_nop 4");
             if (nu > 0) issue_v(0);
             if (MAXT > 1 && nu > 1) issue_v(1 < MAXT ? 1 : 0);
 #pragma unroll
@@ -950,7 +949,6 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             DmaTileF32::load(wK, lk, kl, J * 32 * ild * 4, kx);
         };
         if (nu > 0) {
-            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
             issue(w, tcol[t0 + w]);
             int Jn = tcol[t0 + w + (nu > 1 ? WAVES : 0)];
             for (int i = 0; i < nu; ++i) {
@@ -1001,7 +999,6 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
             DmaTileF32::load(wK, lk + DmaTileF32::TILE, kl, J * 32 * ild * 4 + 128, kx);
         };
         if (nu > 0) {
-            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
             issue(w, tcol[t0 + w]);
             int Jn = tcol[t0 + w + (nu > 1 ? WAVES : 0)];
             for (int i = 0; i < nu; ++i) {
@@ -1113,7 +1110,6 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
         };
         settle(vt);
         if (nu > 0) {
-            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
             issue(desc[w]);
             int4 dn = desc[w + (nu > 1 ? WAVES : 0)];
             for (int i = 0; i < nu; ++i) {
@@ -1174,7 +1170,6 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
         };
         settle(vt);
         if (nu > 0) {
-            asm volatile("s_nop 4");  // the resource words above come out of vector instructions
             int4 dn = desc[w];
             issue(dn);
             float gl = ld1(rG, li * 4, dn.x * 128);
