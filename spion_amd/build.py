@@ -59,6 +59,62 @@ def build_autograd_node(verbose: bool = False) -> str:
     return out
 
 
+def emit_device_asm(src: str, out: str) -> str:
+    """Device-only assembly of one HIP source (same flags as the library build)."""
+    _run([HIPCC, *HIP_FLAGS, "--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", out], False)
+    return out
+
+
+def scan_sgpr_hazards(asm_text: str):
+    """Inline-assembly buffer instructions that read a scalar register fewer than five wait states after a vector
+    instruction wrote it (v_readlane when the compiler restores a spilled scalar, v_readfirstlane, v_cmp into a scalar
+    pair).  The compiler keeps that distance for the instructions it emits itself but does not look inside assembly
+    blocks, so the loads into LDS (csrc/tile_kernels.h, csrc/bf16_kernels.h) have to carry it themselves.
+    Returns (number of assembly blocks seen, list of findings)."""
+    import re
+
+    def sregs(tok):
+        regs = set()
+        for m in re.finditer(r"\bs\[(\d+):(\d+)\]", tok):
+            regs.update(range(int(m.group(1)), int(m.group(2)) + 1))
+        for m in re.finditer(r"\bs(\d+)\b", tok):
+            regs.add(int(m.group(1)))
+        return regs
+
+    lines = asm_text.split("\n")
+    kernel, in_asm, blocks, found = None, False, 0, []
+    for idx, ln in enumerate(lines):
+        t = ln.strip()
+        if re.match(r"^_Z\w+:", ln):
+            kernel = ln.split(":")[0]
+        if t.startswith(";;#ASMSTART"):
+            in_asm, blocks = True, blocks + 1
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not (in_asm and t.startswith("buffer_")):
+            continue
+        need = sregs(t.split(None, 1)[1] if " " in t else "")
+        waited, j = 0, idx - 1
+        while j >= 0 and waited < 5:
+            u = lines[j].strip()
+            j -= 1
+            if not u or u.startswith(";"):
+                continue
+            if u.endswith(":") or u.startswith("."):
+                break  # a label: what ran before is not known from the text
+            m = re.match(r"(?:v_readlane_b32|v_readfirstlane_b32)\s+s(\d+)", u)
+            hit = m is not None and int(m.group(1)) in need
+            m = re.match(r"v_cmp\w*\s+(s\[\d+:\d+\])", u)
+            hit = hit or (m is not None and bool(sregs(m.group(1)) & need))
+            if hit:
+                found.append(f"{kernel} line {idx + 1}: '{t}' {waited} wait states after '{u}'")
+            m = re.match(r"s_nop\s+(\d+)", u)
+            waited += int(m.group(1)) + 1 if m else 1
+    return blocks, found
+
+
 def build_all(verbose: bool = False, jobs: int = 4) -> str:
     os.makedirs(OBJ, exist_ok=True)
 
