@@ -14,7 +14,7 @@ algorithmic FLOPs over its own HIP-event time); ``cpu_baseline`` is the dense Py
 the same semantics (the oracle) timed on the host cores over a bounded sample of the batch.
 ``window_ms`` holds five further 20-step timings of the same step and their median.  The default run
 adds the other measured workloads as sub-objects of the same line (``config1``, ``config4``,
-``config5``, ``config2``, ``dense_phase``: step time, windows and roofline of each; ``--no-config1``
+``config5``, ``config5_fp32``, ``config2``, ``dense_phase``: step time, windows and roofline of each; ``--no-config1``
 and ``--no-extra`` leave them out); their CPU baselines are part of their own ``--workload`` runs.
 """
 from __future__ import annotations
@@ -532,7 +532,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-config1", action="store_true", help="north_star only: leave out the L = 1024 sub-object")
     ap.add_argument("--no-extra", action="store_true",
-                    help="north_star only: leave out the config4 / config5 / config2 / dense_phase sub-objects")
+                    help="north_star only: leave out the config4 / config5 / config5_fp32 / config2 / dense_phase sub-objects")
     ap.add_argument("--spinup-ms", type=float, default=300.0,
                     help="untimed repetitions of the step for this long before the warm-up (clock ramp)")
     ap.add_argument("--copy-probe", action="store_true",
@@ -588,6 +588,7 @@ def main():
         if not args.no_extra:
             extra += [("config4", lambda: bench_sparse_layer(sub, dev, "config4", full=False)),
                       ("config5", lambda: bench_bf16_scale_up(sub, dev)),
+                      ("config5_fp32", lambda: bench_sparse_layer(sub, dev, "config5_fp32", full=False)),
                       ("config2", lambda: bench_pattern_discovery(sub, dev)),
                       ("dense_phase", lambda: bench_dense_phase(sub, dev))]
         for name, run in extra:
