@@ -28,7 +28,6 @@
 namespace spion {
 
 #define SPION_TILE_KERNEL(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(2, 2)))
-#define SPION_TILE_KERNEL3(W) __global__ __launch_bounds__(64 * (W)) __attribute__((amdgpu_waves_per_eu(3, 3)))
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
@@ -207,11 +206,6 @@ __device__ __forceinline__ void lds_put_lin(float* T, int l, const f32x4 (&raw)[
 __device__ __forceinline__ void lds_get_lin(const float* T, int l, f32x4 (&raw)[4]) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) raw[i] = *reinterpret_cast<const f32x4*>(T + (8 * i + (l >> 3)) * TS + 4 * (l & 7));
-}
-// operand over 32 features from a feature-major tile T[feature][row]: x[s] = T[16h + s][li]
-__device__ __forceinline__ void lds_get_featcols32(const float* T, int li, int h, float (&x)[16]) {
-#pragma unroll
-    for (int s = 0; s < 16; ++s) x[s] = T[(16 * h + s) * TS + li];
 }
 
 // -------------------------------------------------------------------------------------------------
