@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_bf16|dense_phase|config1|config1_b256|config2|config3|config4|config5|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_global|north_star_bf16|dense_phase|config1|config1_b256|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -119,10 +119,14 @@ def build_workload(name):
     from spion_amd import workloads
     from spion_amd.csr import block_mask_to_csr_host
 
-    if name in ("north_star", "north_star_bs64"):
+    if name in ("north_star", "north_star_bs64", "north_star_global"):
         # bs64: the block size the reference uses on its L = 4000 tasks (config.py:99,181), same density
+        # global: plus one block row and one block column that span the sequence (as configuration 5 has)
         B, H, L, d, bs = 32, 2, 4096, 32, 64 if name == "north_star_bs64" else 32
         mat = workloads.north_star_mask(bs)
+        if name == "north_star_global":
+            mat[0, :] = 1.0
+            mat[:, 0] = 1.0
         scale = 1.0
     elif name in ("config1", "config1_b256"):
         # b256: the same layer at the batch size the reference trains its L = 1024 tasks with (config.py:60)

@@ -37,9 +37,13 @@ int spion_debug_bf16_plan(const int* tile_ptr, int nstrips, int pairs, int num_b
                           int cap_items, int* lane_ptr, int cap_ptr, int* lane_ent, int cap_ent, int* longs,
                           int cap_longs, int* counts);
 
-/* Environment switches read once per process, for A/B measurements only (results are the same either way):
+/* Environment switches read once per process, for A/B measurements only (results are the same to rounding either way):
  *   SPION_NO_FWD_SPLIT   the fp32 tile forward runs all strips in one launch, eight logit tiles per wavefront
  *                        (default: strips of at most 16 tiles in a launch of their own, three work-groups to a CU);
+ *   SPION_NO_LONG_SPLIT  patterns with a few strips far longer than the rest (global rows / columns) run every pass of
+ *                        the fp32 tile path as one launch with four wavefronts to every strip (default: the long strips
+ *                        in a launch of their own on the caller's stream, the others beside it on the handle's side
+ *                        stream; the summation order inside the short strips differs between the two);
  *   SPION_BF16_NO_PAIRS  the bf16 forward and row pass take one strip per wavefront on every pattern (default: two
  *                        strips per wavefront on masks of 64 x 64 blocks and larger, contiguous heads);
  *   SPION_BF16_ROW_PAIRS=0  the same for the row pass alone.

@@ -409,6 +409,9 @@ struct PatternIndex {
     int max_row_tiles = 0, max_col_tiles = 0;
     int n_fwd_long = 0;  // strips of more than 16 tiles: the first entries of the forward's strip order
     int n_fwd_long24 = 0;  // strips of more than 24 tiles
+    // block rows / block columns longer than long_strip_threshold (global rows and columns): the first entries of
+    // the row pass's and of the column pass's strip order
+    int n_long_rows = 0, n_long_cols = 0;
     int* d_blob = nullptr;  // one allocation holding every array below
     int *d_trp = nullptr, *d_tcol = nullptr, *d_tcp = nullptr;
     int* d_tcdesc = nullptr;  // per tile of the transposed index: {block row I, offset of the tile in P, row stride, 0}
@@ -468,6 +471,20 @@ struct SparseAttn {
     size_t ws_ds_count = 0;
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
     size_t ws_part_floats = 0;
+    // Side stream (default priority) on which the fp32 backward runs the few long strips of a pattern beside the
+    // launch of the others; forked from and joined to the caller's stream by the two events.  Created at first use.
+    hipStream_t side = nullptr;
+    hipEvent_t side_fork = nullptr, side_join = nullptr;
+    bool ensure_side() {
+        if (side) return true;
+        if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) return side = nullptr, false;
+        if (hipEventCreateWithFlags(&side_fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&side_join, hipEventDisableTiming) != hipSuccess) {
+            (void)hipStreamDestroy(side);
+            return side = nullptr, false;
+        }
+        return true;
+    }
     // Buffers a grown workspace has replaced.  They stay allocated until the handle is destroyed: a HIP graph
     // recorded earlier on this handle has their addresses in its kernel nodes and may still be replayed.
     std::vector<void*> retired;
@@ -524,6 +541,12 @@ void sparse_destroy(void* h) {
     SparseAttn* a = as_sparse(h, "destroy");
     if (!a) return;
     a->release_patterns();
+    if (a->side) {
+        (void)hipStreamSynchronize(a->side);
+        (void)hipEventDestroy(a->side_fork);
+        (void)hipEventDestroy(a->side_join);
+        (void)hipStreamDestroy(a->side);
+    }
     if (a->ws_rowsum) (void)hipFree(a->ws_rowsum);
     if (a->ws_trans) (void)hipFree(a->ws_trans);
     if (a->ws_stats) (void)hipFree(a->ws_stats);
@@ -776,9 +799,11 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             for (int i = 0; i < nbr; ++i) order[i] = i;
             auto bucket = [&](int i) {
                 const int len = ptr[i + 1] - ptr[i];
-                if (rows) return len > 2 * maxt ? 0 : len > maxt ? 1 : 2;
+                if (rows) return len > long_len ? -1 : len > 2 * maxt ? 0 : len > maxt ? 1 : 2;
                 return len > long_len ? 0 : 1;
             };
+            for (int i = 0; i < nbr; ++i)
+                if (ptr[i + 1] - ptr[i] > long_len) (rows ? pi.n_long_rows : pi.n_long_cols)++;
             std::stable_sort(order.begin(), order.end(), [&](int x, int y) { return bucket(x) < bucket(y); });
             ptr.insert(ptr.end(), order.begin(), order.end());
         };
@@ -815,6 +840,7 @@ static bool analyse_pattern(SparseAttn* a, const int* Offsets, const int* Column
             cdesc[4 * p + 2] = tcp[J + 1] - tcp[J];
             cdesc[4 * p + 3] = 0;
         }
+        if (pi.n_long_rows > 0 || pi.n_long_cols > 0) (void)a->ensure_side();  // see launch_tile_bwd
         for (int p = 0; p < nbr; ++p)
             if (fdesc[4 * p + 2] > 16) pi.n_fwd_long++;
         for (int p = 0; p < nbr; ++p)
@@ -1192,6 +1218,24 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
     // to a CU in a launch of their own, the few longer ones first with eight tiles per wavefront (north star:
     // forward 0.1756 -> 0.1721 ms; six wavefronts of four tiles for the long strips instead: 44 against 36 us)
     static const bool no_split = getenv("SPION_NO_FWD_SPLIT") != nullptr;
+    // A pattern with a few strips far longer than the rest (global rows): those, and whatever else exceeds 24 tiles,
+    // take the two sweeps with eight wavefronts to a strip in a launch of their own, which goes first on the caller's
+    // stream; all other strips follow on the handle's side stream with six logit tiles per wavefront (see
+    // launch_tile_bwd for the streams).
+    static const bool no_long = getenv("SPION_NO_LONG_SPLIT") != nullptr;
+    const int n24 = pi.n_fwd_long24;
+    if (!no_long && a->side && wv == 4 && pi.n_long_rows > 0 && n24 * 8 <= nbr) {
+        (void)hipEventRecord(a->side_fork, a->hdr.stream);
+        (void)hipStreamWaitEvent(a->side, a->side_fork, 0);
+        hipLaunchKernelGGL((tile_fwd_kernel<D, 8, MASK, 0, KROW, ST>), dim3(n24 * a->NB), dim3(512), 0, a->hdr.stream, Q,
+                           Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, 0, n24, hc, ly);
+        hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 6, KROW, ST>), dim3((nbr - n24) * a->NB), dim3(256), 0, a->side,
+                           Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, n24,
+                           nbr - n24, hc, ly);
+        (void)hipEventRecord(a->side_join, a->side);
+        (void)hipStreamWaitEvent(a->hdr.stream, a->side_join, 0);
+        return;
+    }
     if constexpr (D == 32) {
         // longest strip of 17 to 24 tiles: six logit tiles per wavefront still fit three work-groups to a CU (161
         // registers), so one launch takes every strip (north star: forward 0.171 -> 0.166 ms against the split)
@@ -1199,6 +1243,14 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
             hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 6, KROW, ST>), dim3(nbr * a->NB), dim3(256), 0, a->hdr.stream,
                                Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, 0, nbr,
                                hc, ly);
+            return;
+        }
+        // a few strips of more than 32 tiles (global rows) among strips of at most 24: the six-tile kernel with the two
+        // sweeps for the long ones inside the same launch, instead of the two sweeps for every strip
+        if (wv == 4 && pi.max_row_tiles > 4 * MAXT && pi.n_fwd_long24 * 4 < nbr) {
+            hipLaunchKernelGGL((tile_fwd_kernel<D, 4, MASK, 6, KROW, ST, true>), dim3(nbr * a->NB), dim3(256), 0,
+                               a->hdr.stream, Q, Kt, V, pen, P, O, ocache, pi.d_fdesc, pi.d_tcol, a->L, nbr, a->NB, nnz,
+                               a->scale, 0, nbr, hc, ly);
             return;
         }
         if (wv == 4 && !no_split && pi.max_row_tiles <= 4 * MAXT && pi.n_fwd_long < nbr && pi.max_row_tiles > 16) {
@@ -1240,42 +1292,120 @@ static void launch_tile_fwd(SparseAttn* a, const float* Q, const float* Kt, cons
 #undef SPION_LAUNCH
 }
 
+// One launch of a backward pass over the strips s0 .. s0+ns-1 of every head's strip order, W wavefronts per strip.
+template <int D, int W, bool VROW, bool ST>
+static void launch_tile_bwd_rows(SparseAttn* a, hipStream_t stream, const float* K, const float* Vt, const float* P,
+                                 const float* dO, const float* ocache, float* rowsum, float* dQ, int nnz, int hc,
+                                 const Layouts& ly, int s0, int ns) {
+    const PatternIndex& pi = a->pat;
+    const int nbr = a->L / 32;
+    const dim3 grid(ns * a->NB), block(64 * W);
+    if (ocache) {
+        hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, block, 0, stream, K, Vt, P, dO, ocache,
+                           rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, hc, ly, s0, ns);
+    } else {
+        if constexpr (!ST)
+            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, block, 0, stream, K, Vt, P, dO, ocache,
+                               rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB, nnz, a->scale, hc, ly, s0, ns);
+    }
+}
+template <int D, int W, bool VROW, bool ST>
+static void launch_tile_bwd_cols(SparseAttn* a, hipStream_t stream, const float* Q, const float* Vt, const float* P,
+                                 const float* dO, const float* rowsum, float* dK, float* dV, int nnz, int hc,
+                                 const Layouts& ly, int s0, int ns) {
+    const PatternIndex& pi = a->pat;
+    const int nbr = a->L / 32;
+    hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), dim3(ns * a->NB), dim3(64 * W), 0, stream, Q, Vt, P, dO,
+                       rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale, hc, ly, s0, ns);
+}
+
+// Wavefronts per strip of a backward launch over strips of at most `longest` tiles.
+static int bwd_waves(const SparseAttn* a, const PatternIndex& pi, int nbr, int strips_per_head) {
+    const int avg = nbr ? (pi.ntiles + nbr - 1) / nbr : 0;
+    const long long strips = (long long)strips_per_head * a->NB;
+    if (strips >= 2048 || avg <= 2) return 1;
+    if (strips >= 1024 || avg <= 4) return 2;
+    return 4;
+}
+
 template <int D, bool VROW, bool ST = false>
 static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const float* Vt, const float* P,
                             const float* dO, float* dQ, float* dK, float* dV, const int* offs, int nnz,
                             const float* Out, const Layouts& ly = Layouts{}, float* rowsum = nullptr) {
     const PatternIndex& pi = a->pat;
+    // the entry point that allocates nothing brings its own row-sum array and creates nothing either
+    const bool side_ok = rowsum == nullptr;
     if (!rowsum) rowsum = a->ws_rowsum;
     const int nbr = a->L / 32;
-    const dim3 grid(nbr * a->NB);
-    const int wv = pick_waves(a, pi, nbr, false);
     const int hc = heads_per_group(a);
     const float* ocache = Out ? Out : ocache_for_backward(a, P);
-#define SPION_LAUNCH(W)                                                                                             \
-    do {                                                                                                            \
-        if ((a->bwd_passes & 1) && ocache) {                                                                        \
-            PhaseRange range("spion backward: row pass (dQ)");                                                      \
-            hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, true, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, K,   \
-                               Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr, a->NB,    \
-                               nnz, a->scale, hc, ly);                                                              \
-        } else if (a->bwd_passes & 1) {                                                                             \
-            PhaseRange range("spion backward: row pass (dQ)");                                                      \
-            if constexpr (!ST)                                                                                      \
-                hipLaunchKernelGGL((tile_bwd_row_kernel<D, W, false, VROW>), grid, dim3(64 * W), 0, a->hdr.stream,  \
-                                   K, Vt, P, dO, ocache, rowsum, dQ, pi.d_rdesc, pi.d_tcol, a->L, nbr,    \
-                                   a->NB, nnz, a->scale, hc, ly);                                                   \
-        }                                                                                                           \
-        if (a->bwd_passes & 2) {                                                                                    \
-            PhaseRange range("spion backward: column pass (dK, dV)");                                               \
-            hipLaunchKernelGGL((tile_bwd_col_kernel<D, W, VROW, ST>), grid, dim3(64 * W), 0, a->hdr.stream, Q, Vt, P, \
-                               dO, rowsum, dK, dV, pi.d_cdesc, pi.d_tcdesc, a->L, nbr, a->NB, nnz, a->scale,    \
-                               hc, ly);                                                                             \
-        }                                                                                                           \
+    // A pattern with a few strips far longer than the rest (global rows, global columns): those run four wavefronts
+    // to a strip in a small launch of their own, all other strips in a launch with the wavefront count their own
+    // number calls for -- instead of four wavefronts to every strip of the pattern because of the few.  The small
+    // launch goes to a side stream of the handle (made when such a pattern is analysed), beside the large one; without
+    // that stream the two launches follow one another, with the same results.
+    static const bool no_split = getenv("SPION_NO_LONG_SPLIT") != nullptr;
+    const int nlr = pi.n_long_rows, nlc = pi.n_long_cols;
+    const bool split = !no_split && (nlr > 0 || nlc > 0) && nlr * 8 <= nbr && nlc * 8 <= nbr;
+    const bool side = split && side_ok && a->side != nullptr;
+    // the long strips go first, on the caller's stream, so that they hold their places on the CUs before the many
+    // short work-groups arrive; those follow on the side stream
+    hipStream_t rest_stream = side ? a->side : a->hdr.stream;
+    auto fork = [&]() {
+        if (!side) return;
+        (void)hipEventRecord(a->side_fork, a->hdr.stream);
+        (void)hipStreamWaitEvent(a->side, a->side_fork, 0);
+    };
+    auto join = [&]() {
+        if (!side) return;
+        (void)hipEventRecord(a->side_join, a->side);
+        (void)hipStreamWaitEvent(a->hdr.stream, a->side_join, 0);
+    };
+#define SPION_ROWS(W, STREAM, S0, NS) \
+    launch_tile_bwd_rows<D, W, VROW, ST>(a, STREAM, K, Vt, P, dO, ocache, rowsum, dQ, nnz, hc, ly, S0, NS)
+#define SPION_COLS(W, STREAM, S0, NS) \
+    launch_tile_bwd_cols<D, W, VROW, ST>(a, STREAM, Q, Vt, P, dO, rowsum, dK, dV, nnz, hc, ly, S0, NS)
+#define SPION_BY_WAVES(WV, WHAT, STREAM, S0, NS)      \
+    do {                                              \
+        if ((WV) == 1) WHAT(1, STREAM, S0, NS);       \
+        else if ((WV) == 2) WHAT(2, STREAM, S0, NS);  \
+        else WHAT(4, STREAM, S0, NS);                 \
     } while (0)
-    if (wv == 1) SPION_LAUNCH(1);
-    else if (wv == 2) SPION_LAUNCH(2);
-    else SPION_LAUNCH(4);
-#undef SPION_LAUNCH
+    if (split) {
+        if (a->bwd_passes & 1) {
+            PhaseRange range("spion backward: row pass (dQ)");
+            const int wv = bwd_waves(a, pi, nbr, nbr - nlr);
+            if (nlr > 0) {
+                fork();
+                SPION_ROWS(8, a->hdr.stream, 0, nlr);
+            }
+            SPION_BY_WAVES(wv, SPION_ROWS, nlr > 0 ? rest_stream : a->hdr.stream, nlr, nbr - nlr);
+            if (nlr > 0) join();
+        }
+        if (a->bwd_passes & 2) {
+            PhaseRange range("spion backward: column pass (dK, dV)");
+            const int wv = bwd_waves(a, pi, nbr, nbr - nlc);
+            if (nlc > 0) {
+                fork();
+                SPION_COLS(8, a->hdr.stream, 0, nlc);
+            }
+            SPION_BY_WAVES(wv, SPION_COLS, nlc > 0 ? rest_stream : a->hdr.stream, nlc, nbr - nlc);
+            if (nlc > 0) join();
+        }
+    } else {
+        const int wv = pick_waves(a, pi, nbr, false);
+        if (a->bwd_passes & 1) {
+            PhaseRange range("spion backward: row pass (dQ)");
+            SPION_BY_WAVES(wv, SPION_ROWS, a->hdr.stream, 0, nbr);
+        }
+        if (a->bwd_passes & 2) {
+            PhaseRange range("spion backward: column pass (dK, dV)");
+            SPION_BY_WAVES(wv, SPION_COLS, a->hdr.stream, 0, nbr);
+        }
+    }
+#undef SPION_ROWS
+#undef SPION_COLS
+#undef SPION_BY_WAVES
 }
 
 // Hybrid patterns (dense tiles + remainder, d = 32).  Every operand row-major; ST: heads located by `ly`.

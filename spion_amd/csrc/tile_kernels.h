@@ -509,8 +509,11 @@ __device__ __forceinline__ void tile_pipeline(int n, Pre& a, Pre& b, Fetch fetch
 // for contiguous heads therefore still transpose once; only the strided entry points use it.
 // MAXT <= 6 at d = 32 (at most six logit tiles per wavefront) fits three wavefronts per SIMD: the buffer of the
 // final reduction then shares the space of the wave-private tiles (a barrier in between).
-template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false>
-__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(D == 32 && MAXT > 0 && MAXT <= 6 ? 3 : 2, D == 32 && MAXT > 0 && MAXT <= 6 ? 3 : 2)))
+// LONG (with MAXT > 0): a strip too long for the registers of its wavefronts takes the two sweeps inside the same
+// launch, so the few long strips of a pattern -- global rows -- do not force the sweeps on all of them.  Always on
+// at d = 64; at d = 32 it is an instantiation of its own, which leaves the kernel of the other patterns as it is.
+template <int D, int WAVES, bool MASK, int MAXT, bool KROW = false, bool ST = false, bool LONG = D == 64>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(D == 32 && MAXT > 0 && MAXT <= 6 && !LONG ? 3 : 2, D == 32 && MAXT > 0 && MAXT <= 6 && !LONG ? 3 : 2)))
 void tile_fwd_kernel(
     const float* __restrict__ Q, const float* __restrict__ Kt, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ P, float* __restrict__ O, float* __restrict__ Ocache,
@@ -643,9 +646,7 @@ void tile_fwd_kernel(
                 });
         }
     };
-    // d = 64: a strip too long for the registers of its wavefronts takes the two sweeps inside the same launch (one
-    // launch then serves patterns whose few long strips -- global rows -- would force the sweeps on all)
-    constexpr bool FALLBACK = D == 64 && MAXT > 0;
+    constexpr bool FALLBACK = LONG && MAXT > 0;
     if constexpr (MAXT > 0) {
       if (FALLBACK && cnt > MAXT * WAVES) {
         two_sweeps();
@@ -826,7 +827,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
     const float* __restrict__ K, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ Ocache, float* __restrict__ G,
     float* __restrict__ dQ, const int* __restrict__ rdesc, const int* __restrict__ tcol,
-    int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly) {
+    int L, int nbr, int NB, int nnz, float scale, int hc, Layouts ly, int s0, int ns) {
     static_assert(!ST || (VROW && HAVE_O), "strided heads: row-major operands, Out given");
     constexpr int KH = D / 2;
     // LDS of a wavefront: the V, P and K tiles of one pattern tile, 4 KB per 32 features.  d = 64 needs 20 KB, which
@@ -842,11 +843,12 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_row_kernel(
         return reinterpret_cast<float*>(CARVE ? smem + ww * WB + WB - 128 : smem + WAVES * WB + RED + ww * 128);
     };
     // Last head first: the forward wrote P front to back, so its tail is what the memory-side cache still holds.
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    // This launch covers strips s0 .. s0+ns-1 of every head's strip order.
+    const int item = xcd_remap(blockIdx.x, ns * NB);
     int bh, pos;
-    item_to_head_strip(item, nbr, hc, bh, pos);
+    item_to_head_strip(item, ns, hc, bh, pos);
     bh = NB - 1 - bh;
-    const int4 sd = reinterpret_cast<const int4*>(rdesc)[pos];  // strips longest first: {strip, first tile, tiles, P offset}
+    const int4 sd = reinterpret_cast<const int4*>(rdesc)[s0 + pos];  // strips longest first: {strip, first tile, tiles, P offset}
     const int I = sd.x, t0 = sd.y, cnt = sd.z;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     const int rn = cnt * 32;
@@ -1032,7 +1034,7 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     const float* __restrict__ Q, const float* __restrict__ Vt, const float* __restrict__ P,
     const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
     const int* __restrict__ cdesc, const int* __restrict__ tcdesc, int L, int nbr, int NB, int nnz, float scale,
-    int hc, Layouts ly) {
+    int hc, Layouts ly, int s0, int ns) {
     static_assert(!ST || VROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
     // LDS of a wavefront: d = 32, the P, Q and dO tiles and 64 floats of -g; d = 64, the P tile and two tiles each for
@@ -1044,10 +1046,10 @@ SPION_TILE_KERNEL(WAVES) void tile_bwd_col_kernel(
     static_assert(!CARVE || RED <= WAVES * WB, "the reduction fits in the tile space");
     __shared__ __attribute__((aligned(16))) char smem[CARVE ? WAVES * WB : WAVES * WB + (RED ? RED : 4)];
     float* lds = reinterpret_cast<float*>(CARVE ? smem : smem + WAVES * WB);
-    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int item = xcd_remap(blockIdx.x, ns * NB);  // strips s0 .. s0+ns-1 of every head's strip order
     int bh, pos;
-    item_to_head_strip(item, nbr, hc, bh, pos);
-    const int4 sd = reinterpret_cast<const int4*>(cdesc)[pos];  // strips longest first: {strip, first tile, tiles, 0}
+    item_to_head_strip(item, ns, hc, bh, pos);
+    const int4 sd = reinterpret_cast<const int4*>(cdesc)[s0 + pos];  // strips longest first: {strip, first tile, tiles, 0}
     const int J = sd.x, e0 = sd.y, cnt = sd.z;
     const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
     size_t ib, ob, gb, hbytes, obytes, gbytes;

@@ -42,13 +42,23 @@ def _eager_step(module, args, q, k, v, do):
 
 
 @pytest.mark.parametrize("kind", ["block", "blockmask", "dense", "bf16", "block_views", "blockmask_views", "dense_views",
-                                  "bf16_views", "hybrid", "hybrid_views", "hybridmask_views"])
+                                  "bf16_views", "hybrid", "hybrid_views", "hybridmask_views", "global",
+                                  "global_views"])
 def test_whole_step_graph_replays_match_eager(kind):
     views = kind.endswith("_views")  # heads as views of [B, L, H*d] projections: the strided entry points
     kind = kind.split("_")[0]
     B, H, L, d, bs = 2, 2, 256, 32, 32
     hybrid = kind.startswith("hybrid")  # element-sparse pattern (window + scattered entries): seven launches a step
-    if hybrid:
+    if kind == "global":
+        # a block row and a block column that span the sequence: every pass is two launches, the long strips on the
+        # caller's stream and the others on the handle's side stream, forked and joined by events inside the capture
+        L = 2048
+        pattern = workloads.band_random_block_mask(L // bs, 1, extra_frac=0.05, seed=3)
+        pattern[0, :] = 1.0
+        pattern[:, 0] = 1.0
+        mat = torch.from_numpy(pattern).cuda()
+        kind = "block"
+    elif hybrid:
         bs = 1
         sm, off, col = workloads.window_random_csr(L, 40, 100, seed=3)
         pattern = np.zeros((L, L), dtype=np.float32)
@@ -59,7 +69,7 @@ def test_whole_step_graph_replays_match_eager(kind):
         mat = torch.from_numpy(workloads.band_random_block_mask(L // bs, 1, extra_frac=0.1, seed=3)).cuda()
     cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
     key_mask = torch.ones(B, L)
-    key_mask[1, 200:] = 0
+    key_mask[1, L - 56:] = 0
     key_mask = key_mask.cuda()
     if kind == "block":
         cpp = Attention._blockcuda_compile_module()

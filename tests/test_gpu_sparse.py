@@ -105,11 +105,14 @@ def test_tile_path_with_key_mask(d):
     abi.close()
 
 
-@pytest.mark.parametrize("L,d,with_mask", [(2048, 32, False), (2048, 32, True), (1024, 64, False), (1024, 64, True)])
+@pytest.mark.parametrize("L,d,with_mask", [(2048, 32, False), (2048, 32, True), (1024, 64, False), (1024, 64, True),
+                                           (2048, 64, False), (2048, 64, True)])
 def test_tile_path_global_row_and_column(L, d, with_mask):
     """A block row and a block column that span the whole sequence: rows too long for the register-resident
     forward (two-sweep kernel), long strips walked by several wavefronts in the backward passes, and the
-    one-pass backward without the kept copy of O."""
+    one-pass backward without the kept copy of O.  At L = 2048 the global strips count as long against the rest
+    (more than 32 tiles): every pass is then two launches -- the long strips with eight wavefronts each on the
+    caller's stream, the others on the handle's side stream."""
     from spion_amd import _lib
     bs, B, H = 32, 1, 2
     NB, nb = B * H, L // bs

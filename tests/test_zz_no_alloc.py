@@ -10,12 +10,15 @@ from spion_amd import _lib
 from tests.abi_utils import SparseABI, assert_close, oracle_fwd_bwd
 
 
-def _case(L, bs, NB, p, seed, with_mask):
+def _case(L, bs, NB, p, seed, with_mask, global_strips=False):
     d = 32
     rng = np.random.default_rng(seed)
     nb = L // bs
     mat = (rng.random((nb, nb)) < p).astype(np.float32)
     mat[np.arange(nb), np.arange(nb)] = 1
+    if global_strips:
+        mat[0, :] = 1
+        mat[:, 0] = 1
     sm, off, col = osa.build_csr_from_block_mask(mat, bs)
     abi = SparseABI(d, L, NB, bs, with_mask=with_mask)
     abi.set_pattern(sm, off, col)
@@ -56,6 +59,22 @@ def test_noalloc_backward_matches_rowmajor_backward_twice():
             for name, g_ in zip(("dQ", "dK", "dV"), got):
                 assert_close(g_.cpu().numpy(), ref[name], what=f"no-alloc {name}")
         abi.close()
+
+
+@pytest.mark.gpu
+def test_noalloc_backward_on_a_pattern_with_global_strips():
+    """A block row and a block column that span the sequence: the allocating entry point runs the long strips and the
+    others as two launches on two streams, this one as the same two launches one after the other on the caller's
+    stream (it creates no stream either).  Same kernels, same split: bit-identical results."""
+    abi, _, (Q, K, V, dO), pen = _case(2048, 32, 4, 0.05, 5, False, global_strips=True)
+    O, P = abi.forward_rowmajor(Q, K, V, pen)
+    want = abi.backward_rowmajor(Q, K, V, P, O, dO)
+    got = _noalloc_backward(abi, Q, K, V, P, O, dO)
+    torch.cuda.synchronize()
+    assert abi.last_path() == 1
+    for name, g_, w_ in zip(("dQ", "dK", "dV"), got, want):
+        assert torch.equal(g_, w_), f"{name} of the no-alloc entry differs from spion_attn_backward_rowmajor"
+    abi.close()
 
 
 @pytest.mark.gpu
