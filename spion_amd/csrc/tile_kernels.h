@@ -521,14 +521,15 @@ void tile_fwd_kernel(
     int NB, int nnz, float scale, int s0, int ns, int hc, Layouts ly) {
     static_assert(!ST || KROW, "strided heads: row-major operands");
     constexpr int KH = D / 2;
-    constexpr bool SHARE = D == 32 && MAXT > 0 && MAXT <= 6 && WAVES > 1;  // reduction buffer inside the tile space
+    // reduction buffer inside the tile space
+    constexpr bool SHARE = (D == 32 ? MAXT > 0 && MAXT <= 6 : MAXT > 0) && WAVES > 1;
     __shared__ float lds_own[!SHARE && WAVES > 1 ? WAVES * (D / 32) * 16 * 64 : 1];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
-    // per wavefront: one padded tile (layout changes of P) and, d = 32 with the logits in registers, two 4 KB
-    // tiles filled straight from global memory
-    constexpr int TW = 32 * TS + (D == 32 && MAXT > 0 ? 2 * 1024 + (MASK ? 128 : 0) : 0);
+    // per wavefront: one padded tile (layout changes of P) and, with the logits in registers, 8 KB filled straight
+    // from global memory (d = 32: two tiles in turn; d = 64: the two halves of one tile), plus key penalties
+    constexpr int TW = 32 * TS + (MAXT > 0 ? 2 * 1024 + (MASK ? 128 : 0) : 0);
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][TW];
-    static_assert(!SHARE || WAVES * TW >= WAVES * 16 * 64, "the reduction fits in the tile space");
+    static_assert(!SHARE || WAVES * TW >= WAVES * (D / 32) * 16 * 64, "the reduction fits in the tile space");
     float* lds = SHARE ? &lds_t[0][0] : lds_own;
     // this launch covers strips s0 .. s0+ns-1 of the longest-first order of every head
     const int item = xcd_remap(blockIdx.x, ns * NB);
@@ -711,13 +712,46 @@ void tile_fwd_kernel(
                 }
             }
         } else {
-            float kbuf[2][KH];
-            if (nu > 0) load_kf(Js[0], kbuf[0]);
+            // d = 64: a K tile is two 4 KB tiles (features 0..31 and 32..63) in one place; the operand of tile u is
+            // read out into registers, then the place is requested for tile u + 1, which has the chain to arrive.
+            static_assert(D == 64, "head dimension 32 or 64");
+            const u32x4 wK = rsrc_words(Kt + ib, hbytes);
+            const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+            const int kl = DmaTileF32::voff(l, kld), kx = DmaTileF32::extra_step(kld);
+            const int KHALF = KROW ? 128 : 32 * L * 4;
+            const unsigned lb64 = lds_address(Tb);
+            const auto a_k = [&] {  // features 32h .. 32h+31 of key li: the half-wave's own tile
+                if constexpr (KROW) return DmaTileF32::own8_addr(Tb + h * DmaTileF32::TILE, li);
+                else return DmaTileF32::featcols_addr(Tb + h * DmaTileF32::TILE, li, 0);
+            }();
+            const char* Tm = Tb + 2 * DmaTileF32::TILE + 16 * h;
+            auto issue_k = [&](int u) {
+                DmaTileF32::load(wK, lb64, kl, Js[u] * KSTEP, kx);
+                DmaTileF32::load(wK, lb64 + DmaTileF32::TILE, kl, Js[u] * KSTEP + KHALF, kx);
+                if constexpr (MASK) dma_b32(wM, lb64 + 2 * DmaTileF32::TILE, l * 4, Js[u] * 128);
+            };
+            if (nu > 0) issue_k(0);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
-                    if (u + 1 < MAXT) load_kf(Js[u + 1 < MAXT ? u + 1 : u], kbuf[(u + 1) & 1]);
-                    S[u] = mma_feat_init<D>(kbuf[u & 1], q, chain_init(Js[u]));
+                    wait_vm<0>();
+                    float kf[KH];
+                    DmaTileF32::get32(a_k, kf);
+                    f32x16 init = splat16(0.f);
+                    if constexpr (MASK) {  // minus the key penalties, in the log2 domain
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const f32x4 v = *reinterpret_cast<const f32x4*>(Tm + 32 * g);
+                            init[4 * g + 0] = -LOG2E * v.x;
+                            init[4 * g + 1] = -LOG2E * v.y;
+                            init[4 * g + 2] = -LOG2E * v.z;
+                            init[4 * g + 3] = -LOG2E * v.w;
+                        }
+                    }
+                    wait_lgkm0();
+                    if (u + 1 < MAXT && u + 1 < nu) issue_k(u + 1 < MAXT ? u + 1 : u);
+                    __builtin_amdgcn_sched_barrier(0);
+                    S[u] = mma_feat_init<D>(kf, q, init);
                     m = max16(S[u], m);
                 }
             }
@@ -791,18 +825,35 @@ void tile_fwd_kernel(
                 }
             }
         } else {
-            float vbuf[2][D / 32][16];
-            if (nu > 0) ldr_tile_b<D>(rV, b_voff, Js[0] * 32 * ild * 4, vbuf[0], ild);
+            // d = 64: the V tiles take the place of the K tiles, one tile ahead; after the loads of tile u only the
+            // four P stores of tile u - 1 were issued.
+            const u32x4 wV = rsrc_words(V + ib, hbytes);
+            const int vl = DmaTileF32::voff(l, ild), vx = DmaTileF32::extra_step(ild);
+            const unsigned lb64 = lds_address(Tb);
+            const auto a_v = DmaTileF32::cols_addr(Tb, li, h);
+            auto issue_v = [&](int u) {
+                DmaTileF32::load(wV, lb64, vl, Js[u] * 32 * ild * 4, vx);
+                DmaTileF32::load(wV, lb64 + DmaTileF32::TILE, vl, Js[u] * 32 * ild * 4 + 128, vx);
+            };
+            if (nu > 0) issue_v(0);
 #pragma unroll
             for (int u = 0; u < MAXT; ++u) {
                 if (u < nu) {
                     const int t = w + u * WAVES;
-                    if (u + 1 < MAXT) ldr_tile_b<D>(rV, b_voff, Js[u + 1 < MAXT ? u + 1 : u] * 32 * ild * 4, vbuf[(u + 1) & 1], ild);
-                    float p[16];
+                    wait_vm_upto(u == 0 ? 0 : 4);
+                    float p[16], vb[2][16];
 #pragma unroll
                     for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
-                    store_p(p, t);
-                    mma_b<D>(p, vbuf[u & 1], o);
+                    lds_put_rows(T, li, h, p);
+                    DmaTileF32::get(a_v, vb[0]);
+                    DmaTileF32::get(a_v, vb[1], DmaTileF32::TILE);
+                    f32x4 pl[4];
+                    lds_get_lin(T, l, pl);
+                    wait_lgkm0();
+                    if (u + 1 < MAXT && u + 1 < nu) issue_v(u + 1 < MAXT ? u + 1 : u);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mma_b<D>(p, vb, o);
+                    str_tile_lin(rP, plin, p_base + t * 128, rn, pl);
                 }
             }
         }
