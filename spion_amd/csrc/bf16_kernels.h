@@ -82,9 +82,11 @@ __device__ __forceinline__ void pack16(const float (&p)[16], bf16x8 (&pb)[2]) {
 // tile in flight and no ds_write is spent on it.  One instruction moves 64 x 16 bytes to 1 KB of consecutive LDS
 // addresses starting at M0 (+ the instruction's immediate offset, which is added to the global address as well);
 // which 16-byte piece of global memory a lane fetches is free, so the LDS image of a tile is unpadded rows with
-// the pieces of a row permuted: piece c of tile row r lies at position c ^ swz(r).  With that permutation both
-// kinds of LDS reads are free of bank conflicts: eight consecutive rows of one piece (operand over the head
-// dimension, ds_read_b128) and four consecutive rows of two adjacent pieces (transposing read).
+// the pieces of a row permuted: piece c of tile row r lies at position c ^ swz(r).  With that permutation the
+// transposing reads (four consecutive rows of two adjacent pieces, thirty-two lanes at a time) are free of bank
+// conflicts; the 16-byte reads of an operand over the head dimension (sixteen consecutive rows of one piece at a
+// time, 64 banks) meet rows r and r + 8 on the same banks and take 8 cycles instead of 4 -- measured, and measured
+// not to matter: the LDS pipe is a third busy in these kernels.
 // The loads are inline assembly, so the compiler neither tracks them in its s_waitcnt bookkeeping nor knows that
 // they write LDS: the kernels wait for them with wait_vm<N> (N = loads issued after the ones waited for; loads
 // return in order, and the compiler's own counts can only wait longer than needed) and order them against their

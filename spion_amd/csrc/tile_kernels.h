@@ -214,9 +214,11 @@ __device__ __forceinline__ void lds_get_lin(const float* T, int l, f32x4 (&raw)[
 // clock of loads into registers.  One instruction moves 64 x 16 bytes to 1 KB of consecutive LDS addresses starting
 // at M0 (+ the instruction's immediate offset, which is added to the global address as well): eight 128-byte tile
 // rows.  Which 16-byte piece of a row a lane fetches is free, so the LDS image is unpadded rows with the pieces of
-// row r permuted: piece c lies at position c ^ (r % 8).  Every read the kernels make of such a tile is then free of
-// bank conflicts: a lane's own row in 16-byte pieces (eight consecutive rows of one piece land in eight different
-// positions) and one column of a given row across a half-wave (the 32 floats of a row, in some order).
+// row r permuted: piece c lies at position c ^ (r % 8).  One column of a given row across a half-wave (the 32 floats
+// of a row, in some order) is then free of bank conflicts; a lane's own row in 16-byte pieces, which the 64-bank LDS
+// serves sixteen lanes at a time, meets rows r and r + 8 on the same banks (8 cycles instead of 4 per instruction).
+// A permutation without that (c ^ ((r/2 % 2)*4 + r/4 % 4)) was measured in these kernels and changes nothing: the LDS
+// pipe is not what they wait for, and it costs a second lane offset and more address registers.
 // The loads are inline assembly: the compiler neither counts them in its s_waitcnt bookkeeping nor knows that they
 // write LDS.  The kernels wait for them with wait_vm<N> (N = loads issued after the ones waited for; loads return
 // in order, and the compiler's own counts can then only wait longer than needed) and finish their LDS reads with
