@@ -111,6 +111,42 @@ def test_whole_step_graph_replays_match_eager(kind):
     assert np.isfinite(ref_out.float().cpu().numpy()).all()
 
 
+def test_long_strip_split_follows_the_callers_stream():
+    """A pattern with a global block row and column (every pass: the long strips on the caller's stream, the others on
+    the handle's side stream, joined by events): steps issued on torch's default stream and on two side streams in
+    turn, without host synchronisation in between, give what the first step gave, bit for bit."""
+    B, H, L, d, bs = 2, 2, 2048, 32, 32
+    pattern = workloads.band_random_block_mask(L // bs, 1, extra_frac=0.05, seed=3)
+    pattern[0, :] = 1.0
+    pattern[:, 0] = 1.0
+    mat = torch.from_numpy(pattern).cuda()
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=bs)
+    cpp = Attention._blockcuda_compile_module()
+    module = spion_amd.CUDABlockAttention(cfg, cpp, cpp.init(d, L, B * H, bs))
+    args = (torch.ones(B, L, device="cuda"), mat)
+    q, k, v, do = workloads.qkv(B, H, L, d, seed=5, device="cuda")
+    for t in (q, k, v):
+        t.requires_grad_()
+    ref_out, ref_grads = _eager_step(module, args, q, k, v, do)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.current_stream(), torch.cuda.Stream(), torch.cuda.Stream()]
+    results = []
+    prev = streams[0]
+    for i in range(6):
+        s_ = streams[i % 3]
+        s_.wait_stream(prev)  # the steps share the leaves' .grad and the handle's workspaces: one after the other
+        with torch.cuda.stream(s_):
+            results.append(_eager_step(module, args, q, k, v, do))
+        prev = s_
+    torch.cuda.current_stream().wait_stream(prev)
+    torch.cuda.synchronize()
+    for i, (out, grads) in enumerate(results):
+        assert torch.equal(out, ref_out), f"step {i}: output differs"
+        for name, g, r in zip("qkv", grads, ref_grads):
+            assert torch.equal(g, r), f"step {i}: d{name} differs"
+    cpp.destroy(module.attn_handle)
+
+
 @pytest.mark.parametrize("sparse", [True, False])
 def test_attention_layer_graph_replays_match_eager(sparse):
     """The whole ``Attention`` layer -- one GEMM for the three projections, heads read in place by the strided entry
