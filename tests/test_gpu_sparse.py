@@ -137,6 +137,24 @@ def test_tile_path_global_row_and_column(L, d, with_mask):
     abi.close()
 
 
+@pytest.mark.parametrize("d", [32, 64])
+def test_tile_path_global_strips_beside_one_wavefront_strips(d):
+    """Many heads (2560 strips a launch): the strips other than the global ones take one wavefront each in the
+    backward passes -- the launch on the side stream -- while the global row and column take eight."""
+    L, bs, NB = 2048, 32, 40
+    nb = L // bs
+    mat = _random_block_mask(nb, 0.05, seed=77 + d)
+    mat[3, :] = 1
+    mat[:, 5] = 1
+    sm, off, col = osa.build_csr_from_block_mask(mat, bs)
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    Q, K, V, dO = _inputs(NB, L, d, seed=31, scale=1.1)
+    run_and_check(abi, Q, K, V, dO, tag=f"global strips, NB={NB}, d={d}")
+    assert abi.last_path() == 1
+    abi.close()
+
+
 @pytest.mark.parametrize("with_mask", [False, True])
 def test_tile_path_d64_mixed_strip_lengths_in_one_forward_launch(with_mask):
     """Head dimension 64, four wavefronts per strip, most strips of 12 to 23 tiles and one global block row of 64: the
