@@ -1,4 +1,4 @@
-"""Benchmark configurations 3 and 4 at their full sizes (GPU box only).
+"""Benchmark configurations 3 and 4, and configuration 5's shape in fp32, at their full sizes (GPU box only).
 
 The float64 oracle cannot run a whole batch of these sizes in seconds, so each case combines (a) the oracle on a
 bounded part of the very tensors the full-size launch produced (two of the 64 heads; four of the 256 samples) with
@@ -118,3 +118,49 @@ def test_config3_full_size_step_properties():
         assert torch.isfinite(p_).all(), n_
         moved += int(not torch.equal(p_, before[n_]))
     assert moved == len(before)
+
+
+def test_config5_shape_in_fp32_matches_oracle_on_bounded_rows():
+    """Configuration 5's shape (B=4, H=8, L=16384, d=64, 64x64 blocks, a global block row and column) through the fp32
+    tile kernels at full size with the benchmark's inputs: every pass is two launches here (the global strips with
+    eight wavefronts each, the others beside them).  The oracle restates a bounded part exactly, as in the bf16
+    test of the same shape: for three heads, the complete rows of a few query strips -- the global block row, the
+    first band strip, one from the middle, the last -- and of every strip that attends to two chosen key blocks.
+    O, P and dQ of those rows depend on nothing else, and neither do dK and dV of the two key blocks."""
+    from spion_amd.csr import block_mask_to_csr_host
+    B, H, L, d, bs = 4, 8, 16384, 64, 64
+    NB, nb = B * H, L // bs
+    mat = workloads.config5_mask()
+    sm, off, col = block_mask_to_csr_host(mat, bs)
+    g = torch.Generator().manual_seed(0)
+    Q, K, V, dO = ((torch.randn(NB, L, d, generator=g) * s).cuda() for s in (0.125, 0.125, 0.125, 1.0))
+    abi = SparseABI(d, L, NB, bs, with_mask=False)
+    abi.set_pattern(sm, off, col)
+    O, P = abi.forward(Q, K, V)
+    dQ, dK, dV = abi.backward(Q, K, V, P, dO)
+    torch.cuda.synchronize()
+    assert abi.last_path() == 1
+    for t in (O, P, dQ, dK, dV):
+        assert torch.isfinite(t).all()
+
+    heads = [0, 13, 31]
+    key_blocks = [nb // 3, nb - 2]
+    query_blocks = sorted({0, 1, nb // 2, nb - 1} | {int(i) for c in key_blocks for i in np.nonzero(mat[:, c])[0]})
+    assert len(query_blocks) < 40, "the bounded part stays small"
+    rows = np.concatenate([np.arange(i * bs, (i + 1) * bs) for i in query_blocks])
+    sm_r = np.zeros_like(sm)
+    sm_r[rows] = sm[rows]
+    off_r = np.zeros(L + 1, dtype=off.dtype)
+    np.cumsum(sm_r, out=off_r[1:])
+    col_r = np.concatenate([col[off[r]:off[r + 1]] for r in rows]).astype(col.dtype)
+    assert int(off_r[-1]) == col_r.size
+    sel = lambda t: t[heads]
+    ref = oracle_fwd_bwd(sel(Q), sel(K), sel(V), sel(dO), sm_r, off_r, col_r)
+    for name, t in (("O", O), ("dQ", dQ)):
+        assert_close(sel(t).cpu().numpy()[:, rows], ref[name][:, rows], what=f"config 5 shape, fp32, rows: {name}")
+    p_idx = np.concatenate([np.arange(off[r], off[r + 1]) for r in rows])
+    assert_close(sel(P).cpu().numpy()[:, p_idx], ref["P"], what="config 5 shape, fp32, rows: P")
+    keys = np.concatenate([np.arange(c * bs, (c + 1) * bs) for c in key_blocks])
+    for name, t in (("dK", dK), ("dV", dV)):
+        assert_close(sel(t).cpu().numpy()[:, keys], ref[name][:, keys], what=f"config 5 shape, fp32, key blocks: {name}")
+    abi.close()
