@@ -345,8 +345,9 @@ void spion_block_bf16_attn_backward_strided(void* handle, const void* Q, const v
  * (models/attn.cu:179-262) take feature-major operands, and hand Out and the gradients back feature-major.
  * Here Q, K, V, Out, dO, dQ, dK, dV are all [B][H][L][d] views described as above (a contiguous [NB][L][d]
  * tensor is the layout {H*L*d, L*d, d}); Attn / P is the same [NB][key][query] map as in attn_forward.  Mask:
- * NULL for a handle of spion_dense_init, the [NB][L] penalty for one of spion_densemask_init.  emb_dim 32 and
- * seq_len <= 16384 only.  No copy of Out is kept: the backward takes Out (required). */
+ * NULL for a handle of spion_dense_init, the [NB][L] penalty for one of spion_densemask_init.  seq_len <= 16384;
+ * with emb_dim 64 the forward serves seq_len <= 1024 (the backward all of them).  No copy of Out is kept: the
+ * backward takes Out (required). */
 void spion_dense_forward_strided(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
                                  float* Attn, float* Out,
                                  int heads, const spion_head_layout* in, const spion_head_layout* out);
@@ -363,7 +364,7 @@ void spion_dense_backward_strided(void* handle, const float* Q, const float* K, 
  * one reduction over a few partial maps finishes the mean, so the maps are not read back.  The handle keeps the
  * partial maps: C * seq_len^2 floats, C = the smallest divisor of num_batches with C * seq_len / 32 >= 512, or
  * num_batches itself when it has none; allocated by the first such call (not under HIP graph capture).  All other arguments and results as in
- * spion_dense_forward_strided (Attn is still written: the API returns it). */
+ * spion_dense_forward_strided (Attn is still written: the API returns it).  emb_dim 32 only. */
 void spion_dense_forward_strided_mean(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
                                       float* Attn, float* Out, float* Mean,
                                       int heads, const spion_head_layout* in, const spion_head_layout* out);

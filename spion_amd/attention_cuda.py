@@ -33,9 +33,10 @@ def _empty_heads(shape, interleaved, device):
 class _DenseAttnFunction(torch.autograd.Function):
     """The reference's function (models/attention_cuda.py:18-74) transposes Q and V for the forward and K and
     grad_output for the backward, because its ABI takes feature-major operands, and returns feature-major results
-    as permuted views.  For head dimension 32 and sequences up to 16384 the library's strided entry points
-    (spion_dense_forward_strided / spion_dense_backward_strided) take every tensor row-major -- also as views of
-    [B, L, H*d] projections -- and nothing is transposed or copied; other shapes go through the reference's ABI."""
+    as permuted views.  For head dimension 32 and sequences up to 16384, and head dimension 64 up to 1024, the
+    library's strided entry points (spion_dense_forward_strided / spion_dense_backward_strided) take every tensor
+    row-major -- also as views of [B, L, H*d] projections -- and nothing is transposed or copied; other shapes go
+    through the reference's ABI."""
 
     @staticmethod
     def forward(ctx, query, key, value, mask, module):
@@ -58,7 +59,7 @@ class _DenseAttnFunction(torch.autograd.Function):
             if m.with_mask:
                 pen = (1e6 * (1.0 - mask.repeat(1, H))).to(torch.float32).contiguous()
                 pen_ptr = pen.data_ptr()
-            if m.emit_score_map:
+            if m.emit_score_map and d == 32:
                 # models/model_transformer.py:136-137 averages the returned maps over batch and heads; the kernel
                 # does it while it writes them
                 mean = torch.empty((L, L), dtype=torch.float32, device=dev)
@@ -71,6 +72,9 @@ class _DenseAttnFunction(torch.autograd.Function):
                     m.attn_handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pen_ptr, attn.data_ptr(),
                     out.data_ptr(), H, ctypes.addressof(lay), ctypes.addressof(lout))
             _lib.check_error("attn_forward")
+            if m.emit_score_map and d != 32:  # head dimension 64: one pass over the maps just written
+                from .pattern import mean_score_map
+                m.score_map = mean_score_map(attn.permute(0, 1, 3, 2))
             ctx.save_for_backward(query, key, value, attn, out)
             ctx.set_materialize_grads(False)
             ctx.module = m
@@ -160,7 +164,8 @@ class _DenseAttentionBase(nn.Module):
         self.attn_handle = attn_handle
         self.attn_func = _DenseAttnFunction
         # shapes the strided entry points serve; everything else goes through the reference's ABI
-        self.reads_views = self.emb_dim == 32 and self.seq_len <= 16384
+        self.reads_views = (self.emb_dim == 32 and self.seq_len <= 16384) or (
+            self.emb_dim == 64 and self.seq_len <= 1024)
         # When set, every forward also leaves ``self.score_map`` [L, L]: the mean of the returned maps over batch and
         # heads (what models/model_transformer.py:136-137 computes from them), taken while the maps are written.
         self.emit_score_map = False

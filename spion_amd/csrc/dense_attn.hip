@@ -304,6 +304,149 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     }
 }
 
+// Forward for d = 64, row-major operands, L <= 1024: the same register-resident scheme.  A K or V tile is two 4 KB
+// tiles (features 0..31 and 32..63) in one place per wavefront: the operands of tile u are read out into registers,
+// then the space is requested for tile u + 1, whose loads have the chains of tile u (32 MFMA) to arrive.
+template <bool MASK, int WAVES = 4>
+SPION_TILE_KERNEL(WAVES) void dense_fwd_reg64_kernel(
+    const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
+    const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out,
+    int L, int nbr, int NB, float scale, Layouts ly) {
+    constexpr int D = 64, KH = 32, MAXT = 32 / WAVES;
+    __shared__ float lds[WAVES * 16 * 64];
+    __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
+    __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS + 2 * 1024 + (MASK ? 64 : 0)];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;  // key tiles w, w + WAVES, ... of this wavefront
+    float* T = lds_t[w];  // map tile on its way to memory
+    const char* Tb = reinterpret_cast<const char*>(T + 32 * TS);  // the two halves of a K tile, later of a V tile
+    const unsigned lb = lds_address(Tb);
+    size_t ib, ob, hbytes, obytes;
+    int ild, old_;
+    head_slice<true, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<true, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    const rsrc_t rA = make_rsrc(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const u32x4 wK = rsrc_words(K + ib, hbytes), wV = rsrc_words(V + ib, hbytes);
+    const u32x4 wM = rsrc_words(MASK ? pen + (size_t)bh * L : pen, MASK ? (size_t)L * 4 : 0);
+    const int alin = lin_voff(l, L);
+    const int kl = DmaTileF32::voff(l, ild), kx = DmaTileF32::extra_step(ild);
+    const float c2 = scale * LOG2E;
+    auto issue = [&](const u32x4& r, int J) {
+        DmaTileF32::load(r, lb, kl, J * 32 * ild * 4, kx);
+        DmaTileF32::load(r, lb + DmaTileF32::TILE, kl, J * 32 * ild * 4 + 128, kx);
+    };
+
+    float q[KH];
+    ldr_rows<D>(make_rsrc(Q + ib, hbytes), (li * ild + h * KH) * 4, I * 32 * ild * 4, q);
+#pragma unroll
+    for (int s = 0; s < KH; ++s) q[s] *= c2;
+    settle(q);
+
+    float m = -10.f * LOG2E, z = 0.f;  // models/attn.cu:17
+    f32x16 S[MAXT];
+    {
+        const auto a_k = DmaTileF32::own8_addr(Tb + h * DmaTileF32::TILE, li);  // K[key li][feature 32h + s]
+        const char* Tm = Tb + 2 * DmaTileF32::TILE + 16 * h;
+        auto issue_k = [&](int u) {
+            const int J = w + u * WAVES;
+            issue(wK, J);
+            if constexpr (MASK) dma_b32(wM, lb + 2 * DmaTileF32::TILE, l * 4, J * 128);
+        };
+        if (nu > 0) issue_k(0);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                wait_vm<0>();
+                float kf[KH];
+                DmaTileF32::get32(a_k, kf);
+                f32x16 init = splat16(0.f);
+                if constexpr (MASK) {  // minus the key penalties of the tile, log2 domain
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        const f32x4 x = *reinterpret_cast<const f32x4*>(Tm + 32 * g);
+                        init[4 * g + 0] = -LOG2E * x.x;
+                        init[4 * g + 1] = -LOG2E * x.y;
+                        init[4 * g + 2] = -LOG2E * x.z;
+                        init[4 * g + 3] = -LOG2E * x.w;
+                    }
+                }
+                wait_lgkm0();
+                if (u + 1 < MAXT && u + 1 < nu) issue_k(u + 1);
+                __builtin_amdgcn_sched_barrier(0);
+                S[u] = mma_feat_init<D>(kf, q, init);  // S^T: register = key, lane = query
+                m = max16(S[u], m);
+            }
+        }
+    }
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+#pragma unroll
+    for (int u = 0; u < MAXT; ++u) {
+        if (u < nu) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float e = __builtin_amdgcn_exp2f(S[u][r] - m);
+                S[u][r] = e;
+                z += e;
+            }
+        }
+    }
+    const float m_own = m;
+    z += __shfl_xor(z, 32, 64);
+    if (h == 0) {
+        lds_m[w][li] = m;
+        lds_z[w][li] = z;
+    }
+    __syncthreads();
+    {
+        float Mx = lds_m[0][li];
+#pragma unroll
+        for (int ww = 1; ww < WAVES; ++ww) Mx = fmaxf(Mx, lds_m[ww][li]);
+        float Z = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < WAVES; ++ww) Z += lds_z[ww][li] * __builtin_amdgcn_exp2f(lds_m[ww][li] - Mx);
+        m = Mx;
+        z = Z;
+    }
+    const float rinv = __builtin_amdgcn_exp2f(m_own - m) * (1.0f / z);
+
+    f32x16 o[2] = {splat16(0.f), splat16(0.f)};  // O^T: register = feature (+32), lane = query
+    {
+        const auto a_v = DmaTileF32::cols_addr(Tb, li, h);  // vb[c][s] = V[key acc_row(s, h)][feature 32c + li]
+        if (nu > 0) issue(wV, w);
+#pragma unroll
+        for (int u = 0; u < MAXT; ++u) {
+            if (u < nu) {
+                const int J = w + u * WAVES;
+                // in flight after the loads of V tile u: the four map stores of tile u - 1
+                if (u == 0) wait_vm<0>();
+                else wait_vm<4>();
+                float p[16], vb[2][16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) p[r] = S[u][r] * rinv;
+                lds_put_cols(T, li, h, p);  // T[key][query]: the map is stored key-major
+                DmaTileF32::get(a_v, vb[0]);
+                DmaTileF32::get(a_v, vb[1], DmaTileF32::TILE);
+                f32x4 pl[4];
+                lds_get_lin(T, l, pl);
+                wait_lgkm0();
+                if (u + 1 < MAXT && u + 1 < nu) issue(wV, w + (u + 1) * WAVES);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < 2; ++c)
+#pragma unroll
+                    for (int s = 0; s < 16; ++s)
+                        o[c] = __builtin_amdgcn_mfma_f32_32x32x2f32(vb[c][s], p[s], o[c], 0, 0, 0);
+                str_tile_lin(rA, alin, (J * 32 * L + I * 32) * 4, L, pl);
+            }
+        }
+    }
+    reduce_store_rows<WAVES>(o[0], Out + ob, I * 32, w, li, h, lds, old_);
+    __syncthreads();
+    reduce_store_rows<WAVES>(o[1], Out + ob + 32, I * 32, w, li, h, lds, old_);
+}
+
 // Forward for d = 32 and any L: two sweeps over the key tiles of a query strip, four wavefronts sharing the strip.
 // Sweep 1 keeps a running maximum and sum of exponentials per wavefront (merged over the work-group afterwards);
 // sweep 2 recomputes the logits with -M folded into the chain's initial accumulator, writes the map and
@@ -793,6 +936,166 @@ SPION_TILE_KERNEL(WAVES) void dense_bwd_col32_kernel(
     reduce_store<D, WAVES, true>(out, dV + hb, J * 32, w, li, h, lds, L);
 }
 
+// Backward passes for d = 64, row-major operands (the strided entry points): the d = 64 schedule of the sparse tile
+// kernels (tile_kernels.h) on the dense map.  A wavefront's LDS holds five 4 KB tiles -- the map tile and two
+// 32-feature halves each of the two operand tiles -- 20 KB, so that four wavefronts take 80 KB and two work-groups
+// fill a CU to the last byte; the buffer of the final reduction lies inside the tile space, a barrier in between.
+template <int WAVES>
+SPION_TILE_KERNEL(WAVES) void dense_bwd_row64_kernel(
+    const float* __restrict__ K, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dO, const float* __restrict__ Out, float* __restrict__ G, float* __restrict__ dQ,
+    int L, int nbr, int NB, float scale, Layouts ly) {
+    constexpr int D = 64, KH = 32, WB = 5 * DmaTileF32::TILE;
+    static_assert(WAVES * 2 * 16 * 64 * 4 <= WAVES * WB, "the reduction fits in the tile space");
+    __shared__ __attribute__((aligned(16))) char smem[WAVES * WB];
+    // last head first: the tail of the map is what the memory-side cache still holds after the forward
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = NB - 1 - item / nbr, I = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<true, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<true, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<true, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+
+    float go[KH], oo[KH];
+    ldr_rows<D>(make_rsrc(dO + ob, obytes), (li * old_ + h * KH) * 4, I * 32 * old_ * 4, go);
+    ldr_rows<D>(make_rsrc(Out + ob, obytes), (li * old_ + h * KH) * 4, I * 32 * old_ * 4, oo);
+    float g = 0.f;
+#pragma unroll
+    for (int s = 0; s < KH; ++s) g = fmaf(go[s], oo[s], g);
+    g += __shfl_xor(g, 32, 64);
+    if (w == 0 && h == 0) G[(size_t)bh * L + I * 32 + li] = -g;
+    const f32x16 gneg = splat16(-g);
+
+    f32x16 acc[2] = {splat16(0.f), splat16(0.f)};  // dQ: register = query, lane = feature
+    const char* Tv = smem + w * WB;
+    const char* Tk = Tv + 2 * DmaTileF32::TILE;
+    const char* Tp = Tv + 4 * DmaTileF32::TILE;
+    const unsigned lv = lds_address(Tv), lk = lv + 2 * DmaTileF32::TILE, lp = lv + 4 * DmaTileF32::TILE;
+    const u32x4 wV = rsrc_words(V + ib, hbytes), wK = rsrc_words(K + ib, hbytes);
+    const u32x4 wP = rsrc_words(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const int vl = DmaTileF32::voff(l, ild), pl = DmaTileF32::voff(l, L);
+    const int vx = DmaTileF32::extra_step(ild), px = DmaTileF32::extra_step(L);
+    const auto a_v = DmaTileF32::own8_addr(Tv + h * DmaTileF32::TILE, li);  // V[key li][feature 32h + s]
+    const auto a_p = DmaTileF32::cols_addr(Tp, li, h);                      // P[query li][key acc_row(r, h)]
+    const auto a_k = DmaTileF32::cols_addr(Tk, li, h);                      // K[key acc_row(s, h)][feature li (+32)]
+    auto issue = [&](int J) {
+        DmaTileF32::load(wV, lv, vl, J * 32 * ild * 4, vx);
+        DmaTileF32::load(wV, lv + DmaTileF32::TILE, vl, J * 32 * ild * 4 + 128, vx);
+        DmaTileF32::load<true>(wP, lp, pl, (J * 32 * L + I * 32) * 4, px);
+        DmaTileF32::load(wK, lk, vl, J * 32 * ild * 4, vx);
+        DmaTileF32::load(wK, lk + DmaTileF32::TILE, vl, J * 32 * ild * 4 + 128, vx);
+    };
+    if (nu > 0) {
+        issue(w);
+        for (int i = 0; i < nu; ++i) {
+            wait_vm<0>();
+            float vt[KH], pr[16], kb[2][16];
+            DmaTileF32::get32(a_v, vt);
+            DmaTileF32::get(a_p, pr);
+            DmaTileF32::get(a_k, kb[0]);
+            DmaTileF32::get(a_k, kb[1], DmaTileF32::TILE);
+            wait_lgkm0();
+            if (i + 1 < nu) issue(w + (i + 1) * WAVES);
+            __builtin_amdgcn_sched_barrier(0);
+            f32x16 dp = mma_feat_init<D>(vt, go, gneg);  // register = key, lane = query: dO_i . v_j - g_i
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pr[r];
+            mma_b<D>(ds, kb, acc);
+        }
+    }
+    if (WAVES > 1) __syncthreads();  // every wavefront is done with its tiles
+    acc[0] *= scale;
+    acc[1] *= scale;
+    reduce_store<D, WAVES>(acc, dQ + gb, I * 32, w, li, h, reinterpret_cast<float*>(smem), gld);
+}
+
+// -g does not fit beside the tiles: each lane loads the value of query row lane % 32 of the next tile with an ordinary
+// load, and one extra MFMA step -- A = that value in the lower half-wave, zero in the upper, B = 1 -- spreads it over
+// the accumulator the dP chain starts from.
+template <int WAVES>
+SPION_TILE_KERNEL(WAVES) void dense_bwd_col64_kernel(
+    const float* __restrict__ Q, const float* __restrict__ V, const float* __restrict__ Attn,
+    const float* __restrict__ dO, const float* __restrict__ G, float* __restrict__ dK, float* __restrict__ dV,
+    int L, int nbr, int NB, float scale, Layouts ly) {
+    constexpr int D = 64, KH = 32, WB = 5 * DmaTileF32::TILE;
+    static_assert(WAVES * 2 * 16 * 64 * 4 <= WAVES * WB, "the reduction fits in the tile space");
+    __shared__ __attribute__((aligned(16))) char smem[WAVES * WB];
+    const int item = xcd_remap(blockIdx.x, nbr * NB);
+    const int bh = item / nbr, J = item % nbr;
+    const int w = wave_index(), l = threadIdx.x & 63, h = l >> 5, li = l & 31;
+    const int nu = nbr > w ? (nbr - w + WAVES - 1) / WAVES : 0;
+    size_t ib, ob, gb, hbytes, obytes, gbytes;
+    int ild, old_, gld;
+    head_slice<true, D>(ly.in, ly.H, bh, L, ib, ild, hbytes);
+    head_slice<true, D>(ly.out, ly.H, bh, L, ob, old_, obytes);
+    head_slice<true, D>(ly.grad, ly.H, bh, L, gb, gld, gbytes);
+    const rsrc_t rG = make_rsrc(G + (size_t)bh * L, (size_t)L * 4);
+
+    float vt[KH];
+    ldr_rows<D>(make_rsrc(V + ib, hbytes), (li * ild + h * KH) * 4, J * 32 * ild * 4, vt);
+
+    f32x16 ak[2] = {splat16(0.f), splat16(0.f)}, av[2] = {splat16(0.f), splat16(0.f)};  // register = key, lane = feature
+    const char* Tp = smem + w * WB;
+    const char* Tq = Tp + DmaTileF32::TILE;
+    const char* To = Tp + 3 * DmaTileF32::TILE;
+    const unsigned lp = lds_address(Tp), lq = lp + DmaTileF32::TILE, lo = lp + 3 * DmaTileF32::TILE;
+    const u32x4 wQ = rsrc_words(Q + ib, hbytes), wO = rsrc_words(dO + ob, obytes);
+    const u32x4 wP = rsrc_words(Attn + (size_t)bh * L * L, (size_t)L * L * 4);
+    const int ql = DmaTileF32::voff(l, ild), ol = DmaTileF32::voff(l, old_), pl = DmaTileF32::voff(l, L);
+    const int qx = DmaTileF32::extra_step(ild), ox = DmaTileF32::extra_step(old_), px = DmaTileF32::extra_step(L);
+    const auto a_p = DmaTileF32::own_addr(Tp, li, h, 2);  // P[query acc_row(r, h)][key li]
+    const auto a_q = DmaTileF32::cols_addr(Tq, li, h);    // Q[query acc_row(s, h)][feature li (+32)]
+    const auto a_o = DmaTileF32::cols_addr(To, li, h);    // dO[query acc_row(s, h)][feature li (+32)]
+    const auto a_go = DmaTileF32::own8_addr(To + h * DmaTileF32::TILE, li);  // dO[query li][feature 32h + s]
+    auto issue = [&](int I) {
+        DmaTileF32::load<true>(wP, lp, pl, (J * 32 * L + I * 32) * 4, px);
+        DmaTileF32::load(wQ, lq, ql, I * 32 * ild * 4, qx);
+        DmaTileF32::load(wQ, lq + DmaTileF32::TILE, ql, I * 32 * ild * 4 + 128, qx);
+        DmaTileF32::load(wO, lo, ol, I * 32 * old_ * 4, ox);
+        DmaTileF32::load(wO, lo + DmaTileF32::TILE, ol, I * 32 * old_ * 4 + 128, ox);
+    };
+    settle(vt);
+    if (nu > 0) {
+        issue(w);
+        float gl = ld1(rG, li * 4, w * 128);
+        for (int i = 0; i < nu; ++i) {
+            wait_vm<0>();
+            settle(gl);
+            const float ga = h == 0 ? gl : 0.f;
+            float pc[16], qb[2][16], ob[2][16], go[KH];
+            DmaTileF32::get32(a_go, go);
+            DmaTileF32::get(a_p, pc);
+            DmaTileF32::get(a_q, qb[0]);
+            DmaTileF32::get(a_q, qb[1], DmaTileF32::TILE);
+            DmaTileF32::get(a_o, ob[0]);
+            DmaTileF32::get(a_o, ob[1], DmaTileF32::TILE);
+            wait_lgkm0();
+            if (i + 1 < nu) {
+                issue(w + (i + 1) * WAVES);
+                gl = ld1(rG, li * 4, (w + (i + 1) * WAVES) * 128);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const f32x16 init = __builtin_amdgcn_mfma_f32_32x32x2f32(ga, 1.0f, splat16(0.f), 0, 0, 0);  // -g_i in every column
+            f32x16 dp = mma_feat_init<D>(go, vt, init);  // register = query, lane = key
+            float ds[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) ds[r] = dp[r] * pc[r];
+            mma_b<D>(ds, qb, ak);
+            mma_b<D>(pc, ob, av);
+        }
+    }
+    if (WAVES > 1) __syncthreads();  // every wavefront is done with its tiles
+    ak[0] *= scale;
+    ak[1] *= scale;
+    reduce_store<D, WAVES>(ak, dK + gb, J * 32, w, li, h, reinterpret_cast<float*>(smem), gld);
+    if (WAVES > 1) __syncthreads();
+    reduce_store<D, WAVES>(av, dV + gb, J * 32, w, li, h, reinterpret_cast<float*>(smem), gld);
+}
+
 // -------------------------------------------------------------------------------------------------
 struct DenseAttn {
     HandleHeader hdr;
@@ -944,13 +1247,14 @@ void dense_backward(void* h, const float* Qt, const float* Kt, const float* V, c
     check_launch("dense_bwd kernels");
 }
 
-// Row-major / strided heads (d = 32, L <= 16384): Q, K, V, Out, dO and the gradients are [B][H][L][32] views with
-// one layout per tensor group (tile_kernels.h), read and written in place; the map stays [NB][key][query].
+// Row-major / strided heads (L <= 16384; d = 64: the forward for L <= 1024 only): Q, K, V, Out, dO and the gradients
+// are [B][H][L][d] views with one layout per tensor group (tile_kernels.h), read and written in place; the map stays
+// [NB][key][query].
 static DenseAttn* dense_strided_handle(void* h, const char* who, int heads, const HeadLayout* const* lays, int n) {
     DenseAttn* a = as_dense(h, who);
     if (!a) return nullptr;
-    if (a->d != 32 || a->L > 16384) {
-        set_error("%s: strided heads are served for emb_dim 32 and seq_len <= 16384 only", who);
+    if (a->L > 16384) {  // 32-bit byte offsets into one head's map: L*L*4 < 2^31
+        set_error("%s: strided heads are served for seq_len <= 16384 only", who);
         return nullptr;
     }
     if (heads <= 0 || a->NB % heads) {
@@ -1005,6 +1309,20 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB), block4(64 * 4);
     a->out_key = nullptr;  // no kept copy: the strided backward is handed Out
+    if (a->d == 64) {
+        if (Mean || nbr > 32) {
+            set_error("%s: emb_dim 64 is served for seq_len <= 1024 and without the mean map", who);
+            return;
+        }
+        if (a->has_mask)
+            hipLaunchKernelGGL(dense_fwd_reg64_kernel<true>, grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out,
+                               a->L, nbr, a->NB, a->scale, ly);
+        else
+            hipLaunchKernelGGL(dense_fwd_reg64_kernel<false>, grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out,
+                               a->L, nbr, a->NB, a->scale, ly);
+        check_launch("dense_fwd kernels");
+        return;
+    }
     if (Mean) {
         // C partial maps: the smallest divisor of NB that fills the device -- one eight-wavefront work-group per CU
         // for the register-resident form (measured at B=256, H=2, L=1024: 0.95 ms with 256 work-groups, 1.05 with
@@ -1120,10 +1438,17 @@ void dense_backward_strided(void* h, const float* Q, const float* K, const float
     ly.H = heads;
     const int nbr = a->L / 32;
     const dim3 grid(nbr * a->NB), block4(64 * 4);
-    hipLaunchKernelGGL((dense_bwd_row32_kernel<4, true>), grid, block4, 0, a->hdr.stream, K, V, P, dO, Out,
-                       a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale, ly);
-    hipLaunchKernelGGL((dense_bwd_col32_kernel<4, true>), grid, block4, 0, a->hdr.stream, Q, V, P, dO, a->ws_rowsum, dK,
-                       dV, a->L, nbr, a->NB, a->scale, ly);
+    if (a->d == 64) {
+        hipLaunchKernelGGL(dense_bwd_row64_kernel<4>, grid, block4, 0, a->hdr.stream, K, V, P, dO, Out, a->ws_rowsum,
+                           dQ, a->L, nbr, a->NB, a->scale, ly);
+        hipLaunchKernelGGL(dense_bwd_col64_kernel<4>, grid, block4, 0, a->hdr.stream, Q, V, P, dO, a->ws_rowsum, dK, dV,
+                           a->L, nbr, a->NB, a->scale, ly);
+    } else {
+        hipLaunchKernelGGL((dense_bwd_row32_kernel<4, true>), grid, block4, 0, a->hdr.stream, K, V, P, dO, Out,
+                           a->ws_rowsum, dQ, a->L, nbr, a->NB, a->scale, ly);
+        hipLaunchKernelGGL((dense_bwd_col32_kernel<4, true>), grid, block4, 0, a->hdr.stream, Q, V, P, dO, a->ws_rowsum,
+                           dK, dV, a->L, nbr, a->NB, a->scale, ly);
+    }
     check_launch("dense_bwd kernels");
 }
 

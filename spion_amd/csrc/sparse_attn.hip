@@ -471,8 +471,9 @@ struct SparseAttn {
     size_t ws_ds_count = 0;
     float* ws_part = nullptr;    // [NB][slots][slot floats] partial results of the chunks of long strips (bf16 family)
     size_t ws_part_floats = 0;
-    // Side stream (default priority) on which the fp32 backward runs the few long strips of a pattern beside the
-    // launch of the others; forked from and joined to the caller's stream by the two events.  Created at first use.
+    // Side stream (default priority) of the fp32 tile passes on a pattern with a few long strips: the long strips'
+    // launch goes to the caller's stream, the launch of all other strips to this one, beside it; forked from and
+    // joined to the caller's stream by the two events.  Created when such a pattern is analysed, never inside a call.
     hipStream_t side = nullptr;
     hipEvent_t side_fork = nullptr, side_join = nullptr;
     bool ensure_side() {
@@ -1341,8 +1342,8 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
     const float* ocache = Out ? Out : ocache_for_backward(a, P);
     // A pattern with a few strips far longer than the rest (global rows, global columns): those run four wavefronts
     // to a strip in a small launch of their own, all other strips in a launch with the wavefront count their own
-    // number calls for -- instead of four wavefronts to every strip of the pattern because of the few.  The small
-    // launch goes to a side stream of the handle (made when such a pattern is analysed), beside the large one; without
+    // number calls for -- instead of four wavefronts to every strip of the pattern because of the few.  The large
+    // launch goes to a side stream of the handle (made when such a pattern is analysed), beside the small one; without
     // that stream the two launches follow one another, with the same results.
     static const bool no_split = getenv("SPION_NO_LONG_SPLIT") != nullptr;
     const int nlr = pi.n_long_rows, nlc = pi.n_long_cols;
