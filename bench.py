@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the sparse-attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_global|north_star_bf16|dense_phase|config1|config1_b256|config2|config3|config4|config5|config5_fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload north_star|north_star_bs64|north_star_global|north_star_bf16|dense_phase|dense_phase_d64|config1|config1_b256|config2|config3|config4|config5|config5_fp32]
 
 A step is one forward+backward of the drop-in sparse attention module (``CUDABlockAttention``:
 layout preparation, the C-ABI forward, the C-ABI backward) on seeded synthetic inputs that are
@@ -400,16 +400,17 @@ def bench_bf16_scale_up(args, dev, shape="config5"):
     return result
 
 
-def bench_dense_phase(args, dev):
+def bench_dense_phase(args, dev, d=32):
     """Dense-phase attention (the phase that feeds pattern discovery) at configuration 3's layer shape: B=256, H=2,
     L=1024, d=32, fp32, forward + backward of the ``CUDAAttention`` module, which materialises the full
-    [B, H, L, L] probability map (2.1 GB) as the reference does.  FLOPs 12*L*L*d*NB; MFMA-bound."""
+    [B, H, L, L] probability map (2.1 GB) as the reference does.  FLOPs 12*L*L*d*NB; MFMA-bound.
+    d=64 (``dense_phase_d64``): the same FLOPs with half the batch."""
     import spion_amd
     from oracle import sparse_attention as osa
     from spion_amd import _lib, workloads
     from spion_amd.attention import Attention
 
-    B, H, L, d = 256, 2, 1024, 32
+    B, H, L = (256 if d == 32 else 128), 2, 1024
     NB = B * H
     cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
     cpp = Attention._cuda_compile_module()
@@ -461,10 +462,12 @@ def bench_dense_phase(args, dev):
     _lib.check_error("dense backward (row-major)")
     # the same forward leaving the mean of all maps as well (what pattern discovery reads)
     mean_map = torch.empty(L, L, device=dev)
-    t_fwd_mean = _event_ms(lambda: core.spion_dense_forward_strided_mean(
-        handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), None, attn.data_ptr(), out_r.data_ptr(),
-        mean_map.data_ptr(), H, A, A), max(10, args.steps // 4))
-    _lib.check_error("dense forward with mean (row-major)")
+    t_fwd_mean = None
+    if d == 32:  # the mean-emitting forward is served for head dimension 32
+        t_fwd_mean = _event_ms(lambda: core.spion_dense_forward_strided_mean(
+            handle, Qr.data_ptr(), Kr.data_ptr(), Vr.data_ptr(), None, attn.data_ptr(), out_r.data_ptr(),
+            mean_map.data_ptr(), H, A, A), max(10, args.steps // 4))
+        _lib.check_error("dense forward with mean (row-major)")
     del Qr, Kr, Vr, dOr, out_r, gq, gk, gv, mean_map
 
     # forward kernel alone at the C ABI (operands in the layouts it takes: Qt, Vt feature-major)
@@ -485,15 +488,19 @@ def bench_dense_phase(args, dev):
                                                 dv.data_ptr()), max(10, args.steps // 4))
     _lib.check_error("dense backward")
     alg_flops = 12.0 * L * L * d * NB
-    roof = dict(bound="mfma", kernel="dense_fwd_reg_kernel", achieved=alg_flops / 3.0 / t_fwd_rm / 1e9,
+    k_fwd = "dense_fwd_reg_kernel" if d == 32 else "dense_fwd_reg64_kernel"
+    k_bwd = f"dense_bwd_row{d}_kernel + dense_bwd_col{d}_kernel"
+    roof = dict(bound="mfma", kernel=k_fwd, achieved=alg_flops / 3.0 / t_fwd_rm / 1e9,
                 peak=PEAK_FP32_MFMA_TFLOPS, unit="TFLOP/s", traffic=None)
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd_rm, 4),
-                         "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd_rm, 4)}
+    roof["kernel_ms"] = {k_fwd: round(t_fwd_rm, 4), k_bwd: round(t_bwd_rm, 4)}
     roof["backward_frac"] = alg_flops * 2.0 / 3.0 / t_bwd_rm / 1e9 / PEAK_FP32_MFMA_TFLOPS
-    roof["forward_with_mean_ms"] = round(t_fwd_mean, 4)  # spion_dense_forward_strided_mean: maps + their mean
-    roof["reference_abi_kernel_ms"] = {"dense_fwd_reg_kernel": round(t_fwd, 4),
-                                       "dense_bwd_row32_kernel + dense_bwd_col32_kernel": round(t_bwd, 4)}
+    if t_fwd_mean is not None:
+        roof["forward_with_mean_ms"] = round(t_fwd_mean, 4)  # spion_dense_forward_strided_mean: maps + their mean
+    # the feature-major ABI: the same kernels at d = 32, the two-sweep kernels with operand-layout loads at d = 64
+    roof["reference_abi_kernel_ms"] = {
+        k_fwd if d == 32 else "dense_fwd_kernel": round(t_fwd, 4),
+        k_bwd if d == 32 else "dense_bwd_row_kernel + dense_bwd_col_kernel": round(t_bwd, 4)}
     result = {
         "metric": "dense-phase attn fwd+bwd effective TFLOP/s (12*L*L*d*NB FLOPs / step time), 1 GPU",
         "value": alg_flops / ms_step / 1e9, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -570,8 +577,8 @@ def main():
     if args.workload == "config5":
         print(json.dumps(bench_bf16_scale_up(args, dev)))
         return
-    if args.workload == "dense_phase":
-        print(json.dumps(bench_dense_phase(args, dev)))
+    if args.workload in ("dense_phase", "dense_phase_d64"):
+        print(json.dumps(bench_dense_phase(args, dev, 32 if args.workload == "dense_phase" else 64)))
         return
     if args.workload == "north_star_bf16":
         print(json.dumps(bench_bf16_scale_up(args, dev, "north_star")))
