@@ -346,7 +346,7 @@ void spion_block_bf16_attn_backward_strided(void* handle, const void* Q, const v
  * Here Q, K, V, Out, dO, dQ, dK, dV are all [B][H][L][d] views described as above (a contiguous [NB][L][d]
  * tensor is the layout {H*L*d, L*d, d}); Attn / P is the same [NB][key][query] map as in attn_forward.  Mask:
  * NULL for a handle of spion_dense_init, the [NB][L] penalty for one of spion_densemask_init.  seq_len <= 16384;
- * with emb_dim 64 the forward serves seq_len <= 1024 (the backward all of them).  No copy of Out is kept: the
+ * with emb_dim 64 the forward serves seq_len <= 2048 (the backward all of them).  No copy of Out is kept: the
  * backward takes Out (required). */
 void spion_dense_forward_strided(void* handle, const float* Q, const float* K, const float* V, const float* Mask,
                                  float* Attn, float* Out,

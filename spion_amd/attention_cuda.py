@@ -33,7 +33,7 @@ def _empty_heads(shape, interleaved, device):
 class _DenseAttnFunction(torch.autograd.Function):
     """The reference's function (models/attention_cuda.py:18-74) transposes Q and V for the forward and K and
     grad_output for the backward, because its ABI takes feature-major operands, and returns feature-major results
-    as permuted views.  For head dimension 32 and sequences up to 16384, and head dimension 64 up to 1024, the
+    as permuted views.  For head dimension 32 and sequences up to 16384, and head dimension 64 up to 2048, the
     library's strided entry points (spion_dense_forward_strided / spion_dense_backward_strided) take every tensor
     row-major -- also as views of [B, L, H*d] projections -- and nothing is transposed or copied; other shapes go
     through the reference's ABI."""
@@ -165,7 +165,7 @@ class _DenseAttentionBase(nn.Module):
         self.attn_func = _DenseAttnFunction
         # shapes the strided entry points serve; everything else goes through the reference's ABI
         self.reads_views = (self.emb_dim == 32 and self.seq_len <= 16384) or (
-            self.emb_dim == 64 and self.seq_len <= 1024)
+            self.emb_dim == 64 and self.seq_len <= 2048)
         # When set, every forward also leaves ``self.score_map`` [L, L]: the mean of the returned maps over batch and
         # heads (what models/model_transformer.py:136-137 computes from them), taken while the maps are written.
         self.emit_score_map = False

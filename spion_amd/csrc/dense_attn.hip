@@ -304,7 +304,7 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     }
 }
 
-// Forward for d = 64, row-major operands, L <= 1024: the same register-resident scheme.  A K or V tile is two 4 KB
+// Forward for d = 64, row-major operands, L <= 256 * WAVES: the same register-resident scheme.  A K or V tile is two 4 KB
 // tiles (features 0..31 and 32..63) in one place per wavefront: the operands of tile u are read out into registers,
 // then the space is requested for tile u + 1, whose loads have the chains of tile u (32 MFMA) to arrive.
 template <bool MASK, int WAVES = 4>
@@ -312,7 +312,7 @@ SPION_TILE_KERNEL(WAVES) void dense_fwd_reg64_kernel(
     const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ V,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out,
     int L, int nbr, int NB, float scale, Layouts ly) {
-    constexpr int D = 64, KH = 32, MAXT = 32 / WAVES;
+    constexpr int D = 64, KH = 32, MAXT = 8;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     __shared__ __attribute__((aligned(16))) float lds_t[WAVES][32 * TS + 2 * 1024 + (MASK ? 64 : 0)];
@@ -1247,7 +1247,7 @@ void dense_backward(void* h, const float* Qt, const float* Kt, const float* V, c
     check_launch("dense_bwd kernels");
 }
 
-// Row-major / strided heads (L <= 16384; d = 64: the forward for L <= 1024 only): Q, K, V, Out, dO and the gradients
+// Row-major / strided heads (L <= 16384; d = 64: the forward for L <= 2048 only): Q, K, V, Out, dO and the gradients
 // are [B][H][L][d] views with one layout per tensor group (tile_kernels.h), read and written in place; the map stays
 // [NB][key][query].
 static DenseAttn* dense_strided_handle(void* h, const char* who, int heads, const HeadLayout* const* lays, int n) {
@@ -1310,16 +1310,22 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
     const dim3 grid(nbr * a->NB), block4(64 * 4);
     a->out_key = nullptr;  // no kept copy: the strided backward is handed Out
     if (a->d == 64) {
-        if (Mean || nbr > 32) {
-            set_error("%s: emb_dim 64 is served for seq_len <= 1024 and without the mean map", who);
+        if (Mean || nbr > 64) {
+            set_error("%s: emb_dim 64 is served for seq_len <= 2048 and without the mean map", who);
             return;
         }
-        if (a->has_mask)
-            hipLaunchKernelGGL(dense_fwd_reg64_kernel<true>, grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out,
-                               a->L, nbr, a->NB, a->scale, ly);
-        else
-            hipLaunchKernelGGL(dense_fwd_reg64_kernel<false>, grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn, Out,
-                               a->L, nbr, a->NB, a->scale, ly);
+        // at most eight logit tiles per wavefront: four wavefronts up to L = 1024, eight up to 2048
+#define SPION_LAUNCH(MM, W)                                                                                          \
+    hipLaunchKernelGGL((dense_fwd_reg64_kernel<MM, W>), grid, dim3(64 * W), 0, a->hdr.stream, Q, K, V, Mask, Attn, Out, \
+                       a->L, nbr, a->NB, a->scale, ly)
+        if (nbr <= 32) {
+            if (a->has_mask) SPION_LAUNCH(true, 4);
+            else SPION_LAUNCH(false, 4);
+        } else {
+            if (a->has_mask) SPION_LAUNCH(true, 8);
+            else SPION_LAUNCH(false, 8);
+        }
+#undef SPION_LAUNCH
         check_launch("dense_fwd kernels");
         return;
     }

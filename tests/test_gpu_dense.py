@@ -89,7 +89,7 @@ def _views(B, H, L, d, layout, n, seed, fill=None):
     ("plain", 256, False, 32), ("proj", 256, True, 32), ("fused", 160, False, 32), ("proj", 1024, False, 32),
     ("proj", 1088, True, 32), ("fused", 2048, False, 32),
     ("plain", 256, False, 64), ("proj", 288, True, 64), ("fused", 160, False, 64), ("proj", 1024, True, 64),
-    ("fused", 32, False, 64)])
+    ("fused", 32, False, 64), ("proj", 2048, False, 64), ("plain", 1056, True, 64)])
 def test_dense_strided_entry_points(layout, L, with_mask, d):
     """spion_dense_forward_strided / spion_dense_backward_strided: row-major heads, possibly interleaved in the
     memory of [B, L, H*d] projections, against the oracle and -- d = 32, where both entries run the same kernels --
@@ -156,9 +156,9 @@ def test_dense_backward_without_the_kept_output():
         assert_close(got[name], ref, what=f"dense, map at another address: {name}")
 
 
-@pytest.mark.parametrize("with_mask,d,L", [(False, 32, 128), (True, 32, 128), (True, 64, 192), (False, 64, 2048)])
+@pytest.mark.parametrize("with_mask,d,L", [(False, 32, 128), (True, 32, 128), (True, 64, 192), (False, 64, 2080)])
 def test_dense_modules_autograd(with_mask, d, L):
-    """The dense modules against float64 autograd; d = 64 takes the row-major entry points up to L = 1024 and the
+    """The dense modules against float64 autograd; d = 64 takes the row-major entry points up to L = 2048 and the
     reference's ABI beyond."""
     import spion_amd
 
