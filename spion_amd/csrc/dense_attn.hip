@@ -99,9 +99,9 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
     }
 }
 
-// Forward for d = 32 and L <= 1024 (at most 32 key tiles per query strip): the register-resident scheme of the
-// sparse forward (tile_kernels.h) on the dense layouts.  Each of the four wavefronts keeps the logit tiles of its
-// share of the strip (at most 8) in registers, so a tile costs one QK^T chain and one PV chain instead of the
+// Forward for d = 32 and L <= 2048: the register-resident scheme of the sparse forward (tile_kernels.h) on the
+// dense layouts.  Each of the WAVES wavefronts (four up to L = 1024, eight beyond) keeps the logit tiles of its
+// share of the strip (at most MAXT) in registers, so a tile costs one QK^T chain and one PV chain instead of the
 // two-sweep kernel's three; K and V tiles go from global memory straight into wave-private LDS tiles, map tiles
 // change layout in a padded LDS tile and leave as four 16-byte instructions, non-temporally.
 // RM: Q, V and Out are row-major head slices located by `ly` (heads possibly interleaved in [B][L][H*32] memory,
@@ -111,13 +111,13 @@ __global__ __launch_bounds__(64 * DENSE_WAVES) void dense_fwd_kernel(
 // heads c, c + C, c + 2C, ... one after the other and adds every probability tile it writes to a register tile of
 // its own, so the sum costs sixteen additions per tile and, once per work-group, the store of its [L][32] slab of
 // Part[c] (key-major like the map).  The mean over batch and heads is then one small reduction of the C partial maps.
-template <bool MASK, bool RM = false, int WAVES = 4, bool MEAN = false>
+template <bool MASK, bool RM = false, int WAVES = 4, bool MEAN = false, int MAXT = 32 / WAVES>
 SPION_TILE_KERNEL(WAVES) void dense_fwd_reg_kernel(
     const float* __restrict__ Qt, const float* __restrict__ K, const float* __restrict__ Vt,
     const float* __restrict__ pen, float* __restrict__ Attn, float* __restrict__ Out, float* __restrict__ OutCopy,
     int L, int nbr, int NB, float scale, Layouts ly, float* __restrict__ Part = nullptr, int C = 0) {
     static_assert(!MEAN || RM, "the mean-emitting forward takes row-major operands");
-    constexpr int D = 32, KH = 16, MAXT = 32 / WAVES;
+    constexpr int D = 32, KH = 16;
     __shared__ float lds[WAVES * 16 * 64];
     __shared__ float lds_m[WAVES][32], lds_z[WAVES][32];
     // per wavefront: one padded tile (the map tile on its way to memory), two 4 KB tiles filled straight from global
@@ -1174,6 +1174,16 @@ static void dense_fwd_launch(DenseAttn* a, const float* Qt, const float* K, cons
                                a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
         return;
     }
+    if (D == 32 && nbr <= 64) {  // eight wavefronts with at most eight logit tiles each
+        const dim3 block8(64 * 8);
+        if (a->has_mask)
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<true, false, 8, false, 8>), grid, block8, 0, a->hdr.stream, Qt, K, Vt,
+                               Mask, Attn, Out, a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
+        else
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<false, false, 8, false, 8>), grid, block8, 0, a->hdr.stream, Qt, K, Vt,
+                               Mask, Attn, Out, a->ws_out, a->L, nbr, a->NB, a->scale, Layouts{});
+        return;
+    }
     if (D == 32 && a->L <= 16384) {  // 32-bit byte offsets into one head's map: L*L*4 < 2^31
         const dim3 block4(64 * 4);
         if (a->has_mask)
@@ -1391,6 +1401,14 @@ static void dense_forward_strided_impl(void* h, const float* Q, const float* K, 
         else
             hipLaunchKernelGGL((dense_fwd_reg_kernel<false, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask, Attn,
                                Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+    } else if (nbr <= 64) {  // eight wavefronts with at most eight logit tiles each
+        const dim3 block8(64 * 8);
+        if (a->has_mask)
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<true, true, 8, false, 8>), grid, block8, 0, a->hdr.stream, Q, K, V,
+                               Mask, Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
+        else
+            hipLaunchKernelGGL((dense_fwd_reg_kernel<false, true, 8, false, 8>), grid, block8, 0, a->hdr.stream, Q, K, V,
+                               Mask, Attn, Out, nullptr, a->L, nbr, a->NB, a->scale, ly);
     } else {
         if (a->has_mask)
             hipLaunchKernelGGL((dense_fwd_sweep32_kernel<true, true>), grid, block4, 0, a->hdr.stream, Q, K, V, Mask,
