@@ -694,4 +694,89 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
     }
 }
 
+// -------------------------------------------------------------------------------------------------
+// The same pass with the gathered operands in LDS instead of L2.  A work-group of sixteen wavefronts owns HYB_CL_COLS
+// columns of a head and walks the sequence in ranges of HYB_CL_ROWS rows, whose Q and dO rows (128 KB) it loads
+// once per range.  A group of eight lanes owns eight columns (lane s holds floats 4s .. 4s+3 of their dK and dV rows,
+// 64 accumulator registers that live across the ranges) and walks each column's entries -- rows ascending, so the
+// entries of a range are the next ones of the column's list -- eight at a time: lane s fetches the s-th entry's row
+// and {dS, P} pair with full-width loads, the eight are handed round the group, and every lane adds its 16-byte
+// pieces of the Q and dO rows, read from LDS, to its sums.  Each column's sum runs in the order of its list, so the
+// result does not depend on the launch.
+// -------------------------------------------------------------------------------------------------
+constexpr int HYB_CL_ROWS = 512, HYB_CL_COLS = 1024, HYB_CL_THREADS = 1024;
+template <bool ST>
+__global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
+    const float* __restrict__ Q, const float* __restrict__ dO, const float2* __restrict__ Pairs,
+    float* __restrict__ dK, float* __restrict__ dV, HybIndex ix, int L, int NB, Layouts ly) {
+    __shared__ f32x4 sq[HYB_CL_ROWS * 8], so[HYB_CL_ROWS * 8];
+    const int ncg = L / HYB_CL_COLS;
+    const int item = xcd_remap((int)blockIdx.x, (int)gridDim.x);  // the work-groups of a head share an XCD's L2
+    const int bh = item / ncg, cg = item % ncg;
+    const int t = threadIdx.x, grp = t >> 3, sub = t & 7, lane = t & 63;
+    size_t ib, ob, gb;
+    int ild, old_, gld;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
+    hyb_head<ST>(ly.grad, ly.H, bh, L, gb, gld);
+    const float2* pairs = Pairs + (size_t)bh * ix.nr;
+    constexpr int NC = HYB_CL_COLS / (HYB_CL_THREADS / 8);  // columns per lane group: 8
+    f32x4 ak[NC], av[NC];
+    int e[NC], eend[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int col = cg * HYB_CL_COLS + c * (HYB_CL_THREADS / 8) + grp;
+        ak[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        av[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        e[c] = ix.c_ptr[col];
+        eend[c] = ix.c_ptr[col + 1];
+    }
+    for (int r0 = 0; r0 < L; r0 += HYB_CL_ROWS) {
+        __syncthreads();  // everybody has finished with the previous range
+#pragma unroll
+        for (int k = 0; k < HYB_CL_ROWS * 8 / HYB_CL_THREADS; ++k) {
+            const int idx = t + k * HYB_CL_THREADS, row = r0 + (idx >> 3), piece = idx & 7;
+            sq[idx] = reinterpret_cast<const f32x4*>(Q + ib + (size_t)row * ild)[piece];
+            so[idx] = reinterpret_cast<const f32x4*>(dO + ob + (size_t)row * old_)[piece];
+        }
+        __syncthreads();
+        const int rend = r0 + HYB_CL_ROWS;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            while (true) {
+                const int my = e[c] + sub;
+                const int row = my < eend[c] ? ix.c_row[my] : 0x7fffffff;
+                const bool in = row < rend;
+                // rows ascend along the list: the entries of this range among the eight are the first n
+                const int n = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                if (n == 0) break;
+                float2 pr = (float2){0.f, 0.f};
+                int lrow = 0;
+                if (in) {
+                    pr = pairs[ix.c_src[my]];
+                    lrow = row - r0;
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int rk = __shfl(lrow, k, 8);
+                    const float wk = __shfl(pr.x, k, 8), wv = __shfl(pr.y, k, 8);
+                    ak[c] += sq[rk * 8 + sub] * wk;
+                    av[c] += so[rk * 8 + sub] * wv;
+                }
+                e[c] += n;
+                if (n < 8) break;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int col = cg * HYB_CL_COLS + c * (HYB_CL_THREADS / 8) + grp;
+        if (eend[c] == ix.c_ptr[col]) continue;  // a column without remainder entries
+        f32x4* kr = reinterpret_cast<f32x4*>(dK + gb + (size_t)col * gld) + sub;
+        f32x4* vr = reinterpret_cast<f32x4*>(dV + gb + (size_t)col * gld) + sub;
+        *kr = *kr + ak[c];
+        *vr = *vr + av[c];
+    }
+}
+
 }  // namespace spion

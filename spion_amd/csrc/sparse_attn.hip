@@ -1485,8 +1485,15 @@ static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const 
         else
             hipLaunchKernelGGL((hyb_tile_bwd_col_kernel<4, ST>), grid_t, dim3(256), 0, a->hdr.stream, Q, V, P, dO,
                                (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
-        hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO, (const float2*)pairs,
-                           dK, dV, a->pat.hyb, a->L, a->NB, ly);
+        // enough work-groups of 1024 columns to occupy the device: the remainder's Q and dO rows come from LDS
+        static const bool col_gather = getenv("SPION_HYB_COL_GATHER") != nullptr;
+        const int ncg = a->L / HYB_CL_COLS;
+        if (!col_gather && a->L % HYB_CL_COLS == 0 && a->NB * ncg >= 128)
+            hipLaunchKernelGGL(hyb_rem_bwd_col_lds_kernel<ST>, dim3(a->NB * ncg), dim3(HYB_CL_THREADS), 0, a->hdr.stream,
+                               Q, dO, (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
+        else
+            hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO,
+                               (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
     }
     check_launch("hyb_bwd kernels");
 }

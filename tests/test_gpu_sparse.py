@@ -299,6 +299,35 @@ def test_hybrid_and_gather_paths_agree(with_mask):
         assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"hybrid vs gather {name}")
 
 
+@pytest.mark.parametrize("L,NB", [(1024, 128), (2048, 64)])
+def test_hybrid_remainder_columns_from_lds_on_many_heads(L, NB):
+    """With enough heads for 128 work-groups of 1024 columns, the remainder's column pass keeps the Q and dO rows of
+    a range of 512 rows in LDS (two and four ranges here): all heads against the pure gather kernels, three of them
+    against the oracle; a second backward gives the same bits."""
+    d = 32
+    sm, off, col = workloads.window_random_csr(L, 48, 110, seed=L)
+    Q, K, V, dO = _inputs(NB, L, d, seed=L + 1)
+    res = {}
+    for force in (False, True):
+        abi = SparseABI(d, L, NB, 1, with_mask=False)
+        abi.force_element(force)
+        abi.set_pattern(sm, off, col)
+        O, P = abi.forward(Q, K, V, None)
+        assert abi.last_path() == (2 if force else 3)
+        res[force] = (O, P) + tuple(abi.backward_rowmajor(Q, K, V, P, O, dO))
+        if not force:
+            again = abi.backward_rowmajor(Q, K, V, P, O, dO)
+            for x, y in zip(res[force][2:], again):
+                assert torch.equal(x, y)
+        abi.close()
+    for a, b, name in zip(res[False], res[True], ["O", "P", "dQ", "dK", "dV"]):
+        assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"hybrid vs gather {name}")
+    for h in (0, NB // 2 + 13, NB - 1):
+        ref = oracle_fwd_bwd(Q[h:h + 1], K[h:h + 1], V[h:h + 1], dO[h:h + 1], sm, off, col)
+        for t, name in zip(res[False], ["O", "P", "dQ", "dK", "dV"]):
+            assert_close(t[h:h + 1].cpu().numpy(), ref[name], what=f"head {h} {name}")
+
+
 def test_hybrid_pattern_with_partial_tiles_empty_rows_and_no_remainder():
     """Dense tiles with holes, rows without any entry and a block row whose entries all sit in dense tiles."""
     L, d, NB = 256, 32, 2
