@@ -701,10 +701,16 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
 // 64 accumulator registers that live across the ranges) and walks each column's entries -- rows ascending, so the
 // entries of a range are the next ones of the column's list -- eight at a time: lane s fetches the s-th entry's row
 // and {dS, P} pair with full-width loads, the eight are handed round the group, and every lane adds its 16-byte
-// pieces of the Q and dO rows, read from LDS, to its sums.  Each column's sum runs in the order of its list, so the
-// result does not depend on the launch.
+// pieces of the Q and dO rows, read from LDS, to its sums.  Each lane's sums run in a fixed order along the column's
+// list, so the result does not depend on the launch.
 // -------------------------------------------------------------------------------------------------
 constexpr int HYB_CL_ROWS = 512, HYB_CL_COLS = 1024, HYB_CL_THREADS = 1024;
+// x of another lane of the same row of sixteen: quad_perm (CTRL = 0x55 * k: lane k of the own quad) or row_half_mirror
+// (0x141: lane 7 - i of the own eight)
+template <int CTRL>
+__device__ __forceinline__ int hyb_dpp(int x) {
+    return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, false);
+}
 template <bool ST>
 __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
     const float* __restrict__ Q, const float* __restrict__ dO, const float2* __restrict__ Pairs,
@@ -741,30 +747,69 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
         }
         __syncthreads();
         const int rend = r0 + HYB_CL_ROWS;
+        // four columns at a time: the index loads of their first eight entries go out together, then the four pair
+        // loads, then the sums; what a column has beyond eight entries in this range follows batch by batch
+        auto fetch_idx = [&](int c, int& row, int& src) {
+            const int my = e[c] + sub;
+            const bool ok = my < eend[c];
+            row = ok ? ix.c_row[my] : 0x7fffffff;
+            src = ok ? ix.c_src[my] : 0;
+        };
+        // The eight entries go round the group by DPP moves: a quad broadcast hands entry k of a lane's own quad to
+        // its four lanes, and the same on the values mirrored within the eight lanes hands over the other quad's
+        // entries -- every lane sees all eight, each quad in an order of its own, which is fixed.
+        auto add_batch = [&](int c, int lrow, float2 pr) {
+            const int wx = __float_as_int(pr.x), wy = __float_as_int(pr.y);
+            const int mrow = hyb_dpp<0x141>(lrow), mx = hyb_dpp<0x141>(wx), my_ = hyb_dpp<0x141>(wy);
+#define SPION_HYB_ENTRY(CTRL, R, X, Y)                                           \
+    {                                                                            \
+        const int rk = hyb_dpp<CTRL>(R);                                         \
+        const float wk = __int_as_float(hyb_dpp<CTRL>(X)), wv = __int_as_float(hyb_dpp<CTRL>(Y)); \
+        ak[c] += sq[rk * 8 + sub] * wk;                                          \
+        av[c] += so[rk * 8 + sub] * wv;                                          \
+    }
+            SPION_HYB_ENTRY(0x00, lrow, wx, wy)
+            SPION_HYB_ENTRY(0x55, lrow, wx, wy)
+            SPION_HYB_ENTRY(0xaa, lrow, wx, wy)
+            SPION_HYB_ENTRY(0xff, lrow, wx, wy)
+            SPION_HYB_ENTRY(0x00, mrow, mx, my_)
+            SPION_HYB_ENTRY(0x55, mrow, mx, my_)
+            SPION_HYB_ENTRY(0xaa, mrow, mx, my_)
+            SPION_HYB_ENTRY(0xff, mrow, mx, my_)
+#undef SPION_HYB_ENTRY
+        };
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            while (true) {
-                const int my = e[c] + sub;
-                const int row = my < eend[c] ? ix.c_row[my] : 0x7fffffff;
-                const bool in = row < rend;
+        for (int c0 = 0; c0 < NC; c0 += 4) {
+            int row[4], src[4], n[4];
+            float2 pr[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) fetch_idx(c0 + j, row[j], src[j]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = row[j] < rend;
                 // rows ascend along the list: the entries of this range among the eight are the first n
-                const int n = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
-                if (n == 0) break;
-                float2 pr = (float2){0.f, 0.f};
-                int lrow = 0;
-                if (in) {
-                    pr = pairs[ix.c_src[my]];
-                    lrow = row - r0;
-                }
+                n[j] = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                pr[j] = in ? pairs[src[j]] : (float2){0.f, 0.f};
+                row[j] = in ? row[j] - r0 : 0;
+            }
 #pragma unroll
-                for (int k = 0; k < 8; ++k) {
-                    const int rk = __shfl(lrow, k, 8);
-                    const float wk = __shfl(pr.x, k, 8), wv = __shfl(pr.y, k, 8);
-                    ak[c] += sq[rk * 8 + sub] * wk;
-                    av[c] += so[rk * 8 + sub] * wv;
+            for (int j = 0; j < 4; ++j) {
+                if (n[j] == 0) continue;
+                add_batch(c0 + j, row[j], pr[j]);
+                e[c0 + j] += n[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                int nn = n[j];
+                while (nn == 8) {
+                    int r1, s1;
+                    fetch_idx(c0 + j, r1, s1);
+                    const bool in = r1 < rend;
+                    nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                    if (nn == 0) break;
+                    add_batch(c0 + j, in ? r1 - r0 : 0, in ? pairs[s1] : (float2){0.f, 0.f});
+                    e[c0 + j] += nn;
                 }
-                e[c] += n;
-                if (n < 8) break;
             }
         }
     }

@@ -1409,6 +1409,13 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 #undef SPION_BY_WAVES
 }
 
+// The remainder's column pass with its gathered operands in LDS (work-groups of 1024 columns of a head): when there
+// are enough such work-groups to occupy the device.  SPION_HYB_GATHER=1 keeps the kernel that gathers from L2.
+static bool hyb_operands_in_lds(const SparseAttn* a) {
+    static const bool gather = getenv("SPION_HYB_GATHER") != nullptr;
+    return !gather && a->L % HYB_CL_COLS == 0 && a->NB * (a->L / HYB_CL_COLS) >= 128;
+}
+
 // Hybrid patterns (dense tiles + remainder, d = 32).  Every operand row-major; ST: heads located by `ly`.
 // ocopy (contiguous heads only): where a second copy of O goes, or null.
 template <bool ST>
@@ -1448,8 +1455,7 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
         SPION_HYB_FWD(false);
 #undef SPION_HYB_FWD
     hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, (const float*)a->ws_raw, Attn, Out,
-                       ocopy,
-                       (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
+                       ocopy, (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
     check_launch("hybrid forward kernels");
 }
 
@@ -1485,12 +1491,9 @@ static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const 
         else
             hipLaunchKernelGGL((hyb_tile_bwd_col_kernel<4, ST>), grid_t, dim3(256), 0, a->hdr.stream, Q, V, P, dO,
                                (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
-        // enough work-groups of 1024 columns to occupy the device: the remainder's Q and dO rows come from LDS
-        static const bool col_gather = getenv("SPION_HYB_COL_GATHER") != nullptr;
-        const int ncg = a->L / HYB_CL_COLS;
-        if (!col_gather && a->L % HYB_CL_COLS == 0 && a->NB * ncg >= 128)
-            hipLaunchKernelGGL(hyb_rem_bwd_col_lds_kernel<ST>, dim3(a->NB * ncg), dim3(HYB_CL_THREADS), 0, a->hdr.stream,
-                               Q, dO, (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
+        if (hyb_operands_in_lds(a))
+            hipLaunchKernelGGL(hyb_rem_bwd_col_lds_kernel<ST>, dim3(a->NB * (a->L / HYB_CL_COLS)), dim3(HYB_CL_THREADS),
+                               0, a->hdr.stream, Q, dO, (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
         else
             hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO,
                                (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
