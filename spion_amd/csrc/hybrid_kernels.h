@@ -747,8 +747,6 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
         }
         __syncthreads();
         const int rend = r0 + HYB_CL_ROWS;
-        // four columns at a time: the index loads of their first eight entries go out together, then the four pair
-        // loads, then the sums; what a column has beyond eight entries in this range follows batch by batch
         auto fetch_idx = [&](int c, int& row, int& src) {
             const int my = e[c] + sub;
             const bool ok = my < eend[c];
@@ -779,37 +777,16 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
 #undef SPION_HYB_ENTRY
         };
 #pragma unroll
-        for (int c0 = 0; c0 < NC; c0 += 4) {
-            int row[4], src[4], n[4];
-            float2 pr[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) fetch_idx(c0 + j, row[j], src[j]);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bool in = row[j] < rend;
-                // rows ascend along the list: the entries of this range among the eight are the first n
-                n[j] = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
-                pr[j] = in ? pairs[src[j]] : (float2){0.f, 0.f};
-                row[j] = in ? row[j] - r0 : 0;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                if (n[j] == 0) continue;
-                add_batch(c0 + j, row[j], pr[j]);
-                e[c0 + j] += n[j];
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                int nn = n[j];
-                while (nn == 8) {
-                    int r1, s1;
-                    fetch_idx(c0 + j, r1, s1);
-                    const bool in = r1 < rend;
-                    nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
-                    if (nn == 0) break;
-                    add_batch(c0 + j, in ? r1 - r0 : 0, in ? pairs[s1] : (float2){0.f, 0.f});
-                    e[c0 + j] += nn;
-                }
+        for (int c = 0; c < NC; ++c) {
+            int nn = 8;
+            while (nn == 8) {
+                int r1, s1;
+                fetch_idx(c, r1, s1);
+                const bool in = r1 < rend;
+                nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                if (nn == 0) break;
+                add_batch(c, in ? r1 - r0 : 0, in ? pairs[s1] : (float2){0.f, 0.f});
+                e[c] += nn;
             }
         }
     }
