@@ -190,3 +190,31 @@ def test_dense_modules_autograd(with_mask, d, L):
     assert_close(attn.detach().cpu().numpy(), p.detach().numpy(), what="dense module attn")
     for name, a, b in (("dq", q, qc), ("dk", k, kc), ("dv", v, vc)):
         assert_close(a.grad.cpu().numpy(), b.grad.numpy(), what=f"dense module {name}")
+
+
+def test_dense_strided_limits_at_head_dimension_64():
+    """Head dimension 64: the row-major forward refuses sequences beyond 2048 and the mean-emitting form, with a
+    message and without touching the outputs; the module then goes through the reference's ABI."""
+    import ctypes
+    d, B, H, L = 64, 1, 2, 2080
+    lib = Attention._cuda_compile_module()
+    h = lib.init(d, L, B * H)
+    _lib.check_error("init")
+    q, k, v = (torch.zeros(B, H, L, d, device="cuda") for _ in range(3))
+    out = torch.full((B, H, L, d), 3.0, device="cuda")
+    attn = torch.full((2, 8), 5.0, device="cuda")  # never written
+    lay = _lib.head_layout(q)
+    A = ctypes.addressof(lay)
+    core = _lib.core()
+    core.spion_dense_forward_strided(h, q.data_ptr(), k.data_ptr(), v.data_ptr(), None, attn.data_ptr(),
+                                     out.data_ptr(), H, A, A)
+    with pytest.raises(_lib.SpionLibraryError, match="seq_len <= 2048"):
+        _lib.check_error("dense forward strided")
+    torch.cuda.synchronize()
+    assert (out == 3.0).all() and (attn == 5.0).all()
+    lib.destroy(h)
+    import spion_amd
+    cfg = dict(head_dim=d, num_head=H, max_seq_len=L, batch_size=B, block_size=32)
+    cpp = Attention._cuda_compile_module()
+    mod = spion_amd.CUDAAttention(cfg, cpp, cpp.init(d, L, B * H))
+    assert not mod.reads_views
