@@ -319,6 +319,18 @@ def test_hybrid_remainder_columns_from_lds_on_many_heads(L, NB):
             again = abi.backward_rowmajor(Q, K, V, P, O, dO)
             for x, y in zip(res[force][2:], again):
                 assert torch.equal(x, y)
+            # the same heads as views of [B, L, H*d] projections: bit for bit
+            H = 2
+            B = NB // H
+            proj = lambda t: t.view(B, H, L, d).transpose(1, 2).contiguous().transpose(1, 2)
+            q, k, v, do = (proj(t) for t in (Q, K, V, dO))
+            out, dq, dk, dv = (proj(torch.full_like(Q, float("nan"))) for _ in range(4))
+            assert not q.is_contiguous()
+            Ps = abi.forward_strided(q, k, v, out)
+            abi.backward_strided(q, k, v, Ps, out, do, dq, dk, dv)
+            assert abi.last_path() == 3
+            for x, y in zip((out, Ps, dq, dk, dv), res[force]):
+                assert torch.equal(x.reshape(y.shape), y)
         abi.close()
     for a, b, name in zip(res[False], res[True], ["O", "P", "dQ", "dK", "dV"]):
         assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"hybrid vs gather {name}")
