@@ -711,10 +711,15 @@ template <int CTRL>
 __device__ __forceinline__ int hyb_dpp(int x) {
     return __builtin_amdgcn_update_dpp(0, x, CTRL, 0xf, 0xf, false);
 }
-template <bool ST>
+// The list of a column: entries c_ptr[j] .. c_ptr[j+1]-1, their rows c_row (ascending) and c_src, the index of the
+// entry's weights -- PAIRS: in the compact {dS, P} list of a head ([NB][n] float2; the sums are added to what the tile
+// part left in dK and dV); otherwise in the head's dS and P arrays ([NB][n] floats each; the sums are the result).
+template <bool ST, bool PAIRS = true>
 __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
     const float* __restrict__ Q, const float* __restrict__ dO, const float2* __restrict__ Pairs,
-    float* __restrict__ dK, float* __restrict__ dV, HybIndex ix, int L, int NB, Layouts ly) {
+    const float* __restrict__ dSa, const float* __restrict__ Pa, float* __restrict__ dK, float* __restrict__ dV,
+    const int* __restrict__ c_ptr, const int* __restrict__ c_row, const int* __restrict__ c_src, int n, int L, int NB,
+    Layouts ly) {
     __shared__ f32x4 sq[HYB_CL_ROWS * 8], so[HYB_CL_ROWS * 8];
     const int ncg = L / HYB_CL_COLS;
     const int item = xcd_remap((int)blockIdx.x, (int)gridDim.x);  // the work-groups of a head share an XCD's L2
@@ -725,7 +730,10 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
     hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
     hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
     hyb_head<ST>(ly.grad, ly.H, bh, L, gb, gld);
-    const float2* pairs = Pairs + (size_t)bh * ix.nr;
+    const float2* pairs = PAIRS ? Pairs + (size_t)bh * n : nullptr;
+    const float* dsh = PAIRS ? nullptr : dSa + (size_t)bh * n;
+    const float* ph = PAIRS ? nullptr : Pa + (size_t)bh * n;
+    auto weights = [&](int src) { return PAIRS ? pairs[src] : (float2){dsh[src], ph[src]}; };
     constexpr int NC = HYB_CL_COLS / (HYB_CL_THREADS / 8);  // columns per lane group: 8
     f32x4 ak[NC], av[NC];
     int e[NC], eend[NC];
@@ -734,8 +742,8 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
         const int col = cg * HYB_CL_COLS + c * (HYB_CL_THREADS / 8) + grp;
         ak[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
         av[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        e[c] = ix.c_ptr[col];
-        eend[c] = ix.c_ptr[col + 1];
+        e[c] = c_ptr[col];
+        eend[c] = c_ptr[col + 1];
     }
     for (int r0 = 0; r0 < L; r0 += HYB_CL_ROWS) {
         __syncthreads();  // everybody has finished with the previous range
@@ -750,8 +758,8 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
         auto fetch_idx = [&](int c, int& row, int& src) {
             const int my = e[c] + sub;
             const bool ok = my < eend[c];
-            row = ok ? ix.c_row[my] : 0x7fffffff;
-            src = ok ? ix.c_src[my] : 0;
+            row = ok ? c_row[my] : 0x7fffffff;
+            src = ok ? c_src[my] : 0;
         };
         // The eight entries go round the group by DPP moves: a quad broadcast hands entry k of a lane's own quad to
         // its four lanes, and the same on the values mirrored within the eight lanes hands over the other quad's
@@ -785,7 +793,7 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
                 const bool in = r1 < rend;
                 nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
                 if (nn == 0) break;
-                add_batch(c, in ? r1 - r0 : 0, in ? pairs[s1] : (float2){0.f, 0.f});
+                add_batch(c, in ? r1 - r0 : 0, in ? weights(s1) : (float2){0.f, 0.f});
                 e[c] += nn;
             }
         }
@@ -793,11 +801,16 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
         const int col = cg * HYB_CL_COLS + c * (HYB_CL_THREADS / 8) + grp;
-        if (eend[c] == ix.c_ptr[col]) continue;  // a column without remainder entries
         f32x4* kr = reinterpret_cast<f32x4*>(dK + gb + (size_t)col * gld) + sub;
         f32x4* vr = reinterpret_cast<f32x4*>(dV + gb + (size_t)col * gld) + sub;
-        *kr = *kr + ak[c];
-        *vr = *vr + av[c];
+        if constexpr (PAIRS) {
+            if (eend[c] == c_ptr[col]) continue;  // a column without remainder entries
+            *kr = *kr + ak[c];
+            *vr = *vr + av[c];
+        } else {
+            *kr = ak[c];
+            *vr = av[c];
+        }
     }
 }
 

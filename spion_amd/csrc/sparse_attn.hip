@@ -1493,7 +1493,8 @@ static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const 
                                (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
         if (hyb_operands_in_lds(a))
             hipLaunchKernelGGL(hyb_rem_bwd_col_lds_kernel<ST>, dim3(a->NB * (a->L / HYB_CL_COLS)), dim3(HYB_CL_THREADS),
-                               0, a->hdr.stream, Q, dO, (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
+                               0, a->hdr.stream, Q, dO, (const float2*)pairs, nullptr, nullptr, dK, dV, a->pat.hyb.c_ptr,
+                               a->pat.hyb.c_row, a->pat.hyb.c_src, a->pat.hyb.nr, a->L, a->NB, ly);
         else
             hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO,
                                (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
@@ -1532,9 +1533,18 @@ static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const
     if (a->bwd_passes & 1)
         hipLaunchKernelGGL((elem_bwd_row_kernel<D, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, K, Vrm, P, dO,
                            dS, dQ, offs, cols, a->L, a->NB, nnz, a->scale, ly);
-    if (a->bwd_passes & 2)
+    if (a->bwd_passes & 2) {
+        if constexpr (D == 32) {
+            if (hyb_operands_in_lds(a)) {  // the Q and dO rows of a range of the sequence in LDS, see hybrid_kernels.h
+                hipLaunchKernelGGL((hyb_rem_bwd_col_lds_kernel<ST, false>), dim3(a->NB * (a->L / HYB_CL_COLS)),
+                                   dim3(HYB_CL_THREADS), 0, a->hdr.stream, Q, dO, nullptr, dS, P, dK, dV, pi.d_ccp,
+                                   pi.d_crow, pi.d_cpos, nnz, a->L, a->NB, ly);
+                return;
+            }
+        }
         hipLaunchKernelGGL((elem_bwd_col_kernel<D, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, dO, P, dS,
                            dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz, ly);
+    }
 }
 
 // krow: Kt is K itself, row-major [NB][L][d], not the transposed copy of the reference's ABI.

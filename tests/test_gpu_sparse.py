@@ -301,9 +301,10 @@ def test_hybrid_and_gather_paths_agree(with_mask):
 
 @pytest.mark.parametrize("L,NB", [(1024, 128), (2048, 64)])
 def test_hybrid_remainder_columns_from_lds_on_many_heads(L, NB):
-    """With enough heads for 128 work-groups of 1024 columns, the remainder's column pass keeps the Q and dO rows of
-    a range of 512 rows in LDS (two and four ranges here): all heads against the pure gather kernels, three of them
-    against the oracle; a second backward gives the same bits."""
+    """With enough heads for 128 work-groups of 1024 columns, the column pass of the remainder (hybrid kernels) and of
+    all entries (element kernels) keeps the Q and dO rows of a range of 512 rows in LDS (two and four ranges here):
+    the two families against each other on all heads, three heads against the oracle; a second backward and the
+    strided entry points give the same bits."""
     d = 32
     sm, off, col = workloads.window_random_csr(L, 48, 110, seed=L)
     Q, K, V, dO = _inputs(NB, L, d, seed=L + 1)
@@ -315,22 +316,21 @@ def test_hybrid_remainder_columns_from_lds_on_many_heads(L, NB):
         O, P = abi.forward(Q, K, V, None)
         assert abi.last_path() == (2 if force else 3)
         res[force] = (O, P) + tuple(abi.backward_rowmajor(Q, K, V, P, O, dO))
-        if not force:
-            again = abi.backward_rowmajor(Q, K, V, P, O, dO)
-            for x, y in zip(res[force][2:], again):
-                assert torch.equal(x, y)
-            # the same heads as views of [B, L, H*d] projections: bit for bit
-            H = 2
-            B = NB // H
-            proj = lambda t: t.view(B, H, L, d).transpose(1, 2).contiguous().transpose(1, 2)
-            q, k, v, do = (proj(t) for t in (Q, K, V, dO))
-            out, dq, dk, dv = (proj(torch.full_like(Q, float("nan"))) for _ in range(4))
-            assert not q.is_contiguous()
-            Ps = abi.forward_strided(q, k, v, out)
-            abi.backward_strided(q, k, v, Ps, out, do, dq, dk, dv)
-            assert abi.last_path() == 3
-            for x, y in zip((out, Ps, dq, dk, dv), res[force]):
-                assert torch.equal(x.reshape(y.shape), y)
+        again = abi.backward_rowmajor(Q, K, V, P, O, dO)
+        for x, y in zip(res[force][2:], again):
+            assert torch.equal(x, y)
+        # the same heads as views of [B, L, H*d] projections: bit for bit
+        H = 2
+        B = NB // H
+        proj = lambda t: t.view(B, H, L, d).transpose(1, 2).contiguous().transpose(1, 2)
+        q, k, v, do = (proj(t) for t in (Q, K, V, dO))
+        out, dq, dk, dv = (proj(torch.full_like(Q, float("nan"))) for _ in range(4))
+        assert not q.is_contiguous()
+        Ps = abi.forward_strided(q, k, v, out)
+        abi.backward_strided(q, k, v, Ps, out, do, dq, dk, dv)
+        assert abi.last_path() == (2 if force else 3)
+        for x, y in zip((out, Ps, dq, dk, dv), res[force]):
+            assert torch.equal(x.reshape(y.shape), y)
         abi.close()
     for a, b, name in zip(res[False], res[True], ["O", "P", "dQ", "dK", "dV"]):
         assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"hybrid vs gather {name}")
