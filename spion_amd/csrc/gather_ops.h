@@ -3,10 +3,12 @@
 // A wavefront holds a chunk of up to 64 pattern entries one per lane and fetches the entries' rows (D floats, D = 4 LPR)
 // LPR lanes to a row, 16 bytes per lane, G = 64 / LPR rows per load instruction.  Lane l owns entry
 // (l % LPR) * G + l / LPR of the chunk, so that the LPR entries group g = l / LPR fetches (entry j*G + g in
-// instruction j) are the entries its own LPR lanes own: every exchange stays inside a group of LPR lanes (DPP
-// moves), nothing goes through LDS memory, and the number of wavefronts in flight -- what bounds these
-// latency-bound kernels -- is not limited by LDS space.  (Staging the gathered rows through a wave-private LDS tile
-// instead made the same kernels three to five times slower.)
+// instruction j) are the entries its own LPR lanes own: every exchange stays inside a group of LPR lanes (a
+// ds_bpermute for the broadcast of an entry's row and weight, DPP moves for the sums), nothing goes through LDS
+// memory, and the number of wavefronts in flight -- what bounds these latency-bound kernels -- is not limited by LDS
+// space.  (Staging the gathered rows through a wave-private LDS tile instead made the same kernels three to five
+// times slower; the broadcasts as two DPP moves each instead of the permute change nothing: 1.245 against 1.247 ms
+// for a step of 20 M entries.)
 #pragma once
 #include <hip/hip_runtime.h>
 
