@@ -761,7 +761,7 @@ def bench_sparse_layer(args, dev, workload, full=True):
              # hybrid: dense window tiles on the MFMA units + gathered remainder; each phase is two or three launches
              3: ("hyb_rem_logits_kernel + hyb_tile_fwd_kernel + hyb_rem_pv_kernel",
                  "hyb_tile_bwd_row_kernel + hyb_rem_bwd_row_kernel",
-                 "hyb_tile_bwd_col_kernel + " + ("hyb_rem_bwd_col_lds_kernel" if L % 1024 == 0 and NB * (L // 1024) >= 128
+                 "hyb_tile_bwd_col_kernel + " + ("hyb_rem_bwd_col_lds_kernel" if L % 1024 == 0 and NB * (L // 256) >= 256
                                                   and "SPION_HYB_GATHER" not in os.environ else "hyb_rem_bwd_col_kernel"))}[path]
     kernels = dict(zip(names, (t_fwd, t_row, t_col)))
     dom = max(kernels, key=kernels.get)

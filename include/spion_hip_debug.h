@@ -48,8 +48,9 @@ int spion_debug_bf16_plan(const int* tile_ptr, int nstrips, int pairs, int num_b
  *                        strips per wavefront on masks of 64 x 64 blocks and larger, contiguous heads);
  *   SPION_BF16_ROW_PAIRS=0  the same for the row pass alone.
  *   SPION_HYB_GATHER     hybrid patterns: the remainder's column pass gathers its Q and dO rows from L2, one wavefront
- *                        per column (default, when seq_len is a multiple of 1024 and num_batches * seq_len / 1024 >= 128:
- *                        work-groups of 1024 columns with the rows of a range of the sequence in LDS);
+ *                        per column (default, when seq_len is a multiple of 1024 and num_batches * seq_len / 256 >= 256:
+ *                        work-groups of 1024, 512 or 256 columns with the rows of a range of the sequence in LDS; the
+ *                        element kernels' column pass at emb_dim 32 likewise);
  * Read whenever a bf16 handle indexes a pattern (tests):
  *   SPION_BF16_LANES     number of persistent wavefronts the bf16 kernels are launched with (default: eight per
  *                        compute unit); a handful makes each one walk many strips of several heads in a row.

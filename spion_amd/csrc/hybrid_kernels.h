@@ -695,16 +695,16 @@ __global__ __launch_bounds__(64 * HYB_GWAVES) void hyb_rem_bwd_col_kernel(  // t
 }
 
 // -------------------------------------------------------------------------------------------------
-// The same pass with the gathered operands in LDS instead of L2.  A work-group of sixteen wavefronts owns HYB_CL_COLS
+// The same pass with the gathered operands in LDS instead of L2.  A work-group of sixteen wavefronts owns 128 * NC
 // columns of a head and walks the sequence in ranges of HYB_CL_ROWS rows, whose Q and dO rows (128 KB) it loads
-// once per range.  A group of eight lanes owns eight columns (lane s holds floats 4s .. 4s+3 of their dK and dV rows,
-// 64 accumulator registers that live across the ranges) and walks each column's entries -- rows ascending, so the
+// once per range.  A group of eight lanes owns NC columns (lane s holds floats 4s .. 4s+3 of their dK and dV rows,
+// 8 * NC accumulator registers that live across the ranges) and walks each column's entries -- rows ascending, so the
 // entries of a range are the next ones of the column's list -- eight at a time: lane s fetches the s-th entry's row
 // and {dS, P} pair with full-width loads, the eight are handed round the group, and every lane adds its 16-byte
 // pieces of the Q and dO rows, read from LDS, to its sums.  Each lane's sums run in a fixed order along the column's
 // list, so the result does not depend on the launch.
 // -------------------------------------------------------------------------------------------------
-constexpr int HYB_CL_ROWS = 512, HYB_CL_COLS = 1024, HYB_CL_THREADS = 1024;
+constexpr int HYB_CL_ROWS = 512, HYB_CL_THREADS = 1024;  // a work-group owns NC * 128 columns: 1024 (NC = 8) or 512
 // x of another lane of the same row of sixteen: quad_perm (CTRL = 0x55 * k: lane k of the own quad) or row_half_mirror
 // (0x141: lane 7 - i of the own eight)
 template <int CTRL>
@@ -714,13 +714,14 @@ __device__ __forceinline__ int hyb_dpp(int x) {
 // The list of a column: entries c_ptr[j] .. c_ptr[j+1]-1, their rows c_row (ascending) and c_src, the index of the
 // entry's weights -- PAIRS: in the compact {dS, P} list of a head ([NB][n] float2; the sums are added to what the tile
 // part left in dK and dV); otherwise in the head's dS and P arrays ([NB][n] floats each; the sums are the result).
-template <bool ST, bool PAIRS = true>
+template <bool ST, bool PAIRS, int NC>
 __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
     const float* __restrict__ Q, const float* __restrict__ dO, const float2* __restrict__ Pairs,
     const float* __restrict__ dSa, const float* __restrict__ Pa, float* __restrict__ dK, float* __restrict__ dV,
     const int* __restrict__ c_ptr, const int* __restrict__ c_row, const int* __restrict__ c_src, int n, int L, int NB,
     Layouts ly) {
     __shared__ f32x4 sq[HYB_CL_ROWS * 8], so[HYB_CL_ROWS * 8];
+    constexpr int HYB_CL_COLS = NC * (HYB_CL_THREADS / 8);
     const int ncg = L / HYB_CL_COLS;
     const int item = xcd_remap((int)blockIdx.x, (int)gridDim.x);  // the work-groups of a head share an XCD's L2
     const int bh = item / ncg, cg = item % ncg;
@@ -734,7 +735,6 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
     const float* dsh = PAIRS ? nullptr : dSa + (size_t)bh * n;
     const float* ph = PAIRS ? nullptr : Pa + (size_t)bh * n;
     auto weights = [&](int src) { return PAIRS ? pairs[src] : (float2){dsh[src], ph[src]}; };
-    constexpr int NC = HYB_CL_COLS / (HYB_CL_THREADS / 8);  // columns per lane group: 8
     f32x4 ak[NC], av[NC];
     int e[NC], eend[NC];
 #pragma unroll

@@ -1409,12 +1409,20 @@ static void launch_tile_bwd(SparseAttn* a, const float* Q, const float* K, const
 #undef SPION_BY_WAVES
 }
 
-// The remainder's column pass with its gathered operands in LDS (work-groups of 1024 columns of a head): when there
-// are enough such work-groups to occupy the device.  SPION_HYB_GATHER=1 keeps the kernel that gathers from L2.
-static bool hyb_operands_in_lds(const SparseAttn* a) {
+// The remainder's column pass with its gathered operands in LDS: columns per lane group (work-groups of 1024, 512 or
+// 256 columns of a head), the most that still gives every CU a work-group -- with half of them idle the kernel that
+// gathers from L2 is as fast (configuration 4 at half its batch: 0.248 against 0.244 ms) -- or 0 for that kernel
+// (also with SPION_HYB_GATHER=1).
+static int hyb_lds_columns(const SparseAttn* a) {
     static const bool gather = getenv("SPION_HYB_GATHER") != nullptr;
-    return !gather && a->L % HYB_CL_COLS == 0 && a->NB * (a->L / HYB_CL_COLS) >= 128;
+    if (gather || a->L % 1024) return 0;
+    for (int nc = 8; nc >= 2; nc >>= 1)
+        if ((long long)a->NB * (a->L / (128 * nc)) >= 256) return nc;
+    return 0;
 }
+#define SPION_HYB_COL_LDS(ST_, PAIRS_, NC_, ...)                                                          \
+    hipLaunchKernelGGL((hyb_rem_bwd_col_lds_kernel<ST_, PAIRS_, NC_>), dim3(a->NB * (a->L / (128 * NC_))), \
+                       dim3(HYB_CL_THREADS), 0, a->hdr.stream, __VA_ARGS__)
 
 // Hybrid patterns (dense tiles + remainder, d = 32).  Every operand row-major; ST: heads located by `ly`.
 // ocopy (contiguous heads only): where a second copy of O goes, or null.
@@ -1491,10 +1499,16 @@ static void launch_hyb_bwd(SparseAttn* a, const float* Q, const float* K, const 
         else
             hipLaunchKernelGGL((hyb_tile_bwd_col_kernel<4, ST>), grid_t, dim3(256), 0, a->hdr.stream, Q, V, P, dO,
                                (const float*)a->ws_rowsum, dK, dV, a->pat.hyb, a->L, nbr, a->NB, nnz, a->scale, ly);
-        if (hyb_operands_in_lds(a))
-            hipLaunchKernelGGL(hyb_rem_bwd_col_lds_kernel<ST>, dim3(a->NB * (a->L / HYB_CL_COLS)), dim3(HYB_CL_THREADS),
-                               0, a->hdr.stream, Q, dO, (const float2*)pairs, nullptr, nullptr, dK, dV, a->pat.hyb.c_ptr,
-                               a->pat.hyb.c_row, a->pat.hyb.c_src, a->pat.hyb.nr, a->L, a->NB, ly);
+        const int nc = hyb_lds_columns(a);
+        if (nc == 8)
+            SPION_HYB_COL_LDS(ST, true, 8, Q, dO, (const float2*)pairs, nullptr, nullptr, dK, dV, a->pat.hyb.c_ptr,
+                              a->pat.hyb.c_row, a->pat.hyb.c_src, a->pat.hyb.nr, a->L, a->NB, ly);
+        else if (nc == 4)
+            SPION_HYB_COL_LDS(ST, true, 4, Q, dO, (const float2*)pairs, nullptr, nullptr, dK, dV, a->pat.hyb.c_ptr,
+                              a->pat.hyb.c_row, a->pat.hyb.c_src, a->pat.hyb.nr, a->L, a->NB, ly);
+        else if (nc == 2)
+            SPION_HYB_COL_LDS(ST, true, 2, Q, dO, (const float2*)pairs, nullptr, nullptr, dK, dV, a->pat.hyb.c_ptr,
+                              a->pat.hyb.c_row, a->pat.hyb.c_src, a->pat.hyb.nr, a->L, a->NB, ly);
         else
             hipLaunchKernelGGL(hyb_rem_bwd_col_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, Q, dO,
                                (const float2*)pairs, dK, dV, a->pat.hyb, a->L, a->NB, ly);
@@ -1535,12 +1549,17 @@ static void launch_elem_bwd(SparseAttn* a, const float* Q, const float* K, const
                            dS, dQ, offs, cols, a->L, a->NB, nnz, a->scale, ly);
     if (a->bwd_passes & 2) {
         if constexpr (D == 32) {
-            if (hyb_operands_in_lds(a)) {  // the Q and dO rows of a range of the sequence in LDS, see hybrid_kernels.h
-                hipLaunchKernelGGL((hyb_rem_bwd_col_lds_kernel<ST, false>), dim3(a->NB * (a->L / HYB_CL_COLS)),
-                                   dim3(HYB_CL_THREADS), 0, a->hdr.stream, Q, dO, nullptr, dS, P, dK, dV, pi.d_ccp,
-                                   pi.d_crow, pi.d_cpos, nnz, a->L, a->NB, ly);
-                return;
-            }
+            const int nc = hyb_lds_columns(a);  // the Q and dO rows of a range of the sequence in LDS, see hybrid_kernels.h
+            if (nc == 8)
+                SPION_HYB_COL_LDS(ST, false, 8, Q, dO, nullptr, dS, P, dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, nnz, a->L,
+                                  a->NB, ly);
+            else if (nc == 4)
+                SPION_HYB_COL_LDS(ST, false, 4, Q, dO, nullptr, dS, P, dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, nnz, a->L,
+                                  a->NB, ly);
+            else if (nc == 2)
+                SPION_HYB_COL_LDS(ST, false, 2, Q, dO, nullptr, dS, P, dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, nnz, a->L,
+                                  a->NB, ly);
+            if (nc) return;
         }
         hipLaunchKernelGGL((elem_bwd_col_kernel<D, ST>), grid, dim3(64 * ELEM_WAVES), 0, a->hdr.stream, Q, dO, P, dS,
                            dK, dV, pi.d_ccp, pi.d_crow, pi.d_cpos, a->L, a->NB, nnz, ly);

@@ -299,10 +299,11 @@ def test_hybrid_and_gather_paths_agree(with_mask):
         assert_close(a.cpu().numpy(), b.cpu().numpy(), what=f"hybrid vs gather {name}")
 
 
-@pytest.mark.parametrize("L,NB", [(1024, 128), (2048, 64)])
+@pytest.mark.parametrize("L,NB", [(1024, 256), (2048, 64), (1024, 64)])
 def test_hybrid_remainder_columns_from_lds_on_many_heads(L, NB):
-    """With enough heads for 128 work-groups of 1024 columns, the column pass of the remainder (hybrid kernels) and of
-    all entries (element kernels) keeps the Q and dO rows of a range of 512 rows in LDS (two and four ranges here):
+    """With enough heads for 256 work-groups of 1024, 512 or 256 columns (the three cases), the column pass of the
+    remainder (hybrid kernels) and of all entries (element kernels) keeps the Q and dO rows of a range of 512 rows in
+    LDS (two and four ranges here):
     the two families against each other on all heads, three heads against the oracle; a second backward and the
     strided entry points give the same bits."""
     d = 32
