@@ -759,7 +759,9 @@ def bench_sparse_layer(args, dev, workload, full=True):
     names = {1: ("tile_fwd_kernel", "tile_bwd_row_kernel", "tile_bwd_col_kernel"),
              2: ("elem_fwd_kernel", "elem_bwd_row_kernel", "elem_bwd_col_kernel"),
              # hybrid: dense window tiles on the MFMA units + gathered remainder; each phase is two or three launches
-             3: ("hyb_rem_logits_kernel + hyb_tile_fwd_kernel + hyb_rem_pv_kernel",
+             3: ("hyb_rem_logits_lds_kernel + hyb_tile_fwd_kernel + hyb_rem_pv_lds_kernel"
+                 if L % 1024 == 0 and NB * (L // 1024) >= 256 and "SPION_HYB_GATHER" not in os.environ
+                 else "hyb_rem_logits_kernel + hyb_tile_fwd_kernel + hyb_rem_pv_kernel",
                  "hyb_tile_bwd_row_kernel + hyb_rem_bwd_row_kernel",
                  "hyb_tile_bwd_col_kernel + " + ("hyb_rem_bwd_col_lds_kernel" if L % 1024 == 0 and NB * (L // 256) >= 256
                                                   and "SPION_HYB_GATHER" not in os.environ else "hyb_rem_bwd_col_kernel"))}[path]

@@ -50,7 +50,8 @@ int spion_debug_bf16_plan(const int* tile_ptr, int nstrips, int pairs, int num_b
  *   SPION_HYB_GATHER     hybrid patterns: the remainder's column pass gathers its Q and dO rows from L2, one wavefront
  *                        per column (default, when seq_len is a multiple of 1024 and num_batches * seq_len / 256 >= 256:
  *                        work-groups of 1024, 512 or 256 columns with the rows of a range of the sequence in LDS; the
- *                        element kernels' column pass at emb_dim 32 likewise);
+ *                        element kernels' column pass at emb_dim 32 likewise), and so do the forward's two remainder
+ *                        kernels (default: operands in LDS when num_batches * seq_len / 512, resp. / 1024, >= 256);
  * Read whenever a bf16 handle indexes a pattern (tests):
  *   SPION_BF16_LANES     number of persistent wavefronts the bf16 kernels are launched with (default: eight per
  *                        compute unit); a handful makes each one walk many strips of several heads in a row.

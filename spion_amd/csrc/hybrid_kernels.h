@@ -17,6 +17,7 @@
 // part of the row pass, the same for the column pass; the remainder kernels add to what the tile kernels wrote
 // (each row or column has exactly one writer per launch).
 #pragma once
+#include <type_traits>
 #include "gather_ops.h"
 #include "tile_kernels.h"
 
@@ -811,6 +812,207 @@ __global__ __launch_bounds__(HYB_CL_THREADS) void hyb_rem_bwd_col_lds_kernel(
             *kr = ak[c];
             *vr = av[c];
         }
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward, step 1, with the K rows in LDS: a work-group of sixteen wavefronts owns 128 * NR query rows of a head and
+// walks the keys in ranges of HYB_LL_KEYS, whose K rows (128 KB; with a key mask their penalties too) it loads once
+// per range.  A group of eight lanes owns NR rows (their scaled Q rows -- lane i of either quad holds pieces i and
+// i + 4 -- and their running {maximum, sum}) and walks each row's remainder entries eight at a time, lane s fetching
+// the s-th entry's column; then either quad of the group takes the four entries its own lanes hold, one after the
+// other: the column goes round the quad by a DPP move, every lane multiplies its two pieces of the K row, read from
+// LDS, two DPP additions make the dot product, and the lane that holds the entry keeps it.  The eight logits are
+// stored, and the row's statistics follow batch by batch (maximum raised, sum rescaled).
+// -------------------------------------------------------------------------------------------------
+constexpr int HYB_LL_KEYS = 1024, HYB_LL_THREADS = 1024;
+template <bool MASK, bool ST, int NR>
+__global__ __launch_bounds__(HYB_LL_THREADS) void hyb_rem_logits_lds_kernel(
+    const float* __restrict__ Q, const float* __restrict__ K, const float* __restrict__ pen, float* __restrict__ Raw,
+    float2* __restrict__ Stats, HybIndex ix, int L, int NB, float scale, Layouts ly) {
+    __shared__ f32x4 sk[HYB_LL_KEYS * 8];
+    __shared__ float spen[MASK ? HYB_LL_KEYS : 1];
+    constexpr int ROWS = NR * (HYB_LL_THREADS / 8);
+    const int nrg = L / ROWS;
+    const int item = xcd_remap((int)blockIdx.x, (int)gridDim.x);  // the work-groups of a head share an XCD's L2
+    const int bh = item / nrg, rg = item % nrg;
+    const int t = threadIdx.x, grp = t >> 3, sub = t & 7, qi = t & 3, lane = t & 63;
+    size_t ib;
+    int ild;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    float* raw = Raw + (size_t)bh * ix.nr;
+    const float c2 = scale * LOG2E;
+    f32x4 q0[NR], q1[NR];
+    float m[NR], z[NR];
+    int e[NR], eend[NR];
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+        const int row = rg * ROWS + c * (HYB_LL_THREADS / 8) + grp;
+        const f32x4* qr = reinterpret_cast<const f32x4*>(Q + ib + (size_t)row * ild);
+        q0[c] = qr[qi] * c2;
+        q1[c] = qr[4 + qi] * c2;
+        m[c] = HYB_ABSENT;
+        z[c] = 0.f;
+        e[c] = ix.r_off[row];
+        eend[c] = ix.r_off[row + 1];
+    }
+    auto fdpp = [](auto ctrl, float x) {
+        return __int_as_float(hyb_dpp<decltype(ctrl)::value>(__float_as_int(x)));
+    };
+    for (int k0 = 0; k0 < L; k0 += HYB_LL_KEYS) {
+        __syncthreads();  // everybody has finished with the previous range
+#pragma unroll
+        for (int k = 0; k < HYB_LL_KEYS * 8 / HYB_LL_THREADS; ++k) {
+            const int idx = t + k * HYB_LL_THREADS;
+            sk[idx] = reinterpret_cast<const f32x4*>(K + ib + (size_t)(k0 + (idx >> 3)) * ild)[idx & 7];
+        }
+        if constexpr (MASK) spen[t] = pen[(size_t)bh * L + k0 + t] * LOG2E;
+        __syncthreads();
+        const int kend = k0 + HYB_LL_KEYS;
+#pragma unroll
+        for (int c = 0; c < NR; ++c) {
+            int nn = 8;
+            while (nn == 8) {
+                const int my = e[c] + sub;
+                const int col = my < eend[c] ? ix.r_col[my] : 0x7fffffff;
+                const bool in = col < kend;
+                // columns ascend along the list: the entries of this range among the eight are the first nn
+                nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                if (nn == 0) break;
+                const int lcol = in ? col - k0 : 0;
+                float v = 0.f;
+#define SPION_HYB_QUAD_STEP(KQ)                                                                       \
+    {                                                                                                 \
+        const int ck = hyb_dpp<0x55 * KQ>(lcol);                                                      \
+        const f32x4 a0 = sk[ck * 8 + qi], a1 = sk[ck * 8 + 4 + qi];                                   \
+        float d = a0.x * q0[c].x;                                                                     \
+        d = fmaf(a0.y, q0[c].y, d);                                                                   \
+        d = fmaf(a0.z, q0[c].z, d);                                                                   \
+        d = fmaf(a0.w, q0[c].w, d);                                                                   \
+        d = fmaf(a1.x, q1[c].x, d);                                                                   \
+        d = fmaf(a1.y, q1[c].y, d);                                                                   \
+        d = fmaf(a1.z, q1[c].z, d);                                                                   \
+        d = fmaf(a1.w, q1[c].w, d);                                                                   \
+        d += fdpp(std::integral_constant<int, 0xB1>{}, d);                                            \
+        d += fdpp(std::integral_constant<int, 0x4E>{}, d);                                            \
+        if constexpr (MASK) d -= spen[ck];                                                            \
+        v = qi == KQ ? d : v;                                                                         \
+    }
+                SPION_HYB_QUAD_STEP(0)
+                SPION_HYB_QUAD_STEP(1)
+                SPION_HYB_QUAD_STEP(2)
+                SPION_HYB_QUAD_STEP(3)
+#undef SPION_HYB_QUAD_STEP
+                if (in) raw[my] = v;
+                else v = HYB_ABSENT;
+                float bm = v;
+                bm = fmaxf(bm, fdpp(std::integral_constant<int, 0xB1>{}, bm));
+                bm = fmaxf(bm, fdpp(std::integral_constant<int, 0x4E>{}, bm));
+                bm = fmaxf(bm, fdpp(std::integral_constant<int, 0x141>{}, bm));
+                const float mnew = fmaxf(m[c], bm);
+                float ex = __builtin_amdgcn_exp2f(v - mnew);  // an absent entry gives exactly 0
+                ex += fdpp(std::integral_constant<int, 0xB1>{}, ex);
+                ex += fdpp(std::integral_constant<int, 0x4E>{}, ex);
+                ex += fdpp(std::integral_constant<int, 0x141>{}, ex);
+                z[c] = z[c] * __builtin_amdgcn_exp2f(m[c] - mnew) + ex;
+                m[c] = mnew;
+                e[c] += nn;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+        const int row = rg * ROWS + c * (HYB_LL_THREADS / 8) + grp;
+        if (sub == 0) Stats[(size_t)bh * L + row] = make_float2(m[c], z[c]);
+    }
+}
+
+// -------------------------------------------------------------------------------------------------
+// Forward, step 3, with the V rows in LDS: a work-group of sixteen wavefronts owns 1024 query rows of a head and walks
+// the keys in ranges of 1024, whose V rows (128 KB) it loads once per range.  A group of eight lanes owns eight rows
+// (their {maximum, 1 / denominator} and lane s's 16 bytes of their O rows in registers) and walks each row's remainder
+// entries eight at a time: lane s fetches the s-th entry's raw logit, column and position and writes its probability
+// (through the cache: a row's probabilities leave in pieces of at most eight as the ranges go by), the eight
+// {column, probability} go round the group as in the column pass above.
+// -------------------------------------------------------------------------------------------------
+constexpr int HYB_RL_ROWS = 1024, HYB_RL_KEYS = 1024, HYB_RL_THREADS = 1024;
+template <bool ST>
+__global__ __launch_bounds__(HYB_RL_THREADS) void hyb_rem_pv_lds_kernel(
+    const float* __restrict__ V, const float* __restrict__ Raw, float* __restrict__ P, float* __restrict__ O,
+    float* __restrict__ Ocache, const float2* __restrict__ Stats, HybIndex ix, int L, int NB, int nnz, Layouts ly) {
+    __shared__ f32x4 sv[HYB_RL_KEYS * 8];
+    const int nrg = L / HYB_RL_ROWS;
+    const int item = xcd_remap((int)blockIdx.x, (int)gridDim.x);  // the work-groups of a head share an XCD's L2
+    const int bh = item / nrg, rg = item % nrg;
+    const int t = threadIdx.x, grp = t >> 3, sub = t & 7, lane = t & 63;
+    size_t ib, ob;
+    int ild, old_;
+    hyb_head<ST>(ly.in, ly.H, bh, L, ib, ild);
+    hyb_head<ST>(ly.out, ly.H, bh, L, ob, old_);
+    float* Ph = P + (size_t)bh * nnz;
+    const float* raw = Raw + (size_t)bh * ix.nr;
+    constexpr int NR = HYB_RL_ROWS / (HYB_RL_THREADS / 8);  // rows per lane group: 8
+    f32x4 acc[NR];
+    float2 st[NR];
+    int e[NR], eend[NR];
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+        const int row = rg * HYB_RL_ROWS + c * (HYB_RL_THREADS / 8) + grp;
+        acc[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        st[c] = Stats[(size_t)bh * L + row];
+        e[c] = ix.r_off[row];
+        eend[c] = ix.r_off[row + 1];
+    }
+    for (int k0 = 0; k0 < L; k0 += HYB_RL_KEYS) {
+        __syncthreads();  // everybody has finished with the previous range
+#pragma unroll
+        for (int k = 0; k < HYB_RL_KEYS * 8 / HYB_RL_THREADS; ++k) {
+            const int idx = t + k * HYB_RL_THREADS;
+            sv[idx] = reinterpret_cast<const f32x4*>(V + ib + (size_t)(k0 + (idx >> 3)) * ild)[idx & 7];
+        }
+        __syncthreads();
+        const int kend = k0 + HYB_RL_KEYS;
+#pragma unroll
+        for (int c = 0; c < NR; ++c) {
+            int nn = 8;
+            while (nn == 8) {
+                const int my = e[c] + sub;
+                const int col = my < eend[c] ? ix.r_col[my] : 0x7fffffff;
+                const bool in = col < kend;
+                // columns ascend along the list: the entries of this range among the eight are the first nn
+                nn = __popcll((__ballot(in) >> (lane & 56)) & 0xffull);
+                if (nn == 0) break;
+                float wgt = 0.f;
+                int lcol = 0;
+                if (in) {
+                    wgt = __builtin_amdgcn_exp2f(raw[my] - st[c].x) * st[c].y;
+                    Ph[ix.r_pos[my]] = wgt;
+                    lcol = col - k0;
+                }
+                const int wx = __float_as_int(wgt);
+                const int mcol = hyb_dpp<0x141>(lcol), mx = hyb_dpp<0x141>(wx);
+#define SPION_HYB_ENTRY(CTRL, C, X) acc[c] += sv[hyb_dpp<CTRL>(C) * 8 + sub] * __int_as_float(hyb_dpp<CTRL>(X));
+                SPION_HYB_ENTRY(0x00, lcol, wx)
+                SPION_HYB_ENTRY(0x55, lcol, wx)
+                SPION_HYB_ENTRY(0xaa, lcol, wx)
+                SPION_HYB_ENTRY(0xff, lcol, wx)
+                SPION_HYB_ENTRY(0x00, mcol, mx)
+                SPION_HYB_ENTRY(0x55, mcol, mx)
+                SPION_HYB_ENTRY(0xaa, mcol, mx)
+                SPION_HYB_ENTRY(0xff, mcol, mx)
+#undef SPION_HYB_ENTRY
+                e[c] += nn;
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < NR; ++c) {
+        const int row = rg * HYB_RL_ROWS + c * (HYB_RL_THREADS / 8) + grp;
+        if (eend[c] == ix.r_off[row]) continue;  // a row without remainder entries
+        f32x4* orow = reinterpret_cast<f32x4*>(O + ob + (size_t)row * old_) + sub;
+        const f32x4 sum = *orow + acc[c];
+        *orow = sum;
+        if (Ocache) reinterpret_cast<f32x4*>(Ocache + ((size_t)bh * L + row) * 32)[sub] = sum;  // own copy: contiguous
     }
 }
 

@@ -1420,6 +1420,12 @@ static int hyb_lds_columns(const SparseAttn* a) {
         if ((long long)a->NB * (a->L / (128 * nc)) >= 256) return nc;
     return 0;
 }
+// The same for the forward's logits of the remainder: work-groups of 512 rows (four per lane group; eight need more
+// registers than a wavefront of sixteen has and are no faster), when every CU gets one.
+static bool hyb_lds_rows(const SparseAttn* a) {
+    static const bool gather = getenv("SPION_HYB_GATHER") != nullptr;
+    return !gather && a->L % 1024 == 0 && (long long)a->NB * (a->L / 512) >= 256;
+}
 #define SPION_HYB_COL_LDS(ST_, PAIRS_, NC_, ...)                                                          \
     hipLaunchKernelGGL((hyb_rem_bwd_col_lds_kernel<ST_, PAIRS_, NC_>), dim3(a->NB * (a->L / (128 * NC_))), \
                        dim3(HYB_CL_THREADS), 0, a->hdr.stream, __VA_ARGS__)
@@ -1444,8 +1450,15 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
     const dim3 grid_t(nbr * a->NB), block_t(one ? 64 : 256);
     const dim3 grid_g((unsigned)((rows + HYB_GWAVES - 1) / HYB_GWAVES)), block_g(64 * HYB_GWAVES);
     float2* stats = reinterpret_cast<float2*>(a->ws_stats);
+    const bool lds_logits = hyb_lds_rows(a);
+#define SPION_HYB_LOGITS_LDS(MASKED, NR_)                                                                            \
+    hipLaunchKernelGGL((hyb_rem_logits_lds_kernel<MASKED, ST, NR_>), dim3(a->NB * (a->L / (128 * NR_))),             \
+                       dim3(HYB_LL_THREADS), 0, a->hdr.stream, Q, K, Mask, a->ws_raw, stats, a->pat.hyb, a->L, a->NB, \
+                       a->scale, ly)
 #define SPION_HYB_FWD(MASKED)                                                                                        \
     do {                                                                                                             \
+        if (lds_logits) SPION_HYB_LOGITS_LDS(MASKED, 4);                                                             \
+        else                                                                                                         \
         hipLaunchKernelGGL((hyb_rem_logits_kernel<MASKED, ST>), grid_g, block_g, 0, a->hdr.stream, Q, K, Mask,       \
                            a->ws_raw, stats, a->pat.hyb, a->L, a->NB, a->scale, ly);                                 \
         if (one)                                                                                                     \
@@ -1462,8 +1475,14 @@ static void launch_hyb_fwd(SparseAttn* a, const float* Q, const float* K, const 
     else
         SPION_HYB_FWD(false);
 #undef SPION_HYB_FWD
-    hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, (const float*)a->ws_raw, Attn, Out,
-                       ocopy, (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
+#undef SPION_HYB_LOGITS_LDS
+    if (hyb_lds_columns(a) == 8)  // a full machine of work-groups of 1024 rows: the V rows in LDS
+        hipLaunchKernelGGL(hyb_rem_pv_lds_kernel<ST>, dim3(a->NB * (a->L / HYB_RL_ROWS)), dim3(HYB_RL_THREADS), 0,
+                           a->hdr.stream, V, (const float*)a->ws_raw, Attn, Out, ocopy, (const float2*)stats, a->pat.hyb,
+                           a->L, a->NB, nnz, ly);
+    else
+        hipLaunchKernelGGL(hyb_rem_pv_kernel<ST>, grid_g, block_g, 0, a->hdr.stream, V, (const float*)a->ws_raw, Attn,
+                           Out, ocopy, (const float2*)stats, a->pat.hyb, a->L, a->NB, nnz, ly);
     check_launch("hybrid forward kernels");
 }
 
